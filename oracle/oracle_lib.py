@@ -1,0 +1,161 @@
+"""ctypes front end of the CPU oracles.  TEST INFRASTRUCTURE ONLY.
+
+Only the test-suite, the smoke check and the bench's cpu_baseline leg may import this module; the
+shipped package never does.  The shared objects are built by ``make -C oracle`` (or by
+``__graft_entry__.build()``) from the C++ restatements that sit next to this file.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_i32p = ctypes.POINTER(ctypes.c_int)
+_int = ctypes.c_int
+
+
+def build(force=False):
+    """Compile the oracle shared objects in place."""
+    if force:
+        subprocess.check_call(["make", "-C", _HERE, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", _HERE], stdout=subprocess.DEVNULL)
+
+
+def _load(name):
+    path = os.path.join(_HERE, name)
+    if not os.path.exists(path):
+        build()
+    return ctypes.CDLL(path)
+
+
+def _p32(a):
+    return a.ctypes.data_as(_f32p)
+
+
+def _p64(a):
+    return a.ctypes.data_as(_f64p)
+
+
+def _c(a, dt):
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a
+
+
+class TVOracle:
+    """Huber-TV FISTA inpainting layer, CPU restatement (oracle/tv_oracle.cpp)."""
+
+    def __init__(self):
+        L = self.lib = _load("libtv_oracle.so")
+        L.tv_oracle_forward.argtypes = [_f32p] * 6 + [_int] * 6
+        L.tv_oracle_backward.argtypes = [_f32p] * 10 + [_int] * 6
+        L.tv_oracle_forward_f64.argtypes = [_f64p] * 6 + [_int] * 6
+        L.tv_oracle_backward_f64.argtypes = [_f64p] * 10 + [_int] * 6
+        L.tv_oracle_set_quirks.argtypes = [_int] * 6
+        L.tv_oracle_set_quirks.restype = None
+        L.tv_oracle_reset_id.argtypes = [_int]
+        L.tv_oracle_reset_id.restype = None
+        L.tv_oracle_get_state.argtypes = [_int, _f64p, _int]
+        L.tv_oracle_set_state.argtypes = [_int, _f64p]
+        L.tv_oracle_schedule.argtypes = [_int, _i32p, _i32p]
+        L.tv_oracle_step_sizes.argtypes = [_int, _f32p]
+        L.tv_oracle_step_sizes.restype = None
+        L.tv_oracle_forward_iter.argtypes = [_f32p] * 8 + [_int] * 3 + [ctypes.c_float]
+        L.tv_oracle_forward_iter.restype = None
+        L.tv_oracle_forward_iter_f64.argtypes = [_f64p] * 8 + [_int] * 3 + [ctypes.c_double]
+        L.tv_oracle_forward_iter_f64.restype = None
+        L.tv_oracle_guard_f64.argtypes = [_f64p, ctypes.c_long, _int, _f64p, _f64p]
+        L.tv_oracle_guard_f32.argtypes = [_f32p, ctypes.c_long, _int, _f64p, _f64p]
+        L.tv_oracle_set_threads.argtypes = [_int]
+        L.tv_oracle_set_threads.restype = None
+
+    # -- whole layer ---------------------------------------------------------------------------
+    def forward(self, dx, dy, c, b, init, its, pid=0, f64=False):
+        """dx, dy, c: (N,1,H,W); b, init: (N,C,H,W).  Returns x after the last iteration."""
+        dt = np.float64 if f64 else np.float32
+        dx, dy, c, b, init = (_c(a, dt) for a in (dx, dy, c, b, init))
+        n, ic, ih, iw = b.shape
+        out = np.empty_like(b)
+        P = _p64 if f64 else _p32
+        fn = self.lib.tv_oracle_forward_f64 if f64 else self.lib.tv_oracle_forward
+        rc = fn(P(dx), P(dy), P(c), P(b), P(init), P(out), n, ic, ih, iw, int(its), int(pid))
+        if rc:
+            raise RuntimeError("tv_oracle_forward failed with code %d" % rc)
+        return out
+
+    def backward(self, gin, dx, dy, c, b, its, pid=0, f64=False):
+        """Returns (gx, gy, gc, gb, gi); `gin` (a writable array) is scrubbed in place."""
+        dt = np.float64 if f64 else np.float32
+        dx, dy, c, b = (_c(a, dt) for a in (dx, dy, c, b))
+        if gin.dtype != dt or not gin.flags["C_CONTIGUOUS"]:
+            gin = _c(gin, dt).copy()
+        n, ic, ih, iw = b.shape
+        gx, gy, gc = np.empty_like(dx), np.empty_like(dy), np.empty_like(c)
+        gb, gi = np.empty_like(b), np.empty_like(b)
+        P = _p64 if f64 else _p32
+        fn = self.lib.tv_oracle_backward_f64 if f64 else self.lib.tv_oracle_backward
+        rc = fn(P(dx), P(dy), P(c), P(b), P(gin), P(gx), P(gy), P(gc), P(gb), P(gi), n, ic, ih, iw,
+                int(its), int(pid))
+        if rc:
+            raise RuntimeError("tv_oracle_backward failed with code %d" % rc)
+        return gx, gy, gc, gb, gi
+
+    # -- pieces --------------------------------------------------------------------------------
+    def set_quirks(self, end_uses_ckpt_y=1, skip_iter0_adjoint=1, getyk_rebuild=1, scale_factors=1,
+                   clamp=1, guard=1):
+        self.lib.tv_oracle_set_quirks(end_uses_ckpt_y, skip_iter0_adjoint, getyk_rebuild,
+                                      scale_factors, clamp, guard)
+
+    def reset_id(self, pid):
+        self.lib.tv_oracle_reset_id(int(pid))
+
+    def get_state(self, pid, f64=False):
+        s = np.zeros(6, np.float64)
+        self.lib.tv_oracle_get_state(int(pid), _p64(s), int(f64))
+        return s
+
+    def set_state(self, pid, state6):
+        s = _c(state6, np.float64)
+        self.lib.tv_oracle_set_state(int(pid), _p64(s))
+
+    def schedule(self, its):
+        buf = np.zeros(max(int(np.floor(np.sqrt(its))), 1), np.int32)
+        m = ctypes.c_int(0)
+        n = self.lib.tv_oracle_schedule(int(its), buf.ctypes.data_as(_i32p), ctypes.byref(m))
+        return [int(v) for v in buf[:n]], m.value
+
+    def step_sizes(self, its):
+        out = np.zeros(its, np.float32)
+        self.lib.tv_oracle_step_sizes(int(its), _p32(out))
+        return out
+
+    def forward_iter(self, wx_scaled, wy_scaled, c, b, x, y, t, want_x05=False, f64=False):
+        """One iteration on one sample: fields (H,W) / (C,H,W).  Returns (x_new, y_new[, x05])."""
+        dt = np.float64 if f64 else np.float32
+        wx, wy, c, b, y = (_c(a, dt) for a in (wx_scaled, wy_scaled, c, b, y))
+        x = _c(x, dt).copy()
+        ic, ih, iw = b.shape
+        yout = np.empty_like(y)
+        x05 = np.empty_like(y) if want_x05 else None
+        P = _p64 if f64 else _p32
+        fn = self.lib.tv_oracle_forward_iter_f64 if f64 else self.lib.tv_oracle_forward_iter
+        fn(P(wx), P(wy), P(c), P(b), P(x), P(y), P(yout), P(x05) if want_x05 else None, ic, ih, iw, t)
+        return (x, yout, x05) if want_x05 else (x, yout)
+
+    def guard(self, g, run, av, f32=False):
+        """Output guard on one gradient tensor.  Returns (g_new, av_new, action, stats4)."""
+        g = _c(g, np.float32 if f32 else np.float64).copy().ravel()
+        avv = ctypes.c_double(av)
+        stats = np.zeros(4, np.float64)
+        fn = self.lib.tv_oracle_guard_f32 if f32 else self.lib.tv_oracle_guard_f64
+        act = fn(_p32(g) if f32 else _p64(g), g.size, int(run), ctypes.byref(avv), _p64(stats))
+        return g, avv.value, act, stats
+
+    def set_threads(self, n):
+        self.lib.tv_oracle_set_threads(int(n))
+
+    def max_threads(self):
+        return self.lib.tv_oracle_max_threads()
