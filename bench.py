@@ -1,0 +1,130 @@
+"""Headline benchmark: TV inpainting forward + backward, 4 x 2 x 384 x 1248, 100 FISTA iterations.
+
+One "step" is one forward and one backward call of the layer on the whole batch, inputs resident
+in HBM.  Prints ONE JSON line.  The metric is pixel-iterations per second (one pixel of one sample,
+all channels, advanced through one iteration of the forward and its share of the backward).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes_per_pixel(c):
+    """One HBM round trip per iteration, fp32: forward 5C+3, recompute 6C+3, adjoint 10C+9 floats."""
+    return dict(forward=4 * (5 * c + 3), recompute=4 * (6 * c + 3), adjoint=4 * (10 * c + 9),
+                total=4 * (21 * c + 15))
+
+
+def cpu_baseline(cfg, seconds_hint=20.0):
+    """The CPU oracle on a bounded sample of the same workload: ONE sample of the batch, all
+    iterations, forward + backward, all host cores (best of 2 after a warm-up) and one core."""
+    import numpy as np
+    from customnetworklayers_amd.workloads import tv_inputs
+    from oracle.oracle_lib import TVOracle
+
+    o = TVOracle()
+    o.set_quirks()
+    d = tv_inputs(1, cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    its = cfg["its"]
+    pxit = cfg["h"] * cfg["w"] * 2 * (its // 2)
+
+    def once():
+        o.reset_id(9)
+        t0 = time.perf_counter()
+        o.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], its, 9)
+        o.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], its, 9)
+        return time.perf_counter() - t0
+
+    cores = min(o.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or o.max_threads()))
+    o.set_threads(cores)
+    once()
+    t_all = min(once(), once())
+    o.set_threads(1)
+    t_one = once()
+    o.set_threads(cores)
+    return dict(value=round(pxit / t_all / 1e6, 3), unit="Mpixel-iter/s", cores=cores, kind="port",
+                sample="1 of 4 samples (2x384x1248), 100 iterations, fwd+bwd, best of 2",
+                one_core_value=round(pxit / t_one / 1e6, 3), host_cpu_count=os.cpu_count())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--config", type=int, default=1, help="workload index (1 = headline)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
+              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from customnetworklayers_amd._lib import lib
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+    from customnetworklayers_amd.workloads import CONFIGS, config_inputs
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    cfg, d = config_inputs(args.config, seed=0)
+    assert cfg["kind"] == "tv"
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    its, pid = cfg["its"], 0
+    n, c, h, w = cfg["n"], cfg["c"], cfg["h"], cfg["w"]
+    pxit = n * h * w * 2 * (its // 2)
+
+    def step():
+        (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, pid)
+        return ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, pid)
+
+    ext.reset_id(pid)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.tvinpaint_profile(1)  # HIP events around every launch of the main adjoint kernel
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    tot_ms, launches = ctypes.c_double(0), ctypes.c_int(0)
+    lib.tvinpaint_profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
+    lib.tvinpaint_profile(0)
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = pxit / (elapsed / args.steps) / 1e6
+    bpp = algorithmic_bytes_per_pixel(c)
+    kernel_ms = tot_ms.value / max(launches.value, 1)
+    kernel_bytes = bpp["adjoint"] * n * h * w
+    achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
+    whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9
+    out = {
+        "metric": "TV-FISTA fwd+bwd Mpixel-iter/s at 4x2x384x1248; achieved HBM GB/s vs peak",
+        "value": round(value, 2), "unit": "Mpixel-iter/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "TV inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
+                               % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
+        "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
+                      "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "kernel": "tv_adjoint_iter<false>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "bytes_per_launch": kernel_bytes, "avg_launch_ms": round(kernel_ms, 5),
+                     "launches_timed": launches.value},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,42 @@
+"""Loader of the HIP library behind the layers.  There is no fallback: if the library is missing
+or cannot be loaded the import fails, and the message says how to build it."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libinpaint_hip.so")
+
+_f32p = ctypes.c_void_p  # device pointers travel as integers
+_int = ctypes.c_int
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `make -C %s` (or `python setup.py build_ext`)"
+            % (LIB_PATH, os.path.join(_HERE, "csrc")))
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.tvinpaint_forward.argtypes = [_f32p] * 6 + [_int] * 6 + [ctypes.c_void_p]
+    lib.tvinpaint_backward.argtypes = [_f32p] * 10 + [_int] * 6 + [ctypes.c_void_p]
+    lib.tvinpaint_get_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tvinpaint_set_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tvinpaint_reset_id.argtypes = [_int]
+    lib.tvinpaint_guard_stats.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tvinpaint_slot_bytes.argtypes = [_int]
+    lib.tvinpaint_slot_bytes.restype = ctypes.c_longlong
+    lib.tvinpaint_schedule.argtypes = [_int, ctypes.POINTER(_int), ctypes.POINTER(_int)]
+    lib.tvinpaint_step_sizes.argtypes = [_int, ctypes.POINTER(ctypes.c_float)]
+    lib.tvinpaint_step_sizes.restype = None
+    lib.tvinpaint_guard_decide.argtypes = [_int, ctypes.c_double, ctypes.c_double,
+                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    lib.tvinpaint_profile.argtypes = [_int]
+    lib.tvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
+    lib.tvinpaint_last_error.restype = ctypes.c_char_p
+    return lib
+
+
+lib = _load()
+
+
+def last_error():
+    return lib.tvinpaint_last_error().decode("utf-8", "replace")

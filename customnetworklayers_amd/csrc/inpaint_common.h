@@ -1,0 +1,266 @@
+// Shared host/device plumbing of the TV and TGV inpainting layers: error reporting, the per-id
+// device arena, the checkpoint schedule, and the on-device output guard.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../include/tvinpaint.h"
+
+namespace inpaint {
+
+constexpr int kUniqueIds = 10;        // reference: __uniqueIds__, TVInpaintFista.h:5
+constexpr int kMaxCheckpoints = 100;  // reference: idStruct vectors, TVInpaintFista.h:9-15
+
+// ---------------------------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------------------------
+inline char* error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+#define INPAINT_HIP(call)                                                                      \
+  do {                                                                                         \
+    hipError_t e_ = (call);                                                                    \
+    if (e_ != hipSuccess)                                                                      \
+      return inpaint::fail(INPAINT_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                           __FILE__, __LINE__);                                                \
+  } while (0)
+
+// ---------------------------------------------------------------------------------------------
+// schedule (reference: TVInpaintFista.cu:1499-1508,1523 and 1525-1532; the TGV driver repeats both)
+// ---------------------------------------------------------------------------------------------
+inline void make_schedule(int its, std::vector<int>& iterations, int& max_inter_its) {
+  const double root = std::sqrt((double)its);
+  iterations.assign((size_t)std::floor(root), 0);
+  max_inter_its = 0;
+  for (size_t i = 0; i < iterations.size(); i++) {
+    iterations[i] = (int)(std::floor(i * root * 0.5) * 2);
+    if (i > 0) max_inter_its = std::max(max_inter_its, iterations[i] - iterations[i - 1]);
+  }
+  if (!iterations.empty()) max_inter_its = std::max(max_inter_its, its - iterations.back());
+}
+
+inline void make_step_sizes(int its, std::vector<float>& s) {
+  s.assign((size_t)std::max(its, 0), 0.f);
+  double t = 1, t_ = 1;
+  for (size_t i = 0; i < s.size(); i++) {
+    t_ = t;
+    t = (1. + std::sqrt(1. + 4. * t * t)) / 2.;
+    s[i] = (float)std::max(0.0, (t_ - 1.) / t);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// device arena: one hipMalloc per slot, re-made only when the shape changes
+// ---------------------------------------------------------------------------------------------
+struct Arena {
+  char* base = nullptr;
+  size_t bytes = 0, used = 0;
+  int device = -1;
+  int release() {
+    if (base) {
+      int cur = -1;
+      (void)hipGetDevice(&cur);
+      if (cur != device && device >= 0) (void)hipSetDevice(device);
+      hipError_t e = hipFree(base);
+      if (cur != device && cur >= 0) (void)hipSetDevice(cur);
+      base = nullptr;
+      bytes = used = 0;
+      if (e != hipSuccess) return fail(INPAINT_ERR_HIP, "hipFree failed: %s", hipGetErrorString(e));
+    }
+    return 0;
+  }
+  int reserve(size_t need) {
+    int rc = release();
+    if (rc) return rc;
+    INPAINT_HIP(hipGetDevice(&device));
+    INPAINT_HIP(hipMalloc((void**)&base, need));
+    bytes = need;
+    used = 0;
+    return 0;
+  }
+  template <class T>
+  T* take(size_t count) {
+    size_t off = (used + 255) & ~size_t(255);
+    used = off + count * sizeof(T);
+    return (used <= bytes) ? reinterpret_cast<T*>(base + off) : nullptr;
+  }
+  static size_t padded(size_t count, size_t elem) { return ((count * elem + 255) & ~size_t(255)) + 256; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// output guard (reference: check_gradUpdate + update_correct_av_step_host,
+// TVInpaintFista.cu:128-175; TGV variant TGVInpaintFistaHelp.cu:119-216)
+// ---------------------------------------------------------------------------------------------
+struct GuardParams {
+  double max_tolerance;  // entries above are zeroed (TV) or clamped to +-clamp_to (TGV)
+  double clamp_to;       // 0: zero them
+  double kill_t, scale_t, memory_t;
+};
+
+struct GuardStats {
+  double sum;                        // sum of |g| over finite entries
+  double tail_sum;                   // sum of |g| behind the last non-finite entry
+  unsigned long long max_bits;       // bit pattern of max |g| (non-negative doubles order like integers)
+  unsigned long long last_invalid1;  // 1 + index of the last non-finite entry, 0 if none
+  unsigned int num_above, num_invalid;
+};
+
+struct GuardState {  // lives in device memory, one per id
+  double av[5];      // running means: C, X, Y, B, I
+  double scale[5];   // multiplier chosen for the current backward (1, mult, or 0)
+  double report[25]; // per tensor: mean |g|, max |g|, num_above, num_invalid, action
+  GuardStats stats[5];
+};
+
+// The decision rule, shared by the device kernel and the host-side test hook.
+// Returns 0 plain / 1 rescaled / 2 killed.
+__host__ __device__ inline int guard_decide_rule(int run, double av_gc, double& av_running, double& mult,
+                                                 const GuardParams& p) {
+  const double run_step = fmin(p.memory_t, double(run) / double(run + 1));
+  if (run >= 10 && av_running * p.kill_t < av_gc) {
+    mult = 0.0;
+    av_running = av_running * run_step + (1. - run_step) * p.scale_t * av_running;
+    return 2;
+  }
+  if (run >= 10 && av_running * p.scale_t < av_gc) {
+    mult = p.scale_t * av_running / av_gc;
+    av_running = av_running * run_step + (1. - run_step) * av_gc * mult;
+    return 1;
+  }
+  mult = 1.0;
+  av_running = av_running * run_step + (1. - run_step) * av_gc;
+  return 0;
+}
+
+template <class T>
+__device__ inline bool finite_value(T v) {
+  return (v == v) && (fabs((double)v) <= (sizeof(T) == 4 ? 3.4028234663852886e38 : 1.7976931348623157e308));
+}
+
+__device__ inline double wave_sum(double v) {
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+__device__ inline unsigned long long wave_max(unsigned long long v) {
+  for (int off = 32; off > 0; off >>= 1) {
+    unsigned long long o = __shfl_down(v, off, 64);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+__device__ inline unsigned int wave_sum_u(unsigned int v) {
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+// pass 1: sum, max, counts, position of the last non-finite entry
+template <class T>
+__global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__ g, long long n,
+                                                           GuardStats* __restrict__ st, double max_tol) {
+  double s = 0;
+  unsigned long long mx = 0, last = 0;
+  unsigned int above = 0, invalid = 0;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    T v = g[i];
+    if (finite_value(v)) {
+      double a = fabs((double)v);
+      s += a;
+      unsigned long long bits = (unsigned long long)__double_as_longlong(a);
+      mx = bits > mx ? bits : mx;
+      above += (a > max_tol);
+    } else {
+      invalid++;
+      last = (unsigned long long)(i + 1);
+    }
+  }
+  s = wave_sum(s);
+  mx = wave_max(mx);
+  last = wave_max(last);
+  above = wave_sum_u(above);
+  invalid = wave_sum_u(invalid);
+  if ((threadIdx.x & 63) == 0) {
+    if (s != 0) atomicAdd(&st->sum, s);
+    if (mx) atomicMax(&st->max_bits, mx);
+    if (last) atomicMax(&st->last_invalid1, last);
+    if (above) atomicAdd(&st->num_above, above);
+    if (invalid) atomicAdd(&st->num_invalid, invalid);
+  }
+}
+
+// pass 2 (does nothing unless pass 1 saw a non-finite entry): sum of |g| behind the last one
+template <class T>
+__global__ __launch_bounds__(256) void guard_tail_kernel(const T* __restrict__ g, long long n,
+                                                         GuardStats* __restrict__ st) {
+  if (st->num_invalid == 0) return;
+  const long long start = (long long)st->last_invalid1;
+  double s = 0;
+  for (long long i = start + (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    s += fabs((double)g[i]);
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0 && s != 0) atomicAdd(&st->tail_sum, s);
+}
+
+struct GuardCounts {
+  long long n[5];
+};
+
+// single thread: turn the statistics into per-tensor multipliers and update the running means.
+// Sequential running mean of the reference, av_{i+1} = (|g_i| + i av_i)/(i+1) with a reset to
+// 1000*running mean at every non-finite entry, in closed form.
+__global__ void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, GuardParams p) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  for (int k = 0; k < 5; k++) {
+    GuardStats& s = gs->stats[k];
+    const double n = (double)cnt.n[k];
+    double av_gc;
+    if (cnt.n[k] <= 0) {
+      av_gc = 0;
+    } else if (s.num_invalid == 0) {
+      av_gc = s.sum / n;
+    } else {
+      av_gc = ((double)s.last_invalid1 * (gs->av[k] * 1000.) + s.tail_sum) / n;
+    }
+    double mult = 1.0;
+    int action = guard_decide_rule(run, av_gc, gs->av[k], mult, p);
+    gs->scale[k] = mult;
+    gs->report[5 * k + 0] = av_gc;
+    gs->report[5 * k + 1] = __longlong_as_double((long long)s.max_bits);
+    gs->report[5 * k + 2] = s.num_above;
+    gs->report[5 * k + 3] = s.num_invalid;
+    gs->report[5 * k + 4] = action;
+  }
+}
+
+__global__ void guard_clear_kernel(GuardState* gs) {
+  int k = threadIdx.x;
+  if (k < 5) {
+    GuardStats z;
+    z.sum = 0; z.tail_sum = 0; z.max_bits = 0; z.last_invalid1 = 0; z.num_above = 0; z.num_invalid = 0;
+    gs->stats[k] = z;
+  }
+}
+
+inline int guard_grid(long long n) {
+  long long blocks = (n + 256 * 8 - 1) / (256 * 8);
+  return (int)std::max<long long>(1, std::min<long long>(blocks, 2048));
+}
+
+}  // namespace inpaint

@@ -1,0 +1,791 @@
+// Huber-TV FISTA inpainting layer for MI355X (gfx950): kernels, per-id state and the C ABI.
+//
+// What the layer computes is fixed by the reference's kernels
+// (cudaTV/cudaCode/TVInpaintFista.cu, cited per function below as TV.cu).  How it is computed is not:
+//   * samples are a grid dimension (n >= 1), weights are scaled by L = 1/8 and masked at the image
+//     border when they are staged into LDS (no scaled copies, no textures);
+//   * checkpoints, the x05 history, the adjoint iterates, the per-segment fp32 accumulators and
+//     their fp64 totals all live in one device arena per id, sized once per shape;
+//   * the y rebuild (get_yk) is fused into the adjoint kernel: y_{k+1} is rebuilt straight into
+//     the LDS tile, halo included, and never written to HBM;
+//   * the output guard runs on the device (two reductions, a one-thread decision, a finalize
+//     pass), so a backward call enqueues work and returns without a host synchronisation.
+//
+// Arithmetic contract: every value that can reach a Huber / prox switch (the iterates y, x, x05,
+// the rebuilt y, the triangle norms) is computed with the operation order of the reference source,
+// IEEE division and square root and no fused multiply-add (build with -ffp-contract=off).  At 100
+// iterations a one-ulp deviation there flips a few hundred switches and moves the gradients by
+// ~5e-3 of their maximum, above the layer's 1e-3 tolerance.
+#include "inpaint_common.h"
+
+#include <cstddef>
+
+namespace {
+
+using namespace inpaint;
+
+// TV.cu:44,52,63-69,84-90
+constexpr float kDelta = 0.1f;
+constexpr float kClipLocalGrad = 10000.0f;
+constexpr float kLocalGCMult = 0.1f;
+constexpr float kLocalGXMult = 0.1f;
+constexpr float kLocalGBMult = 1.0f;
+constexpr float kGlobalGMult = 0.1f;
+constexpr float kL = 0.125f;  // 1/Lipschitz, TV.cu:1478 (a power of two: scaling is exact)
+const GuardParams kGuard = {10000000., 0., 50., 10., 0.975};
+
+constexpr int TW = 64;   // tile width  = one wavefront along W
+constexpr int TH = 16;   // tile height
+constexpr int NTY = 4;   // thread rows; each thread owns TH/NTY pixels of one column
+constexpr int NT = TW * NTY;
+constexpr int RPT = TH / NTY;
+constexpr int YS = TW + 2;  // LDS row length of a haloed tile
+
+// -------------------------------------------------------------------------------------------------
+// device helpers
+// -------------------------------------------------------------------------------------------------
+
+// Masked, L-scaled edge weights of the tile whose first interior pixel is (h0, w0), staged with a
+// one-pixel top/left apron.  wxs[ly][lx] = wx(h0-1+ly, w0-1+lx)/8, forced to 0 outside the image and
+// in the last column (no right neighbour); wys likewise with the last row.  With these, the six
+// weights of TV.cu:1204-1211 are plain LDS reads.
+__device__ __forceinline__ void stage_weights(const float* __restrict__ wx, const float* __restrict__ wy,
+                                              float (*wxs)[TW + 1], float (*wys)[TW + 1], int h0, int w0,
+                                              int H, int W, int tid) {
+  for (int e = tid; e < (TH + 1) * (TW + 1); e += NT) {
+    const int ly = e / (TW + 1), lx = e - ly * (TW + 1);
+    const int gh = h0 - 1 + ly, gw = w0 - 1 + lx;
+    const bool in = gh >= 0 && gh < H && gw >= 0 && gw < W;
+    float a = 0.f, b = 0.f;
+    if (in) {
+      const size_t p = (size_t)gh * W + gw;
+      if (gw < W - 1) a = kL * wx[p];
+      if (gh < H - 1) b = kL * wy[p];
+    }
+    wxs[ly][lx] = a;
+    wys[ly][lx] = b;
+  }
+}
+
+// Zero-padded haloed tile of one channel plane (TV.cu:1221-1239).
+__device__ __forceinline__ void stage_plane(const float* __restrict__ f, float (*s)[YS], int h0, int w0,
+                                            int H, int W, int tid) {
+  for (int e = tid; e < (TH + 2) * YS; e += NT) {
+    const int ly = e / YS, lx = e - ly * YS;
+    const int gh = h0 - 1 + ly, gw = w0 - 1 + lx;
+    s[ly][lx] = (gh >= 0 && gh < H && gw >= 0 && gw < W) ? f[(size_t)gh * W + gw] : 0.f;
+  }
+}
+
+// y_{k+1} from x05[k] (xa), x05[k-1] (xb): TV.cu:1149-1165.
+__device__ __forceinline__ float rebuild_y(float bb, float xa, float xb, float conf, float t) {
+  float diff = bb - xa;
+  float sign = (diff < 0) ? -1.f : 1.f;
+  float yk;
+  if (1. + (double)conf >= (double)(sign * diff)) {
+    const float xk = (conf * bb + xa) / (1.f + conf);
+    const float xkm = (conf * bb + xb) / (1.f + conf);
+    yk = xk + t * (xk - xkm);
+  } else {
+    const float xk = (conf <= sign * diff) ? bb - diff + sign * conf : bb;
+    diff = bb - xb;
+    sign = (diff < 0) ? -1.f : 1.f;
+    yk = xk + t * (xk - ((conf <= sign * diff) ? bb - diff + sign * conf : bb));
+  }
+  return yk;
+}
+
+// -------------------------------------------------------------------------------------------------
+// forward iteration: TV.cu:1194-1319; with x05 != nullptr also TV.cu:1321-1455
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(NT) void tv_forward_iter(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
+    const float* __restrict__ b, const float* xin, float* xout, const float* __restrict__ yin,
+    float* __restrict__ yout, float* __restrict__ x05, int C, int H, int W, float t) {
+  __shared__ float ys[TH + 2][YS];
+  __shared__ float wxs[TH + 1][TW + 1];
+  __shared__ float wys[TH + 1][TW + 1];
+  const int tid = threadIdx.y * TW + threadIdx.x;
+  const int w0 = blockIdx.x * TW, h0 = blockIdx.y * TH;
+  const size_t HW = (size_t)H * W;
+  const size_t sample = (size_t)blockIdx.z;
+  wx += sample * HW;
+  wy += sample * HW;
+  cf += sample * HW;
+  const size_t soff = sample * HW * C;
+  stage_weights(wx, wy, wxs, wys, h0, w0, H, W, tid);
+  const int lx = threadIdx.x, w = w0 + lx;
+  float conf[RPT];
+#pragma unroll
+  for (int r = 0; r < RPT; r++) {
+    const int h = h0 + threadIdx.y + r * NTY;
+    conf[r] = (h < H && w < W) ? cf[(size_t)h * W + w] : 0.f;
+  }
+  for (int ch = 0; ch < C; ch++) {
+    const size_t coff = soff + (size_t)ch * HW;
+    if (ch > 0) __syncthreads();
+    stage_plane(yin + coff, ys, h0, w0, H, W, tid);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RPT; r++) {
+      const int ly = threadIdx.y + r * NTY, h = h0 + ly;
+      if (h >= H || w >= W) continue;
+      const size_t q = coff + (size_t)h * W + w;
+      const float wx_0 = wxs[ly + 1][lx], wx_1 = wxs[ly + 1][lx + 1], wx_2 = wxs[ly][lx + 1];
+      const float wy_0 = wys[ly][lx + 1], wy_1 = wys[ly + 1][lx + 1], wy_2 = wys[ly + 1][lx];
+      const float x_ = xin[q];
+      const float bb = b[q];
+      float yc = ys[ly + 1][lx + 1];
+      float yt = yc;
+      if (h > 0) {
+        const float yu = ys[ly][lx + 1], yur = ys[ly][lx + 2];
+        const float hub = sqrtf((yc - yu) * (yc - yu) * wy_0 + (yu - yur) * (yu - yur) * wx_2);
+        yt -= (yc - yu) * (wy_0 / fmaxf(1.f, hub / kDelta));
+      }
+      if (w > 0) {
+        const float yl = ys[ly + 1][lx], yld = ys[ly + 2][lx];
+        const float hub = sqrtf((yc - yl) * (yc - yl) * wx_0 + (yl - yld) * (yl - yld) * wy_2);
+        yt -= (yc - yl) * (wx_0 / fmaxf(1.f, hub / kDelta));
+      }
+      {
+        const float yd = ys[ly + 2][lx + 1], yr = ys[ly + 1][lx + 2];
+        const float hub = sqrtf((yc - yd) * (yc - yd) * wy_1 + (yc - yr) * (yc - yr) * wx_1);
+        const float m = fmaxf(1.f, hub / kDelta);
+        yt -= (yc - yd) * (wy_1 / m);
+        yt -= (yc - yr) * (wx_1 / m);
+      }
+      if (x05) x05[q] = yt;
+      const float c = conf[r];
+      float x_loc = (c * bb + yt) / (1.f + c);
+      yc = yt - c;
+      yt = yt + c;
+      if (yc > 1.f + bb) x_loc = yc;
+      if (yt < bb - 1.f) x_loc = yt;
+      yout[q] = x_loc + t * (x_loc - x_);
+      xout[q] = x_loc;
+    }
+  }
+}
+
+// Prox adjoint + confidence / rhs gradient: TV.cu:806-828 (and 240-255 for the first step).
+// Only g05 continues down the chain; none of these values reaches a switch.
+template <bool FIRST>
+__device__ __forceinline__ void prox_adjoint(float df_dxk, float bb, float x05v, float conf, float& g05,
+                                             float& gc, float& gb) {
+  const float diff = bb - x05v;
+  const float sign = (diff < 0) ? -1.f : 1.f;
+  if (1. + (double)conf >= (double)(sign * diff)) {
+    gc += df_dxk * (bb / (1.f + conf) - (conf * bb + x05v) / ((1.f + conf) * (1.f + conf))) * kLocalGCMult;
+    g05 = df_dxk / (1.f + conf);
+    gb += df_dxk * conf / (1.f + conf) * kLocalGBMult;
+  } else if (FIRST) {
+    g05 = df_dxk;
+    gc += sign * df_dxk * kLocalGCMult;
+    gb = 0.f;  // TV.cu:254
+  } else if (conf >= sign * diff) {  // TV.cu:818-822, unreachable for conf >= 0
+    g05 = 0.f;
+    gb += df_dxk * kLocalGBMult;
+  } else {
+    g05 = df_dxk;
+    gc += sign * df_dxk * kLocalGCMult;
+  }
+}
+
+// First adjoint step: TV.cu:222-287.
+__global__ __launch_bounds__(256) void tv_adjoint_first(const float* __restrict__ cf, const float* __restrict__ b,
+                                                        const float* __restrict__ x05, float* __restrict__ gc,
+                                                        float* __restrict__ gb, float* __restrict__ g05,
+                                                        const float* __restrict__ gin, int C, long long HW,
+                                                        long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // over n*HW pixels
+  if (i >= total) return;
+  const long long s = i / HW, p = i - s * HW;
+  const float conf = cf[i];
+  float gcv = gc[i];
+  for (int ch = 0; ch < C; ch++) {
+    const long long q = (s * C + ch) * HW + p;
+    float g05v, gbv = gb[q];
+    prox_adjoint<true>(gin[q], b[q], x05[q], conf, g05v, gcv, gbv);
+    g05[q] = g05v;
+    gb[q] = gbv;
+  }
+  gc[i] = gcv;
+}
+
+// Main adjoint step with the y rebuild fused in: TV.cu:586-859 (+1130-1189), and, with END, the
+// segment-start variant TV.cu:862-1126 that linearises at the checkpoint y.
+template <bool END>
+__global__ __launch_bounds__(NT) void tv_adjoint_iter(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
+    const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
+    const float* __restrict__ yck, float* __restrict__ gc, float* __restrict__ gb,
+    float* __restrict__ gwx, float* __restrict__ gwy, const float* __restrict__ g05_in,
+    float* __restrict__ g05_out, float* __restrict__ gxk, float* __restrict__ gxk_m1, int C, int H, int W,
+    float t) {
+  __shared__ float ys[TH + 2][YS];
+  __shared__ float gs[TH + 2][YS];
+  __shared__ float wxs[TH + 1][TW + 1];
+  __shared__ float wys[TH + 1][TW + 1];
+  const int tid = threadIdx.y * TW + threadIdx.x;
+  const int w0 = blockIdx.x * TW, h0 = blockIdx.y * TH;
+  const size_t HW = (size_t)H * W;
+  const size_t sample = (size_t)blockIdx.z;
+  wx += sample * HW;
+  wy += sample * HW;
+  cf += sample * HW;
+  gc += sample * HW;
+  gwx += sample * HW;
+  gwy += sample * HW;
+  const size_t soff = sample * HW * C;
+  stage_weights(wx, wy, wxs, wys, h0, w0, H, W, tid);
+  const int lx = threadIdx.x, w = w0 + lx;
+  float conf[RPT], gcv[RPT], gwxv[RPT], gwyv[RPT];
+#pragma unroll
+  for (int r = 0; r < RPT; r++) {
+    const int h = h0 + threadIdx.y + r * NTY;
+    const bool in = h < H && w < W;
+    const size_t p = (size_t)h * W + w;
+    conf[r] = in ? cf[p] : 0.f;
+    gcv[r] = in ? gc[p] : 0.f;
+    gwxv[r] = in ? gwx[p] : 0.f;
+    gwyv[r] = in ? gwy[p] : 0.f;
+  }
+  for (int ch = 0; ch < C; ch++) {
+    const size_t coff = soff + (size_t)ch * HW;
+    if (ch > 0) __syncthreads();
+    if (END) {
+      stage_plane(yck + coff, ys, h0, w0, H, W, tid);
+    } else {
+      for (int e = tid; e < (TH + 2) * YS; e += NT) {
+        const int ly = e / YS, lxx = e - ly * YS;
+        const int gh = h0 - 1 + ly, gw = w0 - 1 + lxx;
+        float v = 0.f;
+        if (gh >= 0 && gh < H && gw >= 0 && gw < W) {
+          const size_t p = (size_t)gh * W + gw;
+          v = rebuild_y(b[coff + p], x05a[coff + p], x05b[coff + p], cf[p], t);
+        }
+        ys[ly][lxx] = v;
+      }
+    }
+    stage_plane(g05_in + coff, gs, h0, w0, H, W, tid);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RPT; r++) {
+      const int ly = threadIdx.y + r * NTY, h = h0 + ly;
+      if (h >= H || w >= W) continue;
+      const size_t q = coff + (size_t)h * W + w;
+      const float wx_0 = wxs[ly + 1][lx], wx_1 = wxs[ly + 1][lx + 1];
+      const float wy_0 = wys[ly][lx + 1], wy_1 = wys[ly + 1][lx + 1];
+      const float yk = ys[ly + 1][lx + 1];
+      const float df_dy = gs[ly + 1][lx + 1];
+      float df_dy_t = df_dy;
+      if (h > 0) {  // triangle owned by the pixel above, TV.cu:655-686
+        const float wx_2 = wxs[ly][lx + 1];
+        const float yu = ys[ly][lx + 1], yur = ys[ly][lx + 2];
+        const float gu = gs[ly][lx + 1], gur = gs[ly][lx + 2];
+        const float wy_nyy2 = (yk - yu) * (yk - yu) * wy_0;
+        const float wx_nyx2 = (yu - yur) * (yu - yur) * wx_2;
+        const float hub = sqrtf(wx_nyx2 + wy_nyy2);
+        if (hub > kDelta) {
+          const float nom = kDelta / hub;
+          const float denom = nom / (2.f * hub * hub);
+          df_dy_t -= (df_dy - gu) * (wy_0 * nom);
+          const float temp = -denom * 2.0f * (yk - yu) * wy_0;
+          df_dy_t -= (df_dy - gu) * wy_0 * (yk - yu) * temp;
+          df_dy_t -= (gur - gu) * wx_2 * (yur - yu) * temp;
+        } else {
+          df_dy_t -= (df_dy - gu) * wy_0;
+        }
+      }
+      if (w > 0) {  // triangle owned by the pixel to the left, TV.cu:687-720
+        const float wy_2 = wys[ly + 1][lx];
+        const float yl = ys[ly + 1][lx], yld = ys[ly + 2][lx];
+        const float gl = gs[ly + 1][lx], gld = gs[ly + 2][lx];
+        const float wx_nyx2 = (yk - yl) * (yk - yl) * wx_0;
+        const float wy_nyy2 = (yl - yld) * (yl - yld) * wy_2;
+        const float hub = sqrtf(wx_nyx2 + wy_nyy2);
+        if (hub > kDelta) {
+          const float nom = kDelta / hub;
+          const float denom = nom / (2.f * hub * hub);
+          df_dy_t -= (df_dy - gl) * (wx_0 * nom);
+          const float temp = -denom * 2.0f * (yk - yl) * wx_0;
+          df_dy_t -= (df_dy - gl) * wx_0 * (yk - yl) * temp;
+          df_dy_t -= (gld - gl) * wy_2 * (yld - yl) * temp;
+        } else {
+          df_dy_t -= (df_dy - gl) * wx_0;
+        }
+      }
+      {  // the pixel's own triangle, TV.cu:722-771
+        const float yr = ys[ly + 1][lx + 2], yd = ys[ly + 2][lx + 1];
+        const float gr = gs[ly + 1][lx + 2], gd = gs[ly + 2][lx + 1];
+        const float wx_nyx2 = (yk - yr) * (yk - yr) * wx_1;
+        const float wy_nyy2 = (yk - yd) * (yk - yd) * wy_1;
+        const float hub = sqrtf(wx_nyx2 + wy_nyy2);
+        if (hub > kDelta) {
+          const float nom = kDelta / hub;
+          const float denom = nom / (2.f * hub * hub);
+          df_dy_t -= (df_dy - gd) * (wy_1 * nom);
+          df_dy_t -= (df_dy - gr) * (wx_1 * nom);
+          const float temp = denom * 2.0f * ((yd - yk) * wy_1 + (yr - yk) * wx_1);
+          df_dy_t -= (df_dy - gd) * wy_1 * (yk - yd) * temp;
+          df_dy_t -= (df_dy - gr) * wx_1 * (yk - yr) * temp;
+          if (!END) {  // TV.cu:749-759
+            if (w < W - 1)
+              gwxv[r] = gwxv[r] - kLocalGXMult * (yk - yr) *
+                                      ((df_dy - gr) * (nom - wx_nyx2 * denom) -
+                                       (df_dy - gd) * (yk - yr) * (yk - yd) * denom * wy_1);
+            if (h < H - 1)
+              gwyv[r] = gwyv[r] - kLocalGXMult * (yk - yd) *
+                                      ((df_dy - gd) * (nom - wy_nyy2 * denom) -
+                                       (df_dy - gr) * (yk - yd) * (yk - yr) * denom * wx_1);
+          } else {  // TV.cu:1019-1027 (same algebra, other operand order)
+            if (w < W - 1)
+              gwxv[r] = gwxv[r] - kLocalGXMult * ((df_dy - gr) * (yk - yr) * (nom - wx_nyx2 * denom) -
+                                                  (df_dy - gd) * (yk - yr) * (yk - yr) * (yk - yd) * denom * wy_1);
+            if (h < H - 1)
+              gwyv[r] = gwyv[r] - kLocalGXMult * ((df_dy - gd) * (yk - yd) * (nom - wy_nyy2 * denom) -
+                                                  (df_dy - gr) * (yk - yd) * (yk - yd) * (yk - yr) * denom * wx_1);
+          }
+        } else {
+          df_dy_t -= (df_dy - gd) * wy_1;
+          df_dy_t -= (df_dy - gr) * wx_1;
+          if (w < W - 1) gwxv[r] = gwxv[r] - kLocalGXMult * (yk - yr) * (df_dy - gr);
+          if (h < H - 1) gwyv[r] = gwyv[r] - kLocalGXMult * (yk - yd) * (df_dy - gd);
+        }
+      }
+      // momentum adjoint, TV.cu:796-801 (the product is formed in double, as the literal 1. implies)
+      float df_dxk = (float)((double)gxk[q] + (1. + (double)t) * (double)df_dy_t);
+      df_dxk = fmaxf(-kClipLocalGrad, fminf(df_dxk, kClipLocalGrad));
+      gxk[q] = df_dxk;
+      gxk_m1[q] = -t * df_dy_t;
+      float g05v, gbv = gb[q];
+      prox_adjoint<false>(df_dxk, b[q], x05a[q], conf[r], g05v, gcv[r], gbv);
+      g05_out[q] = g05v;
+      gb[q] = gbv;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPT; r++) {
+    const int h = h0 + threadIdx.y + r * NTY;
+    if (h < H && w < W) {
+      const size_t p = (size_t)h * W + w;
+      gc[p] = gcv[r];
+      gwx[p] = gwxv[r];
+      gwy[p] = gwyv[r];
+    }
+  }
+}
+
+// Segment flush: fp32 accumulator into its fp64 total, then zero (copy_and_set_to_0, TV.cu:178-218).
+__global__ __launch_bounds__(256) void flush_kernel(float* __restrict__ acc, double* __restrict__ total,
+                                                    long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    total[i] = (double)acc[i] + total[i] / 1.;
+    acc[i] = 0.f;
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_f32(float* __restrict__ p, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    p[i] = 0.f;
+}
+__global__ __launch_bounds__(256) void fill_zero_f64(double* __restrict__ p, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    p[i] = 0.;
+}
+
+// Upstream scrub, in the caller's buffer: TV.cu:1609-1623.
+__global__ __launch_bounds__(256) void scrub_kernel(float* __restrict__ g, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    const float v = g[i];
+    if (!finite_value(v)) g[i] = 0.f;
+  }
+}
+
+// Guarded fp64 total -> fp32 output: TV.cu:160-171 (zeroing), 136/147 (kill / rescale), 1795-1818.
+// `chain` is 1/8 for the edge-weight gradients (TV.cu:1817-1818) and 1 otherwise.
+__global__ __launch_bounds__(256) void finalize_f64(const double* __restrict__ total, float* __restrict__ out,
+                                                    long long n, const GuardState* __restrict__ gs, int k,
+                                                    double chain) {
+  const double mult = gs->scale[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    double v = total[i];
+    if (!finite_value(v) || fabs(v) > kGuard.max_tolerance) v = 0;
+    if (mult != 1.0) v = (mult == 0.0) ? 0.0 : v * mult;
+    const float f = (float)(v * kGlobalGMult);
+    out[i] = (chain == 1.0) ? f : (float)(chain * (double)f);
+  }
+}
+// Gradient wrt init: g_x[1] after the last step (TV.cu:1784-1791,1816), guarded as a float tensor.
+__global__ __launch_bounds__(256) void finalize_f32(const float* __restrict__ src, float* __restrict__ out,
+                                                    long long n, const GuardState* __restrict__ gs, int k) {
+  const double mult = gs->scale[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    float v = src[i];
+    if (!finite_value(v) || fabs((double)v) > kGuard.max_tolerance) v = 0.f;
+    if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
+    out[i] = 0.0f + v;
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// per-id state (idStruct, TVInpaintFista.h:7-50)
+// -------------------------------------------------------------------------------------------------
+struct Slot {
+  int run = 0;
+  int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
+  bool forward_done = false;
+  std::vector<int> iterations;
+  std::vector<float> steps;
+  int max_inter_its = 0;
+  hipStream_t stream = nullptr;
+  Arena arena;
+  // buffers (field = n*ic*ih*iw floats, plane = n*ih*iw)
+  float *ypp[2] = {nullptr, nullptr}, *xwork = nullptr, *ckpt_y = nullptr, *ckpt_x = nullptr, *x05 = nullptr;
+  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr};
+  float *acc_gc = nullptr, *acc_gx = nullptr, *acc_gy = nullptr, *acc_gb = nullptr;
+  double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
+  GuardState* guard = nullptr;      // device
+  double pending_av[5] = {0, 0, 0, 0, 0};  // running means to upload when the arena is (re)made
+  bool have_guard_state = false;
+};
+
+Slot g_slots[kUniqueIds];
+
+// Optional timing of the main adjoint kernel with HIP events on the launch stream.
+struct KernelTimer {
+  bool enabled = false;
+  std::vector<hipEvent_t> pool;  // start/stop pairs
+  size_t used = 0;
+  void mark(hipStream_t stream) {
+    if (!enabled) return;
+    if (used == pool.size()) {
+      hipEvent_t e;
+      if (hipEventCreate(&e) != hipSuccess) { enabled = false; return; }
+      pool.push_back(e);
+    }
+    (void)hipEventRecord(pool[used++], stream);
+  }
+};
+KernelTimer g_timer;
+
+size_t field_count(const Slot& s) { return (size_t)s.n * s.ic * s.ih * s.iw; }
+size_t plane_count(const Slot& s) { return (size_t)s.n * s.ih * s.iw; }
+
+int fetch_running_means(Slot& s) {
+  if (s.guard) {
+    GuardState host;
+    INPAINT_HIP(hipStreamSynchronize(s.stream));
+    INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+    for (int k = 0; k < 5; k++) s.pending_av[k] = host.av[k];
+  }
+  return 0;
+}
+
+int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t stream) {
+  int dev = -1;
+  INPAINT_HIP(hipGetDevice(&dev));
+  const bool same = s.arena.base && s.arena.device == dev && s.n == n && s.ic == ic && s.ih == ih &&
+                    s.iw == iw && s.its == its;
+  s.stream = stream;
+  if (same) return 0;
+  int rc = fetch_running_means(s);  // the running means survive a change of shape
+  if (rc) return rc;
+  s.n = n; s.ic = ic; s.ih = ih; s.iw = iw; s.its = its;
+  make_schedule(its, s.iterations, s.max_inter_its);
+  make_step_sizes(its, s.steps);
+  const size_t F = field_count(s), P = plane_count(s);
+  const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)std::max(s.max_inter_its, 1);
+  size_t need = 0;
+  need += Arena::padded(F, 4) * (2 + 1 + 2 * nck + ring + 2 + 2 + 1);
+  need += Arena::padded(P, 4) * 3;
+  need += Arena::padded(P, 8) * 3 + Arena::padded(F, 8);
+  need += Arena::padded(1, sizeof(GuardState));
+  rc = s.arena.reserve(need);
+  if (rc) return rc;
+  Arena& a = s.arena;
+  s.ypp[0] = a.take<float>(F); s.ypp[1] = a.take<float>(F);
+  s.xwork = a.take<float>(F);
+  s.ckpt_y = a.take<float>(F * nck); s.ckpt_x = a.take<float>(F * nck);
+  s.x05 = a.take<float>(F * ring);
+  s.g05[0] = a.take<float>(F); s.g05[1] = a.take<float>(F);
+  s.gxk[0] = a.take<float>(F); s.gxk[1] = a.take<float>(F);
+  s.acc_gb = a.take<float>(F);
+  s.acc_gc = a.take<float>(P); s.acc_gx = a.take<float>(P); s.acc_gy = a.take<float>(P);
+  s.tot_gc = a.take<double>(P); s.tot_gx = a.take<double>(P); s.tot_gy = a.take<double>(P);
+  s.tot_gb = a.take<double>(F);
+  s.guard = a.take<GuardState>(1);
+  if (!s.guard) return fail(INPAINT_ERR_HIP, "arena layout overflow");
+  GuardState init;
+  memset(&init, 0, sizeof(init));
+  for (int k = 0; k < 5; k++) { init.av[k] = s.pending_av[k]; init.scale[k] = 1.0; }
+  INPAINT_HIP(hipMemcpyAsync(s.guard, &init, sizeof(init), hipMemcpyHostToDevice, stream));
+  INPAINT_HIP(hipStreamSynchronize(stream));  // `init` is a stack object
+  return 0;
+}
+
+inline int grid1d(long long n) { return (int)std::max<long long>(1, std::min<long long>((n + 255) / 256, 1 << 20)); }
+inline int grid_stride(long long n) { return (int)std::max<long long>(1, std::min<long long>((n + 1023) / 1024, 4096)); }
+
+int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int iw, int its, int id) {
+  if (id < 0 || id >= kUniqueIds)
+    return fail(INPAINT_ERR_ID, "Cannot use an id that is negative or larger/equal than the maximal one: %d/%d", id,
+                kUniqueIds);
+  for (int i = 0; i < nptrs; i++)
+    if (!ptrs[i]) return fail(INPAINT_ERR_ARG, "null pointer argument (position %d)", i);
+  if (n < 1 || ic < 1 || ih < 1 || iw < 1 || its < 0)
+    return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
+  if (n > 65535 || (ih + TH - 1) / TH > 65535)
+    return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
+  if ((int)std::floor(std::sqrt((double)its)) > kMaxCheckpoints)
+    return fail(INPAINT_ERR_ITS, "its=%d needs more than %d checkpoints", its, kMaxCheckpoints);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tvinpaint_forward(const float* dx, const float* dy, const float* c, const float* b, const float* init,
+                      float* out, int n, int ic, int ih, int iw, int its, int id, void* stream_) {
+  const void* ptrs[] = {dx, dy, c, b, init, out};
+  int rc = check_common(ptrs, 6, n, ic, ih, iw, its, id);
+  if (rc) return rc;
+  hipStream_t stream = (hipStream_t)stream_;
+  Slot& s = g_slots[id];
+  s.forward_done = false;
+  rc = prepare_slot(s, n, ic, ih, iw, its, stream);
+  if (rc) return rc;
+  const size_t F = field_count(s), FB = F * sizeof(float);
+  const int K = 2 * (its / 2);
+  const dim3 block(TW, NTY), grid((iw + TW - 1) / TW, (ih + TH - 1) / TH, n);
+  // iterate k reads (Y(k), X(k)) and writes (Y(k+1), X(k+1)); a checkpointed iterate lives in its
+  // checkpoint buffer, so no copies are made (the reference copies to the host, TV.cu:1541-1546)
+  auto ck_index = [&](int k) {
+    for (size_t i = 0; i < s.iterations.size(); i++)
+      if (s.iterations[i] == k) return (int)i;
+    return -1;
+  };
+  auto Ybuf = [&](int k) { int i = ck_index(k); return (i >= 0 && k < K) ? s.ckpt_y + (size_t)i * F : s.ypp[k & 1]; };
+  auto Xbuf = [&](int k) {
+    if (k == K) return out;
+    int i = ck_index(k);
+    return i >= 0 ? s.ckpt_x + (size_t)i * F : s.xwork;
+  };
+  if (K == 0) {
+    INPAINT_HIP(hipMemcpyAsync(out, init, FB, hipMemcpyDeviceToDevice, stream));
+    if (!s.iterations.empty()) {  // its == 1: the reference leaves calloc'ed (zero) checkpoints
+      hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, s.ckpt_y, (long long)F);
+      hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, s.ckpt_x, (long long)F);
+    }
+  } else {
+    INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, FB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
+    INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, FB, hipMemcpyDeviceToDevice, stream));
+    for (int k = 0; k < K; k++) {
+      hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k),
+                         Ybuf(k + 1), (float*)nullptr, ic, ih, iw, s.steps[k]);
+    }
+  }
+  INPAINT_HIP(hipGetLastError());
+  s.forward_done = true;
+  return 0;
+}
+
+int tvinpaint_backward(const float* dx, const float* dy, const float* c, const float* b, float* gin, float* gx,
+                       float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih, int iw, int its, int id,
+                       void* stream_) {
+  const void* ptrs[] = {dx, dy, c, b, gin, gx, gy, gc, gb, gi};
+  int rc = check_common(ptrs, 10, n, ic, ih, iw, its, id);
+  if (rc) return rc;
+  hipStream_t stream = (hipStream_t)stream_;
+  Slot& s = g_slots[id];
+  if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
+    return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
+  s.stream = stream;
+  const size_t F = field_count(s), P = plane_count(s);
+  const dim3 block(TW, NTY), grid((iw + TW - 1) / TW, (ih + TH - 1) / TH, n);
+  const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
+
+  hipLaunchKernelGGL(scrub_kernel, dim3(gF), dim3(256), 0, stream, gin, (long long)F);
+  for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.acc_gb})
+    hipLaunchKernelGGL(fill_zero_f32, dim3(gF), dim3(256), 0, stream, p, (long long)F);
+  for (float* p : {s.acc_gc, s.acc_gx, s.acc_gy})
+    hipLaunchKernelGGL(fill_zero_f32, dim3(gP), dim3(256), 0, stream, p, (long long)P);
+  for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy})
+    hipLaunchKernelGGL(fill_zero_f64, dim3(gP), dim3(256), 0, stream, p, (long long)P);
+  hipLaunchKernelGGL(fill_zero_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, (long long)F);
+
+  // buffer roles of TV.cu:1638-1641: g05[0]/g05[1] and gxk[0]/gxk[1] ping-pong with the parity of
+  // the local iteration index; after the last step gxk[1] holds g_x[1]
+  int lastIt = its;
+  const int nseg = (int)s.iterations.size();
+  for (int outer = nseg - 1; outer >= 0; outer--) {
+    const int k0 = s.iterations[outer];
+    const int len = 2 * ((lastIt - k0) / 2);
+    const float* cky = s.ckpt_y + (size_t)outer * F;
+    const float* ckx = s.ckpt_x + (size_t)outer * F;
+    // recompute the segment, keeping x05 (TV.cu:1678-1687)
+    for (int j = 0; j < len; j++) {
+      const float* yin = (j == 0) ? cky : s.ypp[j & 1];
+      const float* xin = (j == 0) ? ckx : s.xwork;
+      hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, xin, s.xwork, yin,
+                         s.ypp[(j + 1) & 1], s.x05 + (size_t)j * F, ic, ih, iw, s.steps[k0 + j]);
+    }
+    // reverse sweep (TV.cu:1696-1729)
+    for (int j = len - 1; j >= 0; j--) {
+      const float t = s.steps[k0 + j];
+      const float* xa = s.x05 + (size_t)j * F;
+      const int odd = j & 1;
+      if (outer == nseg - 1 && j == len - 1) {
+        hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa, s.acc_gc,
+                           s.acc_gb, s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+      } else if (j > 0) {
+        const float* xb = s.x05 + (size_t)(j - 1) * F;
+        g_timer.mark(stream);
+        hipLaunchKernelGGL(tv_adjoint_iter<false>, grid, block, 0, stream, dx, dy, c, b, xa, xb,
+                           (const float*)nullptr, s.acc_gc, s.acc_gb, s.acc_gx, s.acc_gy, s.g05[odd ? 0 : 1],
+                           s.g05[odd ? 1 : 0], s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], ic, ih, iw, t);
+        g_timer.mark(stream);
+      } else {
+        hipLaunchKernelGGL(tv_adjoint_iter<true>, grid, block, 0, stream, dx, dy, c, b, xa, xa, cky, s.acc_gc,
+                           s.acc_gb, s.acc_gx, s.acc_gy, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0], ic, ih, iw, t);
+      }
+    }
+    // fp32 segment sums into the fp64 totals (TV.cu:1730)
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc, s.tot_gc, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gx, s.tot_gx, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gy, s.tot_gy, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb, s.tot_gb, (long long)F);
+    lastIt = k0;
+  }
+
+  // output guard on the device (TV.cu:1760-1791), then scale and store (TV.cu:1795-1818)
+  hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
+  GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
+  const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
+  const long long cnts[5] = {(long long)P, (long long)P, (long long)P, (long long)F, (long long)F};
+  for (int k = 0; k < 4; k++) {
+    hipLaunchKernelGGL(guard_reduce_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k],
+                       cnts[k], st + k, kGuard.max_tolerance);
+    hipLaunchKernelGGL(guard_tail_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k], cnts[k],
+                       st + k);
+  }
+  hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gxk[1], cnts[4],
+                     st + 4, kGuard.max_tolerance);
+  hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gxk[1], cnts[4],
+                     st + 4);
+  GuardCounts gcnt;
+  for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
+  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gc, gc, (long long)P, s.guard, 0, 1.0);
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gx, gx, (long long)P, s.guard, 1, (double)kL);
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gy, gy, (long long)P, s.guard, 2, (double)kL);
+  hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, 1.0);
+  hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gxk[1], gi, (long long)F, s.guard, 4);
+  INPAINT_HIP(hipGetLastError());
+  s.run++;  // TV.cu:1829
+  return 0;
+}
+
+int tvinpaint_get_state(int id, double* state6) {
+  if (id < 0 || id >= kUniqueIds || !state6) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  int rc = fetch_running_means(s);
+  if (rc) return rc;
+  state6[0] = s.run;
+  for (int k = 0; k < 5; k++) state6[1 + k] = s.pending_av[k];
+  return 0;
+}
+
+int tvinpaint_set_state(int id, const double* state6) {
+  if (id < 0 || id >= kUniqueIds || !state6) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  s.run = (int)state6[0];
+  for (int k = 0; k < 5; k++) s.pending_av[k] = state6[1 + k];
+  if (s.guard) {
+    INPAINT_HIP(hipStreamSynchronize(s.stream));
+    INPAINT_HIP(hipMemcpy(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, av), s.pending_av, 5 * sizeof(double),
+                         hipMemcpyHostToDevice));
+  }
+  return 0;
+}
+
+int tvinpaint_reset_id(int id) {
+  if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  if (s.arena.base) (void)hipStreamSynchronize(s.stream);
+  int rc = s.arena.release();
+  s = Slot();
+  return rc;
+}
+
+int tvinpaint_guard_stats(int id, double* stats25) {
+  if (id < 0 || id >= kUniqueIds || !stats25) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  if (!s.guard) return fail(INPAINT_ERR_PAIRING, "id %d holds no state", id);
+  GuardState host;
+  INPAINT_HIP(hipStreamSynchronize(s.stream));
+  INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+  memcpy(stats25, host.report, sizeof(host.report));
+  return 0;
+}
+
+long long tvinpaint_slot_bytes(int id) {
+  if (id < 0 || id >= kUniqueIds) return 0;
+  return (long long)g_slots[id].arena.bytes;
+}
+
+int tvinpaint_schedule(int its, int* iterations_out, int* max_inter_its) {
+  std::vector<int> it;
+  int m = 0;
+  make_schedule(its, it, m);
+  for (size_t i = 0; i < it.size(); i++) iterations_out[i] = it[i];
+  if (max_inter_its) *max_inter_its = m;
+  return (int)it.size();
+}
+
+void tvinpaint_step_sizes(int its, float* out) {
+  std::vector<float> s;
+  make_step_sizes(its, s);
+  for (size_t i = 0; i < s.size(); i++) out[i] = s[i];
+}
+
+int tvinpaint_guard_decide(int run, double av_gc, double av_running, double* mult_out, double* av_out) {
+  double mult = 1.0, av = av_running;
+  int action = guard_decide_rule(run, av_gc, av, mult, kGuard);
+  if (mult_out) *mult_out = mult;
+  if (av_out) *av_out = av;
+  return action;
+}
+
+int tvinpaint_profile(int enable) {
+  g_timer.enabled = enable != 0;
+  g_timer.used = 0;
+  return 0;
+}
+
+int tvinpaint_profile_read(double* total_ms, int* launches) {
+  double total = 0;
+  int count = 0;
+  for (size_t i = 0; i + 1 < g_timer.used; i += 2) {
+    INPAINT_HIP(hipEventSynchronize(g_timer.pool[i + 1]));
+    float ms = 0;
+    INPAINT_HIP(hipEventElapsedTime(&ms, g_timer.pool[i], g_timer.pool[i + 1]));
+    total += ms;
+    count++;
+  }
+  g_timer.used = 0;
+  if (total_ms) *total_ms = total;
+  if (launches) *launches = count;
+  return 0;
+}
+
+const char* tvinpaint_last_error(void) { return error_buffer(); }
+
+}  // extern "C"

@@ -1,0 +1,79 @@
+/* C ABI of the MI355X TV inpainting layer (libinpaint_hip.so).
+ *
+ * Plain pointers and sizes only; every pointer is a device pointer on the current HIP device unless
+ * the parameter says "host".  All tensors are contiguous NCHW float32.  `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream); the calls enqueue work and return without waiting.
+ * Return value 0 = ok; anything else is an error and tvinpaint_last_error() describes it.
+ */
+#ifndef TVINPAINT_H_
+#define TVINPAINT_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Error codes shared by the TV and TGV entry points. */
+#define INPAINT_OK 0
+#define INPAINT_ERR_ID 1        /* id outside [0, 10)            (reference: returns 1, TV.cu:1468-1472) */
+#define INPAINT_ERR_ARG 2       /* null pointer / non-positive size / its out of range                   */
+#define INPAINT_ERR_ITS 3       /* its needs more than 100 checkpoints (reference: TV.h:9-15 overflows)  */
+#define INPAINT_ERR_PAIRING 4   /* backward does not match the forward that filled this id's state       */
+#define INPAINT_ERR_HIP 5       /* a HIP runtime call failed                                             */
+
+/* Replaces TVInpaintFista::forward (cudaTV/cudaCode/TVInpaintFista.h:71-72,
+ * cudaTV/cudaCode/TVInpaintFista.cu:1463-1559), bound by cudaTV/TVInpaintFista_cuda.cpp:47-88.
+ *   dx, dy, c : (n,1,ih,iw) edge weights along W / along H and confidence, read only
+ *   b, init   : (n,ic,ih,iw) right-hand side and starting point, read only
+ *   out       : (n,ic,ih,iw) x after 2*floor(its/2) FISTA iterations
+ *   id        : state slot in [0,10); the matching backward consumes the checkpoints stored here.
+ * n > 1 runs n independent problems (the reference accepts n == 1 only). */
+int tvinpaint_forward(const float* dx, const float* dy, const float* c, const float* b, const float* init,
+                      float* out, int n, int ic, int ih, int iw, int its, int id, void* stream);
+
+/* Replaces TVInpaintFista::backward (TVInpaintFista.h:82-85, TVInpaintFista.cu:1570-1831), bound by
+ * TVInpaintFista_cuda.cpp:99-143.
+ *   gin            : (n,ic,ih,iw) upstream gradient; non-finite entries are zeroed IN PLACE
+ *                    (TVInpaintFista.cu:1609-1623)
+ *   gx, gy, gc     : (n,1,ih,iw) gradients wrt dx, dy, c   (overwritten)
+ *   gb, gi         : (n,ic,ih,iw) gradients wrt b and init (overwritten)
+ * Must follow a tvinpaint_forward with the same shape, its and id. */
+int tvinpaint_backward(const float* dx, const float* dy, const float* c, const float* b, float* gin,
+                       float* gx, float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih,
+                       int iw, int its, int id, void* stream);
+
+/* Per-id state (idStruct, TVInpaintFista.h:7-50).  state6 (host) = {run, av_GC, av_GX, av_GY, av_GB,
+ * av_GI}.  get waits for the slot's stream; reset frees the slot's device buffers as well. */
+int tvinpaint_get_state(int id, double* state6);
+int tvinpaint_set_state(int id, const double* state6);
+int tvinpaint_reset_id(int id);
+
+/* Statistics of the last backward's output guard (check_gradUpdate, TVInpaintFista.cu:158-175), host
+ * array of 5 tensors (C, X, Y, B, I) x {mean |g|, max |g|, count above 1e7, count non-finite,
+ * action (0 plain, 1 rescaled, 2 killed)}.  Waits for the slot's stream. */
+int tvinpaint_guard_stats(int id, double* stats25);
+
+/* Bytes of device memory the slot currently owns (0 if none). */
+long long tvinpaint_slot_bytes(int id);
+
+/* Host-only: checkpoint schedule and FISTA extrapolation factors the layer uses for `its`
+ * (TVInpaintFista.cu:1499-1508,1523 and 1525-1532).  iterations_out holds floor(sqrt(its)) ints. */
+int tvinpaint_schedule(int its, int* iterations_out, int* max_inter_its);
+void tvinpaint_step_sizes(int its, float* out);
+
+/* Host-only: the guard's decision rule for one tensor (update_correct_av_step_host,
+ * TVInpaintFista.cu:128-155).  Returns the action and writes the multiplier and the new running mean. */
+int tvinpaint_guard_decide(int run, double av_gc, double av_running, double* mult_out, double* av_out);
+
+/* Timing of the main adjoint kernel (the dominant one) with HIP events recorded on the launch
+ * stream around every launch.  profile(1) starts collecting, profile_read waits for the recorded
+ * events, returns their summed duration and count and clears the collection. */
+int tvinpaint_profile(int enable);
+int tvinpaint_profile_read(double* total_ms, int* launches);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* tvinpaint_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TVINPAINT_H_ */

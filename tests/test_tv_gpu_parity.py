@@ -1,0 +1,199 @@
+"""GPU parity of the TV layer: the HIP path through the C ABI against the CPU oracle on the same
+seeded inputs.
+
+Tolerances (the layer's contract): max-abs error / max-abs oracle value <= 1e-4 on the inpainted
+flow and <= 1e-3 on the gradients wrt edge weights, confidence, right-hand side and starting point.
+The kernels reproduce the oracle's arithmetic operation by operation, so the observed errors are
+far smaller (the forward iterates are expected to agree bit for bit); the tests print them.
+"""
+import numpy as np
+import pytest
+import torch
+
+from customnetworklayers_amd.workloads import CONFIGS, tv_inputs
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 1e-4
+GRAD_TOL = 1e-3
+
+
+def rel_err(a, ref):
+    return float(np.abs(a.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext
+
+    return tvInpaint_cuda_ext
+
+
+def run_gpu(ext, d, its, pid, fresh=True):
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    if fresh:
+        ext.reset_id(pid)
+    (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, pid)
+    grads = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, pid)
+    torch.cuda.synchronize()
+    return sol.cpu().numpy(), [g.cpu().numpy() for g in grads], t["grad"].cpu().numpy()
+
+
+def run_oracle(o, d, its, pid, fresh=True):
+    if fresh:
+        o.reset_id(pid)
+    sol = o.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], its, pid)
+    gin = d["grad"].copy()
+    grads = o.backward(gin, d["dx"], d["dy"], d["dc"], d["db"], its, pid)
+    return sol, list(grads), gin
+
+
+def compare(name, got, ref):
+    sol, grads, _ = got
+    rsol, rgrads, _ = ref
+    e_out = rel_err(sol, rsol)
+    errs = [rel_err(g, r) for g, r in zip(grads, rgrads)]
+    exact = float((sol == rsol).mean())
+    print("\n[%s] out rel %.2e (bit-equal %.4f)  gx %.2e gy %.2e gc %.2e gb %.2e gi %.2e"
+          % (name, e_out, exact, *errs), flush=True)
+    assert e_out <= OUT_TOL, (name, e_out)
+    for nm, e in zip(("gx", "gy", "gc", "gb", "gi"), errs):
+        assert e <= GRAD_TOL, (name, nm, e)
+    return e_out, errs
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 2, 64, 128, 20),    # the reference's own single-sample case
+    (1, 1, 16, 64, 2),      # a single pair of iterations, tile-exact
+    (2, 3, 37, 101, 9),     # ragged tiles, odd its, three channels, two samples
+    (1, 2, 5, 3, 6),        # smaller than one tile
+    (1, 2, 1, 70, 4),       # a single row
+    (1, 1, 33, 1, 4),       # a single column
+    (3, 2, 130, 200, 50),   # several segments of unequal length
+])
+def test_forward_backward_match_oracle(ext, tv_oracle, n, c, h, w, its):
+    d = tv_inputs(n, c, h, w, seed=n * 1000 + h + w + its, conf_density=0.3)
+    print("case n=%d c=%d h=%d w=%d its=%d" % (n, c, h, w, its), flush=True)
+    compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2))
+
+
+def test_its_zero_and_one_return_init_and_zero_grads(ext, tv_oracle):
+    d = tv_inputs(1, 2, 20, 30, seed=5)
+    for its in (0, 1):
+        sol, grads, _ = run_gpu(ext, d, its, 3)
+        np.testing.assert_array_equal(sol, d["di"])
+        rsol, rgrads, _ = run_oracle(tv_oracle, d, its, 3)
+        for g, r in zip(grads, rgrads):
+            np.testing.assert_array_equal(g, r)
+            assert not g.any()
+
+
+def test_rectangles_and_dense_confidence(ext, tv_oracle):
+    # the stress configuration's generators at a size the oracle finishes quickly
+    d = tv_inputs(2, 2, 96, 160, seed=4, flow="rectangles", dense_conf=True)
+    compare("rectangles", run_gpu(ext, d, 60, 1), run_oracle(tv_oracle, d, 60, 1))
+
+
+def test_headline_shape_one_sample(ext, tv_oracle):
+    # one sample of the headline configuration (2 x 384 x 1248, 100 iterations)
+    cfg = CONFIGS[1]
+    d = tv_inputs(1, cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    compare("headline/1", run_gpu(ext, d, cfg["its"], 0), run_oracle(tv_oracle, d, cfg["its"], 0))
+
+
+def test_upstream_scrub_is_in_place_and_matches(ext, tv_oracle):
+    d = tv_inputs(1, 2, 40, 50, seed=6)
+    d["grad"][0, 1, 7, 9] = np.nan
+    d["grad"][0, 0, 0, 0] = np.inf
+    got = run_gpu(ext, d, 12, 4)
+    ref = run_oracle(tv_oracle, d, 12, 4)
+    np.testing.assert_array_equal(got[2], ref[2])  # scrubbed upstream tensors agree
+    assert got[2][0, 1, 7, 9] == 0 and got[2][0, 0, 0, 0] == 0
+    compare("scrub", got, ref)
+
+
+def test_ids_are_independent_and_nest(ext, tv_oracle):
+    # forward on ids 0,1,2 then backward 2,1,0 (the hierarchy's calling pattern)
+    dev = torch.device("cuda:0")
+    cases = [tv_inputs(1, 2, 24 * (i + 1), 40 * (i + 1), seed=30 + i) for i in range(3)]
+    its = 10
+    tens = [{k: torch.from_numpy(v).to(dev) for k, v in d.items()} for d in cases]
+    for i in range(3):
+        ext.reset_id(i)
+        tv_oracle.reset_id(i)
+    sols = [ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, i)[0] for i, t in enumerate(tens)]
+    grads = {}
+    for i in (2, 1, 0):
+        t = tens[i]
+        grads[i] = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, i)
+    torch.cuda.synchronize()
+    for i, d in enumerate(cases):
+        ref = run_oracle(tv_oracle, d, its, i)
+        compare("id%d" % i, (sols[i].cpu().numpy(), [g.cpu().numpy() for g in grads[i]], None), ref)
+
+
+def test_guard_rescales_and_kills_like_the_oracle(ext, tv_oracle):
+    d = tv_inputs(1, 2, 32, 48, seed=8)
+    its = 8
+    # learn what the plain gradient means are
+    base = run_gpu(ext, d, its, 5)
+    means = [float(np.abs(g).mean()) for g in base[1]]
+    stats = ext.guard_stats(5)
+    assert all(row[4] == 0 for row in stats)
+    # running means 20x below (C: rescale), 60x below (X: kill), equal (others), after 10 runs.
+    # the guard sees the values before the global 0.1 (and the 1/8 of the edge weights)
+    f = float(np.float32(0.1))
+    pre = [means[2] / f, means[0] / f * 8, means[1] / f * 8, means[3] / f, means[4]]  # C, X, Y, B, I
+    state = [10, pre[0] / 20, pre[1] / 60, pre[2], pre[3], pre[4]]
+    ext.set_state(5, state)
+    tv_oracle.reset_id(5)
+    tv_oracle.set_state(5, state)
+    got = run_gpu(ext, d, its, 5, fresh=False)
+    ref = run_oracle(tv_oracle, d, its, 5, fresh=False)
+    stats = ext.guard_stats(5)
+    assert [int(r[4]) for r in stats] == [1, 2, 0, 0, 0]
+    assert not got[1][0].any()  # gx killed
+    np.testing.assert_allclose(got[1][2], base[1][2] * 0.5, rtol=1e-5, atol=0)  # gc halved
+    compare("guard", got, ref)
+    gs, os_ = ext.get_state(5), tv_oracle.get_state(5)
+    np.testing.assert_allclose(gs, os_, rtol=1e-9)
+    assert gs[0] == 11
+
+
+def test_errors(ext):
+    dev = torch.device("cuda:0")
+    d = {k: torch.from_numpy(v).to(dev) for k, v in tv_inputs(1, 2, 8, 8, seed=1).items()}
+    with pytest.raises(IndexError):
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 4, 10)
+    with pytest.raises(IndexError):
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 4, -1)
+    with pytest.raises(TypeError):
+        ext.forward(d["dx"].double(), d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(RuntimeError):
+        ext.forward(d["dx"].cpu(), d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(RuntimeError):
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"].permute(0, 1, 3, 2), d["di"], 4, 0)
+    ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(RuntimeError):  # its differs from the forward that filled the slot
+        ext.backward(d["grad"], d["dx"], d["dy"], d["dc"], d["db"], 6, 0)
+    with pytest.raises(ValueError):
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 10201 + 300, 0)
+
+
+def test_module_surface_and_autograd(ext, tv_oracle):
+    from customnetworklayers_amd import TVInpaint
+
+    dev = torch.device("cuda:0")
+    d = tv_inputs(1, 2, 30, 44, seed=9)
+    hwc = lambda a: torch.from_numpy(np.ascontiguousarray(a[0].transpose(1, 2, 0))).to(dev).requires_grad_(True)
+    tx, ty, tc, tb, ti = (hwc(d[k]) for k in ("dx", "dy", "dc", "db", "di"))
+    layer = TVInpaint(dev, 14, pid=6)
+    ext.reset_id(6)
+    sol = layer(tx, ty, tc, tb, ti)
+    assert tuple(sol.shape) == (30, 44, 2)
+    up = torch.from_numpy(np.ascontiguousarray(d["grad"][0].transpose(1, 2, 0))).to(dev)
+    sol.backward(up)
+    ref = run_oracle(tv_oracle, d, 14, 6)
+    got_grads = [t.grad.permute(2, 0, 1).unsqueeze(0).cpu().numpy() for t in (tx, ty, tc, tb, ti)]
+    compare("module", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
