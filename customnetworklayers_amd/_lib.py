@@ -31,6 +31,7 @@ def _load():
                                            ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_profile.argtypes = [_int]
     lib.tvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
+    lib.inpaint_selftest_math.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_uint]
     lib.tvinpaint_last_error.restype = ctypes.c_char_p
     return lib
 

@@ -225,7 +225,7 @@ struct GuardCounts {
 // single thread: turn the statistics into per-tensor multipliers and update the running means.
 // Sequential running mean of the reference, av_{i+1} = (|g_i| + i av_i)/(i+1) with a reset to
 // 1000*running mean at every non-finite entry, in closed form.
-__global__ void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, GuardParams p) {
+static __global__ void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, GuardParams p) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   for (int k = 0; k < 5; k++) {
     GuardStats& s = gs->stats[k];
@@ -249,7 +249,7 @@ __global__ void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, Gu
   }
 }
 
-__global__ void guard_clear_kernel(GuardState* gs) {
+static __global__ void guard_clear_kernel(GuardState* gs) {
   int k = threadIdx.x;
   if (k < 5) {
     GuardStats z;

@@ -1,0 +1,69 @@
+// On-device check of the cheap correctly-rounded division / square root against the compiler's
+// IEEE expansions.  Diagnostic entry point of the library, used by the GPU test-suite.
+#include "exact_math.h"
+#include "inpaint_common.h"
+
+namespace {
+
+using namespace inpaint;
+
+__device__ inline bool same_bits(float a, float b) {
+  return (__float_as_uint(a) == __float_as_uint(b)) || (a != a && b != b);
+}
+
+__device__ inline unsigned int mix(unsigned int x) {  // integer hash, good enough to spread operands
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+
+// counts[0]: sqrt over every float in [2^-96, FLT_MAX] plus 0
+// counts[1]: x / 0.1f over 0 and every float in [2^-96, 2^96]
+// counts[2]: n / d on hashed pairs, d in [2^-6, 2^40), |n| in [2^-60, 2^60) or 0, plus structured
+//            denominators (all-ones and single-bit mantissas)
+// counts[3]: shared-reciprocal form, two numerators per denominator in [1, 2^24)
+__global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* counts, unsigned int pair_rounds) {
+  const unsigned int tid = blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned int stride = gridDim.x * blockDim.x;
+  unsigned int bad0 = 0, bad1 = 0, bad2 = 0, bad3 = 0;
+  for (unsigned long long i = tid; i < 0x7f800000ULL; i += stride) {
+    const float x = __uint_as_float((unsigned int)i);
+    if (x == 0.f || x >= 1.2621774e-29f) bad0 += !same_bits(exact_sqrt(x), sqrtf(x));
+    if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) bad1 += !same_bits(exact_div(x, 0.1f), x / 0.1f);
+  }
+  for (unsigned int k = 0; k < pair_rounds; k++) {
+    const unsigned int h1 = mix(tid * 2654435761U + k * 40503U + 17U), h2 = mix(h1 ^ 0x9e3779b9U);
+    // denominator: exponent in [-6, 40), mantissa hashed / structured
+    unsigned int mant = h1 & 0x7fffffU;
+    if ((k & 7) == 1) mant = 0x7fffffU;
+    if ((k & 7) == 2) mant = 1U << (h1 % 23U);
+    if ((k & 7) == 3) mant = 0x7fffffU ^ (1U << (h1 % 23U));
+    const unsigned int dexp = 127U - 6U + ((h1 >> 23) % 46U);
+    const float d = __uint_as_float((dexp << 23) | mant);
+    const unsigned int nexp = 127U - 60U + ((h2 >> 23) % 120U);
+    float n = __uint_as_float((h2 & 0x80000000U) | (nexp << 23) | (h2 & 0x7fffffU));
+    if ((k & 63) == 5) n = 0.f;
+    bad2 += !same_bits(exact_div(n, d), n / d);
+    const float d1 = __uint_as_float(((127U + ((h1 >> 23) % 24U)) << 23) | mant);
+    const float r = rcp_refined(d1);
+    const float n2 = __uint_as_float(((127U - 20U + ((h2 >> 8) % 24U)) << 23) | (h1 & 0x7fffffU));
+    bad3 += !same_bits(div_by(n, d1, r), n / d1);
+    bad3 += !same_bits(div_by(n2, d1, r), n2 / d1);
+  }
+  if (bad0) atomicAdd(&counts[0], (unsigned long long)bad0);
+  if (bad1) atomicAdd(&counts[1], (unsigned long long)bad1);
+  if (bad2) atomicAdd(&counts[2], (unsigned long long)bad2);
+  if (bad3) atomicAdd(&counts[3], (unsigned long long)bad3);
+}
+
+}  // namespace
+
+extern "C" int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds) {
+  unsigned long long* dev = nullptr;
+  INPAINT_HIP(hipMalloc((void**)&dev, 4 * sizeof(unsigned long long)));
+  INPAINT_HIP(hipMemset(dev, 0, 4 * sizeof(unsigned long long)));
+  hipLaunchKernelGGL(selftest_kernel, dim3(4096), dim3(256), 0, 0, dev, pair_rounds);
+  INPAINT_HIP(hipGetLastError());
+  INPAINT_HIP(hipMemcpy(mismatches4_host, dev, 4 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+  INPAINT_HIP(hipFree(dev));
+  return 0;
+}

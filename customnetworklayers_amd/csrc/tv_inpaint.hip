@@ -17,8 +17,10 @@
 // iterations a one-ulp deviation there flips a few hundred switches and moves the gradients by
 // ~5e-3 of their maximum, above the layer's 1e-3 tolerance.
 #include "inpaint_common.h"
+#include "tv_strip_kernels.h"
 
 #include <cstddef>
+#include <cstdlib>
 
 namespace {
 
@@ -548,6 +550,79 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
   return 0;
 }
 
+// -------------------------------------------------------------------------------------------------
+// kernel selection: wave-strip kernels when the width is a multiple of 4 and every pointer is
+// 16-byte aligned (float4 rows), the LDS-tile kernels otherwise.  INPAINT_TV_PATH=tile forces the
+// tile kernels (used by the tests to keep both paths covered).
+// -------------------------------------------------------------------------------------------------
+bool force_tile_path() {
+  const char* e = getenv("INPAINT_TV_PATH");
+  return e && strcmp(e, "tile") == 0;
+}
+bool aligned16(std::initializer_list<const void*> ptrs) {
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & 15) return false;
+  return true;
+}
+int strip_rows(int n, int ih, int iw) {
+  // rows per wavefront: as tall as possible while the launch still holds >= 2 wavefronts per SIMD
+  const long long sx = (iw + tvstrip::kStripCols - 1) / tvstrip::kStripCols;
+  for (int R : {32, 16, 8}) {
+    const long long waves = sx * ((ih + R - 1) / R) * n;
+    if (waves >= 2 * 1024) return R;
+  }
+  return 4;
+}
+
+void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                    const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
+                    float t) {
+  const bool strip = !force_tile_path() && (s.iw % 4 == 0) && aligned16({dx, dy, c, b, xin, xout, yin, yout, x05});
+  if (strip) {
+    constexpr int R = 4;
+    const int sx = (s.iw + tvstrip::kStripCols - 1) / tvstrip::kStripCols, sy = (s.ih + R - 1) / R;
+    const long long waves = (long long)sx * sy * s.n;
+    hipLaunchKernelGGL(tvstrip::tv_forward_strip<R>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, dx, dy,
+                       c, b, xin, xout, yin, yout, x05, s.n, s.ic, s.ih, s.iw, t, sx, sy);
+  } else {
+    const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
+    hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05, s.ic, s.ih,
+                       s.iw, t);
+  }
+}
+
+template <int C, bool END>
+void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                          const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
+                          float* g05_out, float* gxk, float* gxk_m1, float t) {
+  const int R = strip_rows(s.n, s.ih, s.iw);
+  const int sx = (s.iw + tvstrip::kStripCols - 1) / tvstrip::kStripCols, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, dx,
+                     dy, c, b, xa, xb, yck, s.acc_gc, s.acc_gb, s.acc_gx, s.acc_gy, g05_in, g05_out, gxk, gxk_m1, s.n,
+                     s.ih, s.iw, t, R, sx, sy);
+}
+
+template <bool END>
+void launch_adjoint(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                    const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
+                    float* g05_out, float* gxk, float* gxk_m1, float t) {
+  const bool strip = !force_tile_path() && (s.iw % 4 == 0) && s.ic >= 1 && s.ic <= 4 &&
+                     aligned16({dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1});
+  if (strip) {
+    switch (s.ic) {
+      case 1: launch_adjoint_strip<1, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
+      case 2: launch_adjoint_strip<2, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
+      case 3: launch_adjoint_strip<3, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
+      default: launch_adjoint_strip<4, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
+    }
+  } else {
+    const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
+    hipLaunchKernelGGL(tv_adjoint_iter<END>, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc, s.acc_gb,
+                       s.acc_gx, s.acc_gy, g05_in, g05_out, gxk, gxk_m1, s.ic, s.ih, s.iw, t);
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -564,7 +639,6 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   if (rc) return rc;
   const size_t F = field_count(s), FB = F * sizeof(float);
   const int K = 2 * (its / 2);
-  const dim3 block(TW, NTY), grid((iw + TW - 1) / TW, (ih + TH - 1) / TH, n);
   // iterate k reads (Y(k), X(k)) and writes (Y(k+1), X(k+1)); a checkpointed iterate lives in its
   // checkpoint buffer, so no copies are made (the reference copies to the host, TV.cu:1541-1546)
   auto ck_index = [&](int k) {
@@ -588,8 +662,7 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, FB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, FB, hipMemcpyDeviceToDevice, stream));
     for (int k = 0; k < K; k++) {
-      hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k),
-                         Ybuf(k + 1), (float*)nullptr, ic, ih, iw, s.steps[k]);
+      launch_forward(s, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
     }
   }
   INPAINT_HIP(hipGetLastError());
@@ -609,7 +682,6 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
   s.stream = stream;
   const size_t F = field_count(s), P = plane_count(s);
-  const dim3 block(TW, NTY), grid((iw + TW - 1) / TW, (ih + TH - 1) / TH, n);
   const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
 
   hipLaunchKernelGGL(scrub_kernel, dim3(gF), dim3(256), 0, stream, gin, (long long)F);
@@ -634,8 +706,8 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     for (int j = 0; j < len; j++) {
       const float* yin = (j == 0) ? cky : s.ypp[j & 1];
       const float* xin = (j == 0) ? ckx : s.xwork;
-      hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, xin, s.xwork, yin,
-                         s.ypp[(j + 1) & 1], s.x05 + (size_t)j * F, ic, ih, iw, s.steps[k0 + j]);
+      launch_forward(s, stream, dx, dy, c, b, xin, s.xwork, yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * F,
+                     s.steps[k0 + j]);
     }
     // reverse sweep (TV.cu:1696-1729)
     for (int j = len - 1; j >= 0; j--) {
@@ -648,13 +720,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       } else if (j > 0) {
         const float* xb = s.x05 + (size_t)(j - 1) * F;
         g_timer.mark(stream);
-        hipLaunchKernelGGL(tv_adjoint_iter<false>, grid, block, 0, stream, dx, dy, c, b, xa, xb,
-                           (const float*)nullptr, s.acc_gc, s.acc_gb, s.acc_gx, s.acc_gy, s.g05[odd ? 0 : 1],
-                           s.g05[odd ? 1 : 0], s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], ic, ih, iw, t);
+        launch_adjoint<false>(s, stream, dx, dy, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
+                              s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], t);
         g_timer.mark(stream);
       } else {
-        hipLaunchKernelGGL(tv_adjoint_iter<true>, grid, block, 0, stream, dx, dy, c, b, xa, xa, cky, s.acc_gc,
-                           s.acc_gb, s.acc_gx, s.acc_gy, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0], ic, ih, iw, t);
+        launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0], t);
       }
     }
     // fp32 segment sums into the fp64 totals (TV.cu:1730)

@@ -70,6 +70,11 @@ int tvinpaint_guard_decide(int run, double av_gc, double av_running, double* mul
 int tvinpaint_profile(int enable);
 int tvinpaint_profile_read(double* total_ms, int* launches);
 
+/* Diagnostic: compares the library's cheap correctly-rounded division / square root with the
+ * compiler's IEEE expansions on the GPU (exhaustively over single floats, on `pair_rounds` hashed
+ * pairs per thread otherwise) and returns the four mismatch counts (host array).  All must be 0. */
+int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds);
+
 /* Text of the last error on the calling thread ("" if none). */
 const char* tvinpaint_last_error(void);
 
