@@ -169,10 +169,13 @@ __device__ inline unsigned int wave_sum_u(unsigned int v) {
   return v;
 }
 
-// pass 1: sum, max, counts, position of the last non-finite entry
+// pass 1: sum, max, counts, position of the last non-finite entry.  One set of atomics per block.
 template <class T>
 __global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__ g, long long n,
                                                            GuardStats* __restrict__ st, double max_tol) {
+  __shared__ double s_sum[4];
+  __shared__ unsigned long long s_mx[4], s_last[4];
+  __shared__ unsigned int s_above[4], s_invalid[4];
   double s = 0;
   unsigned long long mx = 0, last = 0;
   unsigned int above = 0, invalid = 0;
@@ -195,7 +198,19 @@ __global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__
   last = wave_max(last);
   above = wave_sum_u(above);
   invalid = wave_sum_u(invalid);
+  const int wv = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) {
+    s_sum[wv] = s; s_mx[wv] = mx; s_last[wv] = last; s_above[wv] = above; s_invalid[wv] = invalid;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 4; k++) {
+      s += s_sum[k];
+      mx = s_mx[k] > mx ? s_mx[k] : mx;
+      last = s_last[k] > last ? s_last[k] : last;
+      above += s_above[k];
+      invalid += s_invalid[k];
+    }
     if (s != 0) atomicAdd(&st->sum, s);
     if (mx) atomicMax(&st->max_bits, mx);
     if (last) atomicMax(&st->last_invalid1, last);
@@ -259,8 +274,8 @@ static __global__ void guard_clear_kernel(GuardState* gs) {
 }
 
 inline int guard_grid(long long n) {
-  long long blocks = (n + 256 * 8 - 1) / (256 * 8);
-  return (int)std::max<long long>(1, std::min<long long>(blocks, 2048));
+  long long blocks = (n + 256 * 16 - 1) / (256 * 16);
+  return (int)std::max<long long>(1, std::min<long long>(blocks, 1024));
 }
 
 }  // namespace inpaint

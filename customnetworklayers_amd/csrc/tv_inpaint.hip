@@ -220,9 +220,9 @@ template <bool END>
 __global__ __launch_bounds__(NT) void tv_adjoint_iter(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
-    const float* __restrict__ yck, float* __restrict__ gc, float* __restrict__ gb,
-    float* __restrict__ gwx, float* __restrict__ gwy, const float* __restrict__ g05_in,
-    float* __restrict__ g05_out, float* __restrict__ gxk, float* __restrict__ gxk_m1, int C, int H, int W,
+    const float* __restrict__ yck, const float* gc_in, float* gc, const float* gb_in, float* gb,
+    const float* gwx_in, float* gwx, const float* gwy_in, float* gwy, const float* __restrict__ g05_in,
+    float* __restrict__ g05_out, const float* gxk, float* gxk_m1, float* gx_final, int C, int H, int W,
     float t) {
   __shared__ float ys[TH + 2][YS];
   __shared__ float gs[TH + 2][YS];
@@ -238,6 +238,9 @@ __global__ __launch_bounds__(NT) void tv_adjoint_iter(
   gc += sample * HW;
   gwx += sample * HW;
   gwy += sample * HW;
+  gc_in += sample * HW;
+  gwx_in += sample * HW;
+  gwy_in += sample * HW;
   const size_t soff = sample * HW * C;
   stage_weights(wx, wy, wxs, wys, h0, w0, H, W, tid);
   const int lx = threadIdx.x, w = w0 + lx;
@@ -248,9 +251,9 @@ __global__ __launch_bounds__(NT) void tv_adjoint_iter(
     const bool in = h < H && w < W;
     const size_t p = (size_t)h * W + w;
     conf[r] = in ? cf[p] : 0.f;
-    gcv[r] = in ? gc[p] : 0.f;
-    gwxv[r] = in ? gwx[p] : 0.f;
-    gwyv[r] = in ? gwy[p] : 0.f;
+    gcv[r] = in ? gc_in[p] : 0.f;
+    gwxv[r] = in ? gwx_in[p] : 0.f;
+    gwyv[r] = in ? gwy_in[p] : 0.f;
   }
   for (int ch = 0; ch < C; ch++) {
     const size_t coff = soff + (size_t)ch * HW;
@@ -358,9 +361,9 @@ __global__ __launch_bounds__(NT) void tv_adjoint_iter(
       // momentum adjoint, TV.cu:796-801 (the product is formed in double, as the literal 1. implies)
       float df_dxk = (float)((double)gxk[q] + (1. + (double)t) * (double)df_dy_t);
       df_dxk = fmaxf(-kClipLocalGrad, fminf(df_dxk, kClipLocalGrad));
-      gxk[q] = df_dxk;
+      if (gx_final) gx_final[q] = df_dxk;  // only the last step's g_x is ever read again (TV.cu:800,1785)
       gxk_m1[q] = -t * df_dy_t;
-      float g05v, gbv = gb[q];
+      float g05v, gbv = gb_in[q];
       prox_adjoint<false>(df_dxk, b[q], x05a[q], conf[r], g05v, gcv[r], gbv);
       g05_out[q] = g05v;
       gb[q] = gbv;
@@ -397,6 +400,19 @@ __global__ __launch_bounds__(256) void fill_zero_f64(double* __restrict__ p, lon
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (long long)gridDim.x * blockDim.x)
     p[i] = 0.;
+}
+
+// Zero several buffers in one launch (blockIdx.y picks the buffer).
+struct ZeroList {
+  void* ptr[16];
+  long long bytes[16];
+};
+__global__ __launch_bounds__(256) void fill_zero_many(ZeroList z) {
+  uint32_t* p = static_cast<uint32_t*>(z.ptr[blockIdx.y]);
+  const long long n = z.bytes[blockIdx.y] / 4;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    p[i] = 0u;
 }
 
 // Upstream scrub, in the caller's buffer: TV.cu:1609-1623.
@@ -449,9 +465,12 @@ struct Slot {
   hipStream_t stream = nullptr;
   Arena arena;
   // buffers (field = n*ic*ih*iw floats, plane = n*ih*iw)
-  float *ypp[2] = {nullptr, nullptr}, *xwork = nullptr, *ckpt_y = nullptr, *ckpt_x = nullptr, *x05 = nullptr;
-  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr};
-  float *acc_gc = nullptr, *acc_gx = nullptr, *acc_gy = nullptr, *acc_gb = nullptr;
+  float *ypp[2] = {nullptr, nullptr}, *xpp[2] = {nullptr, nullptr}, *ckpt_y = nullptr, *ckpt_x = nullptr, *x05 = nullptr;
+  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr}, *gx_final = nullptr;
+  // per-segment fp32 accumulators, double-buffered: every adjoint step reads one set and writes the other
+  float *acc_gc[2] = {nullptr, nullptr}, *acc_gx[2] = {nullptr, nullptr}, *acc_gy[2] = {nullptr, nullptr},
+        *acc_gb[2] = {nullptr, nullptr};
+  int acc_cur = 0;
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
   GuardState* guard = nullptr;      // device
   double pending_av[5] = {0, 0, 0, 0, 0};  // running means to upload when the arena is (re)made
@@ -505,21 +524,23 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   const size_t F = field_count(s), P = plane_count(s);
   const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)std::max(s.max_inter_its, 1);
   size_t need = 0;
-  need += Arena::padded(F, 4) * (2 + 1 + 2 * nck + ring + 2 + 2 + 1);
-  need += Arena::padded(P, 4) * 3;
+  need += Arena::padded(F, 4) * (2 + 2 + 2 * nck + ring + 2 + 2 + 1 + 2);
+  need += Arena::padded(P, 4) * 6;
   need += Arena::padded(P, 8) * 3 + Arena::padded(F, 8);
   need += Arena::padded(1, sizeof(GuardState));
   rc = s.arena.reserve(need);
   if (rc) return rc;
   Arena& a = s.arena;
   s.ypp[0] = a.take<float>(F); s.ypp[1] = a.take<float>(F);
-  s.xwork = a.take<float>(F);
+  s.xpp[0] = a.take<float>(F); s.xpp[1] = a.take<float>(F);
   s.ckpt_y = a.take<float>(F * nck); s.ckpt_x = a.take<float>(F * nck);
   s.x05 = a.take<float>(F * ring);
   s.g05[0] = a.take<float>(F); s.g05[1] = a.take<float>(F);
-  s.gxk[0] = a.take<float>(F); s.gxk[1] = a.take<float>(F);
-  s.acc_gb = a.take<float>(F);
-  s.acc_gc = a.take<float>(P); s.acc_gx = a.take<float>(P); s.acc_gy = a.take<float>(P);
+  s.gxk[0] = a.take<float>(F); s.gxk[1] = a.take<float>(F); s.gx_final = a.take<float>(F);
+  for (int i = 0; i < 2; i++) {
+    s.acc_gb[i] = a.take<float>(F);
+    s.acc_gc[i] = a.take<float>(P); s.acc_gx[i] = a.take<float>(P); s.acc_gy[i] = a.take<float>(P);
+  }
   s.tot_gc = a.take<double>(P); s.tot_gx = a.take<double>(P); s.tot_gy = a.take<double>(P);
   s.tot_gb = a.take<double>(F);
   s.guard = a.take<GuardState>(1);
@@ -551,39 +572,56 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
 }
 
 // -------------------------------------------------------------------------------------------------
-// kernel selection: wave-strip kernels when the width is a multiple of 4 and every pointer is
-// 16-byte aligned (float4 rows), the LDS-tile kernels otherwise.  INPAINT_TV_PATH=tile forces the
-// tile kernels (used by the tests to keep both paths covered).
+// kernel selection: wave-strip kernels for 1..4 channels, the LDS-tile kernels otherwise.
+// INPAINT_TV_PATH=tile forces the tile kernels (used by the tests to keep both paths covered).
 // -------------------------------------------------------------------------------------------------
 bool force_tile_path() {
   const char* e = getenv("INPAINT_TV_PATH");
   return e && strcmp(e, "tile") == 0;
 }
-bool aligned16(std::initializer_list<const void*> ptrs) {
-  for (const void* p : ptrs)
-    if (reinterpret_cast<uintptr_t>(p) & 15) return false;
-  return true;
-}
-int strip_rows(int n, int ih, int iw) {
-  // rows per wavefront: as tall as possible while the launch still holds >= 2 wavefronts per SIMD
-  const long long sx = (iw + tvstrip::kStripCols - 1) / tvstrip::kStripCols;
-  for (int R : {32, 16, 8}) {
-    const long long waves = sx * ((ih + R - 1) / R) * n;
-    if (waves >= 2 * 1024) return R;
+int strip_rows(int n, int ih, int iw, int cols, const char* env_name) {
+  // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap
+  // between strips, but the launch should still put about two wavefronts on each of the 1024 SIMDs
+  // (measured on the 4 x 2 x 384 x 1248 workload: 16 rows beat 8 and 24).
+  if (const char* e = getenv(env_name)) {
+    const int v = atoi(e);
+    if (v >= 1 && v <= 4096) return v;
   }
-  return 4;
+  const long long sx = (iw + cols - 1) / cols;
+  for (int R : {16, 12, 8, 6, 4, 3}) {
+    const long long waves = sx * ((ih + R - 1) / R) * n;
+    if (waves >= 1792) return R;
+  }
+  return 2;
+}
+
+template <int C>
+void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                          const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
+                          float t) {
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwdCols, "INPAINT_TV_FWD_ROWS");
+  const int sx = (s.iw + tvstrip::kFwdCols - 1) / tvstrip::kFwdCols, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
+  if (x05)
+    hipLaunchKernelGGL((tvstrip::tv_forward_strip<C, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
+                       x05, s.n, s.ih, s.iw, t, R, sx, sy);
+  else
+    hipLaunchKernelGGL((tvstrip::tv_forward_strip<C, false>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin,
+                       yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
 }
 
 void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
                     float t) {
-  const bool strip = !force_tile_path() && (s.iw % 4 == 0) && aligned16({dx, dy, c, b, xin, xout, yin, yout, x05});
+  const bool strip = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
   if (strip) {
-    constexpr int R = 4;
-    const int sx = (s.iw + tvstrip::kStripCols - 1) / tvstrip::kStripCols, sy = (s.ih + R - 1) / R;
-    const long long waves = (long long)sx * sy * s.n;
-    hipLaunchKernelGGL(tvstrip::tv_forward_strip<R>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, dx, dy,
-                       c, b, xin, xout, yin, yout, x05, s.n, s.ic, s.ih, s.iw, t, sx, sy);
+    switch (s.ic) {
+      case 1: launch_forward_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
+      case 2: launch_forward_strip<2>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
+      case 3: launch_forward_strip<3>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
+      default: launch_forward_strip<4>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
+    }
   } else {
     const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
     hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05, s.ic, s.ih,
@@ -594,33 +632,46 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const fl
 template <int C, bool END>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                           const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
-                          float* g05_out, float* gxk, float* gxk_m1, float t) {
-  const int R = strip_rows(s.n, s.ih, s.iw);
-  const int sx = (s.iw + tvstrip::kStripCols - 1) / tvstrip::kStripCols, sy = (s.ih + R - 1) / R;
+                          float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, "INPAINT_TV_ADJ_ROWS");
+  const int sx = (s.iw + tvstrip::kAdjCols - 1) / tvstrip::kAdjCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
-  hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, dx,
-                     dy, c, b, xa, xb, yck, s.acc_gc, s.acc_gb, s.acc_gx, s.acc_gy, g05_in, g05_out, gxk, gxk_m1, s.n,
-                     s.ih, s.iw, t, R, sx, sy);
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
+  if (gx_final)
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, true>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
+                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih, s.iw, t, R, sx,
+                       sy);
+  else
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, false>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
+                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih, s.iw, t, R, sx,
+                       sy);
 }
 
+// One adjoint step: reads accumulator set acc_cur, writes the other one, then flips acc_cur.
 template <bool END>
-void launch_adjoint(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+bool launch_adjoint(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
-                    float* g05_out, float* gxk, float* gxk_m1, float t) {
-  const bool strip = !force_tile_path() && (s.iw % 4 == 0) && s.ic >= 1 && s.ic <= 4 &&
-                     aligned16({dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1});
+                    float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
+  const bool strip = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
   if (strip) {
     switch (s.ic) {
-      case 1: launch_adjoint_strip<1, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
-      case 2: launch_adjoint_strip<2, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
-      case 3: launch_adjoint_strip<3, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
-      default: launch_adjoint_strip<4, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, t); break;
+      case 1: launch_adjoint_strip<1, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      case 2: launch_adjoint_strip<2, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      case 3: launch_adjoint_strip<3, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      default: launch_adjoint_strip<4, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
     }
   } else {
     const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
-    hipLaunchKernelGGL(tv_adjoint_iter<END>, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc, s.acc_gb,
-                       s.acc_gx, s.acc_gy, g05_in, g05_out, gxk, gxk_m1, s.ic, s.ih, s.iw, t);
+    const int i = s.acc_cur, o = 1 - s.acc_cur;
+    hipLaunchKernelGGL(tv_adjoint_iter<END>, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc[i],
+                       s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in,
+                       g05_out, gxk, gxk_m1, gx_final, s.ic, s.ih, s.iw, t);
   }
+  s.acc_cur = 1 - s.acc_cur;
+  return strip;
 }
 
 }  // namespace
@@ -650,7 +701,7 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   auto Xbuf = [&](int k) {
     if (k == K) return out;
     int i = ck_index(k);
-    return i >= 0 ? s.ckpt_x + (size_t)i * F : s.xwork;
+    return i >= 0 ? s.ckpt_x + (size_t)i * F : s.xpp[k & 1];
   };
   if (K == 0) {
     INPAINT_HIP(hipMemcpyAsync(out, init, FB, hipMemcpyDeviceToDevice, stream));
@@ -685,28 +736,34 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
 
   hipLaunchKernelGGL(scrub_kernel, dim3(gF), dim3(256), 0, stream, gin, (long long)F);
-  for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.acc_gb})
-    hipLaunchKernelGGL(fill_zero_f32, dim3(gF), dim3(256), 0, stream, p, (long long)F);
-  for (float* p : {s.acc_gc, s.acc_gx, s.acc_gy})
-    hipLaunchKernelGGL(fill_zero_f32, dim3(gP), dim3(256), 0, stream, p, (long long)P);
-  for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy})
-    hipLaunchKernelGGL(fill_zero_f64, dim3(gP), dim3(256), 0, stream, p, (long long)P);
-  hipLaunchKernelGGL(fill_zero_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, (long long)F);
+  s.acc_cur = 0;
+  {
+    ZeroList z;
+    int k = 0;
+    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.gx_final, s.acc_gb[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)F * 4; }
+    for (float* p : {s.acc_gc[0], s.acc_gx[0], s.acc_gy[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 4; }
+    for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 8; }
+    z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
+    hipLaunchKernelGGL(fill_zero_many, dim3(gF, k), dim3(256), 0, stream, z);
+  }
 
   // buffer roles of TV.cu:1638-1641: g05[0]/g05[1] and gxk[0]/gxk[1] ping-pong with the parity of
-  // the local iteration index; after the last step gxk[1] holds g_x[1]
+  // the local iteration index.  A step reads the partial g_x[k+1] from one gxk buffer and writes the
+  // partial g_x[k] to the other; the completed g_x[k+1] itself is only ever read after the very last
+  // step (TV.cu:800 calls its store a debugging aid), so only that step stores it, into gx_final.
   int lastIt = its;
   const int nseg = (int)s.iterations.size();
   for (int outer = nseg - 1; outer >= 0; outer--) {
     const int k0 = s.iterations[outer];
     const int len = 2 * ((lastIt - k0) / 2);
+    bool flushed = false;
     const float* cky = s.ckpt_y + (size_t)outer * F;
     const float* ckx = s.ckpt_x + (size_t)outer * F;
     // recompute the segment, keeping x05 (TV.cu:1678-1687)
     for (int j = 0; j < len; j++) {
       const float* yin = (j == 0) ? cky : s.ypp[j & 1];
-      const float* xin = (j == 0) ? ckx : s.xwork;
-      launch_forward(s, stream, dx, dy, c, b, xin, s.xwork, yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * F,
+      const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
+      launch_forward(s, stream, dx, dy, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * F,
                      s.steps[k0 + j]);
     }
     // reverse sweep (TV.cu:1696-1729)
@@ -715,23 +772,28 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       const float* xa = s.x05 + (size_t)j * F;
       const int odd = j & 1;
       if (outer == nseg - 1 && j == len - 1) {
-        hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa, s.acc_gc,
-                           s.acc_gb, s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+        hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
+                           s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = s.x05 + (size_t)(j - 1) * F;
         g_timer.mark(stream);
         launch_adjoint<false>(s, stream, dx, dy, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
-                              s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], t);
+                              s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
         g_timer.mark(stream);
       } else {
-        launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0], t);
+        // the very last step's g_x[k+1] is the gradient wrt the starting point (TV.cu:1785,1816)
+        flushed = launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
+                                       outer == 0 ? s.gx_final : nullptr, t);
       }
     }
-    // fp32 segment sums into the fp64 totals (TV.cu:1730)
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc, s.tot_gc, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gx, s.tot_gx, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gy, s.tot_gy, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb, s.tot_gb, (long long)F);
+    // fp32 segment sums into the fp64 totals (TV.cu:1730); the strip kernel of the segment's first
+    // iteration has already done it
+    if (!flushed) {
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[s.acc_cur], s.tot_gc, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gx[s.acc_cur], s.tot_gx, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gy[s.acc_cur], s.tot_gy, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[s.acc_cur], s.tot_gb, (long long)F);
+    }
     lastIt = k0;
   }
 
@@ -746,9 +808,9 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     hipLaunchKernelGGL(guard_tail_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k], cnts[k],
                        st + k);
   }
-  hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gxk[1], cnts[4],
+  hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gx_final, cnts[4],
                      st + 4, kGuard.max_tolerance);
-  hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gxk[1], cnts[4],
+  hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gx_final, cnts[4],
                      st + 4);
   GuardCounts gcnt;
   for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
@@ -757,7 +819,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gx, gx, (long long)P, s.guard, 1, (double)kL);
   hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gy, gy, (long long)P, s.guard, 2, (double)kL);
   hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, 1.0);
-  hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gxk[1], gi, (long long)F, s.guard, 4);
+  hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gx_final, gi, (long long)F, s.guard, 4);
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TV.cu:1829
   return 0;

@@ -1,17 +1,27 @@
-// Wave-strip kernels of the TV layer: the fast path for image widths that are a multiple of 4.
+// Wave-strip kernels of the TV layer (the default path for up to 4 channels).
 //
-// One wavefront owns a strip of kStripCols output columns x R rows of one sample and runs without
-// LDS and without barriers.  Each lane holds 4 consecutive pixels of a row (float4 loads and
-// stores); lane 0 is an apron lane that covers the 4 columns left of the strip and only supplies
-// its triangle terms to lane 1.  Rows are walked top to bottom, starting one row above the strip.
+// One wavefront owns a strip of one sample: 64 adjacent columns (one pixel per lane) by R rows, and
+// walks it top to bottom without LDS and without barriers.  Lane 0 is an apron lane: it covers the
+// column left of the strip and only feeds its triangle terms to lane 1 (the adjoint kernel also
+// uses lane 63 as an apron on the right, because there a pixel's right neighbour is a rebuilt
+// value and not a plain load).  Neighbouring lanes exchange values with wave-wide DPP shifts.
 //
-// The reference evaluates, per pixel, the Huber weights of the three triangles the pixel belongs
-// to.  The triangle owned by pixel q enters q, q's right neighbour and q's lower neighbour with
-// bit-identical operands (the two squared differences are symmetric under negation and their sum
-// commutes), so here the owner computes the weight once and passes it on: down the column in
-// registers, to the right through one cross-lane move per row.  Results are bit-identical to the
-// per-pixel evaluation; the work per pixel drops from 3 sqrt + 8 div to 1 sqrt + 3 div.
+// Row streaming: row k (k = 0 is the row above the strip) is needed as the "next" row of step k-1
+// and as the "current" row of step k.  Four row buffers rotate, so while step k computes, the loads
+// of rows k+2 and k+3 are in flight; the loop body is four steps with the roles rotated, so no
+// registers are copied.  A row buffer is 4C+4 registers, which keeps the kernels at several
+// wavefronts per SIMD: the layer's images are small for this chip (about 7 rows of work per
+// lane at 1 pixel per lane), so occupancy, not per-lane reuse, is what hides memory latency.
+//
+// Triangle sharing: the reference evaluates, per pixel, the Huber weights of the three triangles
+// the pixel belongs to.  The triangle owned by pixel q enters q, q's right neighbour and q's lower
+// neighbour with bit-identical operands (squared differences are symmetric under negation, their
+// sum commutes), so the owner computes each term once and hands it on: down the column in
+// registers, to the right through a DPP shift.  Results are bit-identical to the per-pixel
+// evaluation; per pixel the work drops from 3 sqrt + 8 div to 1 sqrt + 3 div (forward).
 #pragma once
+
+#include <type_traits>
 
 #include "exact_math.h"
 
@@ -21,202 +31,236 @@ using inpaint::div_by;
 using inpaint::exact_sqrt;
 using inpaint::rcp_refined;
 
-constexpr int kLanePx = 4;
-constexpr int kStripCols = 63 * kLanePx;  // 252 output columns per wavefront (lane 0 is the apron)
-constexpr float kDelta = 0.1f;            // TV.cu:44
-constexpr float kL = 0.125f;              // TV.cu:1478
+constexpr int kFwdCols = 63;      // output columns per wavefront, forward (lane 0 is the apron)
+constexpr int kAdjCols = 62;      // adjoint (lanes 0 and 63 are aprons)
+constexpr float kDelta = 0.1f;    // TV.cu:44
+constexpr float kL = 0.125f;      // TV.cu:1478
+constexpr float kClipLocalGrad = 10000.0f;  // TV.cu:52
+constexpr float kLocalGCMult = 0.1f;        // TV.cu:63
+constexpr float kLocalGXMult = 0.1f;        // TV.cu:65
 
-struct F4 {
-  float v[4];
-};
-
-__device__ __forceinline__ F4 load4(const float* __restrict__ p, bool ok) {
-  F4 r;
-  if (ok) {
-    const float4 t = *reinterpret_cast<const float4*>(p);
-    r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
-  } else {
-    r.v[0] = r.v[1] = r.v[2] = r.v[3] = 0.f;
-  }
-  return r;
+// value of the lane to the left / right; lanes without a source receive 0
+__device__ __forceinline__ float from_left_lane(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x138, 0xf, 0xf, false));  // wave_shr:1
 }
-__device__ __forceinline__ void store4(float* __restrict__ p, const F4& a) {
-  *reinterpret_cast<float4*>(p) = make_float4(a.v[0], a.v[1], a.v[2], a.v[3]);
+__device__ __forceinline__ float from_right_lane(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));  // wave_shl:1
 }
 
-// value held by the lane to the left (lane 0 gets its own back; it is the apron and never uses it)
-__device__ __forceinline__ float from_left_lane(float v, int bperm_addr) {
-  return __int_as_float(__builtin_amdgcn_ds_bpermute(bperm_addr, __float_as_int(v)));
+// element `off_bytes / 4` of a wave-uniform plane: the byte offset is a 32-bit VGPR that is zero-extended
+// and added to the SGPR base by the load / store itself
+__device__ __forceinline__ float ldg(const float* base, unsigned off_bytes) {
+  return *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) + off_bytes);
+}
+__device__ __forceinline__ void stg(float* base, unsigned off_bytes, float v) {
+  *reinterpret_cast<float*>(reinterpret_cast<char*>(base) + off_bytes) = v;
 }
 
 struct StripGeom {
-  int lane, w_first, hs, n;
-  bool col_ok, store_lane;
-  int bperm_left;
+  int lane, w, hs, n;  // w: this lane's column, hs: first output row, n: sample (hs, n wave-uniform)
+  bool col_ok;
 };
 
-__device__ __forceinline__ bool strip_geometry(StripGeom& g, int R, int W, int strips_x, int strips_y, int N) {
-  const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+// The row loop is kept a straight line: loads are unconditional (clamped addresses) and stores sit in
+// blocks small enough to be predicated rather than branched around.  A load or store behind a
+// branch makes the compiler assume the path without it and drain the prefetched rows at every step.
+
+__device__ __forceinline__ bool strip_geometry(StripGeom& g, int cols, int R, int W, int strips_x, int strips_y,
+                                               int N) {
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Neighbouring strips share
+  // halo rows, the apron column and split cache lines, so strips are numbered such that every XCD
+  // works through one contiguous band of the image: workgroup b serves logical block
+  // (b % 8) * (gridDim.x / 8) + b / 8 (the grid is a multiple of 8 workgroups).
+  const int per_xcd = gridDim.x >> 3;
+  const int logical_block = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int wave = __builtin_amdgcn_readfirstlane(logical_block * (blockDim.x >> 6) + (threadIdx.x >> 6));
   g.lane = threadIdx.x & 63;
   const int sx = wave % strips_x;
   const int rest = wave / strips_x;
   const int sy = rest % strips_y;
   g.n = rest / strips_y;
   if (g.n >= N) return false;
-  g.w_first = sx * kStripCols - kLanePx + kLanePx * g.lane;
+  g.w = sx * cols - 1 + g.lane;
   g.hs = sy * R;
-  g.col_ok = g.w_first >= 0 && g.w_first < W;
-  g.store_lane = g.lane > 0 && g.col_ok;
-  g.bperm_left = ((g.lane + 63) & 63) << 2;
+  g.col_ok = g.w >= 0 && g.w < W;
   return true;
 }
 
+// -------------------------------------------------------------------------------------------------
 // Forward iteration, TV.cu:1194-1319 (and 1321-1455 when x05 is given).
-template <int R>
+//
+// Per triangle (owner q) the two products
+//     E1 = (y_q - y_down) * (wy / m),   E2 = (y_q - y_right) * (wx / m),   m = max(1, |.|_q / delta)
+// are formed once; q subtracts both, the pixel below q subtracts -E1 and the pixel right of q
+// subtracts -E2, which are the reference's four updates with identical operands
+// ((y_p - y_up) * q = -(y_up - y_p) * q exactly).
+// -------------------------------------------------------------------------------------------------
+template <int C>
+struct FwdRow {
+  float y[C], yr[C], x[C], bb[C], c, rc1, wxs, wys;
+};
+
+template <int C, bool X05>
 __global__ __launch_bounds__(256) void tv_forward_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
-    const float* __restrict__ b, const float* xin, float* xout, const float* __restrict__ yin,
-    float* __restrict__ yout, float* __restrict__ x05, int N, int C, int H, int W, float t, int strips_x,
-    int strips_y) {
+    const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
+    const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05,
+    int N, int H, int W, float t, int R, int strips_x, int strips_y) {
   StripGeom g;
-  if (!strip_geometry(g, R, W, strips_x, strips_y, N)) return;
+  if (!strip_geometry(g, kFwdCols, R, W, strips_x, strips_y, N)) return;
   const size_t HW = (size_t)H * W;
-  const float* wxp = wx + (size_t)g.n * HW;
-  const float* wyp = wy + (size_t)g.n * HW;
-  const float* cfp = cf + (size_t)g.n * HW;
-  const int w0 = g.w_first;
-  const bool left_ok = w0 - 1 >= 0 && w0 - 1 < W;
-  const bool right_ok = w0 + kLanePx >= 0 && w0 + kLanePx < W;
-
-  // masked, L-scaled weights of rows hs-1 .. hs+R-1, confidence of rows hs .. hs+R-1
-  F4 wxs[R + 1], wys[R + 1], conf[R];
-  float rc1[R][4];  // refined reciprocal of 1 + c
+  const unsigned W4 = 4u * (unsigned)W;           // row pitch in bytes
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;   // clamped column (bytes): every address below is valid
+  const bool right_ok = g.w + 1 < W;
+  const unsigned wr = right_ok ? 4u * (g.w + 1) : 0u;
+  const bool store_lane = g.lane > 0 && g.col_ok;
+  const bool wx_ok = g.col_ok && g.w < W - 1;
+  const int Reff = min(R, H - g.hs);  // output rows of this strip (the last strip may be ragged)
+  // wave-uniform plane pointers + 32-bit element offsets: loads and stores take an SGPR base and a
+  // VGPR offset, so no 64-bit address arithmetic is done per access
+  const float* const wx_p = wx + (size_t)g.n * HW;
+  const float* const wy_p = wy + (size_t)g.n * HW;
+  const float* const cf_p = cf + (size_t)g.n * HW;
+  const float *y_p[C], *x_p[C], *b_p[C];
+  float *yo_p[C], *xo_p[C], *xh_p[C];
 #pragma unroll
-  for (int r = 0; r <= R; r++) {
-    const int h = g.hs - 1 + r;
-    const bool ok = g.col_ok && h >= 0 && h < H;
-    const size_t off = (size_t)(ok ? h : 0) * W + (ok ? w0 : 0);
-    wxs[r] = load4(wxp + off, ok);
-    wys[r] = load4(wyp + off, ok && h < H - 1);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      wxs[r].v[j] = (w0 + j < W - 1) ? kL * wxs[r].v[j] : 0.f;
-      wys[r].v[j] = kL * wys[r].v[j];
-    }
-    if (r > 0) {
-      conf[r - 1] = load4(cfp + off, ok);
-#pragma unroll
-      for (int j = 0; j < 4; j++) rc1[r - 1][j] = rcp_refined(1.f + conf[r - 1].v[j]);
-    }
+  for (int ch = 0; ch < C; ch++) {
+    const size_t q = ((size_t)g.n * C + ch) * HW;
+    y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
+    yo_p[ch] = yout + q; xo_p[ch] = xout + q; xh_p[ch] = X05 ? x05 + q : nullptr;
   }
 
-  for (int ch = 0; ch < C; ch++) {
-    const size_t coff = ((size_t)g.n * C + ch) * HW;
-    const float* yp = yin + coff;
-    // y rows hs-1 .. hs+R: own float4 plus the scalars left and right of it
-    F4 y[R + 2];
-    float yl[R + 2], yr[R + 2];
+  auto load_row = [&](int k, FwdRow<C>& in) {  // row k of the strip = image row hs - 1 + k
+    const int kk = min(k, Reff + 1);  // rows past the last needed one re-read it
+    const int h = g.hs - 1 + kk;
+    const unsigned row = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4;
+    // the rows above and below the strip only contribute y (and, above, the weights); their other
+    // fields are read from the strip's own first / last row instead, which is in L1 anyway, so
+    // that no cache line is fetched for a value that is never used
+    const int hw = g.hs - 1 + min(kk, Reff);
+    const unsigned row_w = (unsigned)(hw < 0 ? 0 : hw) * W4;
+    const unsigned row_p = (unsigned)(g.hs - 1 + max(1, min(kk, Reff))) * W4;
+    in.c = ldg(cf_p, row_p + wc);
+    in.wxs = ldg(wx_p, row_w + wc);
+    in.wys = ldg(wy_p, row_w + wc);
 #pragma unroll
-    for (int r = 0; r < R + 2; r++) {
-      const int h = g.hs - 1 + r;
-      const bool rok = h >= 0 && h < H;
-      const size_t row = (size_t)(rok ? h : 0) * W;
-      y[r] = load4(yp + row + (g.col_ok ? w0 : 0), rok && g.col_ok);
-      yl[r] = (rok && left_ok) ? yp[row + w0 - 1] : 0.f;
-      yr[r] = (rok && right_ok) ? yp[row + w0 + kLanePx] : 0.f;
+    for (int ch = 0; ch < C; ch++) {
+      in.y[ch] = ldg(y_p[ch], row + wc);
+      in.yr[ch] = ldg(y_p[ch], row_w + wr);
+      in.x[ch] = ldg(x_p[ch], row_p + wc);
+      in.bb[ch] = ldg(b_p[ch], row_p + wc);
     }
-    F4 xo[R], bb[R];
+  };
+  // mask what lies outside the image, scale the weights, refine 1/(1+c): in place
+  auto absorb = [&](int k, FwdRow<C>& o) {
+    const int h = g.hs - 1 + k;
+    const bool rok = h >= 0 && h < H;
+    o.rc1 = rcp_refined(1.f + o.c);
+    o.wxs = (rok && wx_ok) ? kL * o.wxs : 0.f;
+    o.wys = (rok && g.col_ok && h < H - 1) ? kL * o.wys : 0.f;
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      const int h = g.hs + r;
-      const bool ok = g.col_ok && h < H;
-      const size_t off = coff + (size_t)(ok ? h : 0) * W + (ok ? w0 : 0);
-      xo[r] = load4(xin + off, ok);
-      bb[r] = load4(b + off, ok);
+    for (int ch = 0; ch < C; ch++) {
+      o.y[ch] = (rok && g.col_ok) ? o.y[ch] : 0.f;
+      o.yr[ch] = (rok && right_ok) ? o.yr[ch] : 0.f;
     }
-    F4 qy_up;  // quotients wy/m of the row above
+  };
+
+  float e1_up[C];
 #pragma unroll
-    for (int r = 0; r <= R; r++) {  // r indexes rows hs-1+r
-      // own triangles of this row (TV.cu:1268-1274): norm, Huber divisor, the two quotients
-      F4 qx, qy, d1, d2;
+  for (int ch = 0; ch < C; ch++) e1_up[ch] = 0.f;
+
+  // one row step; `first` = the row above the strip, which only supplies its triangle terms
+  auto compute = [&](int r, const FwdRow<C>& cur, const FwdRow<C>& nxt, auto first) {
+    const int h = g.hs - 1 + r;
+    const unsigned roff = (unsigned)(h >= 0 ? h : 0) * W4 + wc;
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float yc = y[r].v[j];
-        const float ydn = y[r + 1].v[j];
-        const float yrt = (j < 3) ? y[r].v[j + 1] : yr[r];
-        d1.v[j] = yc - ydn;
-        d2.v[j] = yc - yrt;
-        const float hub = exact_sqrt(d1.v[j] * d1.v[j] * wys[r].v[j] + d2.v[j] * d2.v[j] * wxs[r].v[j]);
-        const float m = fmaxf(1.f, inpaint::exact_div(hub, kDelta));
-        const float rm = rcp_refined(m);
-        qy.v[j] = div_by(wys[r].v[j], m, rm);
-        qx.v[j] = div_by(wxs[r].v[j], m, rm);
+    for (int ch = 0; ch < C; ch++) {
+      // own triangle, TV.cu:1268-1274
+      const float yc = cur.y[ch];
+      const float d1 = yc - nxt.y[ch];
+      const float d2 = yc - cur.yr[ch];
+      const float hub = exact_sqrt(d1 * d1 * cur.wys + d2 * d2 * cur.wxs);
+      const float m = fmaxf(1.f, inpaint::exact_div(hub, kDelta));
+      const float rm = rcp_refined(m);
+      const float e1 = d1 * div_by(cur.wys, m, rm);
+      const float e2 = d2 * div_by(cur.wxs, m, rm);
+      const float e1_above = e1_up[ch];
+      e1_up[ch] = e1;
+      if (first.value) continue;
+      const float e2_left = from_left_lane(e2);
+      float yt = yc;
+      yt -= -e1_above;   // TV.cu:1258
+      yt -= -e2_left;    // TV.cu:1265
+      yt -= e1;          // TV.cu:1272
+      yt -= e2;          // TV.cu:1273
+      const float xh = yt;
+      const float c = cur.c, bv = cur.bb[ch];
+      float x_loc = div_by(c * bv + yt, 1.f + c, cur.rc1);  // TV.cu:1288
+      const float lo = yt - c, hi = yt + c;
+      if (lo > 1.f + bv) x_loc = lo;
+      if (hi < bv - 1.f) x_loc = hi;
+      const float yn = x_loc + t * (x_loc - cur.x[ch]);  // TV.cu:1315
+      if (store_lane) {  // a block this small is predicated, not branched around
+        stg(yo_p[ch], roff, yn);
+        stg(xo_p[ch], roff, x_loc);
+        if (X05) stg(xh_p[ch], roff, xh);
       }
-      if (r > 0) {
-        const int h = g.hs - 1 + r;
-        const float qx_left = from_left_lane(qx.v[3], g.bperm_left);
-        F4 xn, yn, xh;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const float yc = y[r].v[j];
-          const float yu = y[r - 1].v[j];
-          const float ylf = (j > 0) ? y[r].v[j - 1] : yl[r];
-          const float ql = (j > 0) ? qx.v[j - 1] : qx_left;
-          float yt = yc;
-          yt -= (yc - yu) * qy_up.v[j];   // TV.cu:1258
-          yt -= (yc - ylf) * ql;          // TV.cu:1265
-          yt -= d1.v[j] * qy.v[j];        // TV.cu:1272
-          yt -= d2.v[j] * qx.v[j];        // TV.cu:1273
-          xh.v[j] = yt;
-          const float c = conf[r - 1].v[j], bv = bb[r - 1].v[j];
-          float x_loc = div_by(c * bv + yt, 1.f + c, rc1[r - 1][j]);  // TV.cu:1288
-          const float lo = yt - c, hi = yt + c;
-          if (lo > 1.f + bv) x_loc = lo;
-          if (hi < bv - 1.f) x_loc = hi;
-          xn.v[j] = x_loc;
-          yn.v[j] = x_loc + t * (x_loc - xo[r - 1].v[j]);  // TV.cu:1315
-        }
-        if (g.store_lane && h < H) {
-          const size_t off = coff + (size_t)h * W + w0;
-          store4(yout + off, yn);
-          store4(xout + off, xn);
-          if (x05) store4(x05 + off, xh);
-        }
-      }
-      qy_up = qy;
     }
+  };
+  const std::true_type kFirst{};
+  const std::false_type kRow{};
+
+  FwdRow<C> b0, b1, b2, b3;
+  load_row(0, b0);
+  load_row(1, b1);
+  load_row(2, b2);
+  load_row(3, b3);
+  absorb(0, b0);
+  absorb(1, b1);
+  compute(0, b0, b1, kFirst);
+  load_row(4, b0);
+  for (int r = 1; r <= Reff; r += 4) {  // cur / next rotate through (b1,b2) (b2,b3) (b3,b0) (b0,b1)
+    absorb(r + 1, b2);
+    compute(r, b1, b2, kRow);
+    load_row(r + 4, b1);
+    if (r + 1 > Reff) break;
+    absorb(r + 2, b3);
+    compute(r + 1, b2, b3, kRow);
+    load_row(r + 5, b2);
+    if (r + 2 > Reff) break;
+    absorb(r + 3, b0);
+    compute(r + 2, b3, b0, kRow);
+    load_row(r + 6, b3);
+    if (r + 3 > Reff) break;
+    absorb(r + 4, b1);
+    compute(r + 3, b0, b1, kRow);
+    load_row(r + 7, b0);
   }
 }
 
 // -------------------------------------------------------------------------------------------------
 // Adjoint iteration with the y rebuild fused in: TV.cu:586-859 (+1130-1189); END = the
-// segment-start variant TV.cu:862-1126 that reads y from the checkpoint.
+// segment-start variant TV.cu:862-1126 that reads y from the checkpoint.  END is the last step of
+// its segment, so it also performs the segment flush (copy_and_set_to_0, TV.cu:178-218): the fp32
+// segment sums go into the fp64 totals and the accumulators are left at zero.
 //
-// Rows are streamed: the wavefront walks down its strip one row at a time, all channels per row,
-// and prefetches the next row while it works on the current one.  Per triangle (owner q) the
-// kernel forms, once, every term that the reference evaluates at q, at the pixel below q and at
-// the pixel right of q:
-//     O1..O4   the four own-triangle terms subtracted at q                     (TV.cu:732-743)
-//     -O1, P1*tu, P2*tu   the three terms subtracted at the pixel below        (TV.cu:668-677)
-//     -O2, P2*tl, P1*tl   the three terms subtracted at the pixel to the right (TV.cu:701-710)
+// Per triangle (owner q) the kernel forms, once, every term that the reference evaluates at q,
+// at the pixel below q and at the pixel right of q:
+//     O1..O4              the four own-triangle terms subtracted at q               (TV.cu:732-743)
+//     -O1, P1*tu, P2*tu   the three terms subtracted at the pixel below             (TV.cu:668-677)
+//     -O2, P2*tl, P1*tl   the three terms subtracted at the pixel to the right      (TV.cu:701-710)
 // with P1 = (g_q-g_d) wy (y_q-y_d), P2 = (g_q-g_r) wx (y_q-y_r).  The operand order inside every
 // product is the reference's (negating both factors of a product is exact), the order of the
 // subtractions at each pixel is the reference's, and an inactive triangle is the active formula
 // with nom = 1, denom = 0, which reproduces the inactive branch exactly.
 // -------------------------------------------------------------------------------------------------
-constexpr float kClipLocalGrad = 10000.0f;  // TV.cu:52
-constexpr float kLocalGCMult = 0.1f;        // TV.cu:63
-constexpr float kLocalGXMult = 0.1f;        // TV.cu:65
-
-__device__ __forceinline__ float from_right_lane(float v, int bperm_addr) {
-  return __int_as_float(__builtin_amdgcn_ds_bpermute(bperm_addr, __float_as_int(v)));
-}
 
 // y_{k+1} from x05[k] (xa) and x05[k-1] (xb), TV.cu:1149-1165; rc = rcp_refined(1 + conf)
-__device__ __forceinline__ float rebuild_y_fast(float bb, float xa, float xb, float conf, float rc, float t) {
+__device__ __forceinline__ float rebuild_y_fast(float bb, float xa, float xb, float conf, float rc, double opc_d,
+                                                float t) {
   float diff = bb - xa;
   float sign = (diff < 0) ? -1.f : 1.f;
-  const bool quad = (1. + (double)conf >= (double)(sign * diff));
+  const bool quad = (opc_d >= (double)(sign * diff));  // opc_d = 1. + (double)conf
   const float cb = conf * bb;
   const float xk_q = div_by(cb + xa, 1.f + conf, rc);
   const float xkm_q = div_by(cb + xb, 1.f + conf, rc);
@@ -228,253 +272,240 @@ __device__ __forceinline__ float rebuild_y_fast(float bb, float xa, float xb, fl
   return quad ? y_q : y_l;
 }
 
-template <int C, bool END>
+template <int C>
+struct AdjRow {
+  float c, rc1, wxs, wys, xa[C], y[C], bb[C], g[C];  // y is loaded as x05[k-1] (or the checkpoint y) and rebuilt in place
+  float gc_i, gwx_i, gwy_i, gx_i[C], gb_i[C];        // accumulators and partial g_x the row's pixel update continues
+  double opc_d;                                      // 1. + (double)c, the left side of the prox regime test
+};
+
+template <int C, bool END, bool FINAL>
 __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
-    const float* __restrict__ yck, float* __restrict__ gc, float* __restrict__ gb, float* __restrict__ gwx,
-    float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
-    float* __restrict__ gxk, float* __restrict__ gxk_m1, int N, int H, int W, float t, int R, int strips_x,
-    int strips_y) {
+    const float* __restrict__ yck, const float* __restrict__ gc_in, float* __restrict__ gc,
+    const float* __restrict__ gb_in, float* __restrict__ gb, const float* __restrict__ gwx_in,
+    float* __restrict__ gwx, const float* __restrict__ gwy_in, float* __restrict__ gwy,
+    const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
+    float* __restrict__ gxk_m1, float* __restrict__ gx_final, double* __restrict__ tot_gc,
+    double* __restrict__ tot_gb, double* __restrict__ tot_gwx, double* __restrict__ tot_gwy, int N, int H, int W,
+    float t, int R, int strips_x, int strips_y) {
   StripGeom g;
-  if (!strip_geometry(g, R, W, strips_x, strips_y, N)) return;
+  if (!strip_geometry(g, kAdjCols, R, W, strips_x, strips_y, N)) return;
+  const int Reff = min(R, H - g.hs);
   const size_t HW = (size_t)H * W;
-  const size_t poff = (size_t)g.n * HW;
-  const int w0 = g.w_first;
-  const bool last_lane = g.lane == 63;
-  const bool right_ok = w0 + kLanePx < W;
-  const int bperm_right = ((g.lane + 1) & 63) << 2;
+  const unsigned W4 = 4u * (unsigned)W;          // row pitch in bytes
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;  // clamped column (bytes)
+  const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
+  const bool wx_ok = g.col_ok && g.w < W - 1;
   const double opt = 1. + (double)t;
-
-  // raw loads of one row: everything the rebuild and the pixel update of that row need
-  struct RowIn {
-    F4 c, xa[C], xb[C], bb[C], gg[C];
-  };
-  auto load_row = [&](int h, RowIn& in) {
-    const bool ok = g.col_ok && h >= 0 && h < H;
-    const size_t off = (size_t)(ok ? h : 0) * W + (ok ? w0 : 0);
-    in.c = load4(cf + poff + off, ok);
+  // wave-uniform plane pointers + 32-bit element offsets (SGPR base, VGPR offset)
+  const size_t poff = (size_t)g.n * HW;
+  const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
+  const float *const gci_p = gc_in + poff, *const gwxi_p = gwx_in + poff, *const gwyi_p = gwy_in + poff;
+  float *const gco_p = gc + poff, *const gwxo_p = gwx + poff, *const gwyo_p = gwy + poff;
+  const float *xa_p[C], *xb_p[C], *b_p[C], *g_p[C], *gxi_p[C], *gbi_p[C];
+  float *g05o_p[C], *gxm_p[C], *gbo_p[C], *gxf_p[C];
 #pragma unroll
-    for (int ch = 0; ch < C; ch++) {
-      const size_t q = ((size_t)g.n * C + ch) * HW + off;
-      if (END) {
-        in.xa[ch] = load4(x05a + q, ok);
-        in.xb[ch] = load4(yck + q, ok);  // the checkpoint y travels in the xb slot
-      } else {
-        in.xa[ch] = load4(x05a + q, ok);
-        in.xb[ch] = load4(x05b + q, ok);
-      }
-      in.bb[ch] = load4(b + q, ok);
-      in.gg[ch] = load4(g05_in + q, ok);
-    }
-  };
-  // right neighbour of the last lane's fourth pixel: one scalar column, rebuilt the same way
-  auto right_scalar = [&](int h, int ch, float& yv, float& gv) {
-    yv = 0.f;
-    gv = 0.f;
-    if (h >= 0 && h < H && right_ok) {
-      const size_t p = (size_t)h * W + w0 + kLanePx;
-      const size_t q = ((size_t)g.n * C + ch) * HW + p;
-      gv = g05_in[q];
-      if (END) {
-        yv = yck[q];
-      } else {
-        const float cv = cf[poff + p];
-        yv = rebuild_y_fast(b[q], x05a[q], x05b[q], cv, rcp_refined(1.f + cv), t);
-      }
-    }
-  };
-
-  // state of the current row
-  F4 c_cur, rc1_cur, y_cur[C], g_cur[C], xa_cur[C], b_cur[C];
-  F4 dn1[C], dn3[C], dn4[C];  // terms handed down to the row below
-  RowIn nxt;
-  auto absorb = [&](const RowIn& in, F4& c_o, F4& rc1_o, F4* y_o, F4* g_o, F4* xa_o, F4* b_o) {
-    c_o = in.c;
-#pragma unroll
-    for (int j = 0; j < 4; j++) rc1_o.v[j] = rcp_refined(1.f + in.c.v[j]);
-#pragma unroll
-    for (int ch = 0; ch < C; ch++) {
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        y_o[ch].v[j] = END ? in.xb[ch].v[j]
-                           : rebuild_y_fast(in.bb[ch].v[j], in.xa[ch].v[j], in.xb[ch].v[j], in.c.v[j], rc1_o.v[j], t);
-      g_o[ch] = in.gg[ch];
-      xa_o[ch] = in.xa[ch];
-      b_o[ch] = in.bb[ch];
-    }
-  };
-
-  {
-    RowIn first;
-    load_row(g.hs - 1, first);
-    load_row(g.hs, nxt);
-    absorb(first, c_cur, rc1_cur, y_cur, g_cur, xa_cur, b_cur);
+  for (int ch = 0; ch < C; ch++) {
+    const size_t q = ((size_t)g.n * C + ch) * HW;
+    xa_p[ch] = x05a + q; xb_p[ch] = (END ? yck : x05b) + q;  // the checkpoint y travels in the y slot
+    b_p[ch] = b + q; g_p[ch] = g05_in + q; gxi_p[ch] = gxk + q; gbi_p[ch] = gb_in + q;
+    g05o_p[ch] = g05_out + q; gxm_p[ch] = gxk_m1 + q; gbo_p[ch] = gb + q;
+    gxf_p[ch] = FINAL ? gx_final + q : nullptr;
   }
-#pragma unroll
-  for (int ch = 0; ch < C; ch++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) dn1[ch].v[j] = dn3[ch].v[j] = dn4[ch].v[j] = 0.f;
 
-  for (int r = 0; r <= R; r++) {
+  auto load_row = [&](int k, AdjRow<C>& in) {
+    const int kk = min(k, Reff + 1);
+    const int h = g.hs - 1 + kk;
+    const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+    // the rows above and below the strip need y and g (and, above, the weights) only; what they do
+    // not need is read from the strip's own first / last row, which is in L1 anyway
+    const int hw = g.hs - 1 + min(kk, Reff);
+    const unsigned off_w = (unsigned)(hw < 0 ? 0 : hw) * W4 + wc;
+    const unsigned off_p = (unsigned)(g.hs - 1 + max(1, min(kk, Reff))) * W4 + wc;
+    in.c = ldg(cf_p, off);
+    in.wxs = ldg(wx_p, off_w);
+    in.wys = ldg(wy_p, off_w);
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      in.xa[ch] = ldg(xa_p[ch], off);
+      in.y[ch] = ldg(xb_p[ch], off);
+      in.bb[ch] = ldg(b_p[ch], off);
+      in.g[ch] = ldg(g_p[ch], off);
+      in.gx_i[ch] = ldg(gxi_p[ch], off_p);
+      in.gb_i[ch] = ldg(gbi_p[ch], off_p);
+    }
+    in.gc_i = ldg(gci_p, off_p);
+    in.gwx_i = ldg(gwxi_p, off_p);
+    in.gwy_i = ldg(gwyi_p, off_p);
+  };
+  auto absorb = [&](int k, AdjRow<C>& o) {
+    const int h = g.hs - 1 + k;
+    const bool ok = g.col_ok && h >= 0 && h < H;
+    o.c = ok ? o.c : 0.f;
+    o.rc1 = rcp_refined(1.f + o.c);
+    o.opc_d = 1. + (double)o.c;
+    o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
+    o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.y[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+      o.y[ch] = END ? xb : rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
+      o.g[ch] = ok ? o.g[ch] : 0.f;
+      o.xa[ch] = xa;
+      o.bb[ch] = bv;
+    }
+  };
+
+  float dn1[C], dn3[C], dn4[C];  // terms handed down to the row below
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) dn1[ch] = dn3[ch] = dn4[ch] = 0.f;
+
+  auto compute = [&](int r, const AdjRow<C>& cur, const AdjRow<C>& nxt, auto first) {
     const int h = g.hs - 1 + r;  // owner row of this step
-    // next row: turn the prefetched loads into y / g, then prefetch the row after it
-    F4 c_n, rc1_n, y_n[C], g_n[C], xa_n[C], b_n[C];
-    absorb(nxt, c_n, rc1_n, y_n, g_n, xa_n, b_n);
-    if (r < R) load_row(h + 2, nxt);
-
-    // masked, L-scaled weights of the owner row
-    const bool rok = g.col_ok && h >= 0 && h < H;
-    const size_t roff = (size_t)(rok ? h : 0) * W + (rok ? w0 : 0);
-    F4 wxs = load4(wx + poff + roff, rok);
-    F4 wys = load4(wy + poff + roff, rok && h < H - 1);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      wxs.v[j] = (w0 + j < W - 1) ? kL * wxs.v[j] : 0.f;
-      wys.v[j] = kL * wys.v[j];
-    }
-    const bool px_row = r > 0 && h < H;  // rows of this strip that produce output
-    const bool do_store = px_row && g.store_lane;
-    F4 gcv, gwxv, gwyv, rc2;
-    if (r > 0) {
-      gcv = load4(gc + poff + roff, do_store);
-      gwxv = load4(gwx + poff + roff, do_store);
-      gwyv = load4(gwy + poff + roff, do_store);
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float d = (1.f + c_cur.v[j]) * (1.f + c_cur.v[j]);
-        rc2.v[j] = rcp_refined(d);
-      }
-    }
+    const unsigned roff = (unsigned)(h >= 0 ? h : 0) * W4 + wc;
+    float gcv = cur.gc_i, gwxv = cur.gwx_i, gwyv = cur.gwy_i, rc2 = 0.f;
+    if (!first.value) rc2 = rcp_refined((1.f + cur.c) * (1.f + cur.c));
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      const size_t q = ((size_t)g.n * C + ch) * HW + roff;
-      float yr = from_right_lane(y_cur[ch].v[0], bperm_right);
-      float gr = from_right_lane(g_cur[ch].v[0], bperm_right);
-      if (last_lane) right_scalar(h, ch, yr, gr);
-      F4 gxv, gbv;
-      if (r > 0) {
-        gxv = load4(gxk + q, do_store);
-        gbv = load4(gb + q, do_store);
-      }
-      F4 O1, O2, O3, O4, r3, r4, n3, n4;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float yk = y_cur[ch].v[j], yd = y_n[ch].v[j], yrt = (j < 3) ? y_cur[ch].v[j + 1] : yr;
-        const float gk = g_cur[ch].v[j], gd = g_n[ch].v[j], grt = (j < 3) ? g_cur[ch].v[j + 1] : gr;
-        const float wxv = wxs.v[j], wyv = wys.v[j];
-        const float d1 = yk - yd, d2 = yk - yrt;
-        const float a1 = d1 * d1 * wyv;  // wy_nyy2
-        const float a2 = d2 * d2 * wxv;  // wx_nyx2
-        const float hub = exact_sqrt(a2 + a1);
-        const bool act = hub > kDelta;
-        float nom = inpaint::exact_div(kDelta, hub);
-        float denom = inpaint::exact_div(nom, 2.f * hub * hub);
-        nom = act ? nom : 1.f;
-        denom = act ? denom : 0.f;
-        const float gpd = gk - gd, gpr = gk - grt;
-        O1.v[j] = gpd * (wyv * nom);
-        O2.v[j] = gpr * (wxv * nom);
-        const float P1 = gpd * wyv * d1;
-        const float P2 = gpr * wxv * d2;
-        const float dd = denom * 2.0f;
-        const float tp = dd * ((yd - yk) * wyv + (yrt - yk) * wxv);
-        const float tu = dd * d1 * wyv;
-        const float tl = dd * d2 * wxv;
-        O3.v[j] = P1 * tp;
-        O4.v[j] = P2 * tp;
-        n3.v[j] = P1 * tu;
-        n4.v[j] = P2 * tu;
-        r3.v[j] = P2 * tl;
-        r4.v[j] = P1 * tl;
-        if (r > 0) {  // weight gradients of the pixel's own triangle, TV.cu:749-769 / 1019-1037
-          float ux, uy;
-          if (!END) {
-            ux = kLocalGXMult * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
-            uy = kLocalGXMult * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
-          } else {
-            const float ux_a = kLocalGXMult * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
-            const float uy_a = kLocalGXMult * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
-            ux = act ? ux_a : kLocalGXMult * d2 * gpr;
-            uy = act ? uy_a : kLocalGXMult * d1 * gpd;
-          }
-          if (w0 + j < W - 1) gwxv.v[j] = gwxv.v[j] - ux;
-          if (h < H - 1) gwyv.v[j] = gwyv.v[j] - uy;
-        }
-      }
+      const float yrt = from_right_lane(cur.y[ch]);
+      const float grt = from_right_lane(cur.g[ch]);
+      const float gxv = cur.gx_i[ch];
+      float gbv = cur.gb_i[ch];
+      const float yk = cur.y[ch], yd = nxt.y[ch];
+      const float gk = cur.g[ch], gd = nxt.g[ch];
+      const float wxv = cur.wxs, wyv = cur.wys;
+      const float d1 = yk - yd, d2 = yk - yrt;
+      const float a1 = d1 * d1 * wyv;  // wy_nyy2
+      const float a2 = d2 * d2 * wxv;  // wx_nyx2
+      const float hub = exact_sqrt(a2 + a1);
+      const bool act = hub > kDelta;
+      float nom = inpaint::exact_div(kDelta, hub);
+      float denom = inpaint::exact_div(nom, 2.f * hub * hub);
+      nom = act ? nom : 1.f;
+      denom = act ? denom : 0.f;
+      const float gpd = gk - gd, gpr = gk - grt;
+      const float O1 = gpd * (wyv * nom);
+      const float O2 = gpr * (wxv * nom);
+      const float P1 = gpd * wyv * d1;
+      const float P2 = gpr * wxv * d2;
+      const float dd = denom * 2.0f;
+      const float tp = dd * ((yd - yk) * wyv + (yrt - yk) * wxv);
+      const float tu = dd * d1 * wyv;
+      const float tl = dd * d2 * wxv;
+      const float O3 = P1 * tp, O4 = P2 * tp;
+      const float n3 = P1 * tu, n4 = P2 * tu;
       // terms arriving from the triangle of the pixel to the left
-      const float l1 = from_left_lane(O2.v[3], g.bperm_left);
-      const float l3 = from_left_lane(r3.v[3], g.bperm_left);
-      const float l4 = from_left_lane(r4.v[3], g.bperm_left);
-      if (r > 0) {
-        F4 g05v, gxm;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          float tt = g_cur[ch].v[j];
-          tt -= -dn1[ch].v[j];                       // TV.cu:668 / 684
-          tt -= dn3[ch].v[j];                        // TV.cu:675
-          tt -= dn4[ch].v[j];                        // TV.cu:677
-          tt -= -((j > 0) ? O2.v[j - 1] : l1);       // TV.cu:701 / 718
-          tt -= (j > 0) ? r3.v[j - 1] : l3;          // TV.cu:707
-          tt -= (j > 0) ? r4.v[j - 1] : l4;          // TV.cu:710
-          tt -= O1.v[j];                             // TV.cu:732 / 763
-          tt -= O2.v[j];                             // TV.cu:733 / 764
-          tt -= O3.v[j];                             // TV.cu:741
-          tt -= O4.v[j];                             // TV.cu:743
-          // momentum adjoint, TV.cu:796-801
-          float df = (float)((double)gxv.v[j] + opt * (double)tt);
-          df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
-          gxv.v[j] = df;
-          gxm.v[j] = -t * tt;
-          // prox adjoint, TV.cu:806-828
-          const float conf = c_cur.v[j], bv = b_cur[ch].v[j], xh = xa_cur[ch].v[j];
-          const float diff = bv - xh;
-          const float sign = (diff < 0) ? -1.f : 1.f;
-          const bool quad = (1. + (double)conf >= (double)(sign * diff));
-          const float opc = 1.f + conf;
-          const float gc_q = df * (div_by(bv, opc, rc1_cur.v[j]) - div_by(conf * bv + xh, opc * opc, rc2.v[j])) * kLocalGCMult;
-          const float g05_q = div_by(df, opc, rc1_cur.v[j]);
-          const float gb_q = div_by(df * conf, opc, rc1_cur.v[j]) * 1.0f;
-          if (quad) {
-            gcv.v[j] += gc_q;
-            g05v.v[j] = g05_q;
-            gbv.v[j] += gb_q;
-          } else if (conf >= sign * diff) {  // TV.cu:818-822
-            g05v.v[j] = 0.f;
-            gbv.v[j] += df * 1.0f;
+      const float l1 = from_left_lane(O2);
+      const float l3 = from_left_lane(P2 * tl);
+      const float l4 = from_left_lane(P1 * tl);
+      if (!first.value) {
+        // weight gradients of the pixel's own triangle, TV.cu:749-769 / 1019-1037
+        float ux, uy;
+        if (!END) {
+          ux = kLocalGXMult * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
+          uy = kLocalGXMult * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
+        } else {
+          const float ux_a = kLocalGXMult * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
+          const float uy_a = kLocalGXMult * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
+          ux = act ? ux_a : kLocalGXMult * d2 * gpr;
+          uy = act ? uy_a : kLocalGXMult * d1 * gpd;
+        }
+        if (g.w < W - 1) gwxv = gwxv - ux;
+        if (h < H - 1) gwyv = gwyv - uy;
+
+        float tt = gk;
+        tt -= -dn1[ch];  // TV.cu:668 / 684
+        tt -= dn3[ch];   // TV.cu:675
+        tt -= dn4[ch];   // TV.cu:677
+        tt -= -l1;       // TV.cu:701 / 718
+        tt -= l3;        // TV.cu:707
+        tt -= l4;        // TV.cu:710
+        tt -= O1;        // TV.cu:732 / 763
+        tt -= O2;        // TV.cu:733 / 764
+        tt -= O3;        // TV.cu:741
+        tt -= O4;        // TV.cu:743
+        // momentum adjoint, TV.cu:796-801
+        float df = (float)((double)gxv + opt * (double)tt);
+        df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
+        const float gxm = -t * tt;
+        // prox adjoint, TV.cu:806-828
+        const float conf = cur.c, bv = cur.bb[ch], xh = cur.xa[ch];
+        const float diff = bv - xh;
+        const float sign = (diff < 0) ? -1.f : 1.f;
+        const bool quad = (cur.opc_d >= (double)(sign * diff));
+        const float opc = 1.f + conf;
+        const float gc_q = df * (div_by(bv, opc, cur.rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kLocalGCMult;
+        const float g05_q = div_by(df, opc, cur.rc1);
+        const float gb_q = div_by(df * conf, opc, cur.rc1) * 1.0f;
+        // three regimes (quadratic / TV.cu:818-822, unreachable for c >= 0 / linear) as selects;
+        // adding +0 where the reference adds nothing leaves the accumulators unchanged
+        const bool mid = !quad && (conf >= sign * diff);
+        const float g05v = quad ? g05_q : (mid ? 0.f : df);
+        gcv += quad ? gc_q : (mid ? 0.f : sign * df * kLocalGCMult);
+        gbv += quad ? gb_q : (mid ? df * 1.0f : 0.f);
+        if (store_lane) {  // a block this small is predicated, not branched around
+          if (FINAL) stg(gxf_p[ch], roff, df);  // only the last step's g_x is read again (TV.cu:800,1785)
+          stg(gxm_p[ch], roff, gxm);
+          stg(g05o_p[ch], roff, g05v);
+          if (END) {  // segment flush, fused: fp32 segment sum into its fp64 total, then zero (TV.cu:178-218)
+            double* tb = tot_gb + ((size_t)g.n * C + ch) * HW + (roff >> 2);
+            *tb = (double)gbv + *tb / 1.;
+            stg(gbo_p[ch], roff, 0.f);
           } else {
-            g05v.v[j] = df;
-            gcv.v[j] += sign * df * kLocalGCMult;
+            stg(gbo_p[ch], roff, gbv);
           }
         }
-        if (do_store) {
-          store4(gxk + q, gxv);
-          store4(gxk_m1 + q, gxm);
-          store4(g05_out + q, g05v);
-          store4(gb + q, gbv);
-        }
       }
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        dn1[ch].v[j] = O1.v[j];
-        dn3[ch].v[j] = n3.v[j];
-        dn4[ch].v[j] = n4.v[j];
+      dn1[ch] = O1;
+      dn3[ch] = n3;
+      dn4[ch] = n4;
+    }
+    if (!first.value && store_lane) {
+      if (END) {
+        const size_t e = poff + (roff >> 2);
+        tot_gc[e] = (double)gcv + tot_gc[e] / 1.;
+        tot_gwx[e] = (double)gwxv + tot_gwx[e] / 1.;
+        tot_gwy[e] = (double)gwyv + tot_gwy[e] / 1.;
+        stg(gco_p, roff, 0.f);
+        stg(gwxo_p, roff, 0.f);
+        stg(gwyo_p, roff, 0.f);
+      } else {
+        stg(gco_p, roff, gcv);
+        stg(gwxo_p, roff, gwxv);
+        stg(gwyo_p, roff, gwyv);
       }
     }
-    if (do_store) {
-      store4(gc + poff + roff, gcv);
-      store4(gwx + poff + roff, gwxv);
-      store4(gwy + poff + roff, gwyv);
-    }
-    c_cur = c_n;
-    rc1_cur = rc1_n;
-#pragma unroll
-    for (int ch = 0; ch < C; ch++) {
-      y_cur[ch] = y_n[ch];
-      g_cur[ch] = g_n[ch];
-      xa_cur[ch] = xa_n[ch];
-      b_cur[ch] = b_n[ch];
-    }
+  };
+  const std::true_type kFirst{};
+  const std::false_type kRow{};
+
+  AdjRow<C> b0, b1, b2, b3;
+  load_row(0, b0);
+  load_row(1, b1);
+  load_row(2, b2);
+  load_row(3, b3);
+  absorb(0, b0);
+  absorb(1, b1);
+  compute(0, b0, b1, kFirst);
+  load_row(4, b0);
+  for (int r = 1; r <= Reff; r += 4) {  // cur / next rotate through (b1,b2) (b2,b3) (b3,b0) (b0,b1)
+    absorb(r + 1, b2);
+    compute(r, b1, b2, kRow);
+    load_row(r + 4, b1);
+    if (r + 1 > Reff) break;
+    absorb(r + 2, b3);
+    compute(r + 1, b2, b3, kRow);
+    load_row(r + 5, b2);
+    if (r + 2 > Reff) break;
+    absorb(r + 3, b0);
+    compute(r + 2, b3, b0, kRow);
+    load_row(r + 6, b3);
+    if (r + 3 > Reff) break;
+    absorb(r + 4, b1);
+    compute(r + 3, b0, b1, kRow);
+    load_row(r + 7, b0);
   }
 }
 

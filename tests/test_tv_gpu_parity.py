@@ -71,9 +71,12 @@ def compare(name, got, ref):
     (1, 2, 1, 70, 4),       # a single row
     (1, 1, 33, 1, 4),       # a single column
     (3, 2, 130, 200, 50),   # several segments of unequal length
-    (2, 2, 45, 508, 14),    # wave-strip kernels: three strips wide, ragged rows
-    (1, 1, 9, 252, 8),      # exactly one strip wide
-    (1, 4, 19, 256, 6),     # four channels, 256 = one strip + one lane
+    (2, 2, 45, 508, 14),    # several strips wide, ragged rows
+    (1, 1, 9, 63, 8),       # exactly one forward strip wide
+    (1, 2, 11, 62, 8),      # exactly one adjoint strip wide
+    (1, 2, 21, 64, 6),      # one column more than a strip
+    (1, 4, 19, 126, 6),     # four channels, two forward strips
+    (1, 3, 40, 125, 10),    # three channels, ragged
 ])
 def test_forward_backward_match_oracle(ext, tv_oracle, n, c, h, w, its):
     d = tv_inputs(n, c, h, w, seed=n * 1000 + h + w + its, conf_density=0.3)
@@ -83,8 +86,8 @@ def test_forward_backward_match_oracle(ext, tv_oracle, n, c, h, w, its):
 
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
 def test_tile_kernels_when_forced_or_needed(ext, tv_oracle, n, c, h, w, its, monkeypatch):
-    # widths divisible by 4 normally take the wave-strip kernels; force the LDS-tile kernels
-    # (5 channels also exercises the strip forward + tile adjoint combination without forcing)
+    # up to 4 channels normally take the wave-strip kernels; force the LDS-tile kernels
+    # (5 channels always takes them)
     d = tv_inputs(n, c, h, w, seed=77 + c, conf_density=0.3)
     ref = run_oracle(tv_oracle, d, its, 2)
     compare("default path c=%d" % c, run_gpu(ext, d, its, 2), ref)
