@@ -1,0 +1,138 @@
+"""The quoted workloads on the GPU: full-size runs checked through size-independent properties
+(batch independence, channel independence, determinism), the three-level hierarchy against the
+oracle, and the stress configuration's shape at reduced batch against the oracle."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from customnetworklayers_amd.workloads import CONFIGS, edge_weights, smooth_image, tv_inputs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext
+
+    return tvInpaint_cuda_ext
+
+
+def gpu_layer(ext, d, its, pid):
+    t = {k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in d.items()}
+    ext.reset_id(pid)
+    (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, pid)
+    grads = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, pid)
+    torch.cuda.synchronize()
+    return [sol.cpu().numpy()] + [g.cpu().numpy() for g in grads]
+
+
+def test_headline_batch_equals_its_samples_run_alone(ext):
+    # 4 x 2 x 384 x 1248, 100 iterations: the batch must be 4 independent problems, bit for bit
+    cfg = CONFIGS[1]
+    d = tv_inputs(cfg["n"], cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    full = gpu_layer(ext, d, cfg["its"], 0)
+    again = gpu_layer(ext, d, cfg["its"], 1)
+    for a, b in zip(full, again):  # deterministic, and independent of the id used
+        np.testing.assert_array_equal(a, b)
+    for s in (0, 3):
+        one = gpu_layer(ext, {k: v[s:s + 1] for k, v in d.items()}, cfg["its"], 2)
+        for a, b in zip(full, one):
+            np.testing.assert_array_equal(a[s:s + 1], b)
+    assert all(np.isfinite(a).all() for a in full)
+    # channels never couple in the forward pass; the confidence / weight gradients sum over them
+    ch0 = {k: (v[:1, :1] if k in ("db", "di", "grad") else v[:1]) for k, v in d.items()}
+    one_ch = gpu_layer(ext, ch0, cfg["its"], 2)
+    np.testing.assert_array_equal(one_ch[0][0, 0], full[0][0, 0])
+    np.testing.assert_array_equal(one_ch[4][0, 0], full[4][0, 0])  # g_b
+    np.testing.assert_array_equal(one_ch[5][0, 0], full[5][0, 0])  # g_init
+
+
+def test_stress_shape_matches_oracle(ext, tv_oracle):
+    # 16 x 2 x 256 x 512, 200 iterations in the quoted workload; two samples here
+    cfg = CONFIGS[4]
+    d = tv_inputs(2, cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    got = gpu_layer(ext, d, cfg["its"], 3)
+    tv_oracle.reset_id(3)
+    sol = tv_oracle.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], cfg["its"], 3)
+    grads = tv_oracle.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], cfg["its"], 3)
+    rel = lambda a, r: float(np.abs(a - r).max() / max(np.abs(r).max(), 1e-30))
+    errs = [rel(a, r) for a, r in zip(got, [sol] + list(grads))]
+    print("\n[stress 2x2x256x512 its=200] out %.2e grads %s" % (errs[0], ["%.2e" % e for e in errs[1:]]), flush=True)
+    assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3
+
+
+def up2(t):
+    """x2 bilinear upsampling with doubled values (flow vectors scale with the resolution)."""
+    return 2.0 * F.interpolate(t, scale_factor=2, mode="bilinear", align_corners=False)
+
+
+def run_hierarchy(layer_fwd, layer_bwd, levels, inputs, its):
+    """Forward through ids 0,1,2 then backward 2,1,0.  The glue runs on the CPU for both paths so
+    that both see identical layer inputs; returns the solutions and all gradients per level."""
+    sols, feeds = [], []
+    b = torch.from_numpy(inputs[0]["db"])
+    for lvl, d in enumerate(inputs):
+        feed = dict(d, db=b.numpy().copy(), di=b.numpy().copy())
+        sol = layer_fwd(feed, its, lvl)
+        sols.append(sol)
+        feeds.append(feed)
+        if lvl + 1 < len(inputs):
+            b = up2(torch.from_numpy(sol))
+    grads = [None] * len(inputs)
+    upstream = inputs[-1]["grad"].copy()
+    for lvl in reversed(range(len(inputs))):
+        g = layer_bwd(feeds[lvl], upstream, its, lvl)
+        grads[lvl] = g
+        if lvl > 0:  # d loss / d sol_{lvl-1} through b_lvl = init_lvl = up2(sol_{lvl-1})
+            s = torch.from_numpy(sols[lvl - 1]).requires_grad_(True)
+            up2(s).backward(torch.from_numpy(g[3] + g[4]))
+            upstream = s.grad.numpy().copy()
+    return sols, grads
+
+
+def test_three_level_hierarchy_matches_oracle(ext, tv_oracle):
+    cfg = CONFIGS[3]
+    n, c, its = cfg["n"], cfg["c"], cfg["its"]
+    rng = np.random.default_rng(0)
+    top = cfg["levels"][-1]
+    imgs = [smooth_image(rng, *top) for _ in range(n)]
+    inputs = []
+    for lvl, (h, w) in enumerate(cfg["levels"]):
+        d = tv_inputs(n, c, h, w, seed=10 + lvl, **cfg["gen"])
+        f = top[0] // h
+        for s in range(n):  # one image pyramid: the weights of every level come from the same image
+            wx, wy = edge_weights(imgs[s][::f, ::f])
+            d["dx"][s, 0], d["dy"][s, 0] = wx, wy
+        inputs.append(d)
+
+    state = {}
+
+    def gpu_fwd(feed, its, pid):
+        t = {k: torch.from_numpy(v).to(DEV) for k, v in feed.items()}
+        ext.reset_id(pid)
+        state[pid] = t
+        return ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, pid)[0].cpu().numpy()
+
+    def gpu_bwd(feed, upstream, its, pid):
+        t = state[pid]
+        g = ext.backward(torch.from_numpy(upstream).to(DEV), t["dx"], t["dy"], t["dc"], t["db"], its, pid)
+        return [x.cpu().numpy() for x in g]
+
+    def cpu_fwd(feed, its, pid):
+        tv_oracle.reset_id(pid)
+        return tv_oracle.forward(feed["dx"], feed["dy"], feed["dc"], feed["db"], feed["di"], its, pid)
+
+    def cpu_bwd(feed, upstream, its, pid):
+        return list(tv_oracle.backward(upstream.copy(), feed["dx"], feed["dy"], feed["dc"], feed["db"], its, pid))
+
+    gs, gg = run_hierarchy(gpu_fwd, gpu_bwd, cfg["levels"], inputs, its)
+    cs, cg = run_hierarchy(cpu_fwd, cpu_bwd, cfg["levels"], inputs, its)
+    rel = lambda a, r: float(np.abs(a - r).max() / max(np.abs(r).max(), 1e-30))
+    for lvl in range(3):
+        e_out = rel(gs[lvl], cs[lvl])
+        e_g = [rel(a, r) for a, r in zip(gg[lvl], cg[lvl])]
+        print("\n[hierarchy level %d %s] out %.2e grads %s" % (lvl, cfg["levels"][lvl], e_out, ["%.2e" % e for e in e_g]),
+              flush=True)
+        assert e_out <= 1e-4 and max(e_g) <= 1e-3
