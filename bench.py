@@ -15,6 +15,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the main adjoint kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
+# script on the headline workload (2 x 72471 KiB fetched, after the copy-kernel calibration, plus
+# 69740 KiB written; profiles/tv_strip_headline_hbm_traffic.txt).  Other workloads: not measured.
+MEASURED_TRAFFIC_BYTES = {1: (2 * 72471 + 69740) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c):
@@ -116,10 +120,10 @@ def main():
                                % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
         "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
                       "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4)},
-        "roofline": {"bound": "hbm", "kernel": "tv_adjoint_iter<false>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "tvstrip::tv_adjoint_strip<2,false,false>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "bytes_per_launch": kernel_bytes, "avg_launch_ms": round(kernel_ms, 5),
-                     "launches_timed": launches.value},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config), "bytes_per_launch": kernel_bytes,
+                     "avg_launch_ms": round(kernel_ms, 5), "launches_timed": launches.value},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
