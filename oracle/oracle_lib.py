@@ -159,3 +159,132 @@ class TVOracle:
 
     def max_threads(self):
         return self.lib.tv_oracle_max_threads()
+
+
+class TGVOracle:
+    """Huber-TGV FISTA inpainting layer, CPU restatement (oracle/tgv_oracle.cpp).
+
+    Shapes: dx, dy (N,2,H,W) with channel 0 = edge weight and channel 1 = beta; c (N,1,H,W);
+    b (N,C,H,W); init / output / upstream gradient (N,3*C,H,W) in variable-major order (u, v1, v2).
+    """
+
+    def __init__(self):
+        L = self.lib = _load("libtgv_oracle.so")
+        L.tgv_oracle_forward.argtypes = [_f32p] * 6 + [_int] * 6
+        L.tgv_oracle_backward.argtypes = [_f32p] * 10 + [_int] * 6
+        L.tgv_oracle_forward_f64.argtypes = [_f64p] * 6 + [_int] * 6
+        L.tgv_oracle_backward_f64.argtypes = [_f64p] * 10 + [_int] * 6
+        L.tgv_oracle_set_quirks.argtypes = [_int] * 7
+        L.tgv_oracle_set_quirks.restype = None
+        L.tgv_oracle_reset_id.argtypes = [_int]
+        L.tgv_oracle_reset_id.restype = None
+        L.tgv_oracle_get_state.argtypes = [_int, _f64p, _int]
+        L.tgv_oracle_set_state.argtypes = [_int, _f64p]
+        L.tgv_oracle_lipschitz.argtypes = [_f32p, _f32p, _int, _int, _f32p]
+        L.tgv_oracle_lipschitz.restype = ctypes.c_double
+        L.tgv_oracle_lipschitz_f64.argtypes = [_f64p, _f64p, _int, _int, _f64p]
+        L.tgv_oracle_lipschitz_f64.restype = ctypes.c_double
+        L.tgv_oracle_forward_iter.argtypes = [_f32p] * 8 + [_int] * 3 + [ctypes.c_float]
+        L.tgv_oracle_forward_iter.restype = None
+        L.tgv_oracle_forward_iter_f64.argtypes = [_f64p] * 8 + [_int] * 3 + [ctypes.c_double]
+        L.tgv_oracle_forward_iter_f64.restype = None
+        L.tgv_oracle_guard_f64.argtypes = [_f64p, ctypes.c_long, _int, _f64p, _f64p]
+        L.tgv_oracle_guard_f32.argtypes = [_f32p, ctypes.c_long, _int, _f64p, _f64p]
+        L.tgv_oracle_set_threads.argtypes = [_int]
+        L.tgv_oracle_set_threads.restype = None
+        L.tgv_oracle_jt_f64.argtypes = [_f64p] * 4 + [_int] * 4 + [_f64p] * 2
+        L.tgv_oracle_jt_f64.restype = None
+
+    def forward(self, dx, dy, c, b, init, its, pid=0, f64=False):
+        dt = np.float64 if f64 else np.float32
+        dx, dy, c, b, init = (_c(a, dt) for a in (dx, dy, c, b, init))
+        n, ic, ih, iw = b.shape
+        assert dx.shape == (n, 2, ih, iw) and dy.shape == dx.shape and init.shape == (n, 3 * ic, ih, iw)
+        out = np.empty_like(init)
+        P = _p64 if f64 else _p32
+        fn = self.lib.tgv_oracle_forward_f64 if f64 else self.lib.tgv_oracle_forward
+        rc = fn(P(dx), P(dy), P(c), P(b), P(init), P(out), n, ic, ih, iw, int(its), int(pid))
+        if rc:
+            raise RuntimeError("tgv_oracle_forward failed with code %d" % rc)
+        return out
+
+    def backward(self, gin, dx, dy, c, b, its, pid=0, f64=False):
+        """Returns (gx, gy, gc, gb, gi); `gin` (a writable array) may be scrubbed in place."""
+        dt = np.float64 if f64 else np.float32
+        dx, dy, c, b = (_c(a, dt) for a in (dx, dy, c, b))
+        if gin.dtype != dt or not gin.flags["C_CONTIGUOUS"]:
+            gin = _c(gin, dt).copy()
+        n, ic, ih, iw = b.shape
+        assert gin.shape == (n, 3 * ic, ih, iw)
+        gx, gy, gc = np.empty_like(dx), np.empty_like(dy), np.empty_like(c)
+        gb, gi = np.empty_like(b), np.empty_like(gin)
+        P = _p64 if f64 else _p32
+        fn = self.lib.tgv_oracle_backward_f64 if f64 else self.lib.tgv_oracle_backward
+        rc = fn(P(dx), P(dy), P(c), P(b), P(gin), P(gx), P(gy), P(gc), P(gb), P(gi), n, ic, ih, iw,
+                int(its), int(pid))
+        if rc:
+            raise RuntimeError("tgv_oracle_backward failed with code %d" % rc)
+        return gx, gy, gc, gb, gi
+
+    def set_quirks(self, end_uses_ckpt_y=1, skip_iter0_adjoint=1, getyk_rebuild=1, scale_factors=1,
+                   clamp=1, guard=1, dw_div=1):
+        self.lib.tgv_oracle_set_quirks(end_uses_ckpt_y, skip_iter0_adjoint, getyk_rebuild,
+                                       scale_factors, clamp, guard, dw_div)
+
+    def reset_id(self, pid):
+        self.lib.tgv_oracle_reset_id(int(pid))
+
+    def get_state(self, pid, f64=False):
+        s = np.zeros(6, np.float64)
+        self.lib.tgv_oracle_get_state(int(pid), _p64(s), int(f64))
+        return s
+
+    def set_state(self, pid, state6):
+        s = _c(state6, np.float64)
+        self.lib.tgv_oracle_set_state(int(pid), _p64(s))
+
+    def lipschitz(self, dx, dy, f64=False):
+        """dx, dy: (2,H,W) unscaled.  Returns (L, per-pixel bound (H,W))."""
+        dt = np.float64 if f64 else np.float32
+        dx, dy = _c(dx, dt), _c(dy, dt)
+        _, ih, iw = dx.shape
+        st = np.zeros((ih, iw), dt)
+        P = _p64 if f64 else _p32
+        fn = self.lib.tgv_oracle_lipschitz_f64 if f64 else self.lib.tgv_oracle_lipschitz
+        return fn(P(dx), P(dy), ih, iw, P(st)), st
+
+    def forward_iter(self, dx, dy, c, b, x, y, t, want_x05=False, f64=False):
+        """One iteration on one sample: dx, dy (2,H,W) unscaled, c (H,W), b (C,H,W), x / y (3,C,H,W)
+        (any shape with 3*C*H*W elements).  Returns (x_new, y_new[, x05])."""
+        dt = np.float64 if f64 else np.float32
+        dx, dy, c, b, y = (_c(a, dt) for a in (dx, dy, c, b, y))
+        x = _c(x, dt).copy()
+        ic, ih, iw = b.shape
+        yout = np.empty_like(y)
+        x05 = np.empty_like(y) if want_x05 else None
+        P = _p64 if f64 else _p32
+        fn = self.lib.tgv_oracle_forward_iter_f64 if f64 else self.lib.tgv_oracle_forward_iter
+        fn(P(dx), P(dy), P(c), P(b), P(x), P(y), P(yout), P(x05) if want_x05 else None, ic, ih, iw, t)
+        return (x, yout, x05) if want_x05 else (x, yout)
+
+    def jt(self, dx, dy, y, g, end_form=False, q7=False):
+        """J(y)^T g of the gradient step (double precision, one channel): dx, dy (2,H,W) unscaled,
+        y, g (3,H,W).  Returns (out (3,H,W), weight-gradient increments (4,H,W))."""
+        dx, dy, y, g = (_c(a, np.float64) for a in (dx, dy, y, g))
+        _, ih, iw = y.shape
+        out = np.zeros((3, ih, iw))
+        gw = np.zeros((4, ih, iw))
+        self.lib.tgv_oracle_jt_f64(_p64(dx), _p64(dy), _p64(y), _p64(g), ih, iw, int(end_form), int(q7),
+                                   _p64(out), _p64(gw))
+        return out, gw
+
+    def guard(self, g, run, av, f32=False):
+        g = _c(g, np.float32 if f32 else np.float64).copy().ravel()
+        avv = ctypes.c_double(av)
+        stats = np.zeros(4, np.float64)
+        fn = self.lib.tgv_oracle_guard_f32 if f32 else self.lib.tgv_oracle_guard_f64
+        act = fn(_p32(g) if f32 else _p64(g), g.size, int(run), ctypes.byref(avv), _p64(stats))
+        return g, avv.value, act, stats
+
+    def set_threads(self, n):
+        self.lib.tgv_oracle_set_threads(int(n))
