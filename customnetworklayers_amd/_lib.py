@@ -33,6 +33,20 @@ def _load():
     lib.tvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
     lib.inpaint_selftest_math.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_uint]
     lib.tvinpaint_last_error.restype = ctypes.c_char_p
+    lib.tgvinpaint_forward.argtypes = [_f32p] * 6 + [_int] * 6 + [ctypes.c_void_p]
+    lib.tgvinpaint_backward.argtypes = [_f32p] * 10 + [_int] * 6 + [ctypes.c_void_p]
+    lib.tgvinpaint_get_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tgvinpaint_set_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tgvinpaint_reset_id.argtypes = [_int]
+    lib.tgvinpaint_guard_stats.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tgvinpaint_slot_bytes.argtypes = [_int]
+    lib.tgvinpaint_slot_bytes.restype = ctypes.c_longlong
+    lib.tgvinpaint_lipschitz.argtypes = [_int, ctypes.POINTER(ctypes.c_double), _int]
+    lib.tgvinpaint_guard_decide.argtypes = [_int, ctypes.c_double, ctypes.c_double,
+                                            ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    lib.tgvinpaint_profile.argtypes = [_int]
+    lib.tgvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
+    lib.tgvinpaint_last_error.restype = ctypes.c_char_p
     return lib
 
 

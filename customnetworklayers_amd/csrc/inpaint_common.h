@@ -170,9 +170,12 @@ __device__ inline unsigned int wave_sum_u(unsigned int v) {
 }
 
 // pass 1: sum, max, counts, position of the last non-finite entry.  One set of atomics per block.
+// With clamp_mean (TGV) an entry above max_tol enters the mean as max_tol; the TV layer's mean
+// takes it as it is.
 template <class T>
 __global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__ g, long long n,
-                                                           GuardStats* __restrict__ st, double max_tol) {
+                                                           GuardStats* __restrict__ st, double max_tol,
+                                                           bool clamp_mean = false) {
   __shared__ double s_sum[4];
   __shared__ unsigned long long s_mx[4], s_last[4];
   __shared__ unsigned int s_above[4], s_invalid[4];
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__
     T v = g[i];
     if (finite_value(v)) {
       double a = fabs((double)v);
-      s += a;
+      s += (clamp_mean && a > max_tol) ? max_tol : a;
       unsigned long long bits = (unsigned long long)__double_as_longlong(a);
       mx = bits > mx ? bits : mx;
       above += (a > max_tol);
@@ -222,13 +225,16 @@ __global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__
 // pass 2 (does nothing unless pass 1 saw a non-finite entry): sum of |g| behind the last one
 template <class T>
 __global__ __launch_bounds__(256) void guard_tail_kernel(const T* __restrict__ g, long long n,
-                                                         GuardStats* __restrict__ st) {
+                                                         GuardStats* __restrict__ st, double max_tol = 0,
+                                                         bool clamp_mean = false) {
   if (st->num_invalid == 0) return;
   const long long start = (long long)st->last_invalid1;
   double s = 0;
   for (long long i = start + (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x)
-    s += fabs((double)g[i]);
+       i += (long long)gridDim.x * blockDim.x) {
+    const double a = fabs((double)g[i]);
+    s += (clamp_mean && a > max_tol) ? max_tol : a;
+  }
   s = wave_sum(s);
   if ((threadIdx.x & 63) == 0 && s != 0) atomicAdd(&st->tail_sum, s);
 }
@@ -277,5 +283,122 @@ inline int guard_grid(long long n) {
   long long blocks = (n + 256 * 16 - 1) / (256 * 16);
   return (int)std::max<long long>(1, std::min<long long>(blocks, 1024));
 }
+
+// ---------------------------------------------------------------------------------------------
+// small generic kernels shared by both layers
+// ---------------------------------------------------------------------------------------------
+inline int grid1d(long long n) { return (int)std::max<long long>(1, std::min<long long>((n + 255) / 256, 1 << 20)); }
+inline int grid_stride(long long n) { return (int)std::max<long long>(1, std::min<long long>((n + 1023) / 1024, 4096)); }
+
+// Segment flush: fp32 accumulator into its fp64 total, then zero (copy_and_set_to_0,
+// TVInpaintFista.cu:178-218; TGVInpaintFistaHelp.cu:178-216).
+static __global__ __launch_bounds__(256) void flush_kernel(float* __restrict__ acc, double* __restrict__ total,
+                                                           long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    total[i] = (double)acc[i] + total[i] / 1.;
+    acc[i] = 0.f;
+  }
+}
+
+static __global__ __launch_bounds__(256) void fill_zero_f32(float* __restrict__ p, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    p[i] = 0.f;
+}
+
+// Zero several buffers in one launch (blockIdx.y picks the buffer).
+struct ZeroList {
+  void* ptr[24];
+  long long bytes[24];
+};
+static __global__ __launch_bounds__(256) void fill_zero_many(ZeroList z) {
+  uint32_t* p = static_cast<uint32_t*>(z.ptr[blockIdx.y]);
+  const long long n = z.bytes[blockIdx.y] / 4;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    p[i] = 0u;
+}
+
+// Zero the non-finite entries of the caller's upstream gradient in place
+// (TVInpaintFista.cu:1609-1623; TGVInpaintFistaBetas.cu:2690-2701).
+static __global__ __launch_bounds__(256) void scrub_kernel(float* __restrict__ g, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    const float v = g[i];
+    if (!finite_value(v)) g[i] = 0.f;
+  }
+}
+
+// An entry beyond the guard's tolerance: zeroed (TV) or clamped to +-clamp_to (TGV).
+template <class T>
+__device__ inline T guard_limit(T v, const GuardParams& p) {
+  if (!finite_value(v)) return T(0);
+  if (fabs((double)v) > p.max_tolerance) return p.clamp_to > 0 ? (T)(v > 0 ? p.clamp_to : -p.clamp_to) : T(0);
+  return v;
+}
+
+// Guarded fp64 total -> fp32 output: limit, kill / rescale, global multiplier, then the chain
+// factor of the weight scaling (TVInpaintFista.cu:1795-1818; TGVInpaintFistaBetas.cu:3024-3050).
+// The chain factor is chain_const, or chain_per_sample[i / per_sample] when that pointer is given.
+static __global__ __launch_bounds__(256) void finalize_f64(const double* __restrict__ total, float* __restrict__ out,
+                                                           long long n, const GuardState* __restrict__ gs, int k,
+                                                           GuardParams p, float global_mult, double chain_const,
+                                                           const double* __restrict__ chain_per_sample,
+                                                           long long per_sample) {
+  const double mult = gs->scale[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    double v = guard_limit(total[i], p);
+    if (mult != 1.0) v = (mult == 0.0) ? 0.0 : v * mult;
+    const float f = (float)(v * global_mult);
+    const double chain = chain_per_sample ? chain_per_sample[i / per_sample] : chain_const;
+    out[i] = (chain == 1.0) ? f : (float)(chain * (double)f);
+  }
+}
+
+// Gradient wrt the starting point, guarded as a float tensor (TVInpaintFista.cu:1784-1791,1816).
+static __global__ __launch_bounds__(256) void finalize_f32(const float* __restrict__ src, float* __restrict__ out,
+                                                           long long n, const GuardState* __restrict__ gs, int k,
+                                                           GuardParams p) {
+  const double mult = gs->scale[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    float v = guard_limit(src[i], p);
+    if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
+    out[i] = 0.0f + v;
+  }
+}
+
+// Optional timing of a layer's dominant kernel with HIP events on the launch stream.
+struct KernelTimer {
+  bool enabled = false;
+  std::vector<hipEvent_t> pool;  // start/stop pairs
+  size_t used = 0;
+  void mark(hipStream_t stream) {
+    if (!enabled) return;
+    if (used == pool.size()) {
+      hipEvent_t e;
+      if (hipEventCreate(&e) != hipSuccess) { enabled = false; return; }
+      pool.push_back(e);
+    }
+    (void)hipEventRecord(pool[used++], stream);
+  }
+  int read(double* total_ms, int* launches) {
+    double total = 0;
+    int count = 0;
+    for (size_t i = 0; i + 1 < used; i += 2) {
+      INPAINT_HIP(hipEventSynchronize(pool[i + 1]));
+      float ms = 0;
+      INPAINT_HIP(hipEventElapsedTime(&ms, pool[i], pool[i + 1]));
+      total += ms;
+      count++;
+    }
+    used = 0;
+    if (total_ms) *total_ms = total;
+    if (launches) *launches = count;
+    return 0;
+  }
+};
 
 }  // namespace inpaint

@@ -1,0 +1,1080 @@
+// Huber-TGV FISTA inpainting layer for MI355X (gfx950): kernels, per-id state and the C ABI.
+//
+// What the layer computes is fixed by the reference's kernels
+// (cudaTGV/cudaCode/TGVInpaintFistaBetas.cu, cited per function below as TGV.cu; helpers in
+// cudaTGV/cudaCode/TGVInpaintFistaHelp.cu, TGVH.cu).  How it is computed is not:
+//   * samples are a grid dimension (n >= 1), each with its own Lipschitz constant, which is
+//     reduced and applied on the device (no host round trip, no textures);
+//   * state tensors are (n, 3*C, H, W): variable-major (u, v1, v2) inside a sample, as the
+//     reference's (3, C, H, W) tensors are for n == 1;
+//   * checkpoints, the x05 history, the adjoint iterates, the per-segment fp32 accumulators and
+//     their fp64 totals live in one device arena per id;
+//   * the output guard runs on the device.
+//
+// Arithmetic contract: as for the TV layer, every value that can reach a Huber / prox switch is
+// computed with the operation order of the reference source, IEEE division and square root and no
+// fused multiply-add (build with -ffp-contract=off).  CUDA's rsqrtf (2 ulp, bits not recoverable
+// from the sources) is taken as 1.0f / sqrtf(x), both correctly rounded.
+#include "inpaint_common.h"
+#include "../../include/tgvinpaint.h"
+
+#include <cstddef>
+#include <cstdlib>
+
+namespace {
+
+using namespace inpaint;
+
+// TGV.cu:58-60,70,78,87-93; TGVH.cu:24-41
+constexpr float kD0 = 0.2f, kD1 = 0.2f, kD2 = 0.2f;
+constexpr float kBeta = 4.0f;
+constexpr float kClipLocalGrad = 2000.0f;
+constexpr float kLocalGCMult = 0.1f;
+constexpr float kLocalGXMult = 0.1f;
+constexpr float kLocalGBMult = 1.0f;
+constexpr float kGlobalGMult = 0.1f;
+const GuardParams kGuard = {5000000., 5000000., 35., 10., 0.95};
+
+constexpr int BX = 64, BY = 4;  // one pixel per thread, a wavefront per image row segment
+
+// -------------------------------------------------------------------------------------------------
+// device helpers
+// -------------------------------------------------------------------------------------------------
+struct Plane {  // zero outside the image, like the reference's haloed shared-memory tiles (TGV.cu:1581-1597)
+  const float* f;
+  int H, W;
+  __device__ __forceinline__ float at(int h, int w) const {
+    return (h >= 0 && h < H && w >= 0 && w < W) ? f[(size_t)h * W + w] : 0.f;
+  }
+};
+
+__device__ __forceinline__ float rsq(float x) { return 1.0f / sqrtf(x); }
+__device__ __forceinline__ float clampT(const float* f, int h, int w, int H, int W) {
+  h = min(max(h, 0), H - 1);
+  w = min(max(w, 0), W - 1);
+  return f[(size_t)h * W + w];
+}
+
+// -------------------------------------------------------------------------------------------------
+// Lipschitz bound: TGV.cu:101-148 per pixel, TGV.cu:2516-2527 for the reduction.
+// maxbits[s] must hold the bit pattern of 32.0f (= float(max(12, 8*beta) + 0.000001)) on entry.
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BX* BY) void tgv_lipschitz_kernel(const float* __restrict__ dx_, const float* __restrict__ dy_,
+                                                               int H, int W, unsigned int* __restrict__ maxbits) {
+  const int w = blockIdx.x * BX + threadIdx.x, h = blockIdx.y * BY + threadIdx.y;
+  const size_t HW = (size_t)H * W;
+  const float* dx = dx_ + (size_t)blockIdx.z * 2 * HW;
+  const float* dy = dy_ + (size_t)blockIdx.z * 2 * HW;
+  const float* betaX = dx + HW;
+  const float* betaY = dy + HW;
+  float v = 0.f;
+  if (w < W && h < H) {
+    const float wx_0 = (w > 0) ? clampT(dx, h, w - 1, H, W) : 0.f;
+    const float wx_1 = (w < W - 1) ? clampT(dx, h, w, H, W) : 0.f;
+    const float wy_0 = (h > 0) ? clampT(dy, h - 1, w, H, W) : 0.f;
+    const float wy_1 = (h < H - 1) ? clampT(dy, h, w, H, W) : 0.f;
+    const float betaTX_1y = (h < H - 1) ? clampT(betaX, h, w, H, W) : 0.f;
+    const float betaTX_1x = (w < W - 1) ? clampT(betaX, h, w, H, W) : 0.f;
+    const float betaTX_0x = (w > 0) ? clampT(betaX, h - 1, w, H, W) : 0.f;  // sic: (w, h-1) under w > 0 (TGV.cu:116)
+    const float betaTX_0y = (h > 0) ? clampT(betaX, h, w - 1, H, W) : 0.f;  // sic: (w-1, h) under h > 0 (TGV.cu:117)
+    const float betaTY_1y = (h < H - 1) ? clampT(betaY, h, w, H, W) : 0.f;
+    const float betaTY_1x = (w < W - 1) ? clampT(betaY, h, w, H, W) : 0.f;
+    const float betaTY_0x = (w > 0) ? clampT(betaY, h - 1, w, H, W) : 0.f;
+    const float betaTY_0y = (h > 0) ? clampT(betaY, h, w - 1, H, W) : 0.f;
+    float weightx = 0.f, weighty1 = 0.f, weighty2 = 0.f;
+    if (h > 0) {
+      weightx += 3 * wy_0;
+      weighty1 += 2 * betaTX_0y;
+      weighty2 += 2 * betaTY_0y;
+    }
+    if (w > 0) {
+      weightx += 3 * wx_0;
+      weighty1 += 2 * betaTX_0x;
+      weighty2 += 2 * betaTY_0x;
+    }
+    weightx += 3 * (wy_1 + wx_1);
+    weighty1 += 2 * betaTX_1x + 2 * betaTX_1y + 3 * wx_1;
+    weighty2 += 2 * betaTY_1x + 2 * betaTY_1y + 3 * wy_1;
+    v = fmaxf(weightx, fmaxf(weighty1, weighty2));
+  }
+  // non-negative floats order like their bit patterns; anything else (negative, NaN) never wins
+  // against the 32.0f start value in the reference's std::max either
+  unsigned int bits = (v > 0.f) ? __float_as_uint(v) : 0u;
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned int o = __shfl_down(bits, off, 64);
+    bits = o > bits ? o : bits;
+  }
+  if (threadIdx.x == 0 && bits > __float_as_uint(32.0f)) atomicMax(&maxbits[blockIdx.z], bits);
+}
+
+static __global__ void tgv_lipschitz_init(unsigned int* maxbits, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) maxbits[i] = __float_as_uint((float)(fmax(12., 8. * (double)kBeta) + 0.000001));
+}
+
+__device__ __forceinline__ double lipschitz_from_bits(unsigned int bits) {
+  float oneL = __uint_as_float(bits);
+  oneL = (float)(1. / (double)(oneL + 0.01f));  // TGV.cu:2526
+  return (double)oneL;                           // TGV.cu:2527: double L = oneL
+}
+
+// L-scaled private copies of the four weight fields (TGV.cu:2495-2499,2528-2531): (n,H,W) each.
+__global__ __launch_bounds__(256) void tgv_scale_kernel(const float* __restrict__ dx, const float* __restrict__ dy,
+                                                        const unsigned int* __restrict__ maxbits, float* __restrict__ wx,
+                                                        float* __restrict__ wy, float* __restrict__ bx,
+                                                        float* __restrict__ by, double* __restrict__ Ls, long long HW,
+                                                        long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long s = i / HW, p = i - s * HW;
+  const double L = lipschitz_from_bits(maxbits[s]);
+  if (p == 0) Ls[s] = L;
+  wx[i] = (float)(L * (double)dx[s * 2 * HW + p]);
+  wy[i] = (float)(L * (double)dy[s * 2 * HW + p]);
+  bx[i] = (float)(L * (double)dx[s * 2 * HW + HW + p]);
+  by[i] = (float)(L * (double)dy[s * 2 * HW + HW + p]);
+}
+
+// -------------------------------------------------------------------------------------------------
+// forward iteration: TGV.cu:1546-1776; with x05 != nullptr also TGV.cu:2005-2235
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(BX* BY) void tgv_forward_px(
+    const float* __restrict__ wx_, const float* __restrict__ wy_, const float* __restrict__ bx_,
+    const float* __restrict__ by_, const float* __restrict__ cf_, const float* __restrict__ b_,
+    const float* __restrict__ xin_, float* __restrict__ xout_, const float* __restrict__ yin_,
+    float* __restrict__ yout_, float* __restrict__ x05_, int C, int H, int W, float t) {
+  const int w = blockIdx.x * BX + threadIdx.x, h = blockIdx.y * BY + threadIdx.y;
+  if (w >= W || h >= H) return;
+  const size_t HW = (size_t)H * W, CHW = HW * C, S = 3 * CHW;
+  const size_t smp = blockIdx.z;
+  const float *wx = wx_ + smp * HW, *wy = wy_ + smp * HW, *bx = bx_ + smp * HW, *by = by_ + smp * HW;
+  const size_t p = (size_t)h * W + w;
+  const float conf = cf_[smp * HW + p];
+  const float wx_0 = (w > 0) ? wx[p - 1] : 0.f;
+  const float wx_1 = (w < W - 1) ? wx[p] : 0.f;
+  const float wy_0 = (h > 0) ? wy[p - W] : 0.f;
+  const float wy_1 = (h < H - 1) ? wy[p] : 0.f;
+  const float wx_2 = (h > 0 && w < W - 1) ? wx[p - W] : 0.f;
+  const float wy_2 = (w > 0 && h < H - 1) ? wy[p - 1] : 0.f;
+  const float bX_u = (h > 0) ? bx[p - W] : 0.f, bY_u = (h > 0) ? by[p - W] : 0.f;
+  const float bX_l = (w > 0) ? bx[p - 1] : 0.f, bY_l = (w > 0) ? by[p - 1] : 0.f;
+  const float bX_c = bx[p], bY_c = by[p];
+  const float oneL = 1.0f;  // TGV.cu:2527
+  for (int ch = 0; ch < C; ch++) {
+    const size_t o = smp * S + (size_t)ch * HW;
+    const Plane Y0{yin_ + o, H, W}, Y1{yin_ + o + CHW, H, W}, Y2{yin_ + o + 2 * CHW, H, W};
+    const float x_ = xin_[o + p];
+    const float bb = b_[smp * CHW + (size_t)ch * HW + p];
+    float yc = Y0.f[p];
+    float yt = yc;
+    float y1_new = Y1.f[p], y2_new = Y2.f[p];
+    const float y1_c = y1_new, y2_c = y2_new;
+    if (h > 0) {  // TGV.cu:1613-1640
+      const float betaTX = bX_u, betaTY = bY_u;
+      const float zij_1 = (w < W - 1) ? ((Y0.at(h - 1, w + 1) - Y0.at(h - 1, w)) - Y1.at(h - 1, w)) : 0.f;
+      const float zij_2 = ((yc - Y0.at(h - 1, w)) - Y2.at(h - 1, w));
+      const float hwx = fminf(1.f, rsq(zij_2 * zij_2 * wy_0 + zij_1 * zij_1 * wx_2) * kD0);
+      const float uij1_2 = (y1_c - Y1.at(h - 1, w));
+      const float uij1_1 = (w < W - 1) ? (Y1.at(h - 1, w + 1) - Y1.at(h - 1, w)) : 0.f;
+      const float hwy1 = fminf(1.f, rsq(betaTX * (uij1_2 * uij1_2 + uij1_1 * uij1_1)) * kD1);
+      const float uij2_1 = (w < W - 1) ? (Y2.at(h - 1, w + 1) - Y2.at(h - 1, w)) : 0.f;
+      const float uij2_2 = (y2_c - Y2.at(h - 1, w));
+      const float hwy2 = fminf(1.f, rsq(betaTY * (uij2_2 * uij2_2 + uij2_1 * uij2_1)) * kD2);
+      yt -= wy_0 * oneL * (zij_2 * hwx);
+      y1_new -= (betaTX * oneL) * (uij1_2 * hwy1);
+      y2_new -= (betaTY * oneL) * (uij2_2 * hwy2);
+    }
+    if (w > 0) {  // TGV.cu:1641-1668
+      const float betaTX = bX_l, betaTY = bY_l;
+      const float zij_1 = ((yc - Y0.at(h, w - 1)) - Y1.at(h, w - 1));
+      const float zij_2 = (h < H - 1) ? ((Y0.at(h + 1, w - 1) - Y0.at(h, w - 1)) - Y2.at(h, w - 1)) : 0.f;
+      const float hwx = fminf(1.f, rsq(zij_2 * zij_2 * wy_2 + zij_1 * zij_1 * wx_0) * kD0);
+      const float uij1_1 = (y1_c - Y1.at(h, w - 1));
+      const float uij1_2 = (h < H - 1) ? (Y1.at(h + 1, w - 1) - Y1.at(h, w - 1)) : 0.f;
+      const float hwy1 = fminf(1.f, rsq(betaTX * (uij1_2 * uij1_2 + uij1_1 * uij1_1)) * kD1);
+      const float uij2_1 = (y2_c - Y2.at(h, w - 1));
+      const float uij2_2 = (h < H - 1) ? (Y2.at(h + 1, w - 1) - Y2.at(h, w - 1)) : 0.f;
+      const float hwy2 = fminf(1.f, rsq(betaTY * (uij2_2 * uij2_2 + uij2_1 * uij2_1)) * kD2);
+      yt -= wx_0 * oneL * (zij_1 * hwx);
+      y1_new -= (betaTX * oneL) * (uij1_1 * hwy1);
+      y2_new -= (betaTY * oneL) * (uij2_1 * hwy2);
+    }
+    {  // TGV.cu:1669-1691
+      const float betaTX = bX_c, betaTY = bY_c;
+      const float zij_1 = (w < W - 1) ? ((yc - Y0.at(h, w + 1)) + y1_c) : 0.f;
+      const float zij_2 = (h < H - 1) ? ((yc - Y0.at(h + 1, w)) + y2_c) : 0.f;
+      const float hwx = fminf(1.f, rsq(zij_2 * zij_2 * wy_1 + zij_1 * zij_1 * wx_1) * kD0);
+      const float uij1_1 = (w < W - 1) ? (y1_c - Y1.at(h, w + 1)) : 0.f;
+      const float uij1_2 = (h < H - 1) ? (y1_c - Y1.at(h + 1, w)) : 0.f;
+      const float hwy1 = fminf(1.f, rsq(betaTX * (uij1_2 * uij1_2 + uij1_1 * uij1_1)) * kD1);
+      const float uij2_1 = (w < W - 1) ? (y2_c - Y2.at(h, w + 1)) : 0.f;
+      const float uij2_2 = (h < H - 1) ? (y2_c - Y2.at(h + 1, w)) : 0.f;
+      const float hwy2 = fminf(1.f, rsq(betaTY * (uij2_2 * uij2_2 + uij2_1 * uij2_1)) * kD2);
+      yt -= wy_1 * oneL * (zij_2 * hwx);
+      y1_new -= (betaTX * oneL) * (uij1_2 * hwy1);
+      y2_new -= (betaTY * oneL) * (uij2_2 * hwy2) + wy_1 * oneL * (zij_2 * hwx);
+      yt -= wx_1 * oneL * (zij_1 * hwx);
+      y1_new -= (betaTX * oneL) * (uij1_1 * hwy1) + wx_1 * oneL * (zij_1 * hwx);
+      y2_new -= (betaTY * oneL) * (uij2_1 * hwy2);
+    }
+    // aux variables: momentum only (TGV.cu:1686-1690)
+    yout_[o + CHW + p] = y1_new + t * (y1_new - xin_[o + CHW + p]);
+    yout_[o + 2 * CHW + p] = y2_new + t * (y2_new - xin_[o + 2 * CHW + p]);
+    xout_[o + CHW + p] = y1_new;
+    xout_[o + 2 * CHW + p] = y2_new;
+    if (x05_) {  // TGV.cu:2146-2147,2196
+      x05_[o + p] = yt;
+      x05_[o + CHW + p] = y1_new;
+      x05_[o + 2 * CHW + p] = y2_new;
+    }
+    // Huber-1 prox on u (TGV.cu:1740-1744)
+    float x_loc = (conf * bb + yt) / (1.f + conf);
+    yc = yt - conf;
+    yt = yt + conf;
+    if (yc > 1.f + bb) x_loc = yc;
+    if (yt < bb - 1.f) x_loc = yt;
+    yout_[o + p] = x_loc + t * (x_loc - x_);
+    xout_[o + p] = x_loc;
+  }
+}
+
+// y_{k+1} from x05[k] (xa), x05[k-1] (xb): TGV.cu:1478-1541; aux variables are x05[k] itself.
+__global__ __launch_bounds__(256) void tgv_getyk_kernel(const float* __restrict__ cf, const float* __restrict__ b,
+                                                        const float* __restrict__ xa, const float* __restrict__ xb,
+                                                        float* __restrict__ yk, int C, long long HW, long long total,
+                                                        float t) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // over n*HW pixels
+  if (i >= total) return;
+  const long long s = i / HW, p = i - s * HW;
+  const long long CHW = HW * C;
+  const float conf = cf[i];
+  for (int ch = 0; ch < C; ch++) {
+    const long long q = s * 3 * CHW + ch * HW + p;
+    const float bb = b[s * CHW + ch * HW + p];
+    float diff = bb - xa[q];
+    float sign = (diff < 0) ? -1.f : 1.f;
+    float v;
+    if (1. + (double)conf >= (double)(sign * diff)) {
+      const float xk = (conf * bb + xa[q]) / (1.f + conf);
+      const float xkm = (conf * bb + xb[q]) / (1.f + conf);
+      v = xk + t * (xk - xkm);
+    } else {
+      const float xk = (conf <= sign * diff) ? bb - diff + sign * conf : bb;
+      diff = bb - xb[q];
+      sign = (diff < 0) ? -1.f : 1.f;
+      v = xk + t * (xk - ((conf <= sign * diff) ? bb - diff + sign * conf : bb));
+    }
+    yk[q] = v;
+    yk[q + CHW] = xa[q + CHW];
+    yk[q + 2 * CHW] = xa[q + 2 * CHW];
+  }
+}
+
+// Prox adjoint + confidence / rhs gradient: TGV.cu:592-612, 1418-1442 (and 166-182 for the first step).
+template <bool FIRST>
+__device__ __forceinline__ void prox_adjoint(float df_dxk, float bb, float x05v, float conf, float& g05,
+                                             float& gc, float& gb) {
+  const float diff = bb - x05v;
+  const float sign = (diff < 0) ? -1.f : 1.f;
+  if (1. + (double)conf >= (double)(sign * diff)) {
+    gc += df_dxk * (bb / (1.f + conf) - (conf * bb + x05v) / ((1.f + conf) * (1.f + conf))) * kLocalGCMult;
+    g05 = df_dxk / (1.f + conf);
+    gb += df_dxk * conf / (1.f + conf) * kLocalGBMult;
+  } else if (FIRST) {
+    g05 = df_dxk;
+    gc += sign * df_dxk * kLocalGCMult;
+    gb = 0.f;  // TGV.cu:181
+  } else if (conf >= sign * diff) {
+    g05 = 0.f;
+    gb += df_dxk * kLocalGBMult;
+  } else {
+    g05 = df_dxk;
+    gc += sign * df_dxk * kLocalGCMult;
+  }
+}
+
+// First adjoint step: TGV.cu:151-218.
+__global__ __launch_bounds__(256) void tgv_adjoint_first(const float* __restrict__ cf, const float* __restrict__ b,
+                                                         const float* __restrict__ x05, float* __restrict__ gc,
+                                                         float* __restrict__ gb, float* __restrict__ g05,
+                                                         const float* __restrict__ gin, int C, long long HW,
+                                                         long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long s = i / HW, p = i - s * HW;
+  const long long CHW = HW * C;
+  const float conf = cf[i];
+  float gcv = gc[i];
+  for (int ch = 0; ch < C; ch++) {
+    const long long q = s * 3 * CHW + ch * HW + p;
+    const long long qb = s * CHW + ch * HW + p;
+    float g05v, gbv = gb[qb];
+    prox_adjoint<true>(gin[q], b[qb], x05[q], conf, g05v, gcv, gbv);
+    g05[q] = g05v;
+    gb[qb] = gbv;
+    g05[q + CHW] = gin[q + CHW];          // TGV.cu:215
+    g05[q + 2 * CHW] = gin[q + 2 * CHW];  // TGV.cu:216
+  }
+  gc[i] = gcv;
+}
+
+// Huber weight of the segment-start kernel: (float)(1. / (double)max(1, hub / delta)), TGV.cu:1133.
+// For a float m >= 1 the double quotient rounded to float equals the float quotient: a
+// double-rounding slip needs 1/m within 2^-54 (relative) of a 25-bit number M, but 1 - m*M is a
+// multiple of 2^-49 and cannot be that small unless it is zero.
+__device__ __forceinline__ float huber_w_end(float hub, float delta) { return 1.0f / fmaxf(1.f, hub / delta); }
+
+// Main adjoint step (TGV.cu:224-644) and, with END, the segment-start variant (TGV.cu:1061-1472)
+// that linearises at the checkpoint y and writes the same Jacobian with sqrt and divisions.
+// y is y_{k+1} rebuilt by tgv_getyk_kernel, or the checkpoint y.
+template <bool END>
+__global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
+    const float* __restrict__ wx_, const float* __restrict__ wy_, const float* __restrict__ bx_,
+    const float* __restrict__ by_, const float* __restrict__ cf_, const float* __restrict__ b_,
+    const float* __restrict__ x05_, float* __restrict__ gc_, float* __restrict__ gb_, float* __restrict__ gwx_,
+    float* __restrict__ gwy_, const float* __restrict__ g05_in_, float* __restrict__ g05_out_, float* __restrict__ gxk_,
+    float* __restrict__ gxk_m1_, const float* __restrict__ y_, int C, int H, int W, float t) {
+  const int w = blockIdx.x * BX + threadIdx.x, h = blockIdx.y * BY + threadIdx.y;
+  if (w >= W || h >= H) return;
+  const size_t HW = (size_t)H * W, CHW = HW * C, S = 3 * CHW;
+  const size_t smp = blockIdx.z;
+  const float *wx = wx_ + smp * HW, *wy = wy_ + smp * HW, *bx = bx_ + smp * HW, *by = by_ + smp * HW;
+  const size_t p = (size_t)h * W + w;
+  const float conf = cf_[smp * HW + p];
+  const float wx_0 = (w > 0) ? wx[p - 1] : 0.f;
+  const float wx_1 = (w < W - 1) ? wx[p] : 0.f;
+  const float wy_0 = (h > 0) ? wy[p - W] : 0.f;
+  const float wy_1 = (h < H - 1) ? wy[p] : 0.f;
+  const float wx_2 = (h > 0 && w < W - 1) ? wx[p - W] : 0.f;
+  const float wy_2 = (w > 0 && h < H - 1) ? wy[p - 1] : 0.f;
+  const float bX_u = (h > 0) ? bx[p - W] : 0.f, bY_u = (h > 0) ? by[p - W] : 0.f;
+  const float bX_l = (w > 0) ? bx[p - 1] : 0.f, bY_l = (w > 0) ? by[p - 1] : 0.f;
+  const float bX_c = bx[p], bY_c = by[p];
+  const float oneL = 1.0f;
+  const float gxm = kLocalGXMult;
+  float gcv = gc_[smp * HW + p];
+  float gwx0 = gwx_[smp * 2 * HW + p], gwx1 = gwx_[smp * 2 * HW + HW + p];
+  float gwy0 = gwy_[smp * 2 * HW + p], gwy1 = gwy_[smp * 2 * HW + HW + p];
+  for (int ch = 0; ch < C; ch++) {
+    const size_t o = smp * S + (size_t)ch * HW;
+    const Plane Y{y_ + o, H, W}, Y1{y_ + o + CHW, H, W}, Y2{y_ + o + 2 * CHW, H, W};
+    const Plane G{g05_in_ + o, H, W}, G1{g05_in_ + o + CHW, H, W}, G2{g05_in_ + o + 2 * CHW, H, W};
+#define QY(F, dh, dw) F.at(h + (dh), w + (dw))
+    const float yk = Y.f[p];
+    const float df_dy = G.f[p], df_dy1 = G1.f[p], df_dy2 = G2.f[p];
+    float df_dy_t = df_dy, df_dy1_t = df_dy1, df_dy2_t = df_dy2;
+    if (h > 0) {  // triangles owned by the pixel above: TGV.cu:304-360 / 1118-1171
+      const float betaTX = bX_u, betaTY = bY_u;
+      {
+        const float zij_1 = (w < W - 1) ? ((QY(Y, -1, 1) - QY(Y, -1, 0)) - QY(Y1, -1, 0)) : 0.f;
+        const float zij_2 = ((yk - QY(Y, -1, 0)) - QY(Y2, -1, 0));
+        const float A = zij_2 * zij_2 * wy_0 + zij_1 * zij_1 * wx_2;
+        float W_TIJ, dW_TIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(A);
+          W_TIJ = huber_w_end(hub, kD0);
+          active = hub > kD0;
+          dW_TIJ = W_TIJ / (hub * hub);
+        } else {
+          const float hub = rsq(A);
+          W_TIJ = fminf(1.f, hub * kD0);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ * (hub * hub);
+        }
+        df_dy_t -= oneL * W_TIJ * ((df_dy - QY(G, -1, 0)) - QY(G2, -1, 0)) * wy_0;
+        if (active) {
+          const float a2 = zij_2 * wy_0;
+          const float a1 = zij_1 * wx_2;
+          df_dy_t += oneL * (dW_TIJ * a2) * (a1 * (QY(G, -1, 1) - QY(G, -1, 0) - QY(G1, -1, 0)) +
+                                            a2 * (QY(G, 0, 0) - QY(G, -1, 0) - QY(G2, -1, 0)));
+        }
+      }
+      {
+        const float uij_1 = (w < W - 1) ? (QY(Y1, -1, 1) - QY(Y1, -1, 0)) : 0.f;
+        const float uij_2 = (QY(Y1, 0, 0) - QY(Y1, -1, 0));
+        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTX;
+        float W_TIJ, dW_TIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(B);
+          W_TIJ = huber_w_end(hub, kD1);
+          active = hub > kD1;
+          dW_TIJ = W_TIJ / (hub * hub);
+        } else {
+          const float hub = rsq(B);
+          W_TIJ = fminf(1.f, hub * kD1);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ * (hub * hub);
+        }
+        df_dy1_t -= betaTX * oneL * W_TIJ * (df_dy1 - QY(G1, -1, 0));
+        if (active)
+          df_dy1_t += betaTX * oneL * (dW_TIJ * betaTX * uij_2) * (uij_1 * (QY(G1, -1, 1) - QY(G1, -1, 0)) +
+                                                                  uij_2 * (QY(G1, 0, 0) - QY(G1, -1, 0)));
+      }
+      {
+        const float uij_1 = (w < W - 1) ? (QY(Y2, -1, 1) - QY(Y2, -1, 0)) : 0.f;
+        const float uij_2 = (QY(Y2, 0, 0) - QY(Y2, -1, 0));
+        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTY;
+        float W_TIJ, dW_TIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(B);
+          W_TIJ = huber_w_end(hub, kD2);
+          active = hub > kD2;
+          dW_TIJ = W_TIJ / (hub * hub);
+        } else {
+          const float hub = rsq(B);
+          W_TIJ = fminf(1.f, hub * kD2);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ / (hub * hub);  // TGV.cu:355: a division where every sibling block multiplies
+        }
+        df_dy2_t -= betaTY * oneL * W_TIJ * (df_dy2 - QY(G2, -1, 0));
+        if (active)
+          df_dy2_t += betaTY * oneL * (dW_TIJ * betaTY * uij_2) * (uij_1 * (QY(G2, -1, 1) - QY(G2, -1, 0)) +
+                                                                  uij_2 * (QY(G2, 0, 0) - QY(G2, -1, 0)));
+      }
+    }
+    if (w > 0) {  // triangles owned by the pixel to the left: TGV.cu:361-418 / 1172-1227
+      const float betaTX = bX_l, betaTY = bY_l;
+      {
+        const float zij_1 = (yk - QY(Y, 0, -1) - QY(Y1, 0, -1));
+        const float zij_2 = (h < H - 1) ? (QY(Y, 1, -1) - QY(Y, 0, -1) - QY(Y2, 0, -1)) : 0.f;
+        const float A = zij_2 * zij_2 * wy_2 + zij_1 * zij_1 * wx_0;
+        float W_TIJ, dW_TIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(A);
+          W_TIJ = huber_w_end(hub, kD0);
+          active = hub > kD0;
+          dW_TIJ = W_TIJ / (hub * hub);
+        } else {
+          const float hub = rsq(A);
+          W_TIJ = fminf(1.f, hub * kD0);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ * (hub * hub);
+        }
+        df_dy_t -= oneL * W_TIJ * ((df_dy - QY(G, 0, -1)) - QY(G1, 0, -1)) * wx_0;
+        if (active) {
+          const float a1 = zij_1 * wx_0;
+          const float a2 = zij_2 * wy_2;
+          df_dy_t += oneL * (dW_TIJ * a1) * (a1 * (QY(G, 0, 0) - QY(G, 0, -1) - QY(G1, 0, -1)) +
+                                            a2 * (QY(G, 1, -1) - QY(G, 0, -1) - QY(G2, 0, -1)));
+        }
+      }
+      {
+        const float uij_1 = (QY(Y1, 0, 0) - QY(Y1, 0, -1));
+        const float uij_2 = (h < H - 1) ? (QY(Y1, 1, -1) - QY(Y1, 0, -1)) : 0.f;
+        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTX;
+        float W_TIJ, dW_TIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(B);
+          W_TIJ = huber_w_end(hub, kD1);
+          active = hub > kD1;
+          dW_TIJ = W_TIJ / (hub * hub);
+        } else {
+          const float hub = rsq(B);
+          W_TIJ = fminf(1.f, hub * kD1);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ * (hub * hub);
+        }
+        df_dy1_t -= betaTX * oneL * W_TIJ * (df_dy1 - QY(G1, 0, -1));
+        if (active)
+          df_dy1_t += betaTX * oneL * (dW_TIJ * betaTX * uij_1) * (uij_2 * (QY(G1, 1, -1) - QY(G1, 0, -1)) +
+                                                                  uij_1 * (QY(G1, 0, 0) - QY(G1, 0, -1)));
+      }
+      {
+        const float uij_1 = (QY(Y2, 0, 0) - QY(Y2, 0, -1));
+        const float uij_2 = (h < H - 1) ? (QY(Y2, 1, -1) - QY(Y2, 0, -1)) : 0.f;
+        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTY;
+        float W_TIJ, dW_TIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(B);
+          W_TIJ = huber_w_end(hub, kD2);
+          active = hub > kD2;
+          dW_TIJ = W_TIJ / (hub * hub);
+        } else {
+          const float hub = rsq(B);
+          W_TIJ = fminf(1.f, hub * kD2);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ * (hub * hub);
+        }
+        df_dy2_t -= betaTY * oneL * W_TIJ * (df_dy2 - QY(G2, 0, -1));
+        if (active)
+          df_dy2_t += betaTY * oneL * (dW_TIJ * betaTY * uij_1) * (uij_2 * (QY(G2, 1, -1) - QY(G2, 0, -1)) +
+                                                                  uij_1 * (QY(G2, 0, 0) - QY(G2, 0, -1)));
+      }
+    }
+    {  // the pixel's own triangles: TGV.cu:419-507 / 1228-1333
+      const float betaTX = bX_c, betaTY = bY_c;
+      {
+        const float aij_1 = (w < W - 1) ? ((QY(Y, 0, 1) - QY(Y, 0, 0)) - QY(Y1, 0, 0)) : 0.f;
+        const float aij_2 = (h < H - 1) ? ((QY(Y, 1, 0) - QY(Y, 0, 0)) - QY(Y2, 0, 0)) : 0.f;
+        const float A = aij_2 * aij_2 * wy_1 + aij_1 * aij_1 * wx_1;
+        const float gr = QY(G, 0, 1), gd = QY(G, 1, 0);
+        float W_TIJ, dW_TIJ, dyij_1, dyij_2;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(A);
+          W_TIJ = huber_w_end(hub, kD0);
+          active = hub > kD0;
+          dW_TIJ = W_TIJ / (hub * hub);
+          dyij_1 = df_dy - gr + df_dy1;
+          dyij_2 = df_dy - gd + df_dy2;
+          df_dy_t -= oneL * ((df_dy - gd) + df_dy2) * wy_1 * W_TIJ;
+          df_dy_t -= oneL * ((df_dy - gr) + df_dy1) * wx_1 * W_TIJ;
+          df_dy1_t -= oneL * W_TIJ * (df_dy1 - gr + df_dy) * wx_1;
+          df_dy2_t -= oneL * W_TIJ * (df_dy2 - gd + df_dy) * wy_1;
+          gwx0 = gwx0 + oneL * gxm * dyij_1 * aij_1 * W_TIJ;
+          gwy0 = gwy0 + oneL * gxm * dyij_2 * aij_2 * W_TIJ;
+        } else {
+          const float hub = rsq(A);
+          W_TIJ = fminf(1.f, hub * kD0);
+          active = W_TIJ < 1.0f;
+          dW_TIJ = W_TIJ * (hub * hub);
+          dyij_1 = df_dy - gr + df_dy1;
+          dyij_2 = df_dy - gd + df_dy2;
+          df_dy_t -= oneL * W_TIJ * (dyij_2 * wy_1 + dyij_1 * wx_1);
+          df_dy1_t -= oneL * W_TIJ * dyij_1 * wx_1;
+          df_dy2_t -= oneL * W_TIJ * dyij_2 * wy_1;
+          gwx0 = gwx0 + oneL * gxm * dyij_1 * (aij_1 * W_TIJ);
+          gwy0 = gwy0 + oneL * gxm * dyij_2 * (aij_2 * W_TIJ);
+        }
+        if (active) {
+          const float a1 = aij_1 * wx_1;
+          const float a2 = aij_2 * wy_1;
+          const float deriv_Tij = (dyij_1 * a1 + dyij_2 * a2) * oneL;
+          df_dy_t += deriv_Tij * ((a1 + a2) * dW_TIJ);
+          df_dy2_t += deriv_Tij * (a2 * dW_TIJ);
+          df_dy1_t += deriv_Tij * (a1 * dW_TIJ);
+          // the literal 0.5 makes these two updates double (TGV.cu:452-453)
+          gwy0 = (float)((double)gwy0 - (double)(gxm * (aij_2 * dW_TIJ * aij_2)) * 0.5 * (double)deriv_Tij);
+          gwx0 = (float)((double)gwx0 - (double)(gxm * (aij_1 * dW_TIJ * aij_1)) * 0.5 * (double)deriv_Tij);
+        }
+      }
+      {
+        const float uij_1 = (w < W - 1) ? (QY(Y1, 0, 1) - QY(Y1, 0, 0)) : 0.f;
+        const float uij_2 = (h < H - 1) ? (QY(Y1, 1, 0) - QY(Y1, 0, 0)) : 0.f;
+        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTX;
+        const float gr = QY(G1, 0, 1), gd = QY(G1, 1, 0);
+        float W_YIJ, dW_YIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(B);
+          W_YIJ = huber_w_end(hub, kD1);
+          active = hub > kD1;
+          dW_YIJ = W_YIJ / (hub * hub);
+          if (h < H - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gd);  // TGV.cu:1271-1274: y first
+          if (w < W - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gr);
+        } else {
+          const float hub = rsq(B);
+          W_YIJ = fminf(1.f, hub * kD1);
+          active = W_YIJ < 1.0f;
+          dW_YIJ = W_YIJ * (hub * hub);
+          if (w < W - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gr);
+          if (h < H - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gd);
+        }
+        gwx1 = gwx1 + oneL * gxm * ((df_dy1 - gr) * uij_1 + (df_dy1 - gd) * uij_2) * W_YIJ;
+        if (active) {
+          const float deriv_Yij = ((df_dy1 - gr) * uij_1 * betaTX + (df_dy1 - gd) * uij_2 * betaTX) * oneL;
+          df_dy1_t += betaTX * dW_YIJ * (uij_1 + uij_2) * deriv_Yij;
+          gwx1 = (float)((double)gwx1 -
+                         (double)(gxm * (uij_2 * dW_YIJ * uij_2 + uij_1 * dW_YIJ * uij_1)) * 0.5 * (double)deriv_Yij);
+        }
+      }
+      {
+        const float uij_1 = (w < W - 1) ? (QY(Y2, 0, 1) - QY(Y2, 0, 0)) : 0.f;
+        const float uij_2 = (h < H - 1) ? (QY(Y2, 1, 0) - QY(Y2, 0, 0)) : 0.f;
+        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTY;
+        const float gr = QY(G2, 0, 1), gd = QY(G2, 1, 0);
+        float W_YIJ, dW_YIJ;
+        bool active;
+        if (END) {
+          const float hub = sqrtf(B);
+          W_YIJ = huber_w_end(hub, kD2);
+          active = hub > kD2;
+          dW_YIJ = W_YIJ / (hub * hub);
+        } else {
+          const float hub = rsq(B);
+          W_YIJ = fminf(1.f, hub * kD2);
+          active = W_YIJ < 1.0f;
+          dW_YIJ = W_YIJ * (hub * hub);
+        }
+        if (w < W - 1) df_dy2_t -= betaTY * oneL * W_YIJ * (df_dy2 - gr);
+        if (h < H - 1) df_dy2_t -= betaTY * oneL * W_YIJ * (df_dy2 - gd);
+        gwy1 = gwy1 + oneL * gxm * ((df_dy2 - gr) * uij_1 + (df_dy2 - gd) * uij_2) * W_YIJ;
+        if (active) {
+          const float deriv_Yij = ((df_dy2 - gr) * uij_1 * betaTY + (df_dy2 - gd) * uij_2 * betaTY) * oneL;
+          df_dy2_t += betaTY * dW_YIJ * (uij_1 + uij_2) * deriv_Yij;
+          gwy1 = (float)((double)gwy1 -
+                         (double)(gxm * (uij_2 * dW_YIJ * uij_2 + uij_1 * dW_YIJ * uij_1)) * 0.5 * (double)deriv_Yij);
+        }
+      }
+    }
+#undef QY
+    // aux variables: momentum adjoint only (TGV.cu:560-577 / 1383-1399); the literal 1. makes the
+    // product double
+    const size_t q = o + p;
+    gxk_m1_[q + CHW] = -t * df_dy1_t;
+    df_dy1_t = (float)((double)gxk_[q + CHW] + (1. + (double)t) * (double)df_dy1_t);
+    df_dy1_t = fmaxf(-kClipLocalGrad, fminf(df_dy1_t, kClipLocalGrad));
+    g05_out_[q + CHW] = df_dy1_t;
+    gxk_[q + CHW] = df_dy1_t;
+    gxk_m1_[q + 2 * CHW] = -t * df_dy2_t;
+    df_dy2_t = (float)((double)gxk_[q + 2 * CHW] + (1. + (double)t) * (double)df_dy2_t);
+    df_dy2_t = fmaxf(-kClipLocalGrad, fminf(df_dy2_t, kClipLocalGrad));
+    g05_out_[q + 2 * CHW] = df_dy2_t;
+    gxk_[q + 2 * CHW] = df_dy2_t;
+    // u (TGV.cu:579-612 / 1403-1442)
+    float df_dxk = (float)((double)gxk_[q] + (1. + (double)t) * (double)df_dy_t);
+    df_dxk = fmaxf(-kClipLocalGrad, fminf(df_dxk, kClipLocalGrad));
+    gxk_[q] = df_dxk;
+    gxk_m1_[q] = -t * df_dy_t;
+    const size_t qb = smp * CHW + (size_t)ch * HW + p;
+    float g05v, gbv = gb_[qb];
+    prox_adjoint<false>(df_dxk, b_[qb], x05_[q], conf, g05v, gcv, gbv);
+    g05_out_[q] = g05v;
+    gb_[qb] = gbv;
+  }
+  gc_[smp * HW + p] = gcv;
+  gwx_[smp * 2 * HW + p] = gwx0;
+  gwx_[smp * 2 * HW + HW + p] = gwx1;
+  gwy_[smp * 2 * HW + p] = gwy0;
+  gwy_[smp * 2 * HW + HW + p] = gwy1;
+}
+
+// Upstream check (TGV.cu:2686-2703): counts[0] = non-finite entries, counts[1] = non-zero finite ones.
+__global__ __launch_bounds__(256) void tgv_upstream_check(const float* __restrict__ g, long long n,
+                                                          unsigned int* __restrict__ counts) {
+  unsigned int bad = 0, nz = 0;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    const float v = g[i];
+    if (!finite_value(v)) bad++;
+    else if (v != 0.f) nz++;
+  }
+  bad = wave_sum_u(bad);
+  nz = wave_sum_u(nz);
+  if ((threadIdx.x & 63) == 0) {
+    if (bad) atomicAdd(&counts[0], bad);
+    if (nz) atomicAdd(&counts[1], nz > 0 ? 1u : 0u);
+  }
+}
+
+// The guard on the gradient wrt the starting point inspects only the u block (TGV.cu:3014-3021):
+// gather the u blocks of all samples into one contiguous tensor ...
+__global__ __launch_bounds__(256) void tgv_gather_u(const float* __restrict__ src, float* __restrict__ dst,
+                                                    long long CHW, long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long s = i / CHW, r = i - s * CHW;
+  dst[i] = src[s * 3 * CHW + r];
+}
+// ... and apply its verdict to the u blocks only; v1 / v2 gradients pass through (TGV.cu:3047).
+__global__ __launch_bounds__(256) void tgv_finalize_init(const float* __restrict__ src, float* __restrict__ out,
+                                                         long long CHW, long long total,
+                                                         const GuardState* __restrict__ gs, GuardParams p) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long r = i % (3 * CHW);
+  float v = src[i];
+  if (r < CHW) {
+    const double mult = gs->scale[4];
+    v = guard_limit(v, p);
+    if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
+  }
+  out[i] = v;
+}
+
+// -------------------------------------------------------------------------------------------------
+// per-id state (idStructBs, TGVInpaintFista.h:7-50)
+// -------------------------------------------------------------------------------------------------
+struct Slot {
+  int run = 0;
+  int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
+  bool forward_done = false;
+  std::vector<int> iterations;
+  std::vector<float> steps;
+  int max_inter_its = 0;
+  hipStream_t stream = nullptr;
+  Arena arena;
+  // S3 = n*3*ic*ih*iw floats (state), F = n*ic*ih*iw, P = n*ih*iw
+  float *wx = nullptr, *wy = nullptr, *bx = nullptr, *by = nullptr;  // L-scaled weights, P each
+  double* Ls = nullptr;                                              // per-sample L
+  unsigned int* maxbits = nullptr;                                   // per-sample Lipschitz bound (float bits)
+  unsigned int* counts = nullptr;                                    // upstream check
+  float *ypp[2] = {nullptr, nullptr}, *xpp[2] = {nullptr, nullptr}, *ckpt_y = nullptr, *ckpt_x = nullptr, *x05 = nullptr;
+  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr}, *yk = nullptr, *gi_u = nullptr;
+  float *acc_gc = nullptr, *acc_gx = nullptr, *acc_gy = nullptr, *acc_gb = nullptr;
+  double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
+  GuardState* guard = nullptr;
+  double pending_av[5] = {0, 0, 0, 0, 0};
+};
+
+Slot g_slots[kUniqueIds];
+KernelTimer g_timer;
+
+size_t state_count(const Slot& s) { return (size_t)s.n * 3 * s.ic * s.ih * s.iw; }
+size_t field_count(const Slot& s) { return (size_t)s.n * s.ic * s.ih * s.iw; }
+size_t plane_count(const Slot& s) { return (size_t)s.n * s.ih * s.iw; }
+
+int fetch_running_means(Slot& s) {
+  if (s.guard) {
+    GuardState host;
+    INPAINT_HIP(hipStreamSynchronize(s.stream));
+    INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+    for (int k = 0; k < 5; k++) s.pending_av[k] = host.av[k];
+  }
+  return 0;
+}
+
+int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t stream) {
+  int dev = -1;
+  INPAINT_HIP(hipGetDevice(&dev));
+  const bool same = s.arena.base && s.arena.device == dev && s.n == n && s.ic == ic && s.ih == ih &&
+                    s.iw == iw && s.its == its;
+  s.stream = stream;
+  if (same) return 0;
+  int rc = fetch_running_means(s);
+  if (rc) return rc;
+  s.n = n; s.ic = ic; s.ih = ih; s.iw = iw; s.its = its;
+  make_schedule(its, s.iterations, s.max_inter_its);
+  make_step_sizes(its, s.steps);
+  const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
+  const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)std::max(s.max_inter_its, 1);
+  size_t need = 0;
+  need += Arena::padded(S3, 4) * (2 + 2 + 2 + 2 + 1) + Arena::padded(S3 * nck, 4) * 2 + Arena::padded(S3 * ring, 4);
+  need += Arena::padded(F, 4) * 2 + Arena::padded(F, 8);
+  need += Arena::padded(P, 4) * (4 + 1) + Arena::padded(2 * P, 4) * 2;
+  need += Arena::padded(P, 8) + Arena::padded(2 * P, 8) * 2;
+  need += Arena::padded((size_t)n, 8) + Arena::padded((size_t)n, 4) + Arena::padded(2, 4);
+  need += Arena::padded(1, sizeof(GuardState));
+  rc = s.arena.reserve(need);
+  if (rc) return rc;
+  Arena& a = s.arena;
+  s.wx = a.take<float>(P); s.wy = a.take<float>(P); s.bx = a.take<float>(P); s.by = a.take<float>(P);
+  s.Ls = a.take<double>((size_t)n);
+  s.maxbits = a.take<unsigned int>((size_t)n);
+  s.counts = a.take<unsigned int>(2);
+  s.ypp[0] = a.take<float>(S3); s.ypp[1] = a.take<float>(S3);
+  s.xpp[0] = a.take<float>(S3); s.xpp[1] = a.take<float>(S3);
+  s.ckpt_y = a.take<float>(S3 * nck); s.ckpt_x = a.take<float>(S3 * nck);
+  s.x05 = a.take<float>(S3 * ring);
+  s.g05[0] = a.take<float>(S3); s.g05[1] = a.take<float>(S3);
+  s.gxk[0] = a.take<float>(S3); s.gxk[1] = a.take<float>(S3);
+  s.yk = a.take<float>(S3);
+  s.gi_u = a.take<float>(F);
+  s.acc_gb = a.take<float>(F);
+  s.acc_gc = a.take<float>(P); s.acc_gx = a.take<float>(2 * P); s.acc_gy = a.take<float>(2 * P);
+  s.tot_gc = a.take<double>(P); s.tot_gx = a.take<double>(2 * P); s.tot_gy = a.take<double>(2 * P);
+  s.tot_gb = a.take<double>(F);
+  s.guard = a.take<GuardState>(1);
+  if (!s.guard) return fail(INPAINT_ERR_HIP, "arena layout overflow");
+  GuardState init;
+  memset(&init, 0, sizeof(init));
+  for (int k = 0; k < 5; k++) { init.av[k] = s.pending_av[k]; init.scale[k] = 1.0; }
+  INPAINT_HIP(hipMemcpyAsync(s.guard, &init, sizeof(init), hipMemcpyHostToDevice, stream));
+  INPAINT_HIP(hipStreamSynchronize(stream));
+  return 0;
+}
+
+int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int iw, int its, int id) {
+  if (id < 0 || id >= kUniqueIds)
+    return fail(INPAINT_ERR_ID, "Cannot use an id that is negative or larger/equal than the maximal one: %d/%d", id,
+                kUniqueIds);
+  for (int i = 0; i < nptrs; i++)
+    if (!ptrs[i]) return fail(INPAINT_ERR_ARG, "null pointer argument (position %d)", i);
+  if (n < 1 || ic < 1 || ih < 1 || iw < 1 || its < 0)
+    return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
+  if (n > 65535 || (ih + BY - 1) / BY > 65535)
+    return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
+  if ((int)std::floor(std::sqrt((double)its)) > kMaxCheckpoints)
+    return fail(INPAINT_ERR_ITS, "its=%d needs more than %d checkpoints", its, kMaxCheckpoints);
+  return 0;
+}
+
+// Lipschitz reduction + scaled weight copies for the weights of this call (forward and backward both
+// redo it, TGV.cu:2513-2531 and 2667-2679).
+void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const float* dy) {
+  const long long P = (long long)plane_count(s), HW = (long long)s.ih * s.iw;
+  hipLaunchKernelGGL(tgv_lipschitz_init, dim3((s.n + 255) / 256), dim3(256), 0, stream, s.maxbits, s.n);
+  hipLaunchKernelGGL(tgv_lipschitz_kernel, dim3((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n), dim3(BX, BY), 0, stream,
+                     dx, dy, s.ih, s.iw, s.maxbits);
+  hipLaunchKernelGGL(tgv_scale_kernel, dim3(grid1d(P)), dim3(256), 0, stream, dx, dy, s.maxbits, s.wx, s.wy, s.bx, s.by,
+                     s.Ls, HW, P);
+}
+
+void launch_forward(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
+                    const float* yin, float* yout, float* x05, float t) {
+  const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
+  hipLaunchKernelGGL(tgv_forward_px, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xout, yin, yout, x05,
+                     s.ic, s.ih, s.iw, t);
+}
+
+template <bool END>
+void launch_adjoint(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* x05,
+                    const float* g05_in, float* g05_out, float* gxk, float* gxk_m1, const float* y, float t) {
+  const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
+  hipLaunchKernelGGL(tgv_adjoint_px<END>, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, x05, s.acc_gc, s.acc_gb,
+                     s.acc_gx, s.acc_gy, g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
+}
+
+}  // namespace
+
+extern "C" {
+
+int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const float* b, const float* init,
+                       float* out, int n, int ic, int ih, int iw, int its, int id, void* stream_) {
+  const void* ptrs[] = {dx, dy, c, b, init, out};
+  int rc = check_common(ptrs, 6, n, ic, ih, iw, its, id);
+  if (rc) return rc;
+  hipStream_t stream = (hipStream_t)stream_;
+  Slot& s = g_slots[id];
+  s.forward_done = false;
+  rc = prepare_slot(s, n, ic, ih, iw, its, stream);
+  if (rc) return rc;
+  const size_t S3 = state_count(s), SB = S3 * sizeof(float);
+  const int K = 2 * (its / 2);
+  auto ck_index = [&](int k) {
+    for (size_t i = 0; i < s.iterations.size(); i++)
+      if (s.iterations[i] == k) return (int)i;
+    return -1;
+  };
+  auto Ybuf = [&](int k) { int i = ck_index(k); return (i >= 0 && k < K) ? s.ckpt_y + (size_t)i * S3 : s.ypp[k & 1]; };
+  auto Xbuf = [&](int k) {
+    if (k == K) return out;
+    int i = ck_index(k);
+    return i >= 0 ? s.ckpt_x + (size_t)i * S3 : s.xpp[k & 1];
+  };
+  if (K == 0) {
+    INPAINT_HIP(hipMemcpyAsync(out, init, SB, hipMemcpyDeviceToDevice, stream));
+    if (!s.iterations.empty()) {  // its == 1: the reference leaves calloc'ed (zero) checkpoints
+      hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)S3)), dim3(256), 0, stream, s.ckpt_y, (long long)S3);
+      hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)S3)), dim3(256), 0, stream, s.ckpt_x, (long long)S3);
+    }
+  } else {
+    scale_weights(s, stream, dx, dy);
+    INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, SB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
+    INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, SB, hipMemcpyDeviceToDevice, stream));
+    for (int k = 0; k < K; k++)
+      launch_forward(s, stream, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
+  }
+  INPAINT_HIP(hipGetLastError());
+  s.forward_done = true;
+  return 0;
+}
+
+int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const float* b, float* gin, float* gx,
+                        float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih, int iw, int its, int id,
+                        void* stream_) {
+  const void* ptrs[] = {dx, dy, c, b, gin, gx, gy, gc, gb, gi};
+  int rc = check_common(ptrs, 10, n, ic, ih, iw, its, id);
+  if (rc) return rc;
+  hipStream_t stream = (hipStream_t)stream_;
+  Slot& s = g_slots[id];
+  if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
+    return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
+  s.stream = stream;
+  const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
+  const int gS = grid_stride((long long)S3), gF = grid_stride((long long)F), gP = grid_stride((long long)P),
+            g2P = grid_stride((long long)(2 * P));
+
+  // Upstream check (TGV.cu:2686-2703): any non-finite entry, or an upstream that is zero everywhere,
+  // returns all-zero gradients, scrubs the caller's tensor and leaves `run` alone.  The verdict
+  // decides a host-side counter, so this is the one host wait of the call.
+  {
+    ZeroList z;
+    z.ptr[0] = s.counts; z.bytes[0] = 8;
+    hipLaunchKernelGGL(fill_zero_many, dim3(1, 1), dim3(256), 0, stream, z);
+    hipLaunchKernelGGL(tgv_upstream_check, dim3(gS), dim3(256), 0, stream, gin, (long long)S3, s.counts);
+    unsigned int host_counts[2] = {0, 0};
+    INPAINT_HIP(hipMemcpyAsync(host_counts, s.counts, 8, hipMemcpyDeviceToHost, stream));
+    INPAINT_HIP(hipStreamSynchronize(stream));
+    if (host_counts[0] != 0 || host_counts[1] == 0) {
+      hipLaunchKernelGGL(scrub_kernel, dim3(gS), dim3(256), 0, stream, gin, (long long)S3);
+      ZeroList o;
+      o.ptr[0] = gi; o.bytes[0] = (long long)S3 * 4;
+      o.ptr[1] = gx; o.bytes[1] = (long long)P * 8;
+      o.ptr[2] = gy; o.bytes[2] = (long long)P * 8;
+      o.ptr[3] = gc; o.bytes[3] = (long long)P * 4;
+      o.ptr[4] = gb; o.bytes[4] = (long long)F * 4;
+      hipLaunchKernelGGL(fill_zero_many, dim3(gS, 5), dim3(256), 0, stream, o);
+      INPAINT_HIP(hipGetLastError());
+      return 0;
+    }
+  }
+
+  scale_weights(s, stream, dx, dy);
+  {
+    ZeroList z;
+    int k = 0;
+    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.yk}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
+    z.ptr[k] = s.acc_gb; z.bytes[k++] = (long long)F * 4;
+    z.ptr[k] = s.acc_gc; z.bytes[k++] = (long long)P * 4;
+    z.ptr[k] = s.acc_gx; z.bytes[k++] = (long long)P * 8;
+    z.ptr[k] = s.acc_gy; z.bytes[k++] = (long long)P * 8;
+    z.ptr[k] = s.tot_gc; z.bytes[k++] = (long long)P * 8;
+    z.ptr[k] = s.tot_gx; z.bytes[k++] = (long long)P * 16;
+    z.ptr[k] = s.tot_gy; z.bytes[k++] = (long long)P * 16;
+    z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
+    hipLaunchKernelGGL(fill_zero_many, dim3(gS, k), dim3(256), 0, stream, z);
+  }
+
+  // buffer roles of TGV.cu:2718-2736: g05[0]/g05[1] and gxk[0]/gxk[1] ping-pong with the parity of the
+  // local iteration index (the copy of the upstream gradient into gxk[0], TGV.cu:2729, is overwritten
+  // before it is read and is not made).
+  int lastIt = its;
+  const int nseg = (int)s.iterations.size();
+  for (int outer = nseg - 1; outer >= 0; outer--) {
+    const int k0 = s.iterations[outer];
+    const int len = 2 * ((lastIt - k0) / 2);
+    const float* cky = s.ckpt_y + (size_t)outer * S3;
+    const float* ckx = s.ckpt_x + (size_t)outer * S3;
+    for (int j = 0; j < len; j++) {  // recompute the segment, keeping x05 (TGV.cu:2775-2814)
+      const float* yin = (j == 0) ? cky : s.ypp[j & 1];
+      const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
+      launch_forward(s, stream, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * S3,
+                     s.steps[k0 + j]);
+    }
+    for (int j = len - 1; j >= 0; j--) {  // reverse sweep (TGV.cu:2851-2933)
+      const float t = s.steps[k0 + j];
+      const float* xa = s.x05 + (size_t)j * S3;
+      const int odd = j & 1;
+      if (outer == nseg - 1 && j == len - 1) {
+        hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa, s.acc_gc,
+                           s.acc_gb, s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+      } else if (j > 0) {
+        const float* xb = s.x05 + (size_t)(j - 1) * S3;
+        hipLaunchKernelGGL(tgv_getyk_kernel, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa, xb, s.yk, ic,
+                           (long long)ih * iw, (long long)P, t);
+        g_timer.mark(stream);
+        launch_adjoint<false>(s, stream, c, b, xa, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0], s.gxk[odd ? 0 : 1],
+                              s.gxk[odd ? 1 : 0], s.yk, t);
+        g_timer.mark(stream);
+      } else {
+        launch_adjoint<true>(s, stream, c, b, xa, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0], cky, t);
+      }
+    }
+    // fp32 segment sums into the fp64 totals (TGV.cu:2944)
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc, s.tot_gc, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx, s.tot_gx, (long long)(2 * P));
+    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy, s.tot_gy, (long long)(2 * P));
+    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb, s.tot_gb, (long long)F);
+    lastIt = k0;
+  }
+
+  // output guard on the device (TGV.cu:2990-3021), then scale and store (TGV.cu:3024-3050)
+  hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
+  hipLaunchKernelGGL(tgv_gather_u, dim3(grid1d((long long)F)), dim3(256), 0, stream, s.gxk[1], s.gi_u,
+                     (long long)ic * ih * iw, (long long)F);
+  GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
+  const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
+  const long long cnts[5] = {(long long)P, (long long)(2 * P), (long long)(2 * P), (long long)F, (long long)F};
+  for (int k = 0; k < 4; k++) {
+    hipLaunchKernelGGL(guard_reduce_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k],
+                       cnts[k], st + k, kGuard.max_tolerance, true);
+    hipLaunchKernelGGL(guard_tail_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k], cnts[k],
+                       st + k, kGuard.max_tolerance, true);
+  }
+  hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gi_u, cnts[4],
+                     st + 4, kGuard.max_tolerance, true);
+  hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gi_u, cnts[4],
+                     st + 4, kGuard.max_tolerance, true);
+  GuardCounts gcnt;
+  for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
+  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
+  const double* no_chain = nullptr;
+  const long long HW2 = 2LL * ih * iw;
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gc, gc, (long long)P, s.guard, 0, kGuard,
+                     kGlobalGMult, 1.0, no_chain, 1LL);
+  hipLaunchKernelGGL(finalize_f64, dim3(g2P), dim3(256), 0, stream, s.tot_gx, gx, (long long)(2 * P), s.guard, 1, kGuard,
+                     kGlobalGMult, 0.0, (const double*)s.Ls, HW2);
+  hipLaunchKernelGGL(finalize_f64, dim3(g2P), dim3(256), 0, stream, s.tot_gy, gy, (long long)(2 * P), s.guard, 2, kGuard,
+                     kGlobalGMult, 0.0, (const double*)s.Ls, HW2);
+  hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, kGuard,
+                     kGlobalGMult, 1.0, no_chain, 1LL);
+  hipLaunchKernelGGL(tgv_finalize_init, dim3(grid1d((long long)S3)), dim3(256), 0, stream, s.gxk[1], gi,
+                     (long long)ic * ih * iw, (long long)S3, s.guard, kGuard);
+  INPAINT_HIP(hipGetLastError());
+  s.run++;  // TGV.cu:3061
+  return 0;
+}
+
+int tgvinpaint_get_state(int id, double* state6) {
+  if (id < 0 || id >= kUniqueIds || !state6) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  int rc = fetch_running_means(s);
+  if (rc) return rc;
+  state6[0] = s.run;
+  for (int k = 0; k < 5; k++) state6[1 + k] = s.pending_av[k];
+  return 0;
+}
+
+int tgvinpaint_set_state(int id, const double* state6) {
+  if (id < 0 || id >= kUniqueIds || !state6) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  s.run = (int)state6[0];
+  for (int k = 0; k < 5; k++) s.pending_av[k] = state6[1 + k];
+  if (s.guard) {
+    INPAINT_HIP(hipStreamSynchronize(s.stream));
+    INPAINT_HIP(hipMemcpy(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, av), s.pending_av, 5 * sizeof(double),
+                         hipMemcpyHostToDevice));
+  }
+  return 0;
+}
+
+int tgvinpaint_reset_id(int id) {
+  if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  if (s.arena.base) (void)hipStreamSynchronize(s.stream);
+  int rc = s.arena.release();
+  s = Slot();
+  return rc;
+}
+
+int tgvinpaint_guard_stats(int id, double* stats25) {
+  if (id < 0 || id >= kUniqueIds || !stats25) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  if (!s.guard) return fail(INPAINT_ERR_PAIRING, "id %d holds no state", id);
+  GuardState host;
+  INPAINT_HIP(hipStreamSynchronize(s.stream));
+  INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+  memcpy(stats25, host.report, sizeof(host.report));
+  return 0;
+}
+
+long long tgvinpaint_slot_bytes(int id) {
+  if (id < 0 || id >= kUniqueIds) return 0;
+  return (long long)g_slots[id].arena.bytes;
+}
+
+int tgvinpaint_lipschitz(int id, double* L_host, int n) {
+  if (id < 0 || id >= kUniqueIds || !L_host) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  Slot& s = g_slots[id];
+  if (!s.Ls || n != s.n) return fail(INPAINT_ERR_PAIRING, "id %d holds no state for %d samples", id, n);
+  INPAINT_HIP(hipStreamSynchronize(s.stream));
+  INPAINT_HIP(hipMemcpy(L_host, s.Ls, sizeof(double) * (size_t)n, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int tgvinpaint_guard_decide(int run, double av_gc, double av_running, double* mult_out, double* av_out) {
+  double mult = 1.0, av = av_running;
+  int action = guard_decide_rule(run, av_gc, av, mult, kGuard);
+  if (mult_out) *mult_out = mult;
+  if (av_out) *av_out = av;
+  return action;
+}
+
+int tgvinpaint_profile(int enable) {
+  g_timer.enabled = enable != 0;
+  g_timer.used = 0;
+  return 0;
+}
+
+int tgvinpaint_profile_read(double* total_ms, int* launches) { return g_timer.read(total_ms, launches); }
+
+const char* tgvinpaint_last_error(void) { return error_buffer(); }
+
+}  // extern "C"

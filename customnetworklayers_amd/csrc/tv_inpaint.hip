@@ -381,77 +381,6 @@ __global__ __launch_bounds__(NT) void tv_adjoint_iter(
   }
 }
 
-// Segment flush: fp32 accumulator into its fp64 total, then zero (copy_and_set_to_0, TV.cu:178-218).
-__global__ __launch_bounds__(256) void flush_kernel(float* __restrict__ acc, double* __restrict__ total,
-                                                    long long n) {
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    total[i] = (double)acc[i] + total[i] / 1.;
-    acc[i] = 0.f;
-  }
-}
-
-__global__ __launch_bounds__(256) void fill_zero_f32(float* __restrict__ p, long long n) {
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x)
-    p[i] = 0.f;
-}
-__global__ __launch_bounds__(256) void fill_zero_f64(double* __restrict__ p, long long n) {
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x)
-    p[i] = 0.;
-}
-
-// Zero several buffers in one launch (blockIdx.y picks the buffer).
-struct ZeroList {
-  void* ptr[16];
-  long long bytes[16];
-};
-__global__ __launch_bounds__(256) void fill_zero_many(ZeroList z) {
-  uint32_t* p = static_cast<uint32_t*>(z.ptr[blockIdx.y]);
-  const long long n = z.bytes[blockIdx.y] / 4;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x)
-    p[i] = 0u;
-}
-
-// Upstream scrub, in the caller's buffer: TV.cu:1609-1623.
-__global__ __launch_bounds__(256) void scrub_kernel(float* __restrict__ g, long long n) {
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    const float v = g[i];
-    if (!finite_value(v)) g[i] = 0.f;
-  }
-}
-
-// Guarded fp64 total -> fp32 output: TV.cu:160-171 (zeroing), 136/147 (kill / rescale), 1795-1818.
-// `chain` is 1/8 for the edge-weight gradients (TV.cu:1817-1818) and 1 otherwise.
-__global__ __launch_bounds__(256) void finalize_f64(const double* __restrict__ total, float* __restrict__ out,
-                                                    long long n, const GuardState* __restrict__ gs, int k,
-                                                    double chain) {
-  const double mult = gs->scale[k];
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    double v = total[i];
-    if (!finite_value(v) || fabs(v) > kGuard.max_tolerance) v = 0;
-    if (mult != 1.0) v = (mult == 0.0) ? 0.0 : v * mult;
-    const float f = (float)(v * kGlobalGMult);
-    out[i] = (chain == 1.0) ? f : (float)(chain * (double)f);
-  }
-}
-// Gradient wrt init: g_x[1] after the last step (TV.cu:1784-1791,1816), guarded as a float tensor.
-__global__ __launch_bounds__(256) void finalize_f32(const float* __restrict__ src, float* __restrict__ out,
-                                                    long long n, const GuardState* __restrict__ gs, int k) {
-  const double mult = gs->scale[k];
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    float v = src[i];
-    if (!finite_value(v) || fabs((double)v) > kGuard.max_tolerance) v = 0.f;
-    if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
-    out[i] = 0.0f + v;
-  }
-}
-
 // -------------------------------------------------------------------------------------------------
 // per-id state (idStruct, TVInpaintFista.h:7-50)
 // -------------------------------------------------------------------------------------------------
@@ -479,21 +408,6 @@ struct Slot {
 
 Slot g_slots[kUniqueIds];
 
-// Optional timing of the main adjoint kernel with HIP events on the launch stream.
-struct KernelTimer {
-  bool enabled = false;
-  std::vector<hipEvent_t> pool;  // start/stop pairs
-  size_t used = 0;
-  void mark(hipStream_t stream) {
-    if (!enabled) return;
-    if (used == pool.size()) {
-      hipEvent_t e;
-      if (hipEventCreate(&e) != hipSuccess) { enabled = false; return; }
-      pool.push_back(e);
-    }
-    (void)hipEventRecord(pool[used++], stream);
-  }
-};
 KernelTimer g_timer;
 
 size_t field_count(const Slot& s) { return (size_t)s.n * s.ic * s.ih * s.iw; }
@@ -552,9 +466,6 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   INPAINT_HIP(hipStreamSynchronize(stream));  // `init` is a stack object
   return 0;
 }
-
-inline int grid1d(long long n) { return (int)std::max<long long>(1, std::min<long long>((n + 255) / 256, 1 << 20)); }
-inline int grid_stride(long long n) { return (int)std::max<long long>(1, std::min<long long>((n + 1023) / 1024, 4096)); }
 
 int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int iw, int its, int id) {
   if (id < 0 || id >= kUniqueIds)
@@ -804,22 +715,27 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   const long long cnts[5] = {(long long)P, (long long)P, (long long)P, (long long)F, (long long)F};
   for (int k = 0; k < 4; k++) {
     hipLaunchKernelGGL(guard_reduce_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k],
-                       cnts[k], st + k, kGuard.max_tolerance);
+                       cnts[k], st + k, kGuard.max_tolerance, false);
     hipLaunchKernelGGL(guard_tail_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k], cnts[k],
-                       st + k);
+                       st + k, 0.0, false);
   }
   hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gx_final, cnts[4],
-                     st + 4, kGuard.max_tolerance);
+                     st + 4, kGuard.max_tolerance, false);
   hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gx_final, cnts[4],
-                     st + 4);
+                     st + 4, 0.0, false);
   GuardCounts gcnt;
   for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
   hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gc, gc, (long long)P, s.guard, 0, 1.0);
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gx, gx, (long long)P, s.guard, 1, (double)kL);
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gy, gy, (long long)P, s.guard, 2, (double)kL);
-  hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, 1.0);
-  hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gx_final, gi, (long long)F, s.guard, 4);
+  const double* no_chain = nullptr;
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gc, gc, (long long)P, s.guard, 0, kGuard,
+                     kGlobalGMult, 1.0, no_chain, 1LL);
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gx, gx, (long long)P, s.guard, 1, kGuard,
+                     kGlobalGMult, (double)kL, no_chain, 1LL);
+  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gy, gy, (long long)P, s.guard, 2, kGuard,
+                     kGlobalGMult, (double)kL, no_chain, 1LL);
+  hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, kGuard,
+                     kGlobalGMult, 1.0, no_chain, 1LL);
+  hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gx_final, gi, (long long)F, s.guard, 4, kGuard);
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TV.cu:1829
   return 0;
@@ -902,21 +818,7 @@ int tvinpaint_profile(int enable) {
   return 0;
 }
 
-int tvinpaint_profile_read(double* total_ms, int* launches) {
-  double total = 0;
-  int count = 0;
-  for (size_t i = 0; i + 1 < g_timer.used; i += 2) {
-    INPAINT_HIP(hipEventSynchronize(g_timer.pool[i + 1]));
-    float ms = 0;
-    INPAINT_HIP(hipEventElapsedTime(&ms, g_timer.pool[i], g_timer.pool[i + 1]));
-    total += ms;
-    count++;
-  }
-  g_timer.used = 0;
-  if (total_ms) *total_ms = total;
-  if (launches) *launches = count;
-  return 0;
-}
+int tvinpaint_profile_read(double* total_ms, int* launches) { return g_timer.read(total_ms, launches); }
 
 const char* tvinpaint_last_error(void) { return error_buffer(); }
 

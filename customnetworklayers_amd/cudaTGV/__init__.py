@@ -1,0 +1,1 @@
+from .TGVInpainting import TGVInpaint, TGVInpaintingFunction  # noqa: F401

@@ -1,0 +1,73 @@
+/* C ABI of the MI355X TGV inpainting layer (libinpaint_hip.so).
+ *
+ * Same conventions as tvinpaint.h: plain pointers and sizes, device pointers on the current HIP
+ * device unless the parameter says "host", contiguous NCHW float32 tensors, `stream` a hipStream_t
+ * passed as void* (NULL = the default stream).  Return value 0 = ok; the error codes are the
+ * INPAINT_ERR_* values of tvinpaint.h and tgvinpaint_last_error() describes the failure.
+ *
+ * Tensor layout: the layer's state is (u, v1, v2) per flow channel.  `init`, `out`, `gin`, `gi` are
+ * (n, 3*ic, ih, iw) in variable-major order (all u channels, all v1 channels, all v2 channels) -- for
+ * ic == 1 exactly the reference's 3-channel tensor.  `dx`, `dy` are (n, 2, ih, iw): channel 0 the
+ * edge weight in [0,1], channel 1 the weight beta >= 0 of the auxiliary variables' regulariser.
+ */
+#ifndef TGVINPAINT_H_
+#define TGVINPAINT_H_
+
+#include "tvinpaint.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Replaces FistaTGVHuberB2_id::forward (cudaTGV/cudaCode/TGVInpaintFista.h:70-71,
+ * cudaTGV/cudaCode/TGVInpaintFistaBetas.cu:2475-2618), bound by cudaTGV/TGVInpaintFista_cuda.cpp:47-106.
+ *   dx, dy : (n,2,ih,iw) read only (never scaled in place)     c : (n,1,ih,iw)     b : (n,ic,ih,iw)
+ *   init   : (n,3*ic,ih,iw) starting point                    out : (n,3*ic,ih,iw) x after 2*floor(its/2) iterations
+ * The Lipschitz constant (FistaInpaintB2_findLipshitz, TGVInpaintFistaBetas.cu:101-148,2513-2527) is
+ * computed per sample on the device.  n > 1 runs n independent problems (the reference accepts 1). */
+int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const float* b, const float* init,
+                       float* out, int n, int ic, int ih, int iw, int its, int id, void* stream);
+
+/* Replaces FistaTGVHuberB2_id::backward (TGVInpaintFista.h:81-84, TGVInpaintFistaBetas.cu:2621-3063),
+ * bound by TGVInpaintFista_cuda.cpp:117-172.
+ *   gin     : (n,3*ic,ih,iw) upstream gradient.  If it holds any non-finite entry, or is zero
+ *             everywhere, those entries are zeroed IN PLACE, all five outputs are zero and the id's
+ *             run counter is left alone (TGVInpaintFistaBetas.cu:2686-2703).  This check is the call's
+ *             one host wait.
+ *   gx, gy  : (n,2,ih,iw)   gc : (n,1,ih,iw)   gb : (n,ic,ih,iw)   gi : (n,3*ic,ih,iw)   (overwritten)
+ * Must follow a tgvinpaint_forward with the same shape, its and id. */
+int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const float* b, float* gin,
+                        float* gx, float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih,
+                        int iw, int its, int id, void* stream);
+
+/* Per-id state (idStructBs, TGVInpaintFista.h:7-50); separate from the TV layer's ids.
+ * state6 (host) = {run, av_GC, av_GX, av_GY, av_GB, av_GI}. */
+int tgvinpaint_get_state(int id, double* state6);
+int tgvinpaint_set_state(int id, const double* state6);
+int tgvinpaint_reset_id(int id);
+
+/* Statistics of the last backward's output guard (check_gradUpdate, TGVInpaintFistaHelp.cu:155-177):
+ * 5 tensors (C, X, Y, B, I) x {mean |g|, max |g|, count above 5e6, count non-finite, action}.  The
+ * guard on I looks at the u block only (TGVInpaintFistaBetas.cu:3014-3021). */
+int tgvinpaint_guard_stats(int id, double* stats25);
+
+long long tgvinpaint_slot_bytes(int id);
+
+/* The per-sample step scale L = 1 / (max(32, max_p s_p) + 0.01) the last call on this id used
+ * (host array of n doubles).  Waits for the slot's stream. */
+int tgvinpaint_lipschitz(int id, double* L_host, int n);
+
+/* Host-only: the guard's decision rule with this layer's constants (update_correct_av_step_host,
+ * TGVInpaintFistaHelp.cu:119-151). */
+int tgvinpaint_guard_decide(int run, double av_gc, double av_running, double* mult_out, double* av_out);
+
+/* HIP-event timing of the main adjoint kernel, as tvinpaint_profile / tvinpaint_profile_read. */
+int tgvinpaint_profile(int enable);
+int tgvinpaint_profile_read(double* total_ms, int* launches);
+
+const char* tgvinpaint_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TGVINPAINT_H_ */

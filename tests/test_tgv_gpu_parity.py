@@ -1,0 +1,246 @@
+"""GPU parity of the TGV layer: the HIP path through the C ABI against the CPU oracle on the same
+seeded inputs.
+
+Tolerances (the layer's contract): max-abs error / max-abs oracle value <= 1e-4 on the solution
+(u, v1, v2) and <= 1e-3 on the gradients wrt the two-channel edge weights, confidence, right-hand
+side and starting point.  The kernels reproduce the oracle's arithmetic operation by operation, so
+the observed errors are far smaller (bit-equal is expected); the tests print them.
+"""
+import numpy as np
+import pytest
+import torch
+
+from customnetworklayers_amd.workloads import CONFIGS, tgv_inputs
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 1e-4
+GRAD_TOL = 1e-3
+
+
+def rel_err(a, ref):
+    return float(np.abs(a.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from customnetworklayers_amd.cudaTGV import tgvInpaint_cuda_ext
+
+    return tgvInpaint_cuda_ext
+
+
+@pytest.fixture(scope="module")
+def tgv_oracle():
+    from oracle.oracle_lib import TGVOracle
+
+    o = TGVOracle()
+    o.set_quirks()
+    return o
+
+
+def varying_inputs(n, c, h, w, seed, beta_hi=9.0):
+    """Spatially varying beta (exercises the data-dependent Lipschitz branch and its neighbour
+    offsets) and non-zero auxiliary starting values."""
+    d = tgv_inputs(n, c, h, w, seed=seed, conf_density=0.3)
+    rng = np.random.default_rng(seed + 7)
+    d["dx"][:, 1] = rng.uniform(0.2, beta_hi, (n, h, w)).astype(np.float32)
+    d["dy"][:, 1] = rng.uniform(0.2, beta_hi, (n, h, w)).astype(np.float32)
+    d["di"][:, c:] = rng.normal(0, 0.5, (n, 2 * c, h, w)).astype(np.float32)
+    return d
+
+
+def run_gpu(ext, d, its, pid, fresh=True):
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    if fresh:
+        ext.reset_id(pid)
+    (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, pid)
+    grads = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, pid)
+    torch.cuda.synchronize()
+    return sol.cpu().numpy(), [g.cpu().numpy() for g in grads], t["grad"].cpu().numpy()
+
+
+def run_oracle(o, d, its, pid, fresh=True):
+    if fresh:
+        o.reset_id(pid)
+    sol = o.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], its, pid)
+    gin = d["grad"].copy()
+    grads = o.backward(gin, d["dx"], d["dy"], d["dc"], d["db"], its, pid)
+    return sol, list(grads), gin
+
+
+def compare(name, got, ref):
+    sol, grads, _ = got
+    rsol, rgrads, _ = ref
+    e_out = rel_err(sol, rsol)
+    errs = [rel_err(g, r) for g, r in zip(grads, rgrads)]
+    exact = float((sol == rsol).mean())
+    print("\n[%s] out rel %.2e (bit-equal %.4f)  gx %.2e gy %.2e gc %.2e gb %.2e gi %.2e"
+          % (name, e_out, exact, *errs), flush=True)
+    assert e_out <= OUT_TOL, (name, e_out)
+    for nm, e in zip(("gx", "gy", "gc", "gb", "gi"), errs):
+        assert e <= GRAD_TOL, (name, nm, e)
+    return e_out, errs
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 1, 64, 128, 20),    # the reference's own shape: one flow channel, three state channels
+    (1, 1, 16, 64, 2),      # a single pair of iterations
+    (2, 3, 37, 101, 9),     # ragged, odd its, three channels, two samples
+    (1, 2, 5, 3, 6),        # tiny
+    (1, 2, 1, 70, 4),       # a single row
+    (1, 1, 33, 1, 4),       # a single column
+    (2, 2, 70, 130, 50),    # several segments of unequal length
+    (1, 2, 21, 64, 6),      # exactly one wavefront wide
+    (1, 2, 19, 65, 6),      # one column more
+])
+def test_forward_backward_match_oracle(ext, tgv_oracle, n, c, h, w, its):
+    d = tgv_inputs(n, c, h, w, seed=n * 1000 + h + w + its, conf_density=0.3)
+    print("case n=%d c=%d h=%d w=%d its=%d" % (n, c, h, w, its), flush=True)
+    compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
+
+
+def test_varying_beta_and_per_sample_lipschitz(ext, tgv_oracle):
+    # sample 0: beta up to 9 (bound above 32, data dependent); sample 1: small beta (bound 32)
+    d = varying_inputs(2, 2, 40, 56, seed=11)
+    d["dx"][1, 1] *= 0.2
+    d["dy"][1, 1] *= 0.2
+    got = run_gpu(ext, d, 16, 1)
+    Ls = ext.lipschitz(1, 2)
+    ref_L = [tgv_oracle.lipschitz(d["dx"][s], d["dy"][s])[0] for s in range(2)]
+    assert Ls == ref_L, (Ls, ref_L)
+    assert Ls[0] < Ls[1] == float(np.float32(1.0 / np.float64(np.float32(np.float32(32.0) + np.float32(0.01)))))
+    compare("varying beta", got, run_oracle(tgv_oracle, d, 16, 1))
+
+
+def test_its_zero_and_one_return_init_and_zero_grads(ext, tgv_oracle):
+    d = tgv_inputs(1, 2, 20, 30, seed=5)
+    for its in (0, 1):
+        sol, grads, _ = run_gpu(ext, d, its, 3)
+        np.testing.assert_array_equal(sol, d["di"])
+        rsol, rgrads, _ = run_oracle(tgv_oracle, d, its, 3)
+        for g, r in zip(grads, rgrads):
+            np.testing.assert_array_equal(g, r)
+            assert not g.any()
+
+
+def test_headline_shape_one_sample_short(ext, tgv_oracle):
+    # one sample of the TGV configuration's shape (2 x 384 x 1248), 20 iterations
+    cfg = CONFIGS[2]
+    d = tgv_inputs(1, cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    compare("tgv-config/1 its=20", run_gpu(ext, d, 20, 0), run_oracle(tgv_oracle, d, 20, 0))
+
+
+def test_bad_upstream_returns_zeros_and_does_not_count(ext, tgv_oracle):
+    d = tgv_inputs(1, 2, 24, 40, seed=6)
+    its = 8
+    base = run_gpu(ext, d, its, 4)
+    assert ext.get_state(4)[0] == 1 and all(g.any() for g in base[1])
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    bad = t["grad"].clone()
+    bad[0, 1, 7, 9] = float("nan")
+    bad[0, 0, 0, 0] = float("inf")
+    grads = ext.backward(bad, t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+    torch.cuda.synchronize()
+    assert all(not g.any().item() for g in grads)
+    expect = d["grad"].copy(); expect[0, 1, 7, 9] = 0; expect[0, 0, 0, 0] = 0
+    np.testing.assert_array_equal(bad.cpu().numpy(), expect)  # scrubbed in the caller's tensor
+    assert ext.get_state(4)[0] == 1
+    grads = ext.backward(torch.zeros_like(bad), t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+    torch.cuda.synchronize()
+    assert all(not g.any().item() for g in grads) and ext.get_state(4)[0] == 1
+    # and the slot still serves a good upstream afterwards, identically
+    again = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+    torch.cuda.synchronize()
+    for a, b in zip(again, base[1]):
+        np.testing.assert_array_equal(a.cpu().numpy(), b)
+    assert ext.get_state(4)[0] == 2
+
+
+def test_ids_are_independent_and_separate_from_tv(ext, tgv_oracle):
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as tv_ext
+    from customnetworklayers_amd.workloads import tv_inputs
+
+    dev = torch.device("cuda:0")
+    cases = [tgv_inputs(1, 1, 24 * (i + 1), 40 * (i + 1), seed=30 + i) for i in range(3)]
+    its = 10
+    tens = [{k: torch.from_numpy(v).to(dev) for k, v in d.items()} for d in cases]
+    for i in range(3):
+        ext.reset_id(i)
+    sols = [ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, i)[0] for i, t in enumerate(tens)]
+    # a TV forward on the same id numbers in between must not disturb the TGV slots
+    tvd = {k: torch.from_numpy(v).to(dev) for k, v in tv_inputs(1, 2, 16, 16, seed=1).items()}
+    for i in range(3):
+        tv_ext.forward(tvd["dx"], tvd["dy"], tvd["dc"], tvd["db"], tvd["di"], 4, i)
+    grads = {}
+    for i in (2, 1, 0):
+        t = tens[i]
+        grads[i] = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, i)
+    torch.cuda.synchronize()
+    for i, d in enumerate(cases):
+        ref = run_oracle(tgv_oracle, d, its, i)
+        compare("id%d" % i, (sols[i].cpu().numpy(), [g.cpu().numpy() for g in grads[i]], None), ref)
+
+
+def test_guard_rescales_kills_and_touches_u_only(ext, tgv_oracle):
+    c = 2
+    d = tgv_inputs(1, c, 32, 48, seed=8)
+    its = 8
+    base = run_gpu(ext, d, its, 5)
+    st0 = ext.get_state(5)
+    stats = ext.guard_stats(5)
+    assert all(row[4] == 0 for row in stats)
+    # running means 20x below (C: rescale), 40x below (X: kill, threshold 35), 100x below (I: kill)
+    state = [10, st0[1] / 20, st0[2] / 40, st0[3], st0[4], st0[5] / 100]
+    ext.set_state(5, state)
+    tgv_oracle.reset_id(5)
+    tgv_oracle.set_state(5, state)
+    got = run_gpu(ext, d, its, 5, fresh=False)
+    ref = run_oracle(tgv_oracle, d, its, 5, fresh=False)
+    stats = ext.guard_stats(5)
+    assert [int(r[4]) for r in stats] == [1, 2, 0, 0, 2]
+    assert not got[1][0].any()  # gx killed
+    np.testing.assert_allclose(got[1][2], base[1][2] * 0.5, rtol=1e-5, atol=0)  # gc halved
+    assert not got[1][4][0, :c].any()  # u block of gi killed
+    np.testing.assert_array_equal(got[1][4][0, c:], base[1][4][0, c:])  # v1, v2 gradients pass through
+    compare("guard", got, ref)
+    gs, os_ = ext.get_state(5), tgv_oracle.get_state(5)
+    np.testing.assert_allclose(gs, os_, rtol=1e-9)
+    assert gs[0] == 11
+
+
+def test_errors(ext):
+    dev = torch.device("cuda:0")
+    d = {k: torch.from_numpy(v).to(dev) for k, v in tgv_inputs(1, 2, 8, 8, seed=1).items()}
+    with pytest.raises(IndexError):
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 4, 10)
+    with pytest.raises(TypeError):
+        ext.forward(d["dx"].double(), d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(RuntimeError):
+        ext.forward(d["dx"].cpu(), d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(ValueError):  # one-channel diffusion tensor
+        ext.forward(d["dx"][:, :1].contiguous(), d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(ValueError):  # starting point without the auxiliary variables
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"][:, :2].contiguous(), 4, 0)
+    ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 4, 0)
+    with pytest.raises(RuntimeError):  # its differs from the forward that filled the slot
+        ext.backward(d["grad"], d["dx"], d["dy"], d["dc"], d["db"], 6, 0)
+
+
+def test_module_surface_and_autograd(ext, tgv_oracle):
+    from customnetworklayers_amd import TGVInpaint
+
+    dev = torch.device("cuda:0")
+    d = tgv_inputs(1, 1, 30, 44, seed=9)
+    hwc = lambda a: torch.from_numpy(np.ascontiguousarray(a[0].transpose(1, 2, 0))).to(dev).requires_grad_(True)
+    tx, ty, tc, tb, ti = (hwc(d[k]) for k in ("dx", "dy", "dc", "db", "di"))
+    layer = TGVInpaint(dev, 14, pid=3)
+    ext.reset_id(3)
+    sol = layer(tx, ty, tc, tb, ti)
+    assert tuple(sol.shape) == (30, 44, 3)
+    up = torch.from_numpy(np.ascontiguousarray(d["grad"][0].transpose(1, 2, 0))).to(dev)
+    sol.backward(up)
+    ref = run_oracle(tgv_oracle, d, 14, 3)
+    got_grads = [t.grad.permute(2, 0, 1).unsqueeze(0).cpu().numpy() for t in (tx, ty, tc, tb, ti)]
+    compare("module", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
