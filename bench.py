@@ -21,22 +21,36 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {1: (2 * 72471 + 69740) * 1024}
 
 
-def algorithmic_bytes_per_pixel(c):
-    """One HBM round trip per iteration, fp32: forward 5C+3, recompute 6C+3, adjoint 10C+9 floats."""
+def algorithmic_bytes_per_pixel(c, kind="tv"):
+    """One HBM round trip per iteration, fp32.  TV: forward 5C+3, recompute 6C+3, adjoint 10C+9
+    floats.  TGV (three state variables, four weight fields): forward 13C+5, recompute 16C+5,
+    adjoint 22C+15 floats."""
+    if kind == "tgv":
+        return dict(forward=4 * (13 * c + 5), recompute=4 * (16 * c + 5), adjoint=4 * (22 * c + 15),
+                    total=4 * (51 * c + 25))
     return dict(forward=4 * (5 * c + 3), recompute=4 * (6 * c + 3), adjoint=4 * (10 * c + 9),
                 total=4 * (21 * c + 15))
+
+
+def layer_of(kind):
+    """(binding module, C-ABI prefix, input generator, oracle class name, dominant kernel)."""
+    from customnetworklayers_amd import workloads
+    if kind == "tgv":
+        from customnetworklayers_amd.cudaTGV import tgvInpaint_cuda_ext as ext
+        return ext, "tgvinpaint", workloads.tgv_inputs, "TGVOracle", "tgvstrip::tgv_adjoint_strip<2,false,false>"
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+    return ext, "tvinpaint", workloads.tv_inputs, "TVOracle", "tvstrip::tv_adjoint_strip<2,false,false>"
 
 
 def cpu_baseline(cfg, seconds_hint=20.0):
     """The CPU oracle on a bounded sample of the same workload: ONE sample of the batch, all
     iterations, forward + backward, all host cores (best of 2 after a warm-up) and one core."""
-    import numpy as np
-    from customnetworklayers_amd.workloads import tv_inputs
-    from oracle.oracle_lib import TVOracle
+    import oracle.oracle_lib as oracle_lib
 
-    o = TVOracle()
+    _, _, make_inputs, oracle_name, _ = layer_of(cfg["kind"])
+    o = getattr(oracle_lib, oracle_name)()
     o.set_quirks()
-    d = tv_inputs(1, cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    d = make_inputs(1, cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
     its = cfg["its"]
     pxit = cfg["h"] * cfg["w"] * 2 * (its // 2)
 
@@ -47,7 +61,9 @@ def cpu_baseline(cfg, seconds_hint=20.0):
         o.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], its, 9)
         return time.perf_counter() - t0
 
-    cores = min(o.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or o.max_threads()))
+    import multiprocessing
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else multiprocessing.cpu_count()
+    cores = min(avail, int(os.environ.get("OMP_NUM_THREADS", "0") or avail))
     o.set_threads(cores)
     once()
     t_all = min(once(), once())
@@ -55,7 +71,8 @@ def cpu_baseline(cfg, seconds_hint=20.0):
     t_one = once()
     o.set_threads(cores)
     return dict(value=round(pxit / t_all / 1e6, 3), unit="Mpixel-iter/s", cores=cores, kind="port",
-                sample="1 of 4 samples (2x384x1248), 100 iterations, fwd+bwd, best of 2",
+                sample="1 of %d samples (%dx%dx%d), %d iterations, fwd+bwd, best of 2"
+                       % (cfg["n"], cfg["c"], cfg["h"], cfg["w"], its),
                 one_core_value=round(pxit / t_one / 1e6, 3), host_cpu_count=os.cpu_count())
 
 
@@ -74,13 +91,14 @@ def main():
 
     import torch
     from customnetworklayers_amd._lib import lib
-    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
-    from customnetworklayers_amd.workloads import CONFIGS, config_inputs
+    from customnetworklayers_amd.workloads import config_inputs
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     cfg, d = config_inputs(args.config, seed=0)
-    assert cfg["kind"] == "tv"
+    assert cfg["kind"] in ("tv", "tgv")
+    ext, prefix, _, _, kernel_name = layer_of(cfg["kind"])
+    profile, profile_read = getattr(lib, prefix + "_profile"), getattr(lib, prefix + "_profile_read")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     its, pid = cfg["its"], 0
     n, c, h, w = cfg["n"], cfg["c"], cfg["h"], cfg["w"]
@@ -94,33 +112,34 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    lib.tvinpaint_profile(1)  # HIP events around every launch of the main adjoint kernel
+    profile(1)  # HIP events around every launch of the main adjoint kernel
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     tot_ms, launches = ctypes.c_double(0), ctypes.c_int(0)
-    lib.tvinpaint_profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
-    lib.tvinpaint_profile(0)
+    profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
+    profile(0)
 
     ms_per_step = elapsed * 1e3 / args.steps
     value = pxit / (elapsed / args.steps) / 1e6
-    bpp = algorithmic_bytes_per_pixel(c)
+    bpp = algorithmic_bytes_per_pixel(c, cfg["kind"])
     kernel_ms = tot_ms.value / max(launches.value, 1)
     kernel_bytes = bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9
     out = {
-        "metric": "TV-FISTA fwd+bwd Mpixel-iter/s at 4x2x384x1248; achieved HBM GB/s vs peak",
+        "metric": "%s-FISTA fwd+bwd Mpixel-iter/s at %dx%dx%dx%d; achieved HBM GB/s vs peak"
+                  % (cfg["kind"].upper(), n, c, h, w),
         "value": round(value, 2), "unit": "Mpixel-iter/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "TV inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
+        "config": {"workload": cfg["kind"].upper() + " inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
                                % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
         "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
                       "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4)},
-        "roofline": {"bound": "hbm", "kernel": "tvstrip::tv_adjoint_strip<2,false,false>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.config), "bytes_per_launch": kernel_bytes,
                      "avg_launch_ms": round(kernel_ms, 5), "launches_timed": launches.value},

@@ -47,6 +47,7 @@ def _load():
     lib.tgvinpaint_profile.argtypes = [_int]
     lib.tgvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
     lib.tgvinpaint_last_error.restype = ctypes.c_char_p
+    lib.inpaint_selftest_rsqrt.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_uint]
     return lib
 
 

@@ -2,6 +2,7 @@
 // IEEE expansions.  Diagnostic entry point of the library, used by the GPU test-suite.
 #include "exact_math.h"
 #include "inpaint_common.h"
+#include "tgv_strip_kernels.h"
 
 namespace {
 
@@ -55,7 +56,50 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* count
   if (bad3) atomicAdd(&counts[3], (unsigned long long)bad3);
 }
 
+// counts[0]: rsq_exact(x) against 1.0f / sqrtf(x) over 0 and every float in [2^-96, 2^96]
+// counts[1]: x / 0.2f over the same set (the TGV layer's Huber threshold)
+// counts[2]: 1 / m over every float m in [1, 2^40): the segment-start kernel's Huber weight
+// counts[3]: w / h2 on hashed pairs, w in (2^-20, 1], h2 in [2^-14, 2^6): its weight derivative
+__global__ __launch_bounds__(256) void selftest_rsqrt_kernel(unsigned long long* counts, unsigned int pair_rounds) {
+  const unsigned int tid = blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned int stride = gridDim.x * blockDim.x;
+  unsigned int bad0 = 0, bad1 = 0, bad2 = 0, bad3 = 0;
+  for (unsigned long long i = tid; i < 0x7f800000ULL; i += stride) {
+    const float x = __uint_as_float((unsigned int)i);
+    if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) {
+      bad0 += !same_bits(tgvstrip::rsq_exact(x), 1.0f / sqrtf(x));
+      bad1 += !same_bits(exact_div(x, 0.2f), x / 0.2f);
+    }
+    if (x >= 1.0f && x < 1.0995116e12f) bad2 += !same_bits(exact_div(1.0f, x), 1.0f / x);
+  }
+  for (unsigned int k = 0; k < pair_rounds; k++) {
+    const unsigned int h1 = mix(tid * 2654435761U + k * 40503U + 29U), h2 = mix(h1 ^ 0x9e3779b9U);
+    const float w = __uint_as_float(((127U - 20U + ((h1 >> 23) % 21U)) << 23) | (h1 & 0x7fffffU));
+    const float h = __uint_as_float(((127U - 14U + ((h2 >> 23) % 20U)) << 23) | (h2 & 0x7fffffU));
+    bad3 += !same_bits(exact_div(fminf(w, 1.0f), h), fminf(w, 1.0f) / h);
+  }
+  if (bad0) atomicAdd(&counts[0], (unsigned long long)bad0);
+  if (bad1) atomicAdd(&counts[1], (unsigned long long)bad1);
+  if (bad2) atomicAdd(&counts[2], (unsigned long long)bad2);
+  if (bad3) atomicAdd(&counts[3], (unsigned long long)bad3);
+}
+
+int run_selftest(void (*kernel)(unsigned long long*, unsigned int), unsigned long long* host4, unsigned int rounds) {
+  unsigned long long* dev = nullptr;
+  INPAINT_HIP(hipMalloc((void**)&dev, 4 * sizeof(unsigned long long)));
+  INPAINT_HIP(hipMemset(dev, 0, 4 * sizeof(unsigned long long)));
+  hipLaunchKernelGGL(kernel, dim3(4096), dim3(256), 0, 0, dev, rounds);
+  INPAINT_HIP(hipGetLastError());
+  INPAINT_HIP(hipMemcpy(host4, dev, 4 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+  INPAINT_HIP(hipFree(dev));
+  return 0;
+}
+
 }  // namespace
+
+extern "C" int inpaint_selftest_rsqrt(unsigned long long* mismatches4_host, unsigned int pair_rounds) {
+  return run_selftest(selftest_rsqrt_kernel, mismatches4_host, pair_rounds);
+}
 
 extern "C" int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds) {
   unsigned long long* dev = nullptr;

@@ -16,6 +16,7 @@
 // fused multiply-add (build with -ffp-contract=off).  CUDA's rsqrtf (2 ulp, bits not recoverable
 // from the sources) is taken as 1.0f / sqrtf(x), both correctly rounded.
 #include "inpaint_common.h"
+#include "tgv_strip_kernels.h"
 #include "../../include/tgvinpaint.h"
 
 #include <cstddef>
@@ -706,8 +707,11 @@ struct Slot {
   unsigned int* maxbits = nullptr;                                   // per-sample Lipschitz bound (float bits)
   unsigned int* counts = nullptr;                                    // upstream check
   float *ypp[2] = {nullptr, nullptr}, *xpp[2] = {nullptr, nullptr}, *ckpt_y = nullptr, *ckpt_x = nullptr, *x05 = nullptr;
-  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr}, *yk = nullptr, *gi_u = nullptr;
-  float *acc_gc = nullptr, *acc_gx = nullptr, *acc_gy = nullptr, *acc_gb = nullptr;
+  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr}, *yk = nullptr, *gi_u = nullptr, *gx_final = nullptr;
+  // per-segment fp32 accumulators, double-buffered: a strip-kernel step reads one set and writes the other
+  float *acc_gc[2] = {nullptr, nullptr}, *acc_gx[2] = {nullptr, nullptr}, *acc_gy[2] = {nullptr, nullptr},
+        *acc_gb[2] = {nullptr, nullptr};
+  int acc_cur = 0;
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
   GuardState* guard = nullptr;
   double pending_av[5] = {0, 0, 0, 0, 0};
@@ -745,9 +749,9 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
   const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)std::max(s.max_inter_its, 1);
   size_t need = 0;
-  need += Arena::padded(S3, 4) * (2 + 2 + 2 + 2 + 1) + Arena::padded(S3 * nck, 4) * 2 + Arena::padded(S3 * ring, 4);
-  need += Arena::padded(F, 4) * 2 + Arena::padded(F, 8);
-  need += Arena::padded(P, 4) * (4 + 1) + Arena::padded(2 * P, 4) * 2;
+  need += Arena::padded(S3, 4) * (2 + 2 + 2 + 2 + 1 + 1) + Arena::padded(S3 * nck, 4) * 2 + Arena::padded(S3 * ring, 4);
+  need += Arena::padded(F, 4) * 3 + Arena::padded(F, 8);
+  need += Arena::padded(P, 4) * (4 + 2) + Arena::padded(2 * P, 4) * 4;
   need += Arena::padded(P, 8) + Arena::padded(2 * P, 8) * 2;
   need += Arena::padded((size_t)n, 8) + Arena::padded((size_t)n, 4) + Arena::padded(2, 4);
   need += Arena::padded(1, sizeof(GuardState));
@@ -765,9 +769,12 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   s.g05[0] = a.take<float>(S3); s.g05[1] = a.take<float>(S3);
   s.gxk[0] = a.take<float>(S3); s.gxk[1] = a.take<float>(S3);
   s.yk = a.take<float>(S3);
+  s.gx_final = a.take<float>(S3);
   s.gi_u = a.take<float>(F);
-  s.acc_gb = a.take<float>(F);
-  s.acc_gc = a.take<float>(P); s.acc_gx = a.take<float>(2 * P); s.acc_gy = a.take<float>(2 * P);
+  for (int i = 0; i < 2; i++) {
+    s.acc_gb[i] = a.take<float>(F);
+    s.acc_gc[i] = a.take<float>(P); s.acc_gx[i] = a.take<float>(2 * P); s.acc_gy[i] = a.take<float>(2 * P);
+  }
   s.tot_gc = a.take<double>(P); s.tot_gx = a.take<double>(2 * P); s.tot_gy = a.take<double>(2 * P);
   s.tot_gb = a.take<double>(F);
   s.guard = a.take<GuardState>(1);
@@ -806,19 +813,101 @@ void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const flo
                      s.Ls, HW, P);
 }
 
+// -------------------------------------------------------------------------------------------------
+// kernel selection: wave-strip kernels for 1..2 flow channels, the per-pixel kernels otherwise.
+// INPAINT_TGV_PATH=px forces the per-pixel kernels (used by the tests to keep both paths covered).
+// -------------------------------------------------------------------------------------------------
+bool use_strip(const Slot& s) {
+  const char* e = getenv("INPAINT_TGV_PATH");
+  if (e && strcmp(e, "px") == 0) return false;
+  return s.ic >= 1 && s.ic <= 2;
+}
+int strip_rows(int n, int ih, int iw, const char* env_name) {
+  // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap between
+  // strips, but the launch should still keep every SIMD of the chip busy.
+  if (const char* e = getenv(env_name)) {
+    const int v = atoi(e);
+    if (v >= 1 && v <= 4096) return v;
+  }
+  const long long sx = (iw + tgvstrip::kCols - 1) / tgvstrip::kCols;
+  for (int R : {16, 12, 8, 6, 4, 3}) {
+    const long long waves = sx * ((ih + R - 1) / R) * n;
+    if (waves >= 1792) return R;
+  }
+  return 2;
+}
+
+template <int C>
+void launch_forward_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
+                          float* xout, const float* yin, float* yout, float* x05, float t) {
+  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_FWD_ROWS");
+  const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
+  if (x05)
+    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip<C, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
+                       xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
+  else
+    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip<C, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
+                       xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
+}
+
 void launch_forward(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                     const float* yin, float* yout, float* x05, float t) {
+  if (use_strip(s)) {
+    if (s.ic == 1) launch_forward_strip<1>(s, stream, c, b, xin, xout, yin, yout, x05, t);
+    else launch_forward_strip<2>(s, stream, c, b, xin, xout, yin, yout, x05, t);
+    return;
+  }
   const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
   hipLaunchKernelGGL(tgv_forward_px, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xout, yin, yout, x05,
                      s.ic, s.ih, s.iw, t);
 }
 
+template <int C, bool END>
+void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
+                          const float* xb, const float* yck, const float* g05_in, float* g05_out, const float* gxk,
+                          float* gxk_m1, float* gx_final, float t) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
+  const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
+  if (gx_final)
+    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+                       xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
+                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
+  else
+    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+                       xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
+                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
+}
+
+// One adjoint step.  Strip path: y is rebuilt inside the kernel from xa = x05[k], xb = x05[k-1] (END:
+// read from the checkpoint yck); accumulator set acc_cur is read, the other one written, then
+// acc_cur flips; g_x is stored (to gx_final) only when asked.  Per-pixel path: y comes from the yk
+// buffer (or yck), accumulators and g_x are updated in place.
 template <bool END>
-void launch_adjoint(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* x05,
-                    const float* g05_in, float* g05_out, float* gxk, float* gxk_m1, const float* y, float t) {
+void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa, const float* xb,
+                    const float* yck, const float* g05_in, float* g05_out, float* gxk, float* gxk_m1, float* gx_final,
+                    float t) {
+  if (use_strip(s)) {
+    if (s.ic == 1) launch_adjoint_strip<1, END>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
+    else launch_adjoint_strip<2, END>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
+    s.acc_cur = 1 - s.acc_cur;
+    return;
+  }
+  const float* y = yck;
+  if (!END) {
+    const long long P = (long long)plane_count(s);
+    hipLaunchKernelGGL(tgv_getyk_kernel, dim3(grid1d(P)), dim3(256), 0, stream, c, b, xa, xb, s.yk, s.ic,
+                       (long long)s.ih * s.iw, P, t);
+    y = s.yk;
+  }
+  const int a = s.acc_cur;
   const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
-  hipLaunchKernelGGL(tgv_adjoint_px<END>, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, x05, s.acc_gc, s.acc_gb,
-                     s.acc_gx, s.acc_gy, g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
+  hipLaunchKernelGGL(tgv_adjoint_px<END>, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, s.acc_gc[a],
+                     s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
 }
 
 }  // namespace
@@ -910,11 +999,12 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   {
     ZeroList z;
     int k = 0;
-    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.yk}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
-    z.ptr[k] = s.acc_gb; z.bytes[k++] = (long long)F * 4;
-    z.ptr[k] = s.acc_gc; z.bytes[k++] = (long long)P * 4;
-    z.ptr[k] = s.acc_gx; z.bytes[k++] = (long long)P * 8;
-    z.ptr[k] = s.acc_gy; z.bytes[k++] = (long long)P * 8;
+    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.yk, s.gx_final}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
+    s.acc_cur = 0;
+    z.ptr[k] = s.acc_gb[0]; z.bytes[k++] = (long long)F * 4;
+    z.ptr[k] = s.acc_gc[0]; z.bytes[k++] = (long long)P * 4;
+    z.ptr[k] = s.acc_gx[0]; z.bytes[k++] = (long long)P * 8;
+    z.ptr[k] = s.acc_gy[0]; z.bytes[k++] = (long long)P * 8;
     z.ptr[k] = s.tot_gc; z.bytes[k++] = (long long)P * 8;
     z.ptr[k] = s.tot_gx; z.bytes[k++] = (long long)P * 16;
     z.ptr[k] = s.tot_gy; z.bytes[k++] = (long long)P * 16;
@@ -925,6 +1015,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   // buffer roles of TGV.cu:2718-2736: g05[0]/g05[1] and gxk[0]/gxk[1] ping-pong with the parity of the
   // local iteration index (the copy of the upstream gradient into gxk[0], TGV.cu:2729, is overwritten
   // before it is read and is not made).
+  // The strip kernels store g_x only at the very last step (into gx_final); the per-pixel kernels
+  // keep it in gxk[1] as the reference does.
+  const bool strip = use_strip(s);
+  const float* gi_src = strip ? s.gx_final : s.gxk[1];
   int lastIt = its;
   const int nseg = (int)s.iterations.size();
   for (int outer = nseg - 1; outer >= 0; outer--) {
@@ -943,31 +1037,32 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       const float* xa = s.x05 + (size_t)j * S3;
       const int odd = j & 1;
       if (outer == nseg - 1 && j == len - 1) {
-        hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa, s.acc_gc,
-                           s.acc_gb, s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+        hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
+                           s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = s.x05 + (size_t)(j - 1) * S3;
-        hipLaunchKernelGGL(tgv_getyk_kernel, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa, xb, s.yk, ic,
-                           (long long)ih * iw, (long long)P, t);
         g_timer.mark(stream);
-        launch_adjoint<false>(s, stream, c, b, xa, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0], s.gxk[odd ? 0 : 1],
-                              s.gxk[odd ? 1 : 0], s.yk, t);
+        launch_adjoint<false>(s, stream, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
+                              s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
         g_timer.mark(stream);
       } else {
-        launch_adjoint<true>(s, stream, c, b, xa, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0], cky, t);
+        // the very last step's g_x is the gradient wrt the starting point (TGV.cu:3047)
+        launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
+                             (strip && outer == 0) ? s.gx_final : nullptr, t);
       }
     }
     // fp32 segment sums into the fp64 totals (TGV.cu:2944)
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc, s.tot_gc, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx, s.tot_gx, (long long)(2 * P));
-    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy, s.tot_gy, (long long)(2 * P));
-    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb, s.tot_gb, (long long)F);
+    const int a = s.acc_cur;
+    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[a], s.tot_gc, (long long)P);
+    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
+    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
+    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[a], s.tot_gb, (long long)F);
     lastIt = k0;
   }
 
   // output guard on the device (TGV.cu:2990-3021), then scale and store (TGV.cu:3024-3050)
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
-  hipLaunchKernelGGL(tgv_gather_u, dim3(grid1d((long long)F)), dim3(256), 0, stream, s.gxk[1], s.gi_u,
+  hipLaunchKernelGGL(tgv_gather_u, dim3(grid1d((long long)F)), dim3(256), 0, stream, gi_src, s.gi_u,
                      (long long)ic * ih * iw, (long long)F);
   GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
@@ -995,7 +1090,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
                      kGlobalGMult, 0.0, (const double*)s.Ls, HW2);
   hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, kGuard,
                      kGlobalGMult, 1.0, no_chain, 1LL);
-  hipLaunchKernelGGL(tgv_finalize_init, dim3(grid1d((long long)S3)), dim3(256), 0, stream, s.gxk[1], gi,
+  hipLaunchKernelGGL(tgv_finalize_init, dim3(grid1d((long long)S3)), dim3(256), 0, stream, gi_src, gi,
                      (long long)ic * ih * iw, (long long)S3, s.guard, kGuard);
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TGV.cu:3061

@@ -1,0 +1,591 @@
+// Wave-strip kernels of the TGV layer (the default path for up to 2 flow channels).
+//
+// Same execution scheme as the TV layer's strip kernels: one wavefront owns 62 adjacent columns (one
+// pixel per lane, lanes 0 and 63 are aprons) by R rows of one sample and walks them top to bottom
+// without LDS and without barriers; rows stream through rotating register buffers; neighbouring
+// lanes exchange values with wave-wide DPP shifts.
+//
+// Triangle sharing: the pixel q = (h, w) owns the triangle (q, right of q, below q) and with it three
+// Huber terms: the coupling term on z = grad u - v and the two smoothness terms on grad v1, grad v2.
+// The reference evaluates each of them three times (at q, at the pixel below, at the pixel to the
+// right) with operands that are bit-identical or exact negations of each other, so the owner forms
+// every product once and hands the neighbours' shares on: down the column in registers, to the
+// right through a DPP shift.  Results are bit-identical to the per-pixel evaluation.
+//
+// rsqrt: the layer defines CUDA's rsqrtf as 1.0f / sqrtf(x) (both correctly rounded);
+// rsq_exact() below returns those bits (checked exhaustively by inpaint_selftest_rsqrt).
+#pragma once
+
+#include <type_traits>
+
+#include "exact_math.h"
+#include "tv_strip_kernels.h"
+
+namespace tgvstrip {
+
+using inpaint::div_by;
+using inpaint::exact_div;
+using inpaint::exact_sqrt;
+using inpaint::rcp_refined;
+using tvstrip::from_left_lane;
+using tvstrip::from_right_lane;
+using tvstrip::ldg;
+using tvstrip::stg;
+using tvstrip::strip_geometry;
+using tvstrip::StripGeom;
+
+constexpr int kCols = 62;  // output columns per wavefront (lanes 0 and 63 are aprons)
+constexpr float kD0 = 0.2f, kD1 = 0.2f, kD2 = 0.2f;  // TGV.cu:58-60
+constexpr float kClipLocalGrad = 2000.0f;            // TGV.cu:78
+constexpr float kLocalGCMult = 0.1f;                 // TGV.cu:87
+constexpr float kLocalGXMult = 0.1f;                 // TGV.cu:89
+
+// 1.0f / sqrtf(x) with both operations correctly rounded; +inf at 0.  Inputs below 2^-96 may be
+// one ulp off, which no caller can see: their Huber weight is 1 either way.
+__device__ __forceinline__ float rsq_exact(float x) {
+  const float r = exact_div(1.0f, exact_sqrt(x));
+  return (x == 0.0f) ? __builtin_inff() : r;
+}
+
+// Huber weight of the main kernels: min(1, rsqrt(A) * delta)  (TGV.cu:1624 and siblings)
+__device__ __forceinline__ float huber_w(float A, float delta) { return fminf(1.f, rsq_exact(A) * delta); }
+
+// -------------------------------------------------------------------------------------------------
+// Forward iteration, TGV.cu:1546-1776 (and 2005-2235 when x05 is given).
+//
+// Per triangle (owner q) six products are formed once:
+//     Fa = wy (z2 hwx)    Fb = wx (z1 hwx)         z = (y_q - y_right + y1_q, y_q - y_down + y2_q)
+//     G1y = bx (u12 hwy1) G1x = bx (u11 hwy1)      u1 = (y1_q - y1_right, y1_q - y1_down)
+//     G2y = by (u22 hwy2) G2x = by (u21 hwy2)      u2 likewise on y2
+// q subtracts all of them (TGV.cu:1678-1684), the pixel below subtracts -Fa, -G1y, -G2y
+// (TGV.cu:1637-1639) and the pixel to the right -Fb, -G1x, -G2x (TGV.cu:1665-1667).
+// -------------------------------------------------------------------------------------------------
+template <int C>
+struct FwdRow {
+  float y[3][C], x[3][C], bb[C], c, rc1, wxs, wys, bxs, bys;
+};
+
+template <int C, bool X05>
+__global__ __launch_bounds__(256) void tgv_forward_strip(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
+    const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
+    const float* __restrict__ xin, float* __restrict__ xout, const float* __restrict__ yin,
+    float* __restrict__ yout, float* __restrict__ x05, int N, int H, int W, float t, int R, int strips_x,
+    int strips_y) {
+  StripGeom g;
+  if (!strip_geometry(g, kCols, R, W, strips_x, strips_y, N)) return;
+  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
+  const bool rmask = g.col_ok && g.w < W - 1;  // the pixel has a right neighbour
+  const int Reff = min(R, H - g.hs);
+  const size_t poff = (size_t)g.n * HW;
+  const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
+                     *const cf_p = cf + poff;
+  const float *y_p[3][C], *x_p[3][C], *b_p[C];
+  float *yo_p[3][C], *xo_p[3][C], *xh_p[3][C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) {
+    b_p[ch] = b + ((size_t)g.n * C + ch) * HW;
+#pragma unroll
+    for (int v = 0; v < 3; v++) {
+      const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
+      y_p[v][ch] = yin + q; x_p[v][ch] = xin + q;
+      yo_p[v][ch] = yout + q; xo_p[v][ch] = xout + q; xh_p[v][ch] = X05 ? x05 + q : nullptr;
+    }
+  }
+
+  auto load_row = [&](int k, FwdRow<C>& in) {  // row k of the strip = image row hs - 1 + k
+    const int kk = min(k, Reff + 1);
+    const int h = g.hs - 1 + kk;
+    const unsigned row = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4;
+    // the rows above and below the strip contribute y (and, above, the weights) only; their other
+    // fields are read from the strip's own first / last row, which is in L1 anyway
+    const int hw = g.hs - 1 + min(kk, Reff);
+    const unsigned row_w = (unsigned)(hw < 0 ? 0 : hw) * W4;
+    const unsigned row_p = (unsigned)(g.hs - 1 + max(1, min(kk, Reff))) * W4;
+    in.c = ldg(cf_p, row_p + wc);
+    in.wxs = ldg(wx_p, row_w + wc);
+    in.wys = ldg(wy_p, row_w + wc);
+    in.bxs = ldg(bx_p, row_w + wc);
+    in.bys = ldg(by_p, row_w + wc);
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      in.bb[ch] = ldg(b_p[ch], row_p + wc);
+#pragma unroll
+      for (int v = 0; v < 3; v++) {
+        in.y[v][ch] = ldg(y_p[v][ch], row + wc);
+        in.x[v][ch] = ldg(x_p[v][ch], row_p + wc);
+      }
+    }
+  };
+  auto absorb = [&](int k, FwdRow<C>& o) {
+    const int h = g.hs - 1 + k;
+    const bool ok = g.col_ok && h >= 0 && h < H;
+    o.rc1 = rcp_refined(1.f + o.c);
+    o.wxs = (ok && rmask) ? o.wxs : 0.f;
+    o.wys = (ok && h < H - 1) ? o.wys : 0.f;
+    o.bxs = ok ? o.bxs : 0.f;
+    o.bys = ok ? o.bys : 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++)
+#pragma unroll
+      for (int v = 0; v < 3; v++) o.y[v][ch] = ok ? o.y[v][ch] : 0.f;
+  };
+
+  float upFa[C], upG1y[C], upG2y[C];  // terms handed down to the row below
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) upFa[ch] = upG1y[ch] = upG2y[ch] = 0.f;
+
+  auto compute = [&](int r, const FwdRow<C>& cur, const FwdRow<C>& nxt, auto first) {
+    const int h = g.hs - 1 + r;
+    const bool dmask = h >= 0 && h < H - 1;  // the pixel has a lower neighbour
+    const unsigned roff = (unsigned)(h >= 0 ? h : 0) * W4 + wc;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const float yc = cur.y[0][ch], y1c = cur.y[1][ch], y2c = cur.y[2][ch];
+      const float yr = from_right_lane(yc), y1r = from_right_lane(y1c), y2r = from_right_lane(y2c);
+      const float yd = nxt.y[0][ch], y1d = nxt.y[1][ch], y2d = nxt.y[2][ch];
+      // own triangle, TGV.cu:1669-1684
+      const float zij_1 = rmask ? ((yc - yr) + y1c) : 0.f;
+      const float zij_2 = dmask ? ((yc - yd) + y2c) : 0.f;
+      const float hwx = huber_w(zij_2 * zij_2 * cur.wys + zij_1 * zij_1 * cur.wxs, kD0);
+      const float u11 = rmask ? (y1c - y1r) : 0.f;
+      const float u12 = dmask ? (y1c - y1d) : 0.f;
+      const float hwy1 = huber_w(cur.bxs * (u12 * u12 + u11 * u11), kD1);
+      const float u21 = rmask ? (y2c - y2r) : 0.f;
+      const float u22 = dmask ? (y2c - y2d) : 0.f;
+      const float hwy2 = huber_w(cur.bys * (u22 * u22 + u21 * u21), kD2);
+      const float Fa = cur.wys * (zij_2 * hwx), Fb = cur.wxs * (zij_1 * hwx);
+      const float G1y = cur.bxs * (u12 * hwy1), G1x = cur.bxs * (u11 * hwy1);
+      const float G2y = cur.bys * (u22 * hwy2), G2x = cur.bys * (u21 * hwy2);
+      const float aFa = upFa[ch], aG1y = upG1y[ch], aG2y = upG2y[ch];
+      upFa[ch] = Fa; upG1y[ch] = G1y; upG2y[ch] = G2y;
+      if (first.value) continue;
+      const float lFb = from_left_lane(Fb), lG1x = from_left_lane(G1x), lG2x = from_left_lane(G2x);
+      float yt = yc, y1n = y1c, y2n = y2c;
+      yt -= -aFa;    // TGV.cu:1637
+      y1n -= -aG1y;  // TGV.cu:1638
+      y2n -= -aG2y;  // TGV.cu:1639
+      yt -= -lFb;    // TGV.cu:1665
+      y1n -= -lG1x;  // TGV.cu:1666
+      y2n -= -lG2x;  // TGV.cu:1667
+      yt -= Fa;          // TGV.cu:1678
+      y1n -= G1y;        // TGV.cu:1679
+      y2n -= G2y + Fa;   // TGV.cu:1680
+      yt -= Fb;          // TGV.cu:1682
+      y1n -= G1x + Fb;   // TGV.cu:1683
+      y2n -= G2x;        // TGV.cu:1684
+      const float y1o = y1n + t * (y1n - cur.x[1][ch]);  // TGV.cu:1686-1687
+      const float y2o = y2n + t * (y2n - cur.x[2][ch]);
+      const float xh = yt;
+      const float c = cur.c, bv = cur.bb[ch];
+      float x_loc = div_by(c * bv + yt, 1.f + c, cur.rc1);  // TGV.cu:1740
+      const float lo = yt - c, hi = yt + c;
+      if (lo > 1.f + bv) x_loc = lo;
+      if (hi < bv - 1.f) x_loc = hi;
+      const float yn = x_loc + t * (x_loc - cur.x[0][ch]);  // TGV.cu:1772
+      if (store_lane) {
+        stg(yo_p[0][ch], roff, yn);
+        stg(yo_p[1][ch], roff, y1o);
+        stg(yo_p[2][ch], roff, y2o);
+        stg(xo_p[0][ch], roff, x_loc);
+        stg(xo_p[1][ch], roff, y1n);
+        stg(xo_p[2][ch], roff, y2n);
+        if (X05) {
+          stg(xh_p[0][ch], roff, xh);
+          stg(xh_p[1][ch], roff, y1n);
+          stg(xh_p[2][ch], roff, y2n);
+        }
+      }
+    }
+  };
+  const std::true_type kFirst{};
+  const std::false_type kRow{};
+
+  FwdRow<C> b0, b1, b2, b3;
+  load_row(0, b0);
+  load_row(1, b1);
+  load_row(2, b2);
+  load_row(3, b3);
+  absorb(0, b0);
+  absorb(1, b1);
+  compute(0, b0, b1, kFirst);
+  load_row(4, b0);
+  for (int r = 1; r <= Reff; r += 4) {  // cur / next rotate through (b1,b2) (b2,b3) (b3,b0) (b0,b1)
+    absorb(r + 1, b2);
+    compute(r, b1, b2, kRow);
+    load_row(r + 4, b1);
+    if (r + 1 > Reff) break;
+    absorb(r + 2, b3);
+    compute(r + 1, b2, b3, kRow);
+    load_row(r + 5, b2);
+    if (r + 2 > Reff) break;
+    absorb(r + 3, b0);
+    compute(r + 2, b3, b0, kRow);
+    load_row(r + 6, b3);
+    if (r + 3 > Reff) break;
+    absorb(r + 4, b1);
+    compute(r + 3, b0, b1, kRow);
+    load_row(r + 7, b0);
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Adjoint iteration with the y rebuild fused in: TGV.cu:224-644 (+1478-1541); END = the
+// segment-start variant TGV.cu:1061-1472 that reads y from the checkpoint and writes the Huber
+// weights with sqrt and divisions.
+//
+// Per triangle (owner q), with dy = (g_q - g_right + g1_q, g_q - g_down + g2_q), a = (z1 wx, z2 wy),
+// deriv = dy1 a1 + dy2 a2, and for each smoothness term dg = (g1_q - g1_right, g1_q - g1_down),
+// S = dg1 u1 + dg2 u2:
+//     coupling term     Da = (W dy2) wy, Ea = deriv (a2 dW)  -> q's v2 row, negated: u row of the pixel below
+//                       Db = (W dy1) wx, Eb = deriv (a1 dW)  -> q's v1 row, negated: u row of the pixel to the right
+//     smoothness terms  Hy = (b Wy) dg2, Ny = (b ((dWy b) u2)) S -> q (Hy), negated: the pixel below
+//                       Hx = (b Wy) dg1, Nx = (b ((dWy b) u1)) S -> q (Hx), negated: the pixel to the right
+// Every product keeps the reference's operand order; an inactive triangle contributes E = N = 0.
+// -------------------------------------------------------------------------------------------------
+template <int C>
+struct AdjRow {
+  float c, rc1, wxs, wys, bxs, bys;
+  float y[3][C];   // y[0]: loaded as x05[k-1] (or the checkpoint y) and rebuilt in place; y[1], y[2]: x05[k] aux (or checkpoint)
+  float xa[C];     // x05[k] of u, for the prox regime
+  float bb[C], g[3][C];
+  float gx_i[3][C], gb_i[C], gc_i, gwx0_i, gwx1_i, gwy0_i, gwy1_i;
+  double opc_d;
+};
+
+template <int C, bool END, bool FINAL>
+__global__ __launch_bounds__(256) void tgv_adjoint_strip(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
+    const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
+    const float* __restrict__ x05a, const float* __restrict__ x05b, const float* __restrict__ yck,
+    const float* __restrict__ gc_in, float* __restrict__ gc, const float* __restrict__ gb_in, float* __restrict__ gb,
+    const float* __restrict__ gwx_in, float* __restrict__ gwx, const float* __restrict__ gwy_in,
+    float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
+    const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, int N, int H, int W,
+    float t, int R, int strips_x, int strips_y) {
+  StripGeom g;
+  if (!strip_geometry(g, kCols, R, W, strips_x, strips_y, N)) return;
+  const int Reff = min(R, H - g.hs);
+  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
+  const bool rmask = g.col_ok && g.w < W - 1;
+  const double opt = 1. + (double)t;
+  const float gxm = kLocalGXMult;
+  const size_t poff = (size_t)g.n * HW;
+  const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
+                     *const cf_p = cf + poff;
+  const float *const gci_p = gc_in + poff, *const gwx0i_p = gwx_in + 2 * poff, *const gwx1i_p = gwx_in + 2 * poff + HW,
+                     *const gwy0i_p = gwy_in + 2 * poff, *const gwy1i_p = gwy_in + 2 * poff + HW;
+  float *const gco_p = gc + poff, *const gwx0o_p = gwx + 2 * poff, *const gwx1o_p = gwx + 2 * poff + HW,
+               *const gwy0o_p = gwy + 2 * poff, *const gwy1o_p = gwy + 2 * poff + HW;
+  const float *ys_p[3][C], *xa_p[C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
+  float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) {
+    const size_t qb = ((size_t)g.n * C + ch) * HW;
+    b_p[ch] = b + qb; gbi_p[ch] = gb_in + qb; gbo_p[ch] = gb + qb;
+#pragma unroll
+    for (int v = 0; v < 3; v++) {
+      const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
+      // y sources: u from x05[k-1] (rebuilt with x05[k]), aux straight from x05[k] (TGV.cu:1536-1537);
+      // END: all three from the checkpoint y
+      ys_p[v][ch] = (END ? yck : (v == 0 ? x05b : x05a)) + q;
+      g_p[v][ch] = g05_in + q; gxi_p[v][ch] = gxk + q;
+      g05o_p[v][ch] = g05_out + q; gxm_p[v][ch] = gxk_m1 + q; gxf_p[v][ch] = FINAL ? gx_final + q : nullptr;
+    }
+    xa_p[ch] = x05a + (size_t)g.n * 3 * CHW + (size_t)ch * HW;
+  }
+
+  auto load_row = [&](int k, AdjRow<C>& in) {
+    const int kk = min(k, Reff + 1);
+    const int h = g.hs - 1 + kk;
+    const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+    const int hw = g.hs - 1 + min(kk, Reff);
+    const unsigned off_w = (unsigned)(hw < 0 ? 0 : hw) * W4 + wc;
+    const unsigned off_p = (unsigned)(g.hs - 1 + max(1, min(kk, Reff))) * W4 + wc;
+    in.c = ldg(cf_p, off);
+    in.wxs = ldg(wx_p, off_w);
+    in.wys = ldg(wy_p, off_w);
+    in.bxs = ldg(bx_p, off_w);
+    in.bys = ldg(by_p, off_w);
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      in.xa[ch] = ldg(xa_p[ch], off);
+      in.bb[ch] = ldg(b_p[ch], off);
+      in.gb_i[ch] = ldg(gbi_p[ch], off_p);
+#pragma unroll
+      for (int v = 0; v < 3; v++) {
+        in.y[v][ch] = ldg(ys_p[v][ch], off);
+        in.g[v][ch] = ldg(g_p[v][ch], off);
+        in.gx_i[v][ch] = ldg(gxi_p[v][ch], off_p);
+      }
+    }
+    in.gc_i = ldg(gci_p, off_p);
+    in.gwx0_i = ldg(gwx0i_p, off_p);
+    in.gwx1_i = ldg(gwx1i_p, off_p);
+    in.gwy0_i = ldg(gwy0i_p, off_p);
+    in.gwy1_i = ldg(gwy1i_p, off_p);
+  };
+  auto absorb = [&](int k, AdjRow<C>& o) {
+    const int h = g.hs - 1 + k;
+    const bool ok = g.col_ok && h >= 0 && h < H;
+    o.c = ok ? o.c : 0.f;
+    o.rc1 = rcp_refined(1.f + o.c);
+    o.opc_d = 1. + (double)o.c;
+    o.wxs = (ok && rmask) ? o.wxs : 0.f;
+    o.wys = (ok && h < H - 1) ? o.wys : 0.f;
+    o.bxs = ok ? o.bxs : 0.f;
+    o.bys = ok ? o.bys : 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.y[0][ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+      o.y[0][ch] = END ? xb : tvstrip::rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
+      o.y[1][ch] = ok ? o.y[1][ch] : 0.f;
+      o.y[2][ch] = ok ? o.y[2][ch] : 0.f;
+      o.xa[ch] = xa;
+      o.bb[ch] = bv;
+#pragma unroll
+      for (int v = 0; v < 3; v++) o.g[v][ch] = ok ? o.g[v][ch] : 0.f;
+    }
+  };
+
+  // terms handed down to the row below: coupling (Da, Ea) and the two smoothness terms (Hy, Ny)
+  float dDa[C], dEa[C], dH1[C], dN1[C], dH2[C], dN2[C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) dDa[ch] = dEa[ch] = dH1[ch] = dN1[ch] = dH2[ch] = dN2[ch] = 0.f;
+
+  // Huber weight, activity and weight derivative of one term in the kernel's own form
+  auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2) {
+    if (END) {  // TGV.cu:1132-1138
+      const float hub = exact_sqrt(A);
+      Wt = exact_div(1.0f, fmaxf(1.f, exact_div(hub, delta)));
+      act = hub > delta;
+      hub2 = hub * hub;
+      dW = exact_div(Wt, hub2);
+    } else {  // TGV.cu:313-319
+      const float hub = rsq_exact(A);
+      Wt = fminf(1.f, hub * delta);
+      act = Wt < 1.0f;
+      hub2 = hub * hub;
+      dW = Wt * hub2;
+    }
+  };
+
+  auto compute = [&](int r, const AdjRow<C>& cur, const AdjRow<C>& nxt, auto first) {
+    const int h = g.hs - 1 + r;  // owner row of this step
+    const bool dmask = h >= 0 && h < H - 1;
+    const unsigned roff = (unsigned)(h >= 0 ? h : 0) * W4 + wc;
+    float gcv = cur.gc_i, gwx0 = cur.gwx0_i, gwx1 = cur.gwx1_i, gwy0 = cur.gwy0_i, gwy1 = cur.gwy1_i, rc2 = 0.f;
+    if (!first.value) rc2 = rcp_refined((1.f + cur.c) * (1.f + cur.c));
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const float yk = cur.y[0][ch], y1c = cur.y[1][ch], y2c = cur.y[2][ch];
+      const float gk = cur.g[0][ch], g1k = cur.g[1][ch], g2k = cur.g[2][ch];
+      const float yr = from_right_lane(yk), y1r = from_right_lane(y1c), y2r = from_right_lane(y2c);
+      const float gr = from_right_lane(gk), g1r = from_right_lane(g1k), g2r = from_right_lane(g2k);
+      const float yd = nxt.y[0][ch], y1d = nxt.y[1][ch], y2d = nxt.y[2][ch];
+      const float gd = nxt.g[0][ch], g1d = nxt.g[1][ch], g2d = nxt.g[2][ch];
+      const float wxv = cur.wxs, wyv = cur.wys, bX = cur.bxs, bY = cur.bys;
+
+      // ---- coupling term, TGV.cu:421-455 / 1230-1260 ----
+      const float aij_1 = rmask ? ((yr - yk) - y1c) : 0.f;
+      const float aij_2 = dmask ? ((yd - yk) - y2c) : 0.f;
+      float Wt, dW, hub2;
+      bool act;
+      huber(aij_2 * aij_2 * wyv + aij_1 * aij_1 * wxv, kD0, Wt, act, dW, hub2);
+      const float dy1 = gk - gr + g1k;
+      const float dy2 = gk - gd + g2k;
+      const float a1 = aij_1 * wxv, a2 = aij_2 * wyv;
+      const float deriv = dy1 * a1 + dy2 * a2;
+      const float Da = Wt * dy2 * wyv, Db = Wt * dy1 * wxv;
+      const float Ea = act ? deriv * (a2 * dW) : 0.f;
+      const float Eb = act ? deriv * (a1 * dW) : 0.f;
+      const float E0 = act ? deriv * ((a1 + a2) * dW) : 0.f;
+
+      // ---- smoothness term of v1, TGV.cu:457-479 / 1262-1284 ----
+      const float u11 = rmask ? (y1r - y1c) : 0.f;
+      const float u12 = dmask ? (y1d - y1c) : 0.f;
+      float W1, dW1, h1sq;
+      bool act1;
+      huber((u11 * u11 + u12 * u12) * bX, kD1, W1, act1, dW1, h1sq);
+      const float dg1x = g1k - g1r, dg1y = g1k - g1d;
+      const float H1x = rmask ? bX * W1 * dg1x : 0.f;
+      const float H1y = dmask ? bX * W1 * dg1y : 0.f;
+      const float S1 = dg1x * u11 + dg1y * u12;
+      const float dv1 = dg1x * u11 * bX + dg1y * u12 * bX;
+      const float R1 = act1 ? bX * dW1 * (u11 + u12) * dv1 : 0.f;
+      const float N1y = act1 ? bX * (dW1 * bX * u12) * S1 : 0.f;
+      const float N1x = act1 ? bX * (dW1 * bX * u11) * S1 : 0.f;
+
+      // ---- smoothness term of v2, TGV.cu:481-505 / 1286-1310 ----
+      const float u21 = rmask ? (y2r - y2c) : 0.f;
+      const float u22 = dmask ? (y2d - y2c) : 0.f;
+      float W2, dW2, h2sq;
+      bool act2;
+      huber((u21 * u21 + u22 * u22) * bY, kD2, W2, act2, dW2, h2sq);
+      const float dg2x = g2k - g2r, dg2y = g2k - g2d;
+      const float H2x = rmask ? bY * W2 * dg2x : 0.f;
+      const float H2y = dmask ? bY * W2 * dg2y : 0.f;
+      const float S2 = dg2x * u21 + dg2y * u22;
+      const float dv2 = dg2x * u21 * bY + dg2y * u22 * bY;
+      const float R2 = act2 ? bY * dW2 * (u21 + u22) * dv2 : 0.f;
+      // the main kernel's upper-triangle v2 block divides by hub^2 where every sibling multiplies (TGV.cu:355)
+      const float dW2_below = END ? dW2 : exact_div(W2, h2sq);
+      const float N2y = act2 ? bY * (dW2_below * bY * u22) * S2 : 0.f;
+      const float N2x = act2 ? bY * (dW2 * bY * u21) * S2 : 0.f;
+
+      // shares of the pixel to the right
+      const float lDb = from_left_lane(Db), lEb = from_left_lane(Eb);
+      const float lH1 = from_left_lane(H1x), lN1 = from_left_lane(N1x);
+      const float lH2 = from_left_lane(H2x), lN2 = from_left_lane(N2x);
+      // shares handed down from the row above
+      const float aDa = dDa[ch], aEa = dEa[ch], aH1 = dH1[ch], aN1 = dN1[ch], aH2 = dH2[ch], aN2 = dN2[ch];
+      dDa[ch] = Da; dEa[ch] = Ea; dH1[ch] = H1y; dN1[ch] = N1y; dH2[ch] = H2y; dN2[ch] = N2y;
+
+      if (!first.value) {
+        // weight gradients of the pixel's own triangle (edge weights: channel 0, beta: channel 1)
+        if (END) {  // TGV.cu:1245-1246
+          gwx0 = gwx0 + gxm * dy1 * aij_1 * Wt;
+          gwy0 = gwy0 + gxm * dy2 * aij_2 * Wt;
+        } else {  // TGV.cu:438-439
+          gwx0 = gwx0 + gxm * dy1 * (aij_1 * Wt);
+          gwy0 = gwy0 + gxm * dy2 * (aij_2 * Wt);
+        }
+        {  // the literal 0.5 makes these updates double (TGV.cu:452-453)
+          const float ny = (float)((double)gwy0 - (double)(gxm * (aij_2 * dW * aij_2)) * 0.5 * (double)deriv);
+          const float nx = (float)((double)gwx0 - (double)(gxm * (aij_1 * dW * aij_1)) * 0.5 * (double)deriv);
+          gwy0 = act ? ny : gwy0;
+          gwx0 = act ? nx : gwx0;
+        }
+        gwx1 = gwx1 + gxm * S1 * W1;  // TGV.cu:468-469
+        {
+          const float n1 = (float)((double)gwx1 - (double)(gxm * (u12 * dW1 * u12 + u11 * dW1 * u11)) * 0.5 * (double)dv1);
+          gwx1 = act1 ? n1 : gwx1;  // TGV.cu:478
+        }
+        gwy1 = gwy1 + gxm * S2 * W2;  // TGV.cu:494-495
+        {
+          const float n2 = (float)((double)gwy1 - (double)(gxm * (u22 * dW2 * u22 + u21 * dW2 * u21)) * 0.5 * (double)dv2);
+          gwy1 = act2 ? n2 : gwy1;  // TGV.cu:503
+        }
+
+        float t0 = gk, t1 = g1k, t2 = g2k;
+        // triangles of the pixel above (TGV.cu:304-360)
+        t0 -= -aDa;
+        t0 += -aEa;
+        t1 -= -aH1;
+        t1 += -aN1;
+        t2 -= -aH2;
+        t2 += -aN2;
+        // triangles of the pixel to the left (TGV.cu:361-418)
+        t0 -= -lDb;
+        t0 += -lEb;
+        t1 -= -lH1;
+        t1 += -lN1;
+        t2 -= -lH2;
+        t2 += -lN2;
+        // own triangle
+        if (END) {  // TGV.cu:1241-1244
+          t0 -= dy2 * wyv * Wt;
+          t0 -= dy1 * wxv * Wt;
+          t1 -= Wt * (g1k - gr + gk) * wxv;
+          t2 -= Wt * (g2k - gd + gk) * wyv;
+        } else {  // TGV.cu:435-437
+          t0 -= Wt * (dy2 * wyv + dy1 * wxv);
+          t1 -= Db;
+          t2 -= Da;
+        }
+        t0 += E0;  // TGV.cu:447-449
+        t2 += Ea;
+        t1 += Eb;
+        if (END) {  // TGV.cu:1271-1274: the v1 block takes the lower neighbour first
+          t1 -= H1y;
+          t1 -= H1x;
+        } else {  // TGV.cu:463-466
+          t1 -= H1x;
+          t1 -= H1y;
+        }
+        t1 += R1;
+        t2 -= H2x;  // TGV.cu:489-492
+        t2 -= H2y;
+        t2 += R2;
+
+        // aux variables: momentum adjoint only (TGV.cu:560-577)
+        const float gxm1 = -t * t1;
+        float d1 = (float)((double)cur.gx_i[1][ch] + opt * (double)t1);
+        d1 = fmaxf(-kClipLocalGrad, fminf(d1, kClipLocalGrad));
+        const float gxm2 = -t * t2;
+        float d2 = (float)((double)cur.gx_i[2][ch] + opt * (double)t2);
+        d2 = fmaxf(-kClipLocalGrad, fminf(d2, kClipLocalGrad));
+        // u: momentum adjoint (TGV.cu:579-585), then prox adjoint (TGV.cu:592-612)
+        float df = (float)((double)cur.gx_i[0][ch] + opt * (double)t0);
+        df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
+        const float gxm0 = -t * t0;
+        const float conf = cur.c, bv = cur.bb[ch], xh = cur.xa[ch];
+        const float diff = bv - xh;
+        const float sign = (diff < 0) ? -1.f : 1.f;
+        const bool quad = (cur.opc_d >= (double)(sign * diff));
+        const float opc = 1.f + conf;
+        const float gc_q = df * (div_by(bv, opc, cur.rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kLocalGCMult;
+        const float g05_q = div_by(df, opc, cur.rc1);
+        const float gb_q = div_by(df * conf, opc, cur.rc1) * 1.0f;
+        const bool mid = !quad && (conf >= sign * diff);
+        const float g05v = quad ? g05_q : (mid ? 0.f : df);
+        gcv += quad ? gc_q : (mid ? 0.f : sign * df * kLocalGCMult);
+        float gbv = cur.gb_i[ch];
+        gbv += quad ? gb_q : (mid ? df * 1.0f : 0.f);
+        if (store_lane) {
+          if (FINAL) {  // only the last step's g_x is read again (TGV.cu:3047)
+            stg(gxf_p[0][ch], roff, df);
+            stg(gxf_p[1][ch], roff, d1);
+            stg(gxf_p[2][ch], roff, d2);
+          }
+          stg(gxm_p[0][ch], roff, gxm0);
+          stg(gxm_p[1][ch], roff, gxm1);
+          stg(gxm_p[2][ch], roff, gxm2);
+          stg(g05o_p[0][ch], roff, g05v);
+          stg(g05o_p[1][ch], roff, d1);
+          stg(g05o_p[2][ch], roff, d2);
+          stg(gbo_p[ch], roff, gbv);
+        }
+      }
+    }
+    if (!first.value && store_lane) {
+      stg(gco_p, roff, gcv);
+      stg(gwx0o_p, roff, gwx0);
+      stg(gwx1o_p, roff, gwx1);
+      stg(gwy0o_p, roff, gwy0);
+      stg(gwy1o_p, roff, gwy1);
+    }
+  };
+  const std::true_type kFirst{};
+  const std::false_type kRow{};
+
+  AdjRow<C> b0, b1, b2;
+  load_row(0, b0);
+  load_row(1, b1);
+  load_row(2, b2);
+  absorb(0, b0);
+  absorb(1, b1);
+  compute(0, b0, b1, kFirst);
+  load_row(3, b0);
+  for (int r = 1; r <= Reff; r += 3) {  // cur / next rotate through (b1,b2) (b2,b0) (b0,b1)
+    absorb(r + 1, b2);
+    compute(r, b1, b2, kRow);
+    load_row(r + 3, b1);
+    if (r + 1 > Reff) break;
+    absorb(r + 2, b0);
+    compute(r + 1, b2, b0, kRow);
+    load_row(r + 4, b2);
+    if (r + 2 > Reff) break;
+    absorb(r + 3, b1);
+    compute(r + 2, b0, b1, kRow);
+    load_row(r + 5, b0);
+  }
+}
+
+}  // namespace tgvstrip

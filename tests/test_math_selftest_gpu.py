@@ -15,3 +15,13 @@ def test_exact_math_matches_ieee_on_the_gpu():
     assert rc == 0, last_error()
     print("mismatches: sqrt %d, x/0.1 %d, n/d %d, shared-reciprocal n/d %d" % tuple(out), flush=True)
     assert list(out) == [0, 0, 0, 0]
+
+
+def test_tgv_rsqrt_and_divisions_match_ieee_on_the_gpu():
+    from customnetworklayers_amd._lib import last_error, lib
+
+    out = (ctypes.c_ulonglong * 4)()
+    rc = lib.inpaint_selftest_rsqrt(out, 4096)
+    assert rc == 0, last_error()
+    print("mismatches: 1/sqrt %d, x/0.2 %d, 1/m %d, w/h2 %d" % tuple(out), flush=True)
+    assert list(out) == [0, 0, 0, 0]

@@ -100,6 +100,29 @@ def test_forward_backward_match_oracle(ext, tgv_oracle, n, c, h, w, its):
     compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 33, 64, 9), (1, 3, 20, 64, 6)])
+def test_per_pixel_kernels_when_forced_or_needed(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
+    # up to 2 flow channels normally take the wave-strip kernels; force the per-pixel kernels
+    # (3 channels always takes them)
+    d = varying_inputs(n, c, h, w, seed=77 + c)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    compare("default path c=%d" % c, run_gpu(ext, d, its, 2), ref)
+    monkeypatch.setenv("INPAINT_TGV_PATH", "px")
+    compare("per-pixel path c=%d" % c, run_gpu(ext, d, its, 2), ref)
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 1, 9, 62, 8),       # exactly one strip wide
+    (1, 2, 11, 63, 8),      # one column more than a strip
+    (2, 2, 45, 508, 14),    # several strips wide, ragged rows
+    (1, 2, 40, 125, 10),    # two strips and a column
+    (3, 1, 130, 200, 50),   # several segments of unequal length
+])
+def test_strip_edges(ext, tgv_oracle, n, c, h, w, its):
+    d = varying_inputs(n, c, h, w, seed=n * 100 + h + w)
+    compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
+
+
 def test_varying_beta_and_per_sample_lipschitz(ext, tgv_oracle):
     # sample 0: beta up to 9 (bound above 32, data dependent); sample 1: small beta (bound 32)
     d = varying_inputs(2, 2, 40, 56, seed=11)
