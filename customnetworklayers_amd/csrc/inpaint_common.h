@@ -370,13 +370,15 @@ static __global__ __launch_bounds__(256) void finalize_f32(const float* __restri
   }
 }
 
-// Optional timing of a layer's dominant kernel with HIP events on the launch stream.
+// Optional timing of a layer's dominant kernel with HIP events on the launch stream.  An event
+// between two launches costs several microseconds of idle GPU, so a pair of events brackets a run
+// of consecutive launches of that kernel (one reverse sweep), not every launch.
 struct KernelTimer {
   bool enabled = false;
   std::vector<hipEvent_t> pool;  // start/stop pairs
+  std::vector<int> counts;       // launches inside each pair
   size_t used = 0;
-  void mark(hipStream_t stream) {
-    if (!enabled) return;
+  void record(hipStream_t stream) {
     if (used == pool.size()) {
       hipEvent_t e;
       if (hipEventCreate(&e) != hipSuccess) { enabled = false; return; }
@@ -384,6 +386,16 @@ struct KernelTimer {
     }
     (void)hipEventRecord(pool[used++], stream);
   }
+  void begin(hipStream_t stream) {
+    if (enabled) record(stream);
+  }
+  void end(hipStream_t stream, int launches) {
+    if (!enabled) return;
+    record(stream);
+    counts.resize(used / 2, 0);
+    if (used >= 2) counts[used / 2 - 1] = launches;
+  }
+  void reset() { used = 0; counts.clear(); }
   int read(double* total_ms, int* launches) {
     double total = 0;
     int count = 0;
@@ -392,9 +404,9 @@ struct KernelTimer {
       float ms = 0;
       INPAINT_HIP(hipEventElapsedTime(&ms, pool[i], pool[i + 1]));
       total += ms;
-      count++;
+      count += counts[i / 2];
     }
-    used = 0;
+    reset();
     if (total_ms) *total_ms = total;
     if (launches) *launches = count;
     return 0;

@@ -658,9 +658,14 @@ __global__ __launch_bounds__(256) void tgv_upstream_check(const float* __restric
   }
   bad = wave_sum_u(bad);
   nz = wave_sum_u(nz);
-  if ((threadIdx.x & 63) == 0) {
+  __shared__ unsigned int s_bad[4], s_nz[4];
+  if ((threadIdx.x & 63) == 0) { s_bad[threadIdx.x >> 6] = bad; s_nz[threadIdx.x >> 6] = nz; }
+  __syncthreads();
+  if (threadIdx.x == 0) {  // one pair of atomics per block, and only when there is something to report
+    bad = s_bad[0] + s_bad[1] + s_bad[2] + s_bad[3];
+    nz = s_nz[0] + s_nz[1] + s_nz[2] + s_nz[3];
     if (bad) atomicAdd(&counts[0], bad);
-    if (nz) atomicAdd(&counts[1], nz > 0 ? 1u : 0u);
+    if (nz && counts[1] == 0) atomicAdd(&counts[1], 1u);
   }
 }
 
@@ -977,7 +982,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     ZeroList z;
     z.ptr[0] = s.counts; z.bytes[0] = 8;
     hipLaunchKernelGGL(fill_zero_many, dim3(1, 1), dim3(256), 0, stream, z);
-    hipLaunchKernelGGL(tgv_upstream_check, dim3(gS), dim3(256), 0, stream, gin, (long long)S3, s.counts);
+    hipLaunchKernelGGL(tgv_upstream_check, dim3(std::min(gS, 1024)), dim3(256), 0, stream, gin, (long long)S3, s.counts);
     unsigned int host_counts[2] = {0, 0};
     INPAINT_HIP(hipMemcpyAsync(host_counts, s.counts, 8, hipMemcpyDeviceToHost, stream));
     INPAINT_HIP(hipStreamSynchronize(stream));
@@ -1032,6 +1037,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       launch_forward(s, stream, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * S3,
                      s.steps[k0 + j]);
     }
+    int timed_run = 0;
     for (int j = len - 1; j >= 0; j--) {  // reverse sweep (TGV.cu:2851-2933)
       const float t = s.steps[k0 + j];
       const float* xa = s.x05 + (size_t)j * S3;
@@ -1041,10 +1047,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
                            s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = s.x05 + (size_t)(j - 1) * S3;
-        g_timer.mark(stream);
+        if (timed_run == 0) g_timer.begin(stream);
         launch_adjoint<false>(s, stream, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
                               s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
-        g_timer.mark(stream);
+        timed_run++;
+        if (j == 1) g_timer.end(stream, timed_run);  // one event pair around the sweep's run of launches
       } else {
         // the very last step's g_x is the gradient wrt the starting point (TGV.cu:3047)
         launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
@@ -1164,7 +1171,7 @@ int tgvinpaint_guard_decide(int run, double av_gc, double av_running, double* mu
 
 int tgvinpaint_profile(int enable) {
   g_timer.enabled = enable != 0;
-  g_timer.used = 0;
+  g_timer.reset();
   return 0;
 }
 
