@@ -522,6 +522,41 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, co
                        yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
 }
 
+// Two forward iterations in one launch (strip path only): (xin, yin) = iterate k, (xout, yout) = iterate k+2;
+// x05a / x05b receive the pre-prox values of iterations k and k+1 when given.
+template <int C>
+void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                               const float* b, const float* xin, float* xout, const float* yin, float* yout,
+                               float* x05a, float* x05b, float tA, float tB) {
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_FWD_ROWS");
+  const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
+  if (x05a)
+    hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
+                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+  else
+    hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, false>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
+                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+}
+
+bool forward_pairs(const Slot& s) {
+  const char* e = getenv("INPAINT_TV_FUSE");
+  if (e && strcmp(e, "0") == 0) return false;
+  return !force_tile_path() && s.ic >= 1 && s.ic <= 4;
+}
+
+void launch_forward_pair(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                         const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05a,
+                         float* x05b, float tA, float tB) {
+  switch (s.ic) {
+    case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
+    case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
+    case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
+    default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
+  }
+}
+
 void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
                     float t) {
@@ -623,8 +658,21 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   } else {
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, FB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, FB, hipMemcpyDeviceToDevice, stream));
-    for (int k = 0; k < K; k++) {
-      launch_forward(s, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
+    if (forward_pairs(s)) {
+      // two iterations per launch; K is even and so is every checkpoint index.  The intermediate
+      // iterate k+1 stays in registers, so the ping-pong alternates per pair.
+      auto Yp = [&](int k) { int i = ck_index(k); return (i >= 0 && k < K) ? s.ckpt_y + (size_t)i * F : s.ypp[(k >> 1) & 1]; };
+      auto Xp = [&](int k) {
+        if (k == K) return out;
+        int i = ck_index(k);
+        return i >= 0 ? s.ckpt_x + (size_t)i * F : s.xpp[(k >> 1) & 1];
+      };
+      for (int k = 0; k < K; k += 2)
+        launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), nullptr, nullptr, s.steps[k],
+                            s.steps[k + 1]);
+    } else {
+      for (int k = 0; k < K; k++)
+        launch_forward(s, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
     }
   }
   INPAINT_HIP(hipGetLastError());
@@ -671,11 +719,20 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     const float* cky = s.ckpt_y + (size_t)outer * F;
     const float* ckx = s.ckpt_x + (size_t)outer * F;
     // recompute the segment, keeping x05 (TV.cu:1678-1687)
-    for (int j = 0; j < len; j++) {
-      const float* yin = (j == 0) ? cky : s.ypp[j & 1];
-      const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
-      launch_forward(s, stream, dx, dy, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * F,
-                     s.steps[k0 + j]);
+    if (forward_pairs(s)) {
+      for (int j = 0; j < len; j += 2) {  // segments have even length
+        const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
+        const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];
+        launch_forward_pair(s, stream, dx, dy, c, b, xin, s.xpp[((j >> 1) + 1) & 1], yin, s.ypp[((j >> 1) + 1) & 1],
+                            s.x05 + (size_t)j * F, s.x05 + (size_t)(j + 1) * F, s.steps[k0 + j], s.steps[k0 + j + 1]);
+      }
+    } else {
+      for (int j = 0; j < len; j++) {
+        const float* yin = (j == 0) ? cky : s.ypp[j & 1];
+        const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
+        launch_forward(s, stream, dx, dy, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1],
+                       s.x05 + (size_t)j * F, s.steps[k0 + j]);
+      }
     }
     // reverse sweep (TV.cu:1696-1729)
     int timed_run = 0;

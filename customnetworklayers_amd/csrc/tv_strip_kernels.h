@@ -33,6 +33,7 @@ using inpaint::rcp_refined;
 
 constexpr int kFwdCols = 63;      // output columns per wavefront, forward (lane 0 is the apron)
 constexpr int kAdjCols = 62;      // adjoint (lanes 0 and 63 are aprons)
+constexpr int kFwd2Cols = 60;     // two fused forward iterations (lanes 0, 1, 62, 63 are aprons)
 constexpr float kDelta = 0.1f;    // TV.cu:44
 constexpr float kL = 0.125f;      // TV.cu:1478
 constexpr float kClipLocalGrad = 10000.0f;  // TV.cu:52
@@ -66,7 +67,7 @@ struct StripGeom {
 // branch makes the compiler assume the path without it and drain the prefetched rows at every step.
 
 __device__ __forceinline__ bool strip_geometry(StripGeom& g, int cols, int R, int W, int strips_x, int strips_y,
-                                               int N) {
+                                               int N, int left_apron = 1) {
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Neighbouring strips share
   // halo rows, the apron column and split cache lines, so strips are numbered such that every XCD
   // works through one contiguous band of the image: workgroup b serves logical block
@@ -80,7 +81,7 @@ __device__ __forceinline__ bool strip_geometry(StripGeom& g, int cols, int R, in
   const int sy = rest % strips_y;
   g.n = rest / strips_y;
   if (g.n >= N) return false;
-  g.w = sx * cols - 1 + g.lane;
+  g.w = sx * cols - left_apron + g.lane;
   g.hs = sy * R;
   g.col_ok = g.w >= 0 && g.w < W;
   return true;
@@ -235,6 +236,197 @@ __global__ __launch_bounds__(256) void tv_forward_strip(
     absorb(r + 4, b1);
     compute(r + 3, b0, b1, kRow);
     load_row(r + 7, b0);
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Two forward iterations per launch (A = iteration k, B = iteration k+1), same arithmetic as
+// tv_forward_strip applied twice.  B runs one row behind A inside the same wavefront: once A has
+// updated row r+1, B owns everything its triangle of row r needs (A's new y of rows r and r+1, in
+// registers) and, with the term handed down from row r-1, the update of row r.  A's new iterate
+// never touches memory, so a pair moves the bytes of one iteration (plus the two x05 rows when the
+// backward pass recomputes a segment).
+//
+// Lanes cover columns w0-2 .. w0+61.  A's update is valid on lanes 1..62 (it needs the left lane's
+// triangle term and the right lane's y), B's on lanes 2..61, which are the 60 output columns.  Rows:
+// the strip's R output rows need A on R+2 rows and the input y on R+4 rows.  Where A's result lies
+// outside the image B must see the zero padding, so it is masked.
+// -------------------------------------------------------------------------------------------------
+template <int C>
+struct Fwd2Row {
+  float y[C], x[C], bb[C], c, wxs, wys;
+};
+
+template <int C, bool X05>
+__global__ __launch_bounds__(256) void tv_forward_strip2(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
+    const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
+    const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
+    int N, int H, int W, float tA, float tB, int R, int strips_x, int strips_y) {
+  StripGeom g;
+  if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
+  const size_t HW = (size_t)H * W;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
+  const bool wx_ok = g.col_ok && g.w < W - 1;
+  const int Reff = min(R, H - g.hs);
+  const int klast = Reff + 2;  // last step; strip row k is image row hs - 2 + k
+  const float* const wx_p = wx + (size_t)g.n * HW;
+  const float* const wy_p = wy + (size_t)g.n * HW;
+  const float* const cf_p = cf + (size_t)g.n * HW;
+  const float *y_p[C], *x_p[C], *b_p[C];
+  float *yo_p[C], *xo_p[C], *xa_p[C], *xb_p[C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) {
+    const size_t q = ((size_t)g.n * C + ch) * HW;
+    y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
+    yo_p[ch] = yout + q; xo_p[ch] = xout + q;
+    xa_p[ch] = X05 ? x05a + q : nullptr; xb_p[ch] = X05 ? x05b + q : nullptr;
+  }
+  const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
+
+  auto load_row = [&](int k, Fwd2Row<C>& in) {
+    const int kk = min(k, klast + 1);
+    const int h = g.hs - 2 + kk;
+    const unsigned row = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4;
+    // the outermost rows contribute y (and the upper one its weights) only: their other fields are
+    // read from a row the strip needs anyway, so that no cache line is fetched for nothing
+    const unsigned row_w = (unsigned)min(max(h, 0), h_hi) * W4;
+    const unsigned row_p = (unsigned)min(max(h, h_lo), h_hi) * W4;
+    in.c = ldg(cf_p, row_p + wc);
+    in.wxs = ldg(wx_p, row_w + wc);
+    in.wys = ldg(wy_p, row_w + wc);
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      in.y[ch] = ldg(y_p[ch], row + wc);
+      in.x[ch] = ldg(x_p[ch], row_p + wc);
+      in.bb[ch] = ldg(b_p[ch], row_p + wc);
+    }
+  };
+  auto absorb = [&](int k, Fwd2Row<C>& o) {
+    const int h = g.hs - 2 + k;
+    const bool rok = h >= 0 && h < H;
+    o.wxs = (rok && wx_ok) ? kL * o.wxs : 0.f;
+    o.wys = (rok && g.col_ok && h < H - 1) ? kL * o.wys : 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) o.y[ch] = (rok && g.col_ok) ? o.y[ch] : 0.f;
+  };
+
+  // one triangle (owner value yc, lower neighbour yd): the two products of TV.cu:1268-1274
+  auto triangle = [&](float yc, float yd, float wxs, float wys, float& e1, float& e2) {
+    const float d1 = yc - yd;
+    const float d2 = yc - from_right_lane(yc);
+    const float hub = exact_sqrt(d1 * d1 * wys + d2 * d2 * wxs);
+    const float m = fmaxf(1.f, inpaint::exact_div(hub, kDelta));
+    const float rm = rcp_refined(m);
+    e1 = d1 * div_by(wys, m, rm);
+    e2 = d2 * div_by(wxs, m, rm);
+  };
+  // gradient step + Huber-1 prox + extrapolation of one pixel (TV.cu:1258-1316)
+  auto update = [&](float yc, float e1_above, float e2_left, float e1, float e2, float c, float rc1, float bv,
+                    float xold, float t, float& xh, float& x_loc, float& yn) {
+    float yt = yc;
+    yt -= -e1_above;
+    yt -= -e2_left;
+    yt -= e1;
+    yt -= e2;
+    xh = yt;
+    x_loc = div_by(c * bv + yt, 1.f + c, rc1);
+    const float lo = yt - c, hi = yt + c;
+    if (lo > 1.f + bv) x_loc = lo;
+    if (hi < bv - 1.f) x_loc = hi;
+    yn = x_loc + t * (x_loc - xold);
+  };
+
+  float upA[C], upB[C];        // triangle terms handed down to the next row, per iteration
+  float pyB[C], pxB[C], pbb[C], pc = 0.f, pwxs = 0.f, pwys = 0.f;  // row k-1 as iteration B sees it
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) upA[ch] = upB[ch] = pyB[ch] = pxB[ch] = pbb[ch] = 0.f;
+
+  // step k: A's triangle of row k (+ A's update of row k when DO_A), then B's triangle of row k-1
+  // (when TRI_B) and B's update of row k-1 (when DO_B)
+  auto step = [&](int k, const Fwd2Row<C>& cur, const Fwd2Row<C>& nxt, auto do_a, auto tri_b, auto do_b) {
+    const int h = g.hs - 2 + k;
+    const bool in_img = g.col_ok && h >= 0 && h < H;
+    const unsigned roffA = (unsigned)min(max(h, 0), H - 1) * W4 + wc;
+    const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+    const bool storeA = store_lane && k >= 2 && k <= Reff + 1;  // A's pre-prox value, output rows only
+    const float rc1A = rcp_refined(1.f + cur.c);
+    const float rc1B = rcp_refined(1.f + pc);
+    float nyB[C], nxB[C];
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      float e1, e2;
+      triangle(cur.y[ch], nxt.y[ch], cur.wxs, cur.wys, e1, e2);
+      const float e1_above = upA[ch];
+      upA[ch] = e1;
+      nyB[ch] = 0.f;
+      nxB[ch] = 0.f;
+      if (do_a.value) {
+        float xh, x_loc, yn;
+        update(cur.y[ch], e1_above, from_left_lane(e2), e1, e2, cur.c, rc1A, cur.bb[ch], cur.x[ch], tA, xh, x_loc, yn);
+        nyB[ch] = in_img ? yn : 0.f;  // B reads zero padding outside the image (TV.cu:1229,1237)
+        nxB[ch] = x_loc;
+        if (X05 && storeA) stg(xa_p[ch], roffA, xh);
+      }
+    }
+    if (tri_b.value) {
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        float e1, e2;
+        triangle(pyB[ch], nyB[ch], pwxs, pwys, e1, e2);
+        const float e1_above = upB[ch];
+        upB[ch] = e1;
+        if (do_b.value) {
+          float xh, x_loc, yn;
+          update(pyB[ch], e1_above, from_left_lane(e2), e1, e2, pc, rc1B, pbb[ch], pxB[ch], tB, xh, x_loc, yn);
+          if (store_lane) {
+            stg(yo_p[ch], roffB, yn);
+            stg(xo_p[ch], roffB, x_loc);
+            if (X05) stg(xb_p[ch], roffB, xh);
+          }
+        }
+      }
+    }
+    pc = cur.c; pwxs = cur.wxs; pwys = cur.wys;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) { pyB[ch] = nyB[ch]; pxB[ch] = nxB[ch]; pbb[ch] = cur.bb[ch]; }
+  };
+  const std::true_type kYes{};
+  const std::false_type kNo{};
+
+  Fwd2Row<C> b0, b1, b2, b3;
+  load_row(0, b0);
+  load_row(1, b1);
+  load_row(2, b2);
+  load_row(3, b3);
+  absorb(0, b0);
+  absorb(1, b1);
+  step(0, b0, b1, kNo, kNo, kNo);
+  load_row(4, b0);
+  absorb(2, b2);
+  step(1, b1, b2, kYes, kNo, kNo);
+  load_row(5, b1);
+  absorb(3, b3);
+  step(2, b2, b3, kYes, kYes, kNo);
+  load_row(6, b2);
+  for (int k = 3; k <= klast; k += 4) {  // cur / next rotate through (b3,b0) (b0,b1) (b1,b2) (b2,b3)
+    absorb(k + 1, b0);
+    step(k, b3, b0, kYes, kYes, kYes);
+    load_row(k + 4, b3);
+    if (k + 1 > klast) break;
+    absorb(k + 2, b1);
+    step(k + 1, b0, b1, kYes, kYes, kYes);
+    load_row(k + 5, b0);
+    if (k + 2 > klast) break;
+    absorb(k + 3, b2);
+    step(k + 2, b1, b2, kYes, kYes, kYes);
+    load_row(k + 6, b1);
+    if (k + 3 > klast) break;
+    absorb(k + 4, b3);
+    step(k + 3, b2, b3, kYes, kYes, kYes);
+    load_row(k + 7, b2);
   }
 }
 

@@ -95,6 +95,28 @@ def test_tile_kernels_when_forced_or_needed(ext, tv_oracle, n, c, h, w, its, mon
     compare("tile path c=%d" % c, run_gpu(ext, d, its, 2), ref)
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 45, 130, 10)])
+def test_single_iteration_strip_kernels(ext, tv_oracle, n, c, h, w, its, monkeypatch):
+    # the forward and the recompute normally run two iterations per launch; INPAINT_TV_FUSE=0 keeps
+    # the one-iteration strip kernels covered
+    d = tv_inputs(n, c, h, w, seed=91 + c, conf_density=0.3)
+    ref = run_oracle(tv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TV_FUSE", "0")
+    compare("one iteration per launch c=%d" % c, run_gpu(ext, d, its, 2), ref)
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 1, 9, 60, 8),       # exactly one fused strip wide (60 output columns)
+    (1, 2, 11, 61, 8),      # one column more
+    (1, 2, 3, 200, 6),      # fewer rows than the fused kernel's row lag
+    (1, 2, 2, 59, 4),
+    (2, 4, 18, 121, 12),    # four channels, two fused strips and a column
+])
+def test_fused_forward_strip_edges(ext, tv_oracle, n, c, h, w, its):
+    d = tv_inputs(n, c, h, w, seed=n * 100 + h + w, conf_density=0.3)
+    compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2))
+
+
 def test_its_zero_and_one_return_init_and_zero_grads(ext, tv_oracle):
     d = tv_inputs(1, 2, 20, 30, seed=5)
     for its in (0, 1):
