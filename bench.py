@@ -19,7 +19,7 @@ HBM_PEAK_GBS = 8000.0
 # script on the headline workload (2 x 72471 KiB fetched, after the copy-kernel calibration, plus
 # 69740 KiB written; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
 # profiles/tgv_strip_config2_hbm_traffic.txt).  Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: (2 * 72471 + 69740) * 1024, 2: (2 * 142300 + 153730) * 1024}
+MEASURED_TRAFFIC_BYTES = {2: (2 * 142300 + 153730) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):
@@ -40,7 +40,7 @@ def layer_of(kind):
         from customnetworklayers_amd.cudaTGV import tgvInpaint_cuda_ext as ext
         return ext, "tgvinpaint", workloads.tgv_inputs, "TGVOracle", "tgvstrip::tgv_adjoint_strip<2,false,false>"
     from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
-    return ext, "tvinpaint", workloads.tv_inputs, "TVOracle", "tvstrip::tv_adjoint_strip<2,false,false>"
+    return ext, "tvinpaint", workloads.tv_inputs, "TVOracle", "tvstrip::tv_adjoint_strip2<2,false,false>"
 
 
 def cpu_baseline(cfg, seconds_hint=20.0):
@@ -127,7 +127,10 @@ def main():
     value = pxit / (elapsed / args.steps) / 1e6
     bpp = algorithmic_bytes_per_pixel(c, cfg["kind"])
     kernel_ms = tot_ms.value / max(launches.value, 1)
-    kernel_bytes = bpp["adjoint"] * n * h * w
+    # the TV layer's dominant kernel runs two adjoint steps per launch
+    steps_per_launch = 2 if (cfg["kind"] == "tv" and os.environ.get("INPAINT_TV_FUSE", "1") != "0"
+                             and os.environ.get("INPAINT_TV_FUSE_ADJ", "1") != "0") else 1
+    kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9
     out = {
@@ -142,7 +145,7 @@ def main():
                       "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config), "bytes_per_launch": kernel_bytes,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config), "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
                      "avg_launch_ms": round(kernel_ms, 5), "launches_timed": launches.value},
     }
     if not args.no_cpu_baseline:

@@ -620,6 +620,48 @@ bool launch_adjoint(Slot& s, hipStream_t stream, const float* dx, const float* d
   return strip;
 }
 
+// Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
+// (third y source xc = slot j-2, or the checkpoint y when B is the segment's first iteration).
+template <int C, bool BEND>
+void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                               const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
+                               float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_ADJ_ROWS");
+  const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
+  if (gx_final)
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
+                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n,
+                       s.ih, s.iw, tA, tB, R, sx, sy);
+  else
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
+                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n,
+                       s.ih, s.iw, tA, tB, R, sx, sy);
+}
+
+template <bool BEND>
+void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c, const float* b,
+                         const float* xa, const float* xb, const float* xc, const float* g05_in, float* g05_out,
+                         const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
+  switch (s.ic) {
+    case 1: launch_adjoint_pair_strip<1, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
+    case 2: launch_adjoint_pair_strip<2, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
+    case 3: launch_adjoint_pair_strip<3, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
+    default: launch_adjoint_pair_strip<4, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
+  }
+  s.acc_cur = 1 - s.acc_cur;
+}
+
+bool adjoint_pairs(const Slot& s) {
+  const char* e = getenv("INPAINT_TV_FUSE_ADJ");
+  if (e && strcmp(e, "0") == 0) return false;
+  return forward_pairs(s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -711,6 +753,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   // partial g_x[k] to the other; the completed g_x[k+1] itself is only ever read after the very last
   // step (TV.cu:800 calls its store a debugging aid), so only that step stores it, into gx_final.
   int lastIt = its;
+  int pp_src = 1;  // g05 / g_x buffer the next adjoint launch reads (pair path)
   const int nseg = (int)s.iterations.size();
   for (int outer = nseg - 1; outer >= 0; outer--) {
     const int k0 = s.iterations[outer];
@@ -736,6 +779,50 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     }
     // reverse sweep (TV.cu:1696-1729)
     int timed_run = 0;
+    if (adjoint_pairs(s)) {
+      // The g05 / g_x ping-pong flips once per launch: `src` holds what the next launch reads.  The
+      // first step of the whole backward writes g05[1]; a segment's last launch leaves its result
+      // where the next segment picks it up.
+      int j = len - 1;
+      if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
+        hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+                           s.x05 + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                           (long long)ih * iw, (long long)P);
+        pp_src = 1;
+        j--;
+      }
+      if (j >= 0 && ((j + 1) & 1)) {  // an odd number of steps is left: one single step, then pairs
+        const float* xa = s.x05 + (size_t)j * F;
+        if (j > 0)
+          launch_adjoint<false>(s, stream, dx, dy, c, b, xa, s.x05 + (size_t)(j - 1) * F, nullptr, s.g05[pp_src],
+                                s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j]);
+        else
+          flushed = launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[pp_src], s.g05[1 - pp_src],
+                                         s.gxk[pp_src], s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr,
+                                         s.steps[k0 + j]);
+        pp_src = 1 - pp_src;
+        j--;
+      }
+      for (; j >= 1; j -= 2) {
+        const float* xa = s.x05 + (size_t)j * F;
+        const float* xb = s.x05 + (size_t)(j - 1) * F;
+        if (j - 1 > 0) {
+          if (timed_run == 0) g_timer.begin(stream);
+          launch_adjoint_pair<false>(s, stream, dx, dy, c, b, xa, xb, s.x05 + (size_t)(j - 2) * F, s.g05[pp_src],
+                                     s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j],
+                                     s.steps[k0 + j - 1]);
+          timed_run++;
+          if (j - 2 <= 1) g_timer.end(stream, timed_run);  // one event pair around the sweep's run of launches
+        } else {
+          // B is the segment's first iteration; the very last one's g_x is the gradient wrt the start
+          launch_adjoint_pair<true>(s, stream, dx, dy, c, b, xa, xb, cky, s.g05[pp_src], s.g05[1 - pp_src],
+                                    s.gxk[pp_src], s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr,
+                                    s.steps[k0 + j], s.steps[k0 + j - 1]);
+          flushed = true;
+        }
+        pp_src = 1 - pp_src;
+      }
+    } else
     for (int j = len - 1; j >= 0; j--) {
       const float t = s.steps[k0 + j];
       const float* xa = s.x05 + (size_t)j * F;

@@ -105,6 +105,24 @@ def test_single_iteration_strip_kernels(ext, tv_oracle, n, c, h, w, its, monkeyp
     compare("one iteration per launch c=%d" % c, run_gpu(ext, d, its, 2), ref)
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 45, 130, 11)])
+def test_single_step_adjoint_strip_kernels(ext, tv_oracle, n, c, h, w, its, monkeypatch):
+    # the reverse sweep normally runs two adjoint steps per launch; INPAINT_TV_FUSE_ADJ=0 keeps the
+    # one-step strip kernels covered (forward and recompute stay fused)
+    d = tv_inputs(n, c, h, w, seed=93 + c, conf_density=0.3)
+    ref = run_oracle(tv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TV_FUSE_ADJ", "0")
+    compare("one adjoint step per launch c=%d" % c, run_gpu(ext, d, its, 2), ref)
+
+
+@pytest.mark.parametrize("its", [2, 3, 4, 5, 6, 8, 16, 17, 26])
+def test_every_pairing_of_the_reverse_sweep(ext, tv_oracle, its):
+    # its decides how the sweep splits into the first step, an optional single step and pairs:
+    # one segment of 2 (first step + single segment-start step), segments of even and odd remainder
+    d = tv_inputs(1, 2, 23, 75, seed=300 + its, conf_density=0.4)
+    compare("its=%d" % its, run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2))
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [
     (1, 1, 9, 60, 8),       # exactly one fused strip wide (60 output columns)
     (1, 2, 11, 61, 8),      # one column more
