@@ -99,6 +99,8 @@ def main():
     cfg, d = config_inputs(args.config, seed=0)
     assert cfg["kind"] in ("tv", "tgv")
     ext, prefix, _, _, kernel_name = layer_of(cfg["kind"])
+    if cfg["kind"] == "tv" and (os.environ.get("INPAINT_TV_FUSE", "1") == "0" or os.environ.get("INPAINT_TV_FUSE_ADJ", "1") == "0"):
+        kernel_name = "tvstrip::tv_adjoint_strip<2,false,false>"
     profile, profile_read = getattr(lib, prefix + "_profile"), getattr(lib, prefix + "_profile_read")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     its, pid = cfg["its"], 0

@@ -869,6 +869,35 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* c, const flo
                      s.ic, s.ih, s.iw, t);
 }
 
+// Two forward iterations in one launch (strip path): (xin, yin) = iterate k, (xout, yout) = iterate k+2;
+// x05a / x05b receive the x05 rows of iterations k and k+1 when given.
+template <int C>
+void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
+                               float* xout, const float* yin, float* yout, float* x05a, float* x05b, float tA, float tB) {
+  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_FWD_ROWS");
+  const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
+  if (x05a)
+    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
+                       xout, yin, yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+  else
+    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
+                       xout, yin, yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+}
+
+bool forward_pairs(const Slot& s) {
+  const char* e = getenv("INPAINT_TGV_FUSE");
+  if (e && strcmp(e, "0") == 0) return false;
+  return use_strip(s);
+}
+
+void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
+                         const float* yin, float* yout, float* x05a, float* x05b, float tA, float tB) {
+  if (s.ic == 1) launch_forward_pair_strip<1>(s, stream, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB);
+  else launch_forward_pair_strip<2>(s, stream, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB);
+}
+
 template <int C, bool END>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
                           const float* xb, const float* yck, const float* g05_in, float* g05_out, const float* gxk,
@@ -952,8 +981,21 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
     scale_weights(s, stream, dx, dy);
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, SB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, SB, hipMemcpyDeviceToDevice, stream));
-    for (int k = 0; k < K; k++)
-      launch_forward(s, stream, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
+    if (forward_pairs(s)) {
+      // two iterations per launch; K and every checkpoint index are even, the ping-pong alternates per pair
+      auto Yp = [&](int k) { int i = ck_index(k); return (i >= 0 && k < K) ? s.ckpt_y + (size_t)i * S3 : s.ypp[(k >> 1) & 1]; };
+      auto Xp = [&](int k) {
+        if (k == K) return out;
+        int i = ck_index(k);
+        return i >= 0 ? s.ckpt_x + (size_t)i * S3 : s.xpp[(k >> 1) & 1];
+      };
+      for (int k = 0; k < K; k += 2)
+        launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), nullptr, nullptr, s.steps[k],
+                            s.steps[k + 1]);
+    } else {
+      for (int k = 0; k < K; k++)
+        launch_forward(s, stream, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
+    }
   }
   INPAINT_HIP(hipGetLastError());
   s.forward_done = true;
@@ -1031,11 +1073,21 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     const int len = 2 * ((lastIt - k0) / 2);
     const float* cky = s.ckpt_y + (size_t)outer * S3;
     const float* ckx = s.ckpt_x + (size_t)outer * S3;
-    for (int j = 0; j < len; j++) {  // recompute the segment, keeping x05 (TGV.cu:2775-2814)
-      const float* yin = (j == 0) ? cky : s.ypp[j & 1];
-      const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
-      launch_forward(s, stream, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * S3,
-                     s.steps[k0 + j]);
+    // recompute the segment, keeping x05 (TGV.cu:2775-2814)
+    if (forward_pairs(s)) {
+      for (int j = 0; j < len; j += 2) {  // segments have even length
+        const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
+        const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];
+        launch_forward_pair(s, stream, c, b, xin, s.xpp[((j >> 1) + 1) & 1], yin, s.ypp[((j >> 1) + 1) & 1],
+                            s.x05 + (size_t)j * S3, s.x05 + (size_t)(j + 1) * S3, s.steps[k0 + j], s.steps[k0 + j + 1]);
+      }
+    } else {
+      for (int j = 0; j < len; j++) {
+        const float* yin = (j == 0) ? cky : s.ypp[j & 1];
+        const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
+        launch_forward(s, stream, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * S3,
+                       s.steps[k0 + j]);
+      }
     }
     int timed_run = 0;
     for (int j = len - 1; j >= 0; j--) {  // reverse sweep (TGV.cu:2851-2933)

@@ -35,6 +35,7 @@ using tvstrip::strip_geometry;
 using tvstrip::StripGeom;
 
 constexpr int kCols = 62;  // output columns per wavefront (lanes 0 and 63 are aprons)
+constexpr int kCols2 = 60;  // two fused forward iterations (lanes 0, 1, 62, 63 are aprons)
 constexpr float kD0 = 0.2f, kD1 = 0.2f, kD2 = 0.2f;  // TGV.cu:58-60
 constexpr float kClipLocalGrad = 2000.0f;            // TGV.cu:78
 constexpr float kLocalGCMult = 0.1f;                 // TGV.cu:87
@@ -229,6 +230,257 @@ __global__ __launch_bounds__(256) void tgv_forward_strip(
     absorb(r + 4, b1);
     compute(r + 3, b0, b1, kRow);
     load_row(r + 7, b0);
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Two forward iterations per launch (A = iteration k, B = k+1), the arithmetic of tgv_forward_strip
+// applied twice.  B runs one row behind A in the same wavefront and takes A's new y and x from
+// registers (the scheme of tvstrip::tv_forward_strip2).  Lanes cover columns w0-2 .. w0+61; A's
+// update is valid on lanes 1..62, B's on lanes 2..61, the 60 output columns.  A's result outside
+// the image is masked to the zero padding B must see.
+// -------------------------------------------------------------------------------------------------
+template <int C>
+struct Fwd2Row {
+  float y[3][C], x[3][C], bb[C], c, wxs, wys, bxs, bys;
+};
+
+template <int C, bool X05>
+__global__ __launch_bounds__(256) void tgv_forward_strip2(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
+    const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
+    const float* __restrict__ xin, float* __restrict__ xout, const float* __restrict__ yin,
+    float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b, int N, int H, int W, float tA,
+    float tB, int R, int strips_x, int strips_y) {
+  StripGeom g;
+  if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
+  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
+  const bool rmask = g.col_ok && g.w < W - 1;
+  const int Reff = min(R, H - g.hs);
+  const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
+  const size_t poff = (size_t)g.n * HW;
+  const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
+                     *const cf_p = cf + poff;
+  const float *y_p[3][C], *x_p[3][C], *b_p[C];
+  float *yo_p[3][C], *xo_p[3][C], *xa_p[3][C], *xb_p[3][C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) {
+    b_p[ch] = b + ((size_t)g.n * C + ch) * HW;
+#pragma unroll
+    for (int v = 0; v < 3; v++) {
+      const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
+      y_p[v][ch] = yin + q; x_p[v][ch] = xin + q;
+      yo_p[v][ch] = yout + q; xo_p[v][ch] = xout + q;
+      xa_p[v][ch] = X05 ? x05a + q : nullptr; xb_p[v][ch] = X05 ? x05b + q : nullptr;
+    }
+  }
+  const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
+
+  auto load_row = [&](int k, Fwd2Row<C>& in) {
+    const int kk = min(k, klast + 1);
+    const int h = g.hs - 2 + kk;
+    const unsigned row = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4;
+    const unsigned row_w = (unsigned)min(max(h, 0), h_hi) * W4;
+    const unsigned row_p = (unsigned)min(max(h, h_lo), h_hi) * W4;
+    in.c = ldg(cf_p, row_p + wc);
+    in.wxs = ldg(wx_p, row_w + wc);
+    in.wys = ldg(wy_p, row_w + wc);
+    in.bxs = ldg(bx_p, row_w + wc);
+    in.bys = ldg(by_p, row_w + wc);
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      in.bb[ch] = ldg(b_p[ch], row_p + wc);
+#pragma unroll
+      for (int v = 0; v < 3; v++) {
+        in.y[v][ch] = ldg(y_p[v][ch], row + wc);
+        in.x[v][ch] = ldg(x_p[v][ch], row_p + wc);
+      }
+    }
+  };
+  auto absorb = [&](int k, Fwd2Row<C>& o) {
+    const int h = g.hs - 2 + k;
+    const bool ok = g.col_ok && h >= 0 && h < H;
+    o.wxs = (ok && rmask) ? o.wxs : 0.f;
+    o.wys = (ok && h < H - 1) ? o.wys : 0.f;
+    o.bxs = ok ? o.bxs : 0.f;
+    o.bys = ok ? o.bys : 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++)
+#pragma unroll
+      for (int v = 0; v < 3; v++) o.y[v][ch] = ok ? o.y[v][ch] : 0.f;
+  };
+
+  struct Tri {  // the six products of one triangle (TGV.cu:1669-1684)
+    float Fa, Fb, G1y, G1x, G2y, G2x;
+  };
+  auto triangle = [&](float yc, float y1c, float y2c, float yd, float y1d, float y2d, float wxs, float wys, float bxs,
+                      float bys, bool dmask) {
+    Tri r;
+    const float yr = from_right_lane(yc), y1r = from_right_lane(y1c), y2r = from_right_lane(y2c);
+    const float zij_1 = rmask ? ((yc - yr) + y1c) : 0.f;
+    const float zij_2 = dmask ? ((yc - yd) + y2c) : 0.f;
+    const float hwx = huber_w(zij_2 * zij_2 * wys + zij_1 * zij_1 * wxs, kD0);
+    const float u11 = rmask ? (y1c - y1r) : 0.f;
+    const float u12 = dmask ? (y1c - y1d) : 0.f;
+    const float hwy1 = huber_w(bxs * (u12 * u12 + u11 * u11), kD1);
+    const float u21 = rmask ? (y2c - y2r) : 0.f;
+    const float u22 = dmask ? (y2c - y2d) : 0.f;
+    const float hwy2 = huber_w(bys * (u22 * u22 + u21 * u21), kD2);
+    r.Fa = wys * (zij_2 * hwx);
+    r.Fb = wxs * (zij_1 * hwx);
+    r.G1y = bxs * (u12 * hwy1);
+    r.G1x = bxs * (u11 * hwy1);
+    r.G2y = bys * (u22 * hwy2);
+    r.G2x = bys * (u21 * hwy2);
+    return r;
+  };
+  // gradient step on (u, v1, v2), prox on u, extrapolation (TGV.cu:1637-1690, 1740-1773)
+  struct Upd {
+    float xh, y1n, y2n, x_loc, yn, y1o, y2o;
+  };
+  auto update = [&](float yc, float y1c, float y2c, const Tri& t, float aFa, float aG1y, float aG2y, float c, float rc1,
+                    float bv, float x0, float x1, float x2, float tm) {
+    Upd u;
+    const float lFb = from_left_lane(t.Fb), lG1x = from_left_lane(t.G1x), lG2x = from_left_lane(t.G2x);
+    float yt = yc, y1n = y1c, y2n = y2c;
+    yt -= -aFa;
+    y1n -= -aG1y;
+    y2n -= -aG2y;
+    yt -= -lFb;
+    y1n -= -lG1x;
+    y2n -= -lG2x;
+    yt -= t.Fa;
+    y1n -= t.G1y;
+    y2n -= t.G2y + t.Fa;
+    yt -= t.Fb;
+    y1n -= t.G1x + t.Fb;
+    y2n -= t.G2x;
+    u.y1o = y1n + tm * (y1n - x1);
+    u.y2o = y2n + tm * (y2n - x2);
+    u.xh = yt;
+    u.y1n = y1n;
+    u.y2n = y2n;
+    float x_loc = div_by(c * bv + yt, 1.f + c, rc1);
+    const float lo = yt - c, hi = yt + c;
+    if (lo > 1.f + bv) x_loc = lo;
+    if (hi < bv - 1.f) x_loc = hi;
+    u.x_loc = x_loc;
+    u.yn = x_loc + tm * (x_loc - x0);
+    return u;
+  };
+
+  float upA[3][C], upB[3][C];  // terms handed down to the next row (Fa, G1y, G2y), per iteration
+  float pyB[3][C], pxB[3][C], pbb[C], pc = 0.f, pwxs = 0.f, pwys = 0.f, pbxs = 0.f, pbys = 0.f;
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) {
+    pbb[ch] = 0.f;
+#pragma unroll
+    for (int v = 0; v < 3; v++) upA[v][ch] = upB[v][ch] = pyB[v][ch] = pxB[v][ch] = 0.f;
+  }
+
+  auto step = [&](int k, const Fwd2Row<C>& cur, const Fwd2Row<C>& nxt, auto do_a, auto tri_b, auto do_b) {
+    const int h = g.hs - 2 + k;  // A's row; B's row is h - 1
+    const bool in_img = g.col_ok && h >= 0 && h < H;
+    const bool dmaskA = h >= 0 && h < H - 1, dmaskB = h - 1 >= 0 && h - 1 < H - 1;
+    const unsigned roffA = (unsigned)min(max(h, 0), H - 1) * W4 + wc;
+    const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+    const bool storeA = store_lane && k >= 2 && k <= Reff + 1;
+    const float rc1A = rcp_refined(1.f + cur.c);
+    const float rc1B = rcp_refined(1.f + pc);
+    float nyB[3][C], nxB[3][C];
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const Tri t = triangle(cur.y[0][ch], cur.y[1][ch], cur.y[2][ch], nxt.y[0][ch], nxt.y[1][ch], nxt.y[2][ch], cur.wxs,
+                             cur.wys, cur.bxs, cur.bys, dmaskA);
+      const float aFa = upA[0][ch], aG1y = upA[1][ch], aG2y = upA[2][ch];
+      upA[0][ch] = t.Fa; upA[1][ch] = t.G1y; upA[2][ch] = t.G2y;
+#pragma unroll
+      for (int v = 0; v < 3; v++) nyB[v][ch] = nxB[v][ch] = 0.f;
+      if (do_a.value) {
+        const Upd u = update(cur.y[0][ch], cur.y[1][ch], cur.y[2][ch], t, aFa, aG1y, aG2y, cur.c, rc1A, cur.bb[ch],
+                             cur.x[0][ch], cur.x[1][ch], cur.x[2][ch], tA);
+        nyB[0][ch] = in_img ? u.yn : 0.f;  // B reads zero padding outside the image
+        nyB[1][ch] = in_img ? u.y1o : 0.f;
+        nyB[2][ch] = in_img ? u.y2o : 0.f;
+        nxB[0][ch] = u.x_loc; nxB[1][ch] = u.y1n; nxB[2][ch] = u.y2n;
+        if (X05 && storeA) {
+          stg(xa_p[0][ch], roffA, u.xh);
+          stg(xa_p[1][ch], roffA, u.y1n);
+          stg(xa_p[2][ch], roffA, u.y2n);
+        }
+      }
+    }
+    if (tri_b.value) {
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const Tri t = triangle(pyB[0][ch], pyB[1][ch], pyB[2][ch], nyB[0][ch], nyB[1][ch], nyB[2][ch], pwxs, pwys, pbxs,
+                               pbys, dmaskB);
+        const float aFa = upB[0][ch], aG1y = upB[1][ch], aG2y = upB[2][ch];
+        upB[0][ch] = t.Fa; upB[1][ch] = t.G1y; upB[2][ch] = t.G2y;
+        if (do_b.value) {
+          const Upd u = update(pyB[0][ch], pyB[1][ch], pyB[2][ch], t, aFa, aG1y, aG2y, pc, rc1B, pbb[ch], pxB[0][ch],
+                               pxB[1][ch], pxB[2][ch], tB);
+          if (store_lane) {
+            stg(yo_p[0][ch], roffB, u.yn);
+            stg(yo_p[1][ch], roffB, u.y1o);
+            stg(yo_p[2][ch], roffB, u.y2o);
+            stg(xo_p[0][ch], roffB, u.x_loc);
+            stg(xo_p[1][ch], roffB, u.y1n);
+            stg(xo_p[2][ch], roffB, u.y2n);
+            if (X05) {
+              stg(xb_p[0][ch], roffB, u.xh);
+              stg(xb_p[1][ch], roffB, u.y1n);
+              stg(xb_p[2][ch], roffB, u.y2n);
+            }
+          }
+        }
+      }
+    }
+    pc = cur.c; pwxs = cur.wxs; pwys = cur.wys; pbxs = cur.bxs; pbys = cur.bys;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      pbb[ch] = cur.bb[ch];
+#pragma unroll
+      for (int v = 0; v < 3; v++) { pyB[v][ch] = nyB[v][ch]; pxB[v][ch] = nxB[v][ch]; }
+    }
+  };
+  const std::true_type kYes{};
+  const std::false_type kNo{};
+
+  Fwd2Row<C> b0, b1, b2, b3;
+  load_row(0, b0);
+  load_row(1, b1);
+  load_row(2, b2);
+  load_row(3, b3);
+  absorb(0, b0);
+  absorb(1, b1);
+  step(0, b0, b1, kNo, kNo, kNo);
+  load_row(4, b0);
+  absorb(2, b2);
+  step(1, b1, b2, kYes, kNo, kNo);
+  load_row(5, b1);
+  absorb(3, b3);
+  step(2, b2, b3, kYes, kYes, kNo);
+  load_row(6, b2);
+  for (int k = 3; k <= klast; k += 4) {  // cur / next rotate through (b3,b0) (b0,b1) (b1,b2) (b2,b3)
+    absorb(k + 1, b0);
+    step(k, b3, b0, kYes, kYes, kYes);
+    load_row(k + 4, b3);
+    if (k + 1 > klast) break;
+    absorb(k + 2, b1);
+    step(k + 1, b0, b1, kYes, kYes, kYes);
+    load_row(k + 5, b0);
+    if (k + 2 > klast) break;
+    absorb(k + 3, b2);
+    step(k + 2, b1, b2, kYes, kYes, kYes);
+    load_row(k + 6, b1);
+    if (k + 3 > klast) break;
+    absorb(k + 4, b3);
+    step(k + 3, b2, b3, kYes, kYes, kYes);
+    load_row(k + 7, b2);
   }
 }
 

@@ -123,6 +123,28 @@ def test_strip_edges(ext, tgv_oracle, n, c, h, w, its):
     compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 45, 130, 10)])
+def test_single_iteration_strip_kernels(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
+    # the forward and the recompute normally run two iterations per launch; INPAINT_TGV_FUSE=0 keeps
+    # the one-iteration strip kernels covered
+    d = varying_inputs(n, c, h, w, seed=91 + c)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TGV_FUSE", "0")
+    compare("one iteration per launch c=%d" % c, run_gpu(ext, d, its, 2), ref)
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 1, 9, 60, 8),       # exactly one fused strip wide (60 output columns)
+    (1, 2, 11, 61, 8),      # one column more
+    (1, 2, 3, 200, 6),      # fewer rows than the fused kernel's row lag
+    (1, 2, 2, 59, 4),
+    (2, 2, 18, 121, 12),    # two fused strips and a column
+])
+def test_fused_forward_strip_edges(ext, tgv_oracle, n, c, h, w, its):
+    d = varying_inputs(n, c, h, w, seed=n * 100 + h + w)
+    compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
+
+
 def test_varying_beta_and_per_sample_lipschitz(ext, tgv_oracle):
     # sample 0: beta up to 9 (bound above 32, data dependent); sample 1: small beta (bound 32)
     d = varying_inputs(2, 2, 40, 56, seed=11)
