@@ -647,19 +647,19 @@ template <bool BEND>
 void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c, const float* b,
                          const float* xa, const float* xb, const float* xc, const float* g05_in, float* g05_out,
                          const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
-  switch (s.ic) {
-    case 1: launch_adjoint_pair_strip<1, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
-    case 2: launch_adjoint_pair_strip<2, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
-    case 3: launch_adjoint_pair_strip<3, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
-    default: launch_adjoint_pair_strip<4, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB); break;
-  }
+  if (s.ic == 1)
+    launch_adjoint_pair_strip<1, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else
+    launch_adjoint_pair_strip<2, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
 }
 
 bool adjoint_pairs(const Slot& s) {
   const char* e = getenv("INPAINT_TV_FUSE_ADJ");
   if (e && strcmp(e, "0") == 0) return false;
-  return forward_pairs(s);
+  // with 3 or 4 channels the pair kernel needs more than 256 registers (one wavefront per SIMD);
+  // those take the one-step kernels
+  return forward_pairs(s) && s.ic <= 2;
 }
 
 }  // namespace
