@@ -15,11 +15,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the main adjoint kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
-# script on the headline workload (2 x 72471 KiB fetched, after the copy-kernel calibration, plus
-# 69740 KiB written; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script
+# (headline workload: the two-step adjoint kernel fetches 2 x 87000 KiB, after the copy-kernel
+# calibration, and writes 68035 KiB; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
 # profiles/tgv_strip_config2_hbm_traffic.txt).  Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {2: (2 * 142300 + 153730) * 1024}
+MEASURED_TRAFFIC_BYTES = {1: (2 * 87000 + 68035) * 1024, 2: (2 * 142500 + 153510) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):
