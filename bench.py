@@ -38,7 +38,7 @@ def layer_of(kind):
     from customnetworklayers_amd import workloads
     if kind == "tgv":
         from customnetworklayers_amd.cudaTGV import tgvInpaint_cuda_ext as ext
-        return ext, "tgvinpaint", workloads.tgv_inputs, "TGVOracle", "tgvstrip::tgv_adjoint_strip<2,false,false>"
+        return ext, "tgvinpaint", workloads.tgv_inputs, "TGVOracle", "tgvstrip::tgv_adjoint_strip2<2,false,false>"
     from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
     return ext, "tvinpaint", workloads.tv_inputs, "TVOracle", "tvstrip::tv_adjoint_strip2<2,false,false>"
 
@@ -101,6 +101,8 @@ def main():
     ext, prefix, _, _, kernel_name = layer_of(cfg["kind"])
     if cfg["kind"] == "tv" and (os.environ.get("INPAINT_TV_FUSE", "1") == "0" or os.environ.get("INPAINT_TV_FUSE_ADJ", "1") == "0"):
         kernel_name = "tvstrip::tv_adjoint_strip<2,false,false>"
+    if cfg["kind"] == "tgv" and (os.environ.get("INPAINT_TGV_FUSE", "1") == "0" or os.environ.get("INPAINT_TGV_FUSE_ADJ", "1") == "0"):
+        kernel_name = "tgvstrip::tgv_adjoint_strip<2,false,false>"
     profile, profile_read = getattr(lib, prefix + "_profile"), getattr(lib, prefix + "_profile_read")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     its, pid = cfg["its"], 0
@@ -129,9 +131,8 @@ def main():
     value = pxit / (elapsed / args.steps) / 1e6
     bpp = algorithmic_bytes_per_pixel(c, cfg["kind"])
     kernel_ms = tot_ms.value / max(launches.value, 1)
-    # the TV layer's dominant kernel runs two adjoint steps per launch
-    steps_per_launch = 2 if (cfg["kind"] == "tv" and os.environ.get("INPAINT_TV_FUSE", "1") != "0"
-                             and os.environ.get("INPAINT_TV_FUSE_ADJ", "1") != "0") else 1
+    # the dominant kernel runs two adjoint steps per launch
+    steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2
     kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9

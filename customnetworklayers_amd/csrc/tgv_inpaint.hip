@@ -944,6 +944,44 @@ void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b,
                      s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
 }
 
+// Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
+// (xc = slot j-2, or the checkpoint y when B is the segment's first iteration).
+template <int C, bool BEND>
+void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
+                               const float* xb, const float* xc, const float* g05_in, float* g05_out, const float* gxk,
+                               float* gxk_m1, float* gx_final, float tA, float tB) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
+  const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
+  const long long waves = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
+  if (gx_final)
+    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+                       xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
+                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, tA, tB, R, sx,
+                       sy);
+  else
+    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+                       xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
+                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, tA, tB, R, sx,
+                       sy);
+}
+
+template <bool BEND>
+void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa, const float* xb,
+                         const float* xc, const float* g05_in, float* g05_out, const float* gxk, float* gxk_m1,
+                         float* gx_final, float tA, float tB) {
+  if (s.ic == 1) launch_adjoint_pair_strip<1, BEND>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else launch_adjoint_pair_strip<2, BEND>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  s.acc_cur = 1 - s.acc_cur;
+}
+
+bool adjoint_pairs(const Slot& s) {
+  const char* e = getenv("INPAINT_TGV_FUSE_ADJ");
+  if (e && strcmp(e, "0") == 0) return false;
+  return forward_pairs(s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -1067,6 +1105,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   const bool strip = use_strip(s);
   const float* gi_src = strip ? s.gx_final : s.gxk[1];
   int lastIt = its;
+  int pp_src = 1;
   const int nseg = (int)s.iterations.size();
   for (int outer = nseg - 1; outer >= 0; outer--) {
     const int k0 = s.iterations[outer];
@@ -1090,6 +1129,45 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       }
     }
     int timed_run = 0;
+    if (adjoint_pairs(s)) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
+      // `pp_src` = the g05 / g_x buffer the next launch reads; it flips once per launch
+      int j = len - 1;
+      if (outer == nseg - 1 && j >= 0) {
+        hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+                           s.x05 + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                           (long long)ih * iw, (long long)P);
+        pp_src = 1;
+        j--;
+      }
+      if (j >= 0 && ((j + 1) & 1)) {  // an odd number of steps is left: one single step, then pairs
+        const float* xa = s.x05 + (size_t)j * S3;
+        if (j > 0)
+          launch_adjoint<false>(s, stream, c, b, xa, s.x05 + (size_t)(j - 1) * S3, nullptr, s.g05[pp_src],
+                                s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j]);
+        else
+          launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[pp_src], s.g05[1 - pp_src], s.gxk[pp_src],
+                               s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr, s.steps[k0 + j]);
+        pp_src = 1 - pp_src;
+        j--;
+      }
+      for (; j >= 1; j -= 2) {
+        const float* xa = s.x05 + (size_t)j * S3;
+        const float* xb = s.x05 + (size_t)(j - 1) * S3;
+        if (j - 1 > 0) {
+          if (timed_run == 0) g_timer.begin(stream);
+          launch_adjoint_pair<false>(s, stream, c, b, xa, xb, s.x05 + (size_t)(j - 2) * S3, s.g05[pp_src],
+                                     s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j],
+                                     s.steps[k0 + j - 1]);
+          timed_run++;
+          if (j - 2 <= 1) g_timer.end(stream, timed_run);
+        } else {
+          launch_adjoint_pair<true>(s, stream, c, b, xa, xb, cky, s.g05[pp_src], s.g05[1 - pp_src], s.gxk[pp_src],
+                                    s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr, s.steps[k0 + j],
+                                    s.steps[k0 + j - 1]);
+        }
+        pp_src = 1 - pp_src;
+      }
+    } else
     for (int j = len - 1; j >= 0; j--) {  // reverse sweep (TGV.cu:2851-2933)
       const float t = s.steps[k0 + j];
       const float* xa = s.x05 + (size_t)j * S3;

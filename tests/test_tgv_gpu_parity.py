@@ -145,6 +145,25 @@ def test_fused_forward_strip_edges(ext, tgv_oracle, n, c, h, w, its):
     compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 45, 130, 10)])
+def test_single_step_adjoint_strip_kernels(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
+    # the reverse sweep may run two adjoint steps per launch; INPAINT_TGV_FUSE_ADJ=0 keeps the
+    # one-step strip kernels covered
+    d = varying_inputs(n, c, h, w, seed=93 + c)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TGV_FUSE_ADJ", "0")
+    compare("one adjoint step per launch c=%d" % c, run_gpu(ext, d, its, 2), ref)
+
+
+@pytest.mark.parametrize("c", [1, 2])
+@pytest.mark.parametrize("its", [2, 3, 4, 5, 6, 8, 16, 17, 26])
+def test_every_pairing_of_the_reverse_sweep(ext, tgv_oracle, c, its):
+    # segment lengths 2, 4, 6 ... and their mixes: first step + pairs, first + single + pairs,
+    # a pair that ends a segment, a single step that ends a segment
+    d = varying_inputs(1, c, 23, 75, seed=its * 7 + c)
+    compare("c=%d its=%d" % (c, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
+
+
 def test_varying_beta_and_per_sample_lipschitz(ext, tgv_oracle):
     # sample 0: beta up to 9 (bound above 32, data dependent); sample 1: small beta (bound 32)
     d = varying_inputs(2, 2, 40, 56, seed=11)
