@@ -288,3 +288,76 @@ class TGVOracle:
 
     def set_threads(self, n):
         self.lib.tgv_oracle_set_threads(int(n))
+
+
+class FlowAuxOracle:
+    """Quadratic sub-pixel fit (cudaQuadFit) and histogram median (cudaMedian), CPU restatement
+    (oracle/flowaux_oracle.cpp)."""
+
+    def __init__(self):
+        L = self.lib = _load("libflowaux_oracle.so")
+        L.quadfit_oracle_forward.argtypes = [_f32p] * 4 + [_int] * 5
+        L.quadfit_oracle_forward_f64.argtypes = [_f64p] * 4 + [_int] * 5
+        L.quadfit_oracle_backward.argtypes = [_f32p] * 6 + [_int] * 5
+        L.quadfit_oracle_backward_f64.argtypes = [_f64p] * 6 + [_int] * 5
+        L.median_oracle_forward.argtypes = [_f32p] * 2 + [_int] * 4
+        L.median_oracle_forward_f64.argtypes = [_f64p] * 2 + [_int] * 4
+        L.median_oracle_backward.argtypes = [_f32p] * 3 + [_int] * 4
+        L.median_oracle_backward_f64.argtypes = [_f64p] * 3 + [_int] * 4
+        L.flowaux_oracle_set_threads.argtypes = [_int]
+        L.flowaux_oracle_set_threads.restype = None
+
+    def quadfit_forward(self, feat0, feat1, flow, f64=False):
+        """feat0, feat1: (N,C,H,W); flow: (N,F,H,W) with F >= 2.  Returns (N,3,H,W) = (fx, fy, score)."""
+        dt = np.float64 if f64 else np.float32
+        feat0, feat1, flow = (_c(a, dt) for a in (feat0, feat1, flow))
+        n, c, h, w = feat0.shape
+        out = np.empty((n, 3, h, w), dt)
+        P = _p64 if f64 else _p32
+        fn = self.lib.quadfit_oracle_forward_f64 if f64 else self.lib.quadfit_oracle_forward
+        rc = fn(P(feat0), P(feat1), P(flow), P(out), n, c, h, w, flow.shape[1])
+        if rc:
+            raise RuntimeError("quadfit_oracle_forward failed with code %d" % rc)
+        return out
+
+    def quadfit_backward(self, gin, feat0, feat1, flow, f64=False):
+        """gin: (N,3,H,W).  Returns the gradients wrt feat0 and feat1."""
+        dt = np.float64 if f64 else np.float32
+        gin, feat0, feat1, flow = (_c(a, dt) for a in (gin, feat0, feat1, flow))
+        n, c, h, w = feat0.shape
+        g0, g1 = np.empty_like(feat0), np.empty_like(feat1)
+        P = _p64 if f64 else _p32
+        fn = self.lib.quadfit_oracle_backward_f64 if f64 else self.lib.quadfit_oracle_backward
+        rc = fn(P(feat0), P(feat1), P(flow), P(gin), P(g0), P(g1), n, c, h, w, flow.shape[1])
+        if rc:
+            raise RuntimeError("quadfit_oracle_backward failed with code %d" % rc)
+        return g0, g1
+
+    def median_forward(self, vol, f64=False):
+        """vol: (N,H,W,D).  Returns (N,2,H,W) = (median position, mass of its bin)."""
+        dt = np.float64 if f64 else np.float32
+        vol = _c(vol, dt)
+        n, h, w, d = vol.shape
+        out = np.empty((n, 2, h, w), dt)
+        P = _p64 if f64 else _p32
+        fn = self.lib.median_oracle_forward_f64 if f64 else self.lib.median_oracle_forward
+        rc = fn(P(vol), P(out), n, h, w, d)
+        if rc:
+            raise RuntimeError("median_oracle_forward failed with code %d" % rc)
+        return out
+
+    def median_backward(self, gin, vol, f64=False):
+        """gin: (N,2,H,W).  Returns the gradient wrt vol."""
+        dt = np.float64 if f64 else np.float32
+        gin, vol = _c(gin, dt), _c(vol, dt)
+        n, h, w, d = vol.shape
+        g = np.empty_like(vol)
+        P = _p64 if f64 else _p32
+        fn = self.lib.median_oracle_backward_f64 if f64 else self.lib.median_oracle_backward
+        rc = fn(P(vol), P(gin), P(g), n, h, w, d)
+        if rc:
+            raise RuntimeError("median_oracle_backward failed with code %d" % rc)
+        return g
+
+    def set_threads(self, n):
+        self.lib.flowaux_oracle_set_threads(int(n))

@@ -19,3 +19,10 @@ def tv_oracle():
     o = TVOracle()
     o.set_quirks()  # literal reference behaviour
     return o
+
+
+@pytest.fixture(scope="session")
+def flowaux_oracle():
+    from oracle.oracle_lib import FlowAuxOracle
+
+    return FlowAuxOracle()

@@ -1,0 +1,234 @@
+"""Pins of the CPU oracle for the quadratic fit (cudaQuadFit) and the histogram median (cudaMedian)
+against statements written from their definitions: numpy.polyfit parabolas, the inverse of a
+piecewise-linear CDF, torch.autograd and central finite differences.  All CPU."""
+import numpy as np
+import pytest
+import torch
+
+from tests import independent_flowaux as ind
+
+
+def features(n, c, h, w, seed, flow_amp=3.0, fc=2):
+    rng = np.random.default_rng(seed)
+    f0 = rng.standard_normal((n, c, h, w))
+    f1 = rng.standard_normal((n, c, h, w))
+    flow = flow_amp * rng.standard_normal((n, fc, h, w))
+    return f0, f1, flow
+
+
+def peaked_features(n, c, h, w, seed, shift=(1.3, -0.6)):
+    """Second image = first image displaced by a sub-pixel shift of smooth features: most fits are valid."""
+    rng = np.random.default_rng(seed)
+    ys, xs = np.mgrid[0:h, 0:w].astype(np.float64)
+    f0 = np.empty((n, c, h, w))
+    f1 = np.empty((n, c, h, w))
+    for i in range(n):
+        for k in range(0, c, 2):  # quadrature pairs: the summed cost depends on the displacement only
+            fx, fy, ph = rng.uniform(0.2, 0.9), rng.uniform(0.2, 0.9), rng.uniform(0, 6.28)
+            for j, fn in enumerate((np.cos, np.sin)[: min(2, c - k)]):
+                f0[i, k + j] = fn(fx * xs + fy * ys + ph)
+                f1[i, k + j] = fn(fx * (xs - shift[0]) + fy * (ys - shift[1]) + ph)
+    flow = np.zeros((n, 2, h, w))
+    flow[:, 0] = np.round(shift[0]) + 0.2 * rng.standard_normal((n, h, w))
+    flow[:, 1] = np.round(shift[1]) + 0.2 * rng.standard_normal((n, h, w))
+    return f0, f1, flow
+
+
+# ------------------------------------------------------------------------------------------------
+# quadratic fit, forward
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("maker,seed", [(features, 1), (peaked_features, 2)])
+def test_quadfit_forward_matches_polyfit_parabolas(flowaux_oracle, maker, seed):
+    n, c, h, w = 2, 6, 9, 11
+    f0, f1, flow = maker(n, c, h, w, seed)
+    out = flowaux_oracle.quadfit_forward(f0, f1, flow, f64=True)
+    inside, ix, iy = ind.displaced_indices(torch.from_numpy(flow), h, w)
+    costs = [t.numpy() for t in ind.matching_costs(torch.from_numpy(f0), torch.from_numpy(f1), ix, iy)]
+    c0, cxp, cxm, cyp, cym = costs
+    seen = dict(valid_x=0, valid_y=0, outside=0, border=0)
+    for i in range(n):
+        for y in range(h):
+            for x in range(w):
+                if not inside[i, y, x]:
+                    seen["outside"] += 1
+                    assert (out[i, :, y, x] == 0).all()
+                    continue
+                score = c0[i, y, x]
+                for axis, (cp, cm, pos, size) in enumerate([(cxp, cxm, int(ix[i, y, x]), w), (cyp, cym, int(iy[i, y, x]), h)]):
+                    a, b, cc = ind.polyfit_axis(cm[i, y, x], c0[i, y, x], cp[i, y, x])
+                    interior = 0 < pos < size - 1
+                    seen["border"] += (not interior)
+                    if a < 0 and abs(b) <= 2 * abs(a) and interior:
+                        seen["valid_x" if axis == 0 else "valid_y"] += 1
+                        t = -b / (2 * a)
+                        assert abs(out[i, axis, y, x] - t) < 1e-9
+                        score += np.polyval([a, b, cc], t) - cc
+                    else:
+                        assert out[i, axis, y, x] == 0
+                assert abs(out[i, 2, y, x] - score) < 1e-9 * max(1.0, abs(score))
+    assert seen["valid_x"] > 5 and seen["valid_y"] > 5 and seen["border"] > 0, seen
+    if maker is features:
+        assert seen["outside"] > 5, seen
+
+
+def test_quadfit_recovers_a_known_subpixel_shift(flowaux_oracle):
+    # smooth features displaced by a sub-pixel shift along one axis: the fitted offset lands near its
+    # fractional part (the parabola is an approximation of the summed cosines, hence the tolerance)
+    n, c, h, w = 1, 24, 24, 30
+    inner = (slice(None), slice(3, h - 3), slice(3, w - 3))
+    for shift, axis, want in (((1.3, -1.0), 0, 0.3), ((1.0, -0.6), 1, 0.4)):
+        f0, f1, flow = peaked_features(n, c, h, w, seed=5, shift=shift)
+        flow[:, 0], flow[:, 1] = 1.0, -1.0
+        out = flowaux_oracle.quadfit_forward(f0, f1, flow, f64=True)
+        assert np.abs(out[:, axis][inner] - want).max() < 0.05
+
+
+def test_quadfit_float_layer_agrees_with_double(flowaux_oracle):
+    f0, f1, flow = peaked_features(2, 8, 20, 26, seed=7)
+    a = flowaux_oracle.quadfit_forward(f0, f1, flow, f64=False)
+    b = flowaux_oracle.quadfit_forward(f0, f1, flow, f64=True)
+    close = np.abs(a - b) < 1e-4 * np.abs(b).max()
+    assert close.mean() > 0.995  # a validity test may flip at a handful of pixels
+
+
+def test_quadfit_reads_only_the_first_two_flow_channels(flowaux_oracle):
+    f0, f1, flow = features(2, 4, 8, 10, seed=3, fc=3)
+    a = flowaux_oracle.quadfit_forward(f0, f1, flow)
+    b = flowaux_oracle.quadfit_forward(f0, f1, np.ascontiguousarray(flow[:, :2]))
+    assert (a == b).all()
+
+
+# ------------------------------------------------------------------------------------------------
+# quadratic fit, backward
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("maker,seed", [(features, 11), (peaked_features, 12)])
+def test_quadfit_backward_matches_autograd(flowaux_oracle, maker, seed):
+    n, c, h, w = 2, 6, 10, 13
+    f0, f1, flow = maker(n, c, h, w, seed)
+    gin = np.random.default_rng(seed).standard_normal((n, 3, h, w))
+    t0 = torch.from_numpy(f0).requires_grad_(True)
+    t1 = torch.from_numpy(f1).requires_grad_(True)
+    out = ind.quadfit(t0, t1, torch.from_numpy(flow))
+    ref_out = flowaux_oracle.quadfit_forward(f0, f1, flow, f64=True)
+    assert np.abs(out.detach().numpy() - ref_out).max() < 1e-10
+    (out * torch.from_numpy(gin)).sum().backward()
+    g0, g1 = flowaux_oracle.quadfit_backward(gin, f0, f1, flow, f64=True)
+    assert np.abs(g0 - t0.grad.numpy()).max() < 1e-9 * max(1.0, np.abs(g0).max())
+    assert np.abs(g1 - t1.grad.numpy()).max() < 1e-9 * max(1.0, np.abs(g1).max())
+    assert np.abs(g1).max() > 0 and np.abs(g0).max() > 0
+
+
+def test_quadfit_backward_matches_finite_differences(flowaux_oracle):
+    n, c, h, w = 1, 3, 6, 7
+    f0, f1, flow = peaked_features(n, c, h, w, seed=21)
+    rng = np.random.default_rng(21)
+    gin = rng.standard_normal((n, 3, h, w))
+    g0, g1 = flowaux_oracle.quadfit_backward(gin, f0, f1, flow, f64=True)
+
+    def loss(a, b):
+        return float((flowaux_oracle.quadfit_forward(a, b, flow, f64=True) * gin).sum())
+
+    eps = 1e-6
+    for which, g in ((0, g0), (1, g1)):
+        for _ in range(12):
+            idx = tuple(rng.integers(0, s) for s in f0.shape)
+            ap, am = [f0.copy(), f1.copy()], [f0.copy(), f1.copy()]
+            ap[which][idx] += eps
+            am[which][idx] -= eps
+            fd = (loss(*ap) - loss(*am)) / (2 * eps)
+            assert abs(fd - g[idx]) < 1e-5 * max(1.0, abs(fd)), (which, idx, fd, g[idx])
+
+
+def test_quadfit_backward_accumulates_where_pixels_collide(flowaux_oracle):
+    # every pixel is sent to the same target: the gradient wrt the second image is non-zero only in that
+    # target's 5-stencil and its centre collects a term from every pixel
+    n, c, h, w = 1, 2, 7, 9
+    rng = np.random.default_rng(4)
+    f0, f1 = rng.standard_normal((n, c, h, w)), rng.standard_normal((n, c, h, w))
+    ys, xs = np.mgrid[0:h, 0:w]
+    flow = np.stack([4 - xs, 3 - ys])[None].astype(np.float64)
+    gin = np.zeros((n, 3, h, w))
+    gin[:, 2] = 1.0
+    g0, g1 = flowaux_oracle.quadfit_backward(gin, f0, f1, flow, f64=True)
+    mask = np.zeros((h, w), bool)
+    mask[3, 3:6] = mask[2:5, 4] = True
+    assert (g1[0][:, ~mask] == 0).all() and (g1[0][:, mask] != 0).all()
+    t0, t1 = torch.from_numpy(f0), torch.from_numpy(f1).requires_grad_(True)
+    ind.quadfit(t0, t1, torch.from_numpy(flow))[:, 2].sum().backward()
+    assert np.abs(g1 - t1.grad.numpy()).max() < 1e-9
+
+
+def test_quadfit_float_backward_agrees_with_double(flowaux_oracle):
+    f0, f1, flow = peaked_features(2, 8, 20, 26, seed=9)
+    gin = np.random.default_rng(9).standard_normal((2, 3, 20, 26))
+    a = flowaux_oracle.quadfit_backward(gin, f0, f1, flow, f64=False)
+    b = flowaux_oracle.quadfit_backward(gin, f0, f1, flow, f64=True)
+    for x, y in zip(a, b):
+        close = np.abs(x - y) < 1e-4 * np.abs(y).max()
+        assert close.mean() > 0.99
+
+
+# ------------------------------------------------------------------------------------------------
+# median
+# ------------------------------------------------------------------------------------------------
+def histograms(n, h, w, d, seed, sharp=3.0):
+    rng = np.random.default_rng(seed)
+    v = np.exp(sharp * rng.standard_normal((n, h, w, d)))
+    return v / v.sum(-1, keepdims=True)
+
+
+def test_median_forward_is_the_inverse_cdf(flowaux_oracle):
+    vol = histograms(2, 5, 7, 9, seed=1)
+    out = flowaux_oracle.median_forward(vol, f64=True)
+    for i in range(2):
+        for y in range(5):
+            for x in range(7):
+                p = vol[i, y, x]
+                m = ind.histogram_median(p)
+                assert abs(out[i, 0, y, x] - m) < 1e-12
+                k = int(np.floor(m + 0.5))
+                assert out[i, 1, y, x] == p[min(k, len(p) - 1)] or abs(m + 0.5 - k) < 1e-12
+
+
+def test_median_closed_forms(flowaux_oracle):
+    d = 8
+    vol = np.zeros((1, 1, 4, d))
+    vol[0, 0, 0, 5] = 1.0                 # all mass in bin 5: the median is the bin centre
+    vol[0, 0, 1, :] = 1.0 / d             # uniform: the middle of the support
+    vol[0, 0, 2, 2] = vol[0, 0, 2, 6] = 0.5   # half the mass by the end of bin 2: its right edge
+    vol[0, 0, 3, :] = 0.05                # mass below one half: nothing is written
+    out = flowaux_oracle.median_forward(vol, f64=True)
+    assert out[0, 0, 0, 0] == 5.0 and out[0, 1, 0, 0] == 1.0
+    assert abs(out[0, 0, 0, 1] - (d / 2 - 0.5)) < 1e-12
+    assert out[0, 0, 0, 2] == 2.5 and out[0, 1, 0, 2] == 0.5
+    assert out[0, 0, 0, 3] == 0.0 and out[0, 1, 0, 3] == 0.0
+
+
+def test_median_backward_is_the_gradient_of_the_normalised_median(flowaux_oracle):
+    vol = histograms(2, 4, 6, 11, seed=2)
+    gin = np.random.default_rng(2).standard_normal((2, 2, 4, 6))
+    t = torch.from_numpy(vol).requires_grad_(True)
+    med, mass = ind.normalised_median(t)
+    fwd = flowaux_oracle.median_forward(vol, f64=True)
+    assert np.abs(med.detach().numpy() - fwd[:, 0]).max() < 1e-12
+    assert (mass.detach().numpy() == fwd[:, 1]).all()
+    (med * torch.from_numpy(gin[:, 0]) + mass * torch.from_numpy(gin[:, 1])).sum().backward()
+    g = flowaux_oracle.median_backward(gin, vol, f64=True)
+    assert np.abs(g - t.grad.numpy()).max() < 1e-9 * np.abs(g).max()
+
+
+def test_median_backward_without_a_crossing(flowaux_oracle):
+    # mass below one half everywhere: every bin takes -g0 / 2 (the reference's default pmid = 1)
+    vol = np.full((1, 1, 1, 6), 0.05)
+    gin = np.array([3.0, 7.0]).reshape(1, 2, 1, 1)
+    g = flowaux_oracle.median_backward(gin, vol, f64=True)
+    assert (g == -1.5).all()
+
+
+def test_median_float_layer_agrees_with_double(flowaux_oracle):
+    vol = histograms(2, 16, 20, 33, seed=3)
+    gin = np.random.default_rng(3).standard_normal((2, 2, 16, 20))
+    a, b = flowaux_oracle.median_forward(vol), flowaux_oracle.median_forward(vol, f64=True)
+    assert np.abs(a - b).max() < 1e-4 * np.abs(b).max()
+    ga, gb = flowaux_oracle.median_backward(gin, vol), flowaux_oracle.median_backward(gin, vol, f64=True)
+    assert (np.abs(ga - gb) < 1e-4 * np.abs(gb).max()).mean() > 0.999
