@@ -77,13 +77,108 @@ def cpu_baseline(cfg, seconds_hint=20.0):
                 one_core_value=round(pxit / t_one / 1e6, 3), host_cpu_count=os.cpu_count())
 
 
+def flowaux_cpu_baseline(cfg, d):
+    """The CPU oracle on ONE sample of the batch, forward + backward, all host cores (best of 2) and one core."""
+    import multiprocessing
+
+    from oracle.oracle_lib import FlowAuxOracle
+
+    o = FlowAuxOracle()
+    one = {k: v[:1] for k, v in d.items()}
+
+    def once():
+        t0 = time.perf_counter()
+        if cfg["kind"] == "quadfit":
+            o.quadfit_forward(one["feat0"], one["feat1"], one["flow"])
+            o.quadfit_backward(one["grad"], one["feat0"], one["feat1"], one["flow"])
+        else:
+            o.median_forward(one["vol"])
+            o.median_backward(one["grad"], one["vol"])
+        return time.perf_counter() - t0
+
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else multiprocessing.cpu_count()
+    cores = min(avail, int(os.environ.get("OMP_NUM_THREADS", "0") or avail))
+    o.set_threads(cores)
+    once()
+    t_all = min(once(), once())
+    o.set_threads(1)
+    t_one = once()
+    px = cfg["h"] * cfg["w"]
+    # the quadratic fit's backward scatter runs one thread per sample in the oracle
+    used = 1 if cfg["kind"] == "quadfit" else cores
+    return dict(value=round(px / t_all / 1e6, 3), unit="Mpixel/s", cores=cores, kind="port",
+                sample="1 of %d samples, fwd+bwd, best of 2%s" % (cfg["n"], " (backward scatter on %d core)" % used
+                                                                  if cfg["kind"] == "quadfit" else ""),
+                one_core_value=round(px / t_one / 1e6, 3), host_cpu_count=os.cpu_count())
+
+
+def bench_flowaux(args, cfg, d):
+    """Configs 5 and 6: the quadratic fit and the median, forward + backward per step."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    n, h, w = cfg["n"], cfg["h"], cfg["w"]
+    px = n * h * w
+    if cfg["kind"] == "quadfit":
+        from customnetworklayers_amd.cudaQuadFit import QuadFit_cuda_ext as ext
+        c = cfg["c"]
+        fwd = lambda: ext.forward(t["feat0"], t["feat1"], t["flow"])  # noqa: E731
+        bwd = lambda: ext.backward(t["grad"], t["feat0"], t["feat1"], t["flow"])  # noqa: E731
+        # floats per pixel: forward reads both feature maps and the flow, writes 3; backward reads both maps,
+        # flow and upstream, writes g0, zero-fills g1 and read-modify-writes it
+        bpp = dict(forward=4 * (2 * c + 5), backward=4 * (6 * c + 5))
+        kernel = "quadfit_backward_kernel (+ the zero fill of the scatter target)"
+        shape = "features %dx%dx%d" % (c, h, w)
+    else:
+        from customnetworklayers_amd.cudaMedian import median_cuda_ext as ext
+        dd = cfg["d"]
+        fwd = lambda: ext.forward(t["vol"])  # noqa: E731
+        bwd = lambda: ext.backward(t["grad"], t["vol"])  # noqa: E731
+        # forward reads the histogram once (it may stop early) and writes 2; backward reads it, the upstream and writes it
+        bpp = dict(forward=4 * (dd + 2), backward=4 * (2 * dd + 2))
+        kernel = "median_backward_kernel"
+        shape = "histograms %dx%dx%d" % (h, w, dd)
+    bpp["total"] = bpp["forward"] + bpp["backward"]
+    for _ in range(args.warmup):
+        fwd(), bwd()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for e in ev:  # events on the stream the kernels are launched on (torch's current stream)
+        e[0].record(); fwd(); e[1].record(); bwd(); e[2].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    f_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    b_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    value = px / (elapsed / args.steps) / 1e6
+    achieved = bpp["backward"] * px / (b_ms * 1e-3) / 1e9
+    out = {
+        "metric": "%s fwd+bwd Mpixel/s at %d x %s; achieved HBM GB/s vs peak" % (cfg["kind"], n, shape),
+        "value": round(value, 2), "unit": "Mpixel/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s fwd+bwd, N=%d, %s fp32 (config %d)" % (cfg["kind"], n, shape, args.config), "pixels_per_step": px},
+        "whole_job": {"model_bytes_per_pixel": bpp["total"], "achieved_GBps": round(bpp["total"] * px / (elapsed / args.steps) / 1e9, 1),
+                      "forward_ms": round(f_ms, 4), "backward_ms": round(b_ms, 4),
+                      "forward_GBps": round(bpp["forward"] * px / (f_ms * 1e-3) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
+                     "bytes_per_launch": bpp["backward"] * px, "avg_launch_ms": round(b_ms, 5), "launches_timed": args.steps},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = flowaux_cpu_baseline(cfg, d)
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--config", type=int, default=1, help="workload index (1 = headline)")
+    ap.add_argument("--config", type=int, default=1,
+                    help="workload index (1 = headline TV layer, 2 = TGV layer, 5 = quadratic fit, 6 = median)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
@@ -97,6 +192,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     cfg, d = config_inputs(args.config, seed=0)
+    if cfg["kind"] in ("quadfit", "median"):
+        return bench_flowaux(args, cfg, d)
     assert cfg["kind"] in ("tv", "tgv")
     ext, prefix, _, _, kernel_name = layer_of(cfg["kind"])
     if cfg["kind"] == "tv" and (os.environ.get("INPAINT_TV_FUSE", "1") == "0" or os.environ.get("INPAINT_TV_FUSE_ADJ", "1") == "0"):

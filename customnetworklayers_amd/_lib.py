@@ -48,6 +48,11 @@ def _load():
     lib.tgvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
     lib.tgvinpaint_last_error.restype = ctypes.c_char_p
     lib.inpaint_selftest_rsqrt.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_uint]
+    lib.quadfit_forward.argtypes = [_f32p] * 4 + [_int] * 5 + [ctypes.c_void_p]
+    lib.quadfit_backward.argtypes = [_f32p] * 6 + [_int] * 5 + [ctypes.c_void_p]
+    lib.medimax_forward.argtypes = [_f32p] * 2 + [_int] * 4 + [ctypes.c_void_p]
+    lib.medimax_backward.argtypes = [_f32p] * 3 + [_int] * 4 + [ctypes.c_void_p]
+    lib.flowaux_last_error.restype = ctypes.c_char_p
     return lib
 
 

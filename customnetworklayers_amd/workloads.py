@@ -95,6 +95,9 @@ CONFIGS = {
     3: dict(kind="tv_hierarchy", n=2, c=2, levels=[(112, 256), (224, 512), (448, 1024)], its=50,
             gen=dict(conf_density=0.25)),
     4: dict(kind="tv", n=16, c=2, h=256, w=512, its=200, gen=dict(flow="rectangles", dense_conf=True)),
+    # the two layers upstream of the inpainting layer, at the headline image size
+    5: dict(kind="quadfit", n=4, c=32, h=384, w=1248, gen=dict()),
+    6: dict(kind="median", n=4, h=384, w=1248, d=33, gen=dict()),
 }
 
 
@@ -104,6 +107,10 @@ def config_inputs(idx, seed=0):
         return cfg, tv_inputs(cfg["n"], cfg["c"], cfg["h"], cfg["w"], seed=seed, **cfg["gen"])
     if cfg["kind"] == "tgv":
         return cfg, tgv_inputs(cfg["n"], cfg["c"], cfg["h"], cfg["w"], seed=seed, **cfg["gen"])
+    if cfg["kind"] == "quadfit":
+        return cfg, quadfit_inputs(cfg["n"], cfg["c"], cfg["h"], cfg["w"], seed=seed, **cfg["gen"])
+    if cfg["kind"] == "median":
+        return cfg, median_inputs(cfg["n"], cfg["h"], cfg["w"], cfg["d"], seed=seed, **cfg["gen"])
     raise ValueError("config %d is assembled by its caller (hierarchy)" % idx)
 
 
@@ -124,3 +131,57 @@ def tgv_inputs(n, c, h, w, seed=0, conf_density=0.2, alpha0=1.0, alpha1=2.0):
     di[:, :c] = base["db"]
     grad = rng.normal(0, 1, (n, 3 * c, h, w)).astype(np.float32)
     return dict(dx=dx, dy=dy, dc=base["dc"], db=base["db"], di=di, grad=grad)
+
+
+def quadfit_inputs(n, c, h, w, seed=0, flow_channels=2, amplitude=8.0, jitter=0.6):
+    """Inputs of one quadratic-fit call: feat1 is a smooth random feature map, feat0 is feat1 looked up
+    at the true (smooth, sub-pixel) flow, and the flow handed to the layer is the true flow plus a
+    jitter of about half a pixel -- the situation of a matching cost that peaks next to the rounded
+    displaced position.  Near the image border part of the displaced pixels fall outside.
+
+    feat0, feat1: (n,c,h,w); flow: (n,flow_channels,h,w); grad: (n,3,h,w).
+    """
+    from scipy.ndimage import map_coordinates
+
+    rng = np.random.default_rng(seed)
+    feat0 = np.empty((n, c, h, w), np.float32)
+    feat1 = np.empty((n, c, h, w), np.float32)
+    flow = np.zeros((n, flow_channels, h, w), np.float32)
+    ys, xs = np.mgrid[0:h, 0:w].astype(np.float64)
+    for i in range(n):
+        true = sinusoid_flow(rng, 2, h, w, amplitude=amplitude, noise=0.0).astype(np.float64)
+        coords = np.stack([ys + true[1], xs + true[0]])
+        for k in range(c):
+            f = rng.standard_normal((h, w))
+            if gaussian_filter is not None:
+                f = gaussian_filter(f, 1.5, mode="nearest")
+            f = f / max(f.std(), 1e-12)
+            feat1[i, k] = f
+            feat0[i, k] = map_coordinates(f, coords, order=1, mode="nearest")
+        flow[i, 0] = true[0] + rng.normal(0, jitter, (h, w))
+        flow[i, 1] = true[1] + rng.normal(0, jitter, (h, w))
+        if flow_channels > 2:
+            flow[i, 2:] = rng.random((flow_channels - 2, h, w))
+    grad = rng.normal(0, 1, (n, 3, h, w)).astype(np.float32)
+    return dict(feat0=feat0, feat1=feat1, flow=flow, grad=grad)
+
+
+def median_inputs(n, h, w, d, seed=0, spread=2.0, empty_fraction=0.02):
+    """Inputs of one median call: per pixel a normalised histogram over d displacement bins, a noisy
+    bump around a smoothly varying centre; a few pixels carry less than half a unit of mass (the
+    layer leaves them at zero).
+
+    vol: (n,h,w,d) with the bins innermost; grad: (n,2,h,w).
+    """
+    rng = np.random.default_rng(seed)
+    vol = np.empty((n, h, w, d), np.float32)
+    bins = np.arange(d, dtype=np.float64)
+    for i in range(n):
+        centre = (d - 1) * (0.5 + 0.4 * sinusoid_flow(rng, 1, h, w, amplitude=1.0, noise=0.0)[0])
+        logit = -0.5 * ((bins - centre[..., None]) / spread) ** 2 + 0.5 * rng.standard_normal((h, w, d))
+        p = np.exp(logit - logit.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        p[rng.random((h, w)) < empty_fraction] *= 0.3
+        vol[i] = p
+    grad = rng.normal(0, 1, (n, 2, h, w)).astype(np.float32)
+    return dict(vol=vol, grad=grad)

@@ -1,0 +1,2 @@
+"""Top-level alias so that `import median_cuda_ext` keeps working as with the reference build."""
+from customnetworklayers_amd.cudaMedian.median_cuda_ext import backward, dummy, dummy_only, forward  # noqa: F401
