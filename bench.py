@@ -116,6 +116,8 @@ def bench_flowaux(args, cfg, d):
     """Configs 5 and 6: the quadratic fit and the median, forward + backward per step."""
     import torch
 
+    from customnetworklayers_amd._lib import lib
+
     dev = torch.device("cuda:0")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     n, h, w = cfg["n"], cfg["h"], cfg["w"]
@@ -127,8 +129,9 @@ def bench_flowaux(args, cfg, d):
         bwd = lambda: ext.backward(t["grad"], t["feat0"], t["feat1"], t["flow"])  # noqa: E731
         # floats per pixel: forward reads both feature maps and the flow, writes 3; backward reads both maps,
         # flow and upstream, writes g0, zero-fills g1 and read-modify-writes it
-        bpp = dict(forward=4 * (2 * c + 5), backward=4 * (6 * c + 5))
-        kernel = "quadfit_backward_kernel (+ the zero fill of the scatter target)"
+        # per-source pass of the backward (the dominant kernel): both maps, flow, upstream in; g0 and 5 coefficients out
+        bpp = dict(forward=4 * (2 * c + 5), backward=4 * (5 * c + 5), kernel=4 * (3 * c + 10))
+        kernel = "quadfit_tiles<1,2> (backward, per-source pass)"
         shape = "features %dx%dx%d" % (c, h, w)
     else:
         from customnetworklayers_amd.cudaMedian import median_cuda_ext as ext
@@ -136,14 +139,15 @@ def bench_flowaux(args, cfg, d):
         fwd = lambda: ext.forward(t["vol"])  # noqa: E731
         bwd = lambda: ext.backward(t["grad"], t["vol"])  # noqa: E731
         # forward reads the histogram once (it may stop early) and writes 2; backward reads it, the upstream and writes it
-        bpp = dict(forward=4 * (dd + 2), backward=4 * (2 * dd + 2))
-        kernel = "median_backward_kernel"
+        bpp = dict(forward=4 * (dd + 2), backward=4 * (2 * dd + 2), kernel=4 * (2 * dd + 2))
+        kernel = "median_rows_kernel<4,true> (backward)"
         shape = "histograms %dx%dx%d" % (h, w, dd)
-    bpp["total"] = bpp["forward"] + bpp["backward"]
+    bpp["total"] = bpp["forward"] + bpp["backward"]  # "kernel": the dominant kernel alone
     for _ in range(args.warmup):
         fwd(), bwd()
     torch.cuda.synchronize()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    lib.flowaux_profile(1)  # HIP events around the dominant kernel, on the stream it is launched on
     t0 = time.perf_counter()
     for e in ev:  # events on the stream the kernels are launched on (torch's current stream)
         e[0].record(); fwd(); e[1].record(); bwd(); e[2].record()
@@ -151,8 +155,12 @@ def bench_flowaux(args, cfg, d):
     elapsed = time.perf_counter() - t0
     f_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     b_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    tot_ms, launches = ctypes.c_double(0), ctypes.c_int(0)
+    lib.flowaux_profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
+    lib.flowaux_profile(0)
+    k_ms = tot_ms.value / max(launches.value, 1)
     value = px / (elapsed / args.steps) / 1e6
-    achieved = bpp["backward"] * px / (b_ms * 1e-3) / 1e9
+    achieved = bpp["kernel"] * px / (k_ms * 1e-3) / 1e9 if k_ms > 0 else 0.0
     out = {
         "metric": "%s fwd+bwd Mpixel/s at %d x %s; achieved HBM GB/s vs peak" % (cfg["kind"], n, shape),
         "value": round(value, 2), "unit": "Mpixel/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -161,10 +169,11 @@ def bench_flowaux(args, cfg, d):
         "config": {"workload": "%s fwd+bwd, N=%d, %s fp32 (config %d)" % (cfg["kind"], n, shape, args.config), "pixels_per_step": px},
         "whole_job": {"model_bytes_per_pixel": bpp["total"], "achieved_GBps": round(bpp["total"] * px / (elapsed / args.steps) / 1e9, 1),
                       "forward_ms": round(f_ms, 4), "backward_ms": round(b_ms, 4),
-                      "forward_GBps": round(bpp["forward"] * px / (f_ms * 1e-3) / 1e9, 1)},
+                      "forward_GBps": round(bpp["forward"] * px / (f_ms * 1e-3) / 1e9, 1),
+                      "backward_GBps": round(bpp["backward"] * px / (b_ms * 1e-3) / 1e9, 1)},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
-                     "bytes_per_launch": bpp["backward"] * px, "avg_launch_ms": round(b_ms, 5), "launches_timed": args.steps},
+                     "bytes_per_launch": bpp["kernel"] * px, "avg_launch_ms": round(k_ms, 5), "launches_timed": launches.value},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = flowaux_cpu_baseline(cfg, d)

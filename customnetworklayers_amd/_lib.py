@@ -49,10 +49,14 @@ def _load():
     lib.tgvinpaint_last_error.restype = ctypes.c_char_p
     lib.inpaint_selftest_rsqrt.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_uint]
     lib.quadfit_forward.argtypes = [_f32p] * 4 + [_int] * 5 + [ctypes.c_void_p]
-    lib.quadfit_backward.argtypes = [_f32p] * 6 + [_int] * 5 + [ctypes.c_void_p]
+    lib.quadfit_backward.argtypes = [_f32p] * 6 + [_int] * 5 + [ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p]
+    lib.quadfit_backward_workspace_bytes.argtypes = [_int] * 3
+    lib.quadfit_backward_workspace_bytes.restype = ctypes.c_longlong
     lib.medimax_forward.argtypes = [_f32p] * 2 + [_int] * 4 + [ctypes.c_void_p]
     lib.medimax_backward.argtypes = [_f32p] * 3 + [_int] * 4 + [ctypes.c_void_p]
     lib.flowaux_last_error.restype = ctypes.c_char_p
+    lib.flowaux_profile.argtypes = [_int]
+    lib.flowaux_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
     return lib
 
 

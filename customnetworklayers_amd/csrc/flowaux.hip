@@ -23,12 +23,29 @@
 //    found its median.
 #include <hip/hip_runtime.h>
 
+#include <climits>
+#include <cstdlib>
+
 #include "../../include/flowaux.h"
 #include "inpaint_common.h"
 
 namespace {
 
 using inpaint::fail;
+
+// optional timing of the dominant kernel of each backward pass (the bench switches it on)
+inpaint::KernelTimer g_timer;
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Pixels that are close in
+// the image read the same lines of the second feature map (the rows above and below, the shifted
+// segments), so the blocks are renumbered such that every XCD works through one contiguous band of
+// the pixel range.  The grid is a multiple of 8 blocks; blocks past the end return.
+__device__ __forceinline__ long long banded_pixel_index() {
+  const int per_xcd = gridDim.x >> 3;
+  const int logical_block = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  return (long long)logical_block * 256 + threadIdx.x;
+}
+inline dim3 banded_grid(long long pixels) { return dim3((unsigned)(((pixels + 255) / 256 + 7) / 8 * 8)); }
 
 // ---------------------------------------------------------------------------------------------
 // quadratic fit
@@ -40,6 +57,23 @@ struct Fit {
   int ix, iy;
   float c00, ax, ay, bx, by, fx, fy;
 };
+
+// QF.cu:75-104 == QF.cu:198-226: the two parabolas through the five costs, their validity and vertices
+__device__ __forceinline__ void finish_fit(Fit& f, float cost00, float cost0p, float costp0, float cost0m, float costm0,
+                                           int iidx, int iidy, int H, int W) {
+  f.c00 = cost00;
+  f.ax = 0.5 * (cost0p + cost0m - 2. * cost00);  // QF.cu:75-78
+  f.ay = 0.5 * (costp0 + costm0 - 2. * cost00);
+  f.bx = 0.5 * (cost0p - cost0m);
+  f.by = 0.5 * (costp0 - costm0);
+  f.validX = (f.ax < 0 && f.ax * f.ax >= 0.25 * f.bx * f.bx);  // QF.cu:83-89
+  f.validY = (f.ay < 0 && f.ay * f.ay >= 0.25 * f.by * f.by);
+  if (!(iidx < W - 1 && iidx > 0)) f.validX = 0;
+  if (!(iidy < H - 1 && iidy > 0)) f.validY = 0;
+  f.fx = f.fy = 0.f;
+  if (f.validX) f.fx = -0.5 * f.bx / f.ax;  // QF.cu:92-104
+  if (f.validY) f.fy = -0.5 * f.by / f.ay;
+}
 
 // QF.cu:22-104 (forward) == QF.cu:149-226 (backward): displaced position, the five matching
 // costs, the two parabolas and their validity.
@@ -76,17 +110,7 @@ __device__ __forceinline__ Fit fit_pixel(const float* __restrict__ a, const floa
     cost0m += I1 * qc[f.o0m];
     costm0 += I1 * qc[f.om0];
   }
-  f.c00 = cost00;
-  f.ax = 0.5 * (cost0p + cost0m - 2. * cost00);  // QF.cu:75-78
-  f.ay = 0.5 * (costp0 + costm0 - 2. * cost00);
-  f.bx = 0.5 * (cost0p - cost0m);
-  f.by = 0.5 * (costp0 - costm0);
-  f.validX = (f.ax < 0 && f.ax * f.ax >= 0.25 * f.bx * f.bx);  // QF.cu:83-89
-  f.validY = (f.ay < 0 && f.ay * f.ay >= 0.25 * f.by * f.by);
-  if (!(iidx < W - 1 && iidx > 0)) f.validX = 0;
-  if (!(iidy < H - 1 && iidy > 0)) f.validY = 0;
-  if (f.validX) f.fx = -0.5 * f.bx / f.ax;  // QF.cu:92-104
-  if (f.validY) f.fy = -0.5 * f.by / f.ay;
+  finish_fit(f, cost00, cost0p, costp0, cost0m, costm0, iidx, iidy, H, W);
   return f;
 }
 
@@ -95,7 +119,7 @@ __global__ __launch_bounds__(256) void quadfit_forward_kernel(const float* __res
                                                               const float* __restrict__ flow, float* __restrict__ out,
                                                               int N, int d, int H, int W, int fc) {
   const size_t HW = (size_t)H * W;
-  const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long t = banded_pixel_index();
   if (t >= (long long)N * HW) return;
   const int n = (int)(t / HW);
   const unsigned p = (unsigned)(t - (long long)n * HW);
@@ -117,7 +141,7 @@ __global__ __launch_bounds__(256) void quadfit_backward_kernel(const float* __re
                                                                float* __restrict__ g0, float* __restrict__ g1, int N,
                                                                int d, int H, int W, int fc) {
   const size_t HW = (size_t)H * W;
-  const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long t = banded_pixel_index();
   if (t >= (long long)N * HW) return;
   const int n = (int)(t / HW);
   const unsigned p = (unsigned)(t - (long long)n * HW);
@@ -173,6 +197,630 @@ __global__ __launch_bounds__(256) void quadfit_backward_kernel(const float* __re
       const float I2 = q[(size_t)cc * HW + f.o00];
       G0[(size_t)cc * HW + p] = I2 * dFds;
       unsafeAtomicAdd(G1 + (size_t)cc * HW + f.o00, I1 * dFds);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Quadratic fit, backward without float atomics.  Agent-scope float atomics are executed at the
+// memory side on this GPU and run two orders of magnitude below HBM speed, so the scatter into the
+// gradient of the second feature map is turned into a gather through a per-call inverse map:
+//   pass A (per source pixel)  fit, gradient wrt the first map, the five scatter coefficients of the
+//                              pixel (they do not depend on the channel) and one integer atomic that
+//                              appends the pixel to the list of its displaced position (kSlots entries
+//                              per position; what does not fit goes to an overflow list);
+//   pass B (per target pixel)  gathers, per channel, I1 * coefficient from the sources listed at the
+//                              target and at its four neighbours (a source centred on the left
+//                              neighbour reaches the target with its right tap, and so on);
+//   pass C (overflow list)     sources that found their list full scatter with float atomics after
+//                              pass B -- rare: it takes more than kSlots pixels landing on one position.
+// A tap that the image border clamps back onto the centre carries a zero coefficient (the axis is
+// not fitted at the border), so the gather leaves it out.
+// Workspace (caller provided): count[P] | overflow count, pad | slots[P*kSlots] | overflow list[P] | coef[5*P].
+// ---------------------------------------------------------------------------------------------
+constexpr int kSlots = 4;
+
+struct QfWorkspace {
+  int* count;      // sources per displaced position
+  int* ovf_count;  // one counter
+  int* slots;      // [P][kSlots] source pixel (index inside its sample)
+  int* ovf;        // global index of the sources that did not fit
+  float* coef;     // [5][P]: taps 00, 0p, 0m, p0, m0
+};
+long long qf_workspace_bytes(long long P) { return (long long)sizeof(int) * (P * (7 + kSlots) + 64 + 4); }
+QfWorkspace qf_carve(void* base, long long P) {
+  QfWorkspace w;
+  int* p = reinterpret_cast<int*>(base);
+  w.count = p;
+  w.ovf_count = p + P;
+  w.slots = p + (P + 64 + 3) / 4 * 4;  // 16-byte aligned: a position's kSlots entries are read as one int4
+  w.ovf = w.slots + P * kSlots;
+  w.coef = reinterpret_cast<float*>(w.ovf + P);
+  return w;
+}
+
+// the channel-independent factors of QF.cu:244-263,279-297 as multipliers of I1 (scatter) and I2 (g0)
+struct Factors {
+  bool any_valid;
+  double k00;
+  float k0p, k0m, kp0, km0, dFds;
+};
+__device__ __forceinline__ Factors scatter_factors(const Fit& f, const float* __restrict__ gin, size_t n, size_t HW, unsigned p) {
+  Factors k;
+  const int validX = f.validX, validY = f.validY;
+  const float ax = f.ax, ay = f.ay, fx = f.fx, fy = f.fy;
+  const float dfx_dbx = validX ? -1. / (2. * ax) : 0.;  // QF.cu:244-253
+  const float dfx_dax = validX ? -fx / ax : 0.;
+  const float dfy_dby = validY ? -1. / (2. * ay) : 0.;
+  const float dfy_day = validY ? -fy / ay : 0.;
+  const float ds_dax = validX ? fx * fx : 0.;
+  const float ds_dbx = validX ? fx : 0.;
+  const float ds_dc = (validX || validY) ? 1. : 0.;
+  const float ds_day = validY ? fy * fy : 0.;
+  const float ds_dby = validY ? fy : 0.;
+  const float dFdfx = gin[n * 3 * HW + p];  // QF.cu:261-263
+  const float dFdfy = gin[n * 3 * HW + HW + p];
+  const float dFds = gin[n * 3 * HW + 2 * HW + p];
+  k.any_valid = validX || validY;
+  k.dFds = dFds;
+  k.k00 = -2. * dFdfx * dfx_dax - 2. * dFdfy * dfy_day - 2. * dFds * ds_dax - 2. * dFds * ds_day + 2. * dFds * ds_dc;
+  k.k0p = dFdfx * dfx_dax + dFdfx * dfx_dbx + dFds * ds_dax + dFds * ds_dbx;
+  k.k0m = dFdfx * dfx_dax - dFdfx * dfx_dbx + dFds * ds_dax - dFds * ds_dbx;
+  k.kp0 = dFdfy * dfy_day + dFdfy * dfy_dby + dFds * ds_day + dFds * ds_dby;
+  k.km0 = dFdfy * dfy_day - dFdfy * dfy_dby + dFds * ds_day - dFds * ds_dby;
+  return k;
+}
+
+__global__ __launch_bounds__(256) void quadfit_backward_sources(const float* __restrict__ im0, const float* __restrict__ im1,
+                                                                const float* __restrict__ flow, const float* __restrict__ gin,
+                                                                float* __restrict__ g0, QfWorkspace ws, int N, int d, int H,
+                                                                int W, int fc) {
+  const size_t HW = (size_t)H * W;
+  const long long P = (long long)N * HW;
+  const long long t = banded_pixel_index();
+  if (t >= P) return;
+  const int n = (int)(t / HW);
+  const unsigned p = (unsigned)(t - (long long)n * HW);
+  const int h = p / W, w = p - h * W;
+  const float* a = im0 + (size_t)n * d * HW;
+  const float* q = im1 + (size_t)n * d * HW;
+  float* G0 = g0 + (size_t)n * d * HW;
+  const Fit f = fit_pixel(a, q, flow + (size_t)n * fc * HW, d, H, W, HW, h, w);
+  if (!f.inside) {
+    for (int cc = 0; cc < d; cc++) G0[(size_t)cc * HW + p] = 0.f;
+    return;
+  }
+  const Factors k = scatter_factors(f, gin, n, HW, p);
+  // scatter coefficients: contribution to g1 at a tap = I1 * coefficient (QF.cu:279-283,296)
+  ws.coef[0 * P + t] = k.any_valid ? (float)(0.5 * k.k00) : k.dFds;
+  ws.coef[1 * P + t] = k.any_valid ? 0.5f * k.k0p : 0.f;
+  ws.coef[2 * P + t] = k.any_valid ? 0.5f * k.k0m : 0.f;
+  ws.coef[3 * P + t] = k.any_valid ? 0.5f * k.kp0 : 0.f;
+  ws.coef[4 * P + t] = k.any_valid ? 0.5f * k.km0 : 0.f;
+  const long long centre = (long long)n * HW + f.o00;
+  const int pos = atomicAdd(ws.count + centre, 1);
+  if (pos < kSlots) ws.slots[centre * kSlots + pos] = (int)p;
+  else ws.ovf[atomicAdd(ws.ovf_count, 1)] = (int)t;
+  if (k.any_valid) {
+#pragma unroll 4
+    for (int cc = 0; cc < d; cc++) {  // QF.cu:286-290
+      const float* qc = q + (size_t)cc * HW;
+      const float I2 = qc[f.o00], I2_0p = qc[f.o0p], I2_0m = qc[f.o0m], I2_p0 = qc[f.op0], I2_m0 = qc[f.om0];
+      G0[(size_t)cc * HW + p] = 0.5 * (I2 * k.k00 + I2_0p * k.k0p + I2_0m * k.k0m + I2_p0 * k.kp0 + I2_m0 * k.km0);
+    }
+  } else {
+#pragma unroll 4
+    for (int cc = 0; cc < d; cc++) G0[(size_t)cc * HW + p] = q[(size_t)cc * HW + f.o00] * k.dFds;  // QF.cu:295
+  }
+}
+
+__global__ __launch_bounds__(256) void quadfit_backward_gather(const float* __restrict__ im0, float* __restrict__ g1,
+                                                               QfWorkspace ws, int N, int d, int H, int W) {
+  const size_t HW = (size_t)H * W;
+  const long long P = (long long)N * HW;
+  const long long t = banded_pixel_index();
+  if (t >= P) return;
+  const int n = (int)(t / HW);
+  const unsigned p = (unsigned)(t - (long long)n * HW);
+  const int h = p / W, w = p - h * W;
+  const long long base = (long long)n * HW;
+  const float* a = im0 + (size_t)n * d * HW;
+  float* G1 = g1 + (size_t)n * d * HW + p;
+  // (position whose sources reach this pixel, tap they reach it with); -1: outside the image
+  long long ctr[5];
+  ctr[0] = base + p;
+  ctr[1] = w > 0 ? base + p - 1 : -1;      // right tap of the left neighbour
+  ctr[2] = w < W - 1 ? base + p + 1 : -1;  // left tap of the right neighbour
+  ctr[3] = h > 0 ? base + p - W : -1;      // lower tap of the upper neighbour
+  ctr[4] = h < H - 1 ? base + p + W : -1;  // upper tap of the lower neighbour
+  // compact list of the (source, coefficient) pairs that reach this pixel, in registers
+  constexpr int kPairs = 8;
+  unsigned src[kPairs];
+  float cf[kPairs];
+#pragma unroll
+  for (int j = 0; j < kPairs; j++) {
+    src[j] = p;
+    cf[j] = 0.f;
+  }
+  int cnt[5];
+  int np = 0;
+#pragma unroll
+  for (int k = 0; k < 5; k++) {
+    cnt[k] = ctr[k] >= 0 ? min(ws.count[ctr[k]], kSlots) : 0;
+#pragma unroll
+    for (int i = 0; i < kSlots; i++) {
+      if (i < cnt[k]) {
+        const unsigned sidx = (unsigned)ws.slots[ctr[k] * kSlots + i];
+        const float c = ws.coef[(long long)k * P + base + sidx];
+#pragma unroll
+        for (int j = 0; j < kPairs; j++)
+          if (np == j) {
+            src[j] = sidx;
+            cf[j] = c;
+          }
+        np++;
+      }
+    }
+  }
+  // longest list among the wavefront's active lanes: the unrolled gathers beyond it are skipped by a uniform branch
+  unsigned need = 0;
+#pragma unroll
+  for (int j = 0; j < kPairs; j++)
+    if (__ballot(np > j) != 0) need |= 1u << j;
+  if (np <= kPairs) {
+    for (int cc = 0; cc < d; cc++) {
+      const float* ac = a + (size_t)cc * HW;
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < kPairs; j++)
+        if (need & (1u << j)) acc += ac[src[j]] * cf[j];
+      G1[(size_t)cc * HW] = acc;
+    }
+    return;
+  }
+  for (int cc = 0; cc < d; cc++) {  // more pairs than registers: walk the lists per channel
+    const float* ac = a + (size_t)cc * HW;
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < 5; k++)
+      for (int i = 0; i < cnt[k]; i++) {
+        const unsigned sidx = (unsigned)ws.slots[ctr[k] * kSlots + i];
+        acc += ac[sidx] * ws.coef[(long long)k * P + base + sidx];
+      }
+    G1[(size_t)cc * HW] = acc;
+  }
+}
+
+// sources whose list was full: float atomics, after the gather has written g1
+__global__ __launch_bounds__(256) void quadfit_backward_overflow(const float* __restrict__ im0, const float* __restrict__ flow,
+                                                                 float* __restrict__ g1, QfWorkspace ws, int N, int d, int H,
+                                                                 int W, int fc) {
+  const size_t HW = (size_t)H * W;
+  const long long P = (long long)N * HW;
+  const long long total = (long long)*ws.ovf_count * d;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
+    const int e = (int)(i / d), cc = (int)(i - (long long)e * d);  // one lane per (source, channel)
+    const long long t = ws.ovf[e];
+    const int n = (int)(t / HW);
+    const unsigned p = (unsigned)(t - (long long)n * HW);
+    const int h = p / W, w = p - h * W;
+    const float* fl = flow + (size_t)n * fc * HW;
+    const float idx = w + fl[p], idy = h + fl[HW + p];  // QF.cu:31-32,47-53 (the pixel is inside the image)
+    const int iidx = (int)floor(idx + 0.5), iidy = (int)floor(idy + 0.5);
+    const unsigned o[5] = {(unsigned)iidy * W + iidx, (unsigned)iidy * W + min(iidx + 1, W - 1),
+                           (unsigned)iidy * W + max(iidx - 1, 0), (unsigned)min(iidy + 1, H - 1) * W + iidx,
+                           (unsigned)max(iidy - 1, 0) * W + iidx};
+    const float I1 = im0[((size_t)n * d + cc) * HW + p];
+    float* gc = g1 + ((size_t)n * d + cc) * HW;
+#pragma unroll
+    for (int k = 0; k < 5; k++) {
+      const float cf = ws.coef[(long long)k * P + t];
+      if (cf != 0.f) unsafeAtomicAdd(gc + o[k], I1 * cf);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tiled kernels.  A lane that reads its five taps straight from memory issues gathers whose
+// addresses follow the (jittery) flow; the vector L1 then handles them almost lane by lane and
+// becomes the bound.  Here a block owns a 64 x 16 tile of pixels (4 rows per lane), finds the
+// bounding box of all taps of the tile, and per channel stages that window of the second feature
+// map in LDS with row-wise coalesced loads (double buffered: the next channel's window is in flight
+// while the taps of the current one are read from LDS).  A pixel whose taps do not fit the window's
+// capacity reads them from memory as before.
+// ---------------------------------------------------------------------------------------------
+constexpr int kTW = 64;  // tile width: one pixel column per lane
+constexpr int kMaxWinW = 128;  // widest window
+template <int PX>              // PX pixels per lane (rows PX * wave + i): tile height, window capacity in floats
+struct TileCfg {
+  static constexpr int TH = 4 * PX, ELEMS = 96 * (4 * PX + 16);
+};
+constexpr int kChannelsPerStep = 1;
+constexpr int kPxForward = 2, kPxSources = 2;
+
+struct Box {
+  int x0, y0, w, h;
+};
+struct TilePx {
+  bool inside, far;
+  int ix, iy, xm, xp, ym, yp;
+  unsigned p;     // the pixel's offset inside a channel plane
+  unsigned o[5];  // taps 00, 0p, 0m, p0, m0: offsets into the window, or into the plane when far
+};
+
+// QF.cu:31-53: displaced position and tap coordinates of pixel (x, y); widens the tile's bounding box
+__device__ __forceinline__ void locate(TilePx& s, const float* __restrict__ fl, size_t HW, int H, int W, int x, int y,
+                                       bool valid, int& minx, int& maxx, int& miny, int& maxy) {
+  s.inside = s.far = false;
+  s.ix = s.iy = s.xm = s.xp = s.ym = s.yp = 0;
+  s.p = valid ? (unsigned)y * W + x : 0u;
+  if (!valid) return;
+  const float idx = x + fl[s.p];
+  const float idy = y + fl[HW + s.p];
+  if (idx > W - 1 || idx < 0 || idy > H - 1 || idy < 0) return;
+  s.inside = true;
+  s.ix = (int)floor(idx + 0.5);
+  s.iy = (int)floor(idy + 0.5);
+  s.xm = max(s.ix - 1, 0); s.ym = max(s.iy - 1, 0);
+  s.xp = min(s.ix + 1, W - 1); s.yp = min(s.iy + 1, H - 1);
+  minx = min(minx, s.xm); maxx = max(maxx, s.xp);
+  miny = min(miny, s.ym); maxy = max(maxy, s.yp);
+}
+
+__device__ __forceinline__ Box block_box(int minx, int maxx, int miny, int maxy, int* red, int capacity) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    minx = min(minx, __shfl_xor(minx, o));
+    maxx = max(maxx, __shfl_xor(maxx, o));
+    miny = min(miny, __shfl_xor(miny, o));
+    maxy = max(maxy, __shfl_xor(maxy, o));
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    red[wave * 4 + 0] = minx; red[wave * 4 + 1] = maxx; red[wave * 4 + 2] = miny; red[wave * 4 + 3] = maxy;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    minx = min(minx, red[k * 4 + 0]); maxx = max(maxx, red[k * 4 + 1]);
+    miny = min(miny, red[k * 4 + 2]); maxy = max(maxy, red[k * 4 + 3]);
+  }
+  Box b{0, 0, 0, 0};
+  if (maxx >= minx) {
+    b.x0 = minx; b.y0 = miny;
+    b.w = min(maxx - minx + 1, kMaxWinW);
+    b.h = min(maxy - miny + 1, capacity / b.w);
+  }
+  return b;
+}
+
+__device__ __forceinline__ void place(TilePx& s, const Box& b, int W) {
+  if (!s.inside) return;
+  s.far = !(s.xp - b.x0 < b.w && s.yp - b.y0 < b.h);
+  if (s.far) {
+    s.o[0] = (unsigned)s.iy * W + s.ix; s.o[1] = (unsigned)s.iy * W + s.xp; s.o[2] = (unsigned)s.iy * W + s.xm;
+    s.o[3] = (unsigned)s.yp * W + s.ix; s.o[4] = (unsigned)s.ym * W + s.ix;
+  } else {
+    const int cx = s.ix - b.x0, cy = s.iy - b.y0;
+    s.o[0] = cy * b.w + cx; s.o[1] = cy * b.w + (s.xp - b.x0); s.o[2] = cy * b.w + (s.xm - b.x0);
+    s.o[3] = (s.yp - b.y0) * b.w + cx; s.o[4] = (s.ym - b.y0) * b.w + cx;
+  }
+}
+
+// CH channels per step: stage the windows of planes q[cc .. cc+CH) in LDS (dense, pitch box.w), then
+// consume(cc, window, plane) for each of them.  The next step's windows are in flight meanwhile.
+template <int PX, int CH, typename Consume>
+__device__ __forceinline__ void window_pass(const float* __restrict__ q, int d, size_t HW, int W, const Box& box,
+                                            float (*win)[CH][TileCfg<PX>::ELEMS], Consume consume) {
+  constexpr int kPer = (TileCfg<PX>::ELEMS + 255) / 256;
+  const int count = box.w * box.h;
+  // window elements of this thread: e = threadIdx.x + 256 k, row e / w, column e % w (exact in float for these sizes)
+  unsigned goff[kPer];
+  const float inv_w = 1.0f / (float)max(box.w, 1);
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    const int e = threadIdx.x + 256 * k;
+    const int r = (int)(((float)e + 0.5f) * inv_w);
+    goff[k] = (unsigned)(r * W + (e - r * box.w));
+  }
+  float regs[CH][kPer];
+  auto fetch = [&](int c0) {
+#pragma unroll
+    for (int ch = 0; ch < CH; ch++) {
+      if (c0 + ch < d) {
+        const float* src = q + (size_t)(c0 + ch) * HW + (size_t)box.y0 * W + box.x0;
+#pragma unroll
+        for (int k = 0; k < kPer; k++)
+          if ((int)threadIdx.x + 256 * k < count) regs[ch][k] = src[goff[k]];
+      }
+    }
+  };
+  auto stash = [&](int c0, float (*buf)[TileCfg<PX>::ELEMS]) {
+#pragma unroll
+    for (int ch = 0; ch < CH; ch++) {
+      if (c0 + ch < d) {
+#pragma unroll
+        for (int k = 0; k < kPer; k++)
+          if ((int)threadIdx.x + 256 * k < count) buf[ch][threadIdx.x + 256 * k] = regs[ch][k];
+      }
+    }
+  };
+  fetch(0);
+  stash(0, win[0]);
+  __syncthreads();
+  int parity = 0;
+  for (int c0 = 0; c0 < d; c0 += CH) {
+    if (c0 + CH < d) fetch(c0 + CH);
+#pragma unroll
+    for (int ch = 0; ch < CH; ch++)
+      if (c0 + ch < d) consume(c0 + ch, win[parity][ch], q + (size_t)(c0 + ch) * HW);
+    if (c0 + CH < d) stash(c0 + CH, win[parity ^ 1]);
+    parity ^= 1;
+    __syncthreads();
+  }
+}
+
+// the five taps of every inside pixel of the lane, from the window or (far pixels) from the plane
+template <int PX, typename Body>
+__device__ __forceinline__ void each_pixel_taps(const TilePx (&px)[PX], const float* buf, const float* plane, Body body) {
+#pragma unroll
+  for (int i = 0; i < PX; i++) {
+    if (px[i].inside) {
+      float t[5];
+      if (!px[i].far) {
+#pragma unroll
+        for (int k = 0; k < 5; k++) t[k] = buf[px[i].o[k]];
+      } else {
+#pragma unroll
+        for (int k = 0; k < 5; k++) t[k] = plane[px[i].o[k]];
+      }
+      body(i, t);
+    }
+  }
+}
+
+// decode the block's tile (XCD-banded numbering); false: the block has no tile
+__device__ __forceinline__ bool tile_of_block(int N, int tiles_x, int tiles_y, int& n, int& tx, int& ty) {
+  const int per_xcd = gridDim.x >> 3;
+  const int lb = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int tiles = tiles_x * tiles_y;
+  if (lb >= N * tiles) return false;
+  n = lb / tiles;
+  const int r = lb - n * tiles;
+  ty = r / tiles_x;
+  tx = r - ty * tiles_x;
+  return true;
+}
+
+// MODE 0: the forward pass (QF.cu:14-139).  MODE 1: pass A of the backward pass (fit, g0, coefficients, lists).
+template <int MODE, int PX>
+__global__ __launch_bounds__(256) void quadfit_tiles(const float* __restrict__ im0, const float* __restrict__ im1,
+                                                     const float* __restrict__ flow, const float* __restrict__ gin,
+                                                     float* __restrict__ res, QfWorkspace ws, int N, int d, int H, int W,
+                                                     int fc, int tiles_x, int tiles_y) {
+  constexpr int kPX = PX, kTH = TileCfg<PX>::TH, CH = kChannelsPerStep;
+  __shared__ float win[2][CH][TileCfg<PX>::ELEMS];
+  __shared__ int red[16];
+  int n, tx, ty;
+  if (!tile_of_block(N, tiles_x, tiles_y, n, tx, ty)) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t HW = (size_t)H * W;
+  const long long P = (long long)N * HW;
+  const float* a = im0 + (size_t)n * d * HW;
+  const float* q = im1 + (size_t)n * d * HW;
+  const float* fl = flow + (size_t)n * fc * HW;
+  const int x = tx * kTW + lane;
+  TilePx px[kPX];
+  bool valid[kPX];
+  int minx = INT_MAX, maxx = INT_MIN, miny = INT_MAX, maxy = INT_MIN;
+#pragma unroll
+  for (int i = 0; i < kPX; i++) {
+    const int y = ty * kTH + wave * kPX + i;
+    valid[i] = x < W && y < H;
+    locate(px[i], fl, HW, H, W, x, y, valid[i], minx, maxx, miny, maxy);
+  }
+  const Box box = block_box(minx, maxx, miny, maxy, red, TileCfg<PX>::ELEMS);
+#pragma unroll
+  for (int i = 0; i < kPX; i++) place(px[i], box, W);
+
+  float cost[kPX][5];
+#pragma unroll
+  for (int i = 0; i < kPX; i++)
+#pragma unroll
+    for (int k = 0; k < 5; k++) cost[i][k] = 0.f;
+  window_pass<PX, CH>(q, d, HW, W, box, win, [&](int cc, const float* buf, const float* plane) {
+    each_pixel_taps<PX>(px, buf, plane, [&](int i, const float (&t)[5]) {  // QF.cu:63-71
+      const float I1 = a[(size_t)cc * HW + px[i].p];
+#pragma unroll
+      for (int k = 0; k < 5; k++) cost[i][k] += I1 * t[k];
+    });
+  });
+
+  Fit f[kPX];
+#pragma unroll
+  for (int i = 0; i < kPX; i++) {
+    f[i].inside = px[i].inside;
+    f[i].validX = f[i].validY = 0;
+    f[i].c00 = f[i].ax = f[i].ay = f[i].bx = f[i].by = f[i].fx = f[i].fy = 0.f;
+    if (px[i].inside) finish_fit(f[i], cost[i][0], cost[i][1], cost[i][3], cost[i][2], cost[i][4], px[i].ix, px[i].iy, H, W);
+  }
+  if (MODE == 0) {
+#pragma unroll
+    for (int i = 0; i < kPX; i++) {
+      if (!valid[i]) continue;
+      float* o = res + (size_t)n * 3 * HW + px[i].p;
+      float score = 0.f;
+      if (f[i].inside)  // QF.cu:136
+        score = f[i].ax * f[i].fx * f[i].fx + f[i].bx * f[i].fx + f[i].c00 + f[i].ay * f[i].fy * f[i].fy + f[i].by * f[i].fy;
+      o[0] = f[i].fx;
+      o[HW] = f[i].fy;
+      o[2 * HW] = score;
+    }
+    return;
+  }
+  float* G0 = res + (size_t)n * d * HW;
+  Factors k[kPX];
+#pragma unroll
+  for (int i = 0; i < kPX; i++) {
+    k[i].any_valid = false;
+    k[i].k00 = 0.;
+    k[i].k0p = k[i].k0m = k[i].kp0 = k[i].km0 = k[i].dFds = 0.f;
+    if (valid[i] && !px[i].inside)
+      for (int cc = 0; cc < d; cc++) G0[(size_t)cc * HW + px[i].p] = 0.f;
+    if (!px[i].inside) continue;
+    k[i] = scatter_factors(f[i], gin, n, HW, px[i].p);
+    const long long t = (long long)n * HW + px[i].p;
+    ws.coef[0 * P + t] = k[i].any_valid ? (float)(0.5 * k[i].k00) : k[i].dFds;  // QF.cu:279-283,296
+    ws.coef[1 * P + t] = k[i].any_valid ? 0.5f * k[i].k0p : 0.f;
+    ws.coef[2 * P + t] = k[i].any_valid ? 0.5f * k[i].k0m : 0.f;
+    ws.coef[3 * P + t] = k[i].any_valid ? 0.5f * k[i].kp0 : 0.f;
+    ws.coef[4 * P + t] = k[i].any_valid ? 0.5f * k[i].km0 : 0.f;
+    const long long centre = (long long)n * HW + (long long)px[i].iy * W + px[i].ix;
+    const int pos = atomicAdd(ws.count + centre, 1);
+    if (pos < kSlots) ws.slots[centre * kSlots + pos] = (int)px[i].p;
+    else ws.ovf[atomicAdd(ws.ovf_count, 1)] = (int)t;
+  }
+  window_pass<PX, CH>(q, d, HW, W, box, win, [&](int cc, const float* buf, const float* plane) {
+    each_pixel_taps<PX>(px, buf, plane, [&](int i, const float (&t)[5]) {
+      float g;
+      if (k[i].any_valid)  // QF.cu:286-290
+        g = 0.5 * (t[0] * k[i].k00 + t[1] * k[i].k0p + t[2] * k[i].k0m + t[3] * k[i].kp0 + t[4] * k[i].km0);
+      else  // QF.cu:295
+        g = t[0] * k[i].dFds;
+      G0[(size_t)cc * HW + px[i].p] = g;
+    });
+  });
+}
+
+// Pass B of the backward pass on tiles of target pixels: the (source, coefficient) pairs of every pixel are
+// collected once; per channel the window of the FIRST feature map that covers the tile's sources is
+// staged in LDS and the pairs are summed from it.
+constexpr int kPairs = 12;
+constexpr int kPxGather = 2;
+
+template <int PX>
+__global__ __launch_bounds__(256) void quadfit_gather_tiles(const float* __restrict__ im0, float* __restrict__ g1, QfWorkspace ws,
+                                                            int N, int d, int H, int W, int tiles_x, int tiles_y) {
+  constexpr int kTH = TileCfg<PX>::TH, CH = kChannelsPerStep;
+  __shared__ float win[2][CH][TileCfg<PX>::ELEMS];
+  __shared__ int red[16];
+  int n, tx, ty;
+  if (!tile_of_block(N, tiles_x, tiles_y, n, tx, ty)) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t HW = (size_t)H * W;
+  const long long P = (long long)N * HW, base = (long long)n * HW;
+  const float* a = im0 + (size_t)n * d * HW;
+  float* G1 = g1 + (size_t)n * d * HW;
+  const int x = tx * kTW + lane;
+  const float inv_w = 1.0f / (float)W;
+  bool valid[PX];
+  unsigned pix[PX];
+  int np[PX];
+  unsigned off[PX][kPairs];  // packed (y << 16 | x) of the source, then its offset in the window
+  float cf[PX][kPairs];
+  int minx = INT_MAX, maxx = INT_MIN, miny = INT_MAX, maxy = INT_MIN;
+#pragma unroll
+  for (int i = 0; i < PX; i++) {
+    const int y = ty * kTH + wave * PX + i;
+    valid[i] = x < W && y < H;
+    pix[i] = valid[i] ? (unsigned)y * W + x : 0u;
+    np[i] = 0;
+#pragma unroll
+    for (int j = 0; j < kPairs; j++) {
+      off[i][j] = 0u;
+      cf[i][j] = 0.f;
+    }
+    if (!valid[i]) continue;
+    // (position whose sources reach this pixel, tap they reach it with); -1: outside the image
+    long long ctr[5];
+    ctr[0] = base + pix[i];
+    ctr[1] = x > 0 ? base + pix[i] - 1 : -1;      // right tap of the left neighbour
+    ctr[2] = x < W - 1 ? base + pix[i] + 1 : -1;  // left tap of the right neighbour
+    ctr[3] = y > 0 ? base + pix[i] - W : -1;      // lower tap of the upper neighbour
+    ctr[4] = y < H - 1 ? base + pix[i] + W : -1;  // upper tap of the lower neighbour
+#pragma unroll
+    for (int k = 0; k < 5; k++) {
+      const int cnt = ctr[k] >= 0 ? min(ws.count[ctr[k]], kSlots) : 0;
+      int4 sl = make_int4(0, 0, 0, 0);
+      if (cnt > 0) sl = *reinterpret_cast<const int4*>(ws.slots + ctr[k] * kSlots);
+      const int sv[4] = {sl.x, sl.y, sl.z, sl.w};
+#pragma unroll
+      for (int s = 0; s < kSlots; s++) {
+        if (s < cnt) {
+          const unsigned sp = (unsigned)sv[s];  // source pixel, offset in its plane (below 2^24: the float quotient is off by one at most)
+          int sy = (int)((float)sp * inv_w), sx = (int)sp - sy * W;
+          if (sx < 0) { sy--; sx += W; }
+          if (sx >= W) { sy++; sx -= W; }
+          const float c = ws.coef[(long long)k * P + base + sp];
+#pragma unroll
+          for (int j = 0; j < kPairs; j++)
+            if (np[i] == j) {
+              off[i][j] = ((unsigned)sy << 16) | (unsigned)sx;
+              cf[i][j] = c;
+            }
+          if (np[i] < kPairs) {
+            minx = min(minx, sx); maxx = max(maxx, sx);
+            miny = min(miny, sy); maxy = max(maxy, sy);
+          }
+          np[i]++;
+        }
+      }
+    }
+  }
+  const Box box = block_box(minx, maxx, miny, maxy, red, TileCfg<PX>::ELEMS);
+  // a pixel with more pairs than registers, or with a source outside the window, walks its lists from memory instead
+  bool slow[PX];
+  unsigned need = 0;
+#pragma unroll
+  for (int i = 0; i < PX; i++) {
+    slow[i] = np[i] > kPairs;
+#pragma unroll
+    for (int j = 0; j < kPairs; j++) {
+      const int sx = off[i][j] & 0xffff, sy = off[i][j] >> 16;
+      const bool used = j < np[i];
+      if (used && !(sx - box.x0 < box.w && sy - box.y0 < box.h)) slow[i] = true;
+      off[i][j] = used ? (unsigned)((sy - box.y0) * box.w + (sx - box.x0)) : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < kPairs; j++) {
+      if (slow[i]) {
+        off[i][j] = 0u;
+        cf[i][j] = 0.f;
+      }
+      if (__ballot(!slow[i] && j < np[i]) != 0) need |= 1u << j;  // pairs nobody in the wavefront has are skipped by a uniform branch
+    }
+  }
+  window_pass<PX, CH>(a, d, HW, W, box, win, [&](int cc, const float* buf, const float* plane) {
+#pragma unroll
+    for (int i = 0; i < PX; i++) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < kPairs; j++)
+        if (need & (1u << j)) acc = __builtin_fmaf(buf[off[i][j]], cf[i][j], acc);
+      if (valid[i] && !slow[i]) G1[(size_t)cc * HW + pix[i]] = acc;
+    }
+  });
+#pragma unroll
+  for (int i = 0; i < PX; i++) {
+    if (!valid[i] || !slow[i]) continue;
+    const int y = ty * kTH + wave * PX + i;
+    long long ctr[5];
+    ctr[0] = base + pix[i];
+    ctr[1] = x > 0 ? base + pix[i] - 1 : -1;
+    ctr[2] = x < W - 1 ? base + pix[i] + 1 : -1;
+    ctr[3] = y > 0 ? base + pix[i] - W : -1;
+    ctr[4] = y < H - 1 ? base + pix[i] + W : -1;
+    for (int cc = 0; cc < d; cc++) {
+      const float* ac = a + (size_t)cc * HW;
+      float acc = 0.f;
+      for (int k = 0; k < 5; k++) {
+        const int cnt = ctr[k] >= 0 ? min(ws.count[ctr[k]], kSlots) : 0;
+        for (int s = 0; s < cnt; s++) {
+          const unsigned sp = (unsigned)ws.slots[ctr[k] * kSlots + s];
+          acc += ac[sp] * ws.coef[(long long)k * P + base + sp];
+        }
+      }
+      G1[(size_t)cc * HW + pix[i]] = acc;
     }
   }
 }
@@ -299,11 +947,135 @@ __global__ __launch_bounds__(256) void median_backward_kernel(const float* __res
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Median, whole histograms in LDS (up to 255 bins): the histograms of 64 consecutive pixels are one
+// contiguous run of 64*D floats, staged with 16-byte loads into rows of odd pitch; each lane walks its
+// row; the backward pass writes the gradients over the row and the run goes back out the same way.
+// HBM sees the histogram once per pass.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxRowBins = 255;
+
+template <int VEC, bool OUT>
+__device__ __forceinline__ void stage_rows(const float* __restrict__ src, float* __restrict__ dst, float* tile, int total,
+                                           int D, int Dp, int lane) {
+  constexpr int kStep = 64 * VEC;
+  const int qs = kStep / D, rs = kStep - qs * D;
+  int i = lane * VEC;
+  int px = i / D, b = i - px * D;
+  for (; i < total; i += kStep) {
+    if (VEC == 4 && i + 3 < total) {
+      float4 v;
+      if (!OUT) v = *reinterpret_cast<const float4*>(src + i);
+      float* e[4];
+      int pe = px, be = b;
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        e[k] = tile + pe * Dp + be;
+        if (++be >= D) { be = 0; pe++; }
+      }
+      if (OUT) {
+        v.x = *e[0]; v.y = *e[1]; v.z = *e[2]; v.w = *e[3];
+        *reinterpret_cast<float4*>(dst + i) = v;
+      } else {
+        *e[0] = v.x; *e[1] = v.y; *e[2] = v.z; *e[3] = v.w;
+      }
+    } else {
+      int pe = px, be = b;
+      for (int k = 0; k < VEC && i + k < total; k++) {
+        if (OUT) dst[i + k] = tile[pe * Dp + be];
+        else tile[pe * Dp + be] = src[i + k];
+        if (++be >= D) { be = 0; pe++; }
+      }
+    }
+    b += rs;
+    px += qs;
+    if (b >= D) { b -= D; px++; }
+  }
+}
+
+template <int VEC, bool BACKWARD>
+__global__ __launch_bounds__(64) void median_rows_kernel(const float* __restrict__ vol, const float* __restrict__ gin,
+                                                         float* __restrict__ res, long long P, long long HW, int D, int Dp) {
+  extern __shared__ float tile[];  // 64 rows of pitch Dp
+  const int lane = threadIdx.x;
+  const long long p0 = (long long)blockIdx.x * 64;
+  const int npx = (int)min((long long)64, P - p0);
+  const int total = npx * D;
+  stage_rows<VEC, false>(vol + p0 * D, nullptr, tile, total, D, Dp, lane);
+  __syncthreads();
+  float* row = tile + lane * Dp;
+  // the walk of MM.cu:26-43 == MM.cu:59-75, without the early exit (the bins past the crossing are skipped by `found`)
+  bool found = false;
+  int cidx = 0;
+  float score = 0.f, pmid = 1.f, alpha = 0.f;
+  if (lane < npx) {
+    for (int c = 0; c < D; c++) {
+      const float cScore = row[c];
+      const bool hit = !found && score < 0.5 && score + cScore >= 0.5;
+      if (hit) {
+        alpha = (1. - 2. * score - cScore) / (2. * cScore);  // MM.cu:34
+        pmid = cScore;
+        cidx = c;
+        found = true;
+      }
+      if (!found) score = score + cScore;
+    }
+  }
+  const long long p = p0 + lane;
+  const long long n = p / HW, q = p - n * HW;
+  if (!BACKWARD) {
+    if (lane < npx) {
+      res[n * 2 * HW + q] = found ? (float)cidx - 0.f + alpha : 0.f;  // MM.cu:35
+      res[n * 2 * HW + HW + q] = found ? pmid : 0.f;
+    }
+    return;
+  }
+  if (lane < npx) {
+    const float g0v = gin[n * 2 * HW + q], g1v = gin[n * 2 * HW + HW + q];
+    const float cross = g0v * alpha / (-pmid) + g1v;  // MM.cu:69
+    const float neg = -g0v / (2. * pmid);             // MM.cu:85
+    const float pos = +g0v / (2. * pmid);             // MM.cu:88
+    score = 0.f;
+    for (int c = 0; c < D; c++) {  // MM.cu:77-92; the crossing bin keeps the value of MM.cu:69
+      const float cScore = row[c];
+      float g = (found && c == cidx) ? cross : 0.f;
+      if (score + cScore < 0.5) g = neg;
+      else if (score >= 0.5) g = pos;
+      row[c] = g;
+      score = score + cScore;
+    }
+  }
+  __syncthreads();
+  stage_rows<VEC, true>(nullptr, res + p0 * D, tile, total, D, Dp, lane);
+}
+
+template <bool BACKWARD>
+void launch_median_rows(const float* vol, const float* gin, float* res, long long P, long long HW, int D, bool aligned,
+                        hipStream_t stream) {
+  const int Dp = D | 1;
+  const dim3 grid((unsigned)((P + 63) / 64)), block(64);
+  const size_t lds = (size_t)64 * Dp * sizeof(float);
+  if (aligned && D >= 4)
+    hipLaunchKernelGGL((median_rows_kernel<4, BACKWARD>), grid, block, lds, stream, vol, gin, res, P, HW, D, Dp);
+  else
+    hipLaunchKernelGGL((median_rows_kernel<1, BACKWARD>), grid, block, lds, stream, vol, gin, res, P, HW, D, Dp);
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
 }  // namespace
 
 extern "C" {
 
 const char* flowaux_last_error(void) { return inpaint::error_buffer(); }
+
+int flowaux_profile(int enable) {
+  g_timer.enabled = enable != 0;
+  g_timer.reset();
+  return 0;
+}
+
+int flowaux_profile_read(double* total_ms, int* launches) { return g_timer.read(total_ms, launches); }
 
 int quadfit_forward(const float* im0, const float* im1, const float* flow, float* out, int n, int ic, int ih, int iw,
                     int flow_channels, void* stream) {
@@ -312,22 +1084,67 @@ int quadfit_forward(const float* im0, const float* im1, const float* flow, float
   if (flow_channels < 2) return fail(INPAINT_ERR_ARG, "quadfit_forward: the flow needs at least 2 channels, got %d", flow_channels);
   if ((long long)ih * iw >= (1ll << 31)) return fail(INPAINT_ERR_ARG, "quadfit_forward: image too large");
   const long long P = (long long)n * ih * iw;
-  hipLaunchKernelGGL(quadfit_forward_kernel, dim3((unsigned)((P + 255) / 256)), dim3(256), 0, (hipStream_t)stream, im0, im1,
-                     flow, out, n, ic, ih, iw, flow_channels);
+  const int tiles_x = (iw + kTW - 1) / kTW, tiles_y = (ih + TileCfg<kPxForward>::TH - 1) / TileCfg<kPxForward>::TH;
+  const long long tiles = (long long)n * tiles_x * tiles_y;
+  if (tiles >= (1ll << 31) - 8) return fail(INPAINT_ERR_ARG, "quadfit_forward: too many tiles");
+  if (getenv("INPAINT_QUADFIT_PATH") && strcmp(getenv("INPAINT_QUADFIT_PATH"), "px") == 0)
+    hipLaunchKernelGGL(quadfit_forward_kernel, banded_grid(P), dim3(256), 0, (hipStream_t)stream, im0, im1, flow, out, n,
+                       ic, ih, iw, flow_channels);
+  else
+    hipLaunchKernelGGL((quadfit_tiles<0, kPxForward>), dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), 0, (hipStream_t)stream, im0, im1,
+                       flow, nullptr, out, QfWorkspace{}, n, ic, ih, iw, flow_channels, tiles_x, tiles_y);
   INPAINT_HIP(hipGetLastError());
   return 0;
 }
 
+long long quadfit_backward_workspace_bytes(int n, int ih, int iw) {
+  if (n < 1 || ih < 1 || iw < 1) return 0;
+  return qf_workspace_bytes((long long)n * ih * iw);
+}
+
 int quadfit_backward(const float* im0, const float* im1, const float* flow, const float* gin, float* g0, float* g1, int n,
-                     int ic, int ih, int iw, int flow_channels, void* stream) {
+                     int ic, int ih, int iw, int flow_channels, void* workspace, long long workspace_bytes, void* stream) {
   if (!im0 || !im1 || !flow || !gin || !g0 || !g1) return fail(INPAINT_ERR_ARG, "quadfit_backward: null pointer");
   if (n < 1 || ic < 1 || ih < 1 || iw < 1) return fail(INPAINT_ERR_ARG, "quadfit_backward: bad shape %dx%dx%dx%d", n, ic, ih, iw);
   if (flow_channels < 2) return fail(INPAINT_ERR_ARG, "quadfit_backward: the flow needs at least 2 channels, got %d", flow_channels);
   if ((long long)ih * iw >= (1ll << 31)) return fail(INPAINT_ERR_ARG, "quadfit_backward: image too large");
   const long long P = (long long)n * ih * iw, total = P * ic;
-  hipLaunchKernelGGL(inpaint::fill_zero_f32, dim3(inpaint::grid_stride(total)), dim3(256), 0, (hipStream_t)stream, g1, total);
-  hipLaunchKernelGGL(quadfit_backward_kernel, dim3((unsigned)((P + 255) / 256)), dim3(256), 0, (hipStream_t)stream, im0, im1,
-                     flow, gin, g0, g1, n, ic, ih, iw, flow_channels);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid = banded_grid(P), block(256);
+  if (!workspace) {  // no workspace: scatter with float atomics
+    hipLaunchKernelGGL(inpaint::fill_zero_f32, dim3(inpaint::grid_stride(total)), dim3(256), 0, st, g1, total);
+    hipLaunchKernelGGL(quadfit_backward_kernel, grid, block, 0, st, im0, im1, flow, gin, g0, g1, n, ic, ih, iw, flow_channels);
+    INPAINT_HIP(hipGetLastError());
+    return 0;
+  }
+  if (workspace_bytes < qf_workspace_bytes(P))
+    return fail(INPAINT_ERR_ARG, "quadfit_backward: workspace of %lld bytes, %lld needed", workspace_bytes, qf_workspace_bytes(P));
+  if (((uintptr_t)workspace & 15) != 0) return fail(INPAINT_ERR_ARG, "quadfit_backward: workspace must be 16-byte aligned");
+  if (P >= (1ll << 31)) return fail(INPAINT_ERR_ARG, "quadfit_backward: too many pixels for the inverse map");
+  const QfWorkspace ws = qf_carve(workspace, P);
+  // the counters start at zero (a fill kernel, so that the call can be captured into a graph)
+  hipLaunchKernelGGL(inpaint::fill_zero_f32, dim3(inpaint::grid_stride(P + 64)), dim3(256), 0, st,
+                     reinterpret_cast<float*>(ws.count), P + 64);
+  const int tiles_x = (iw + kTW - 1) / kTW, tiles_y = (ih + TileCfg<kPxSources>::TH - 1) / TileCfg<kPxSources>::TH;
+  const long long tiles = (long long)n * tiles_x * tiles_y;
+  const bool px_path = getenv("INPAINT_QUADFIT_PATH") && strcmp(getenv("INPAINT_QUADFIT_PATH"), "px") == 0;
+  if (px_path)
+    hipLaunchKernelGGL(quadfit_backward_sources, grid, block, 0, st, im0, im1, flow, gin, g0, ws, n, ic, ih, iw, flow_channels);
+  else {
+    g_timer.begin(st);
+    hipLaunchKernelGGL((quadfit_tiles<1, kPxSources>), dim3((unsigned)((tiles + 7) / 8 * 8)), block, 0, st, im0, im1, flow, gin, g0, ws, n,
+                       ic, ih, iw, flow_channels, tiles_x, tiles_y);
+    g_timer.end(st, 1);
+  }
+  if (px_path || ih > 65535 || iw > 65535 || (long long)ih * iw >= (1ll << 24)) {
+    hipLaunchKernelGGL(quadfit_backward_gather, grid, block, 0, st, im0, g1, ws, n, ic, ih, iw);
+  } else {
+    const int gy = (ih + TileCfg<kPxGather>::TH - 1) / TileCfg<kPxGather>::TH;
+    const long long gt = (long long)n * tiles_x * gy;
+    hipLaunchKernelGGL((quadfit_gather_tiles<kPxGather>), dim3((unsigned)((gt + 7) / 8 * 8)), block, 0, st, im0, g1, ws, n, ic,
+                       ih, iw, tiles_x, gy);
+  }
+  hipLaunchKernelGGL(quadfit_backward_overflow, dim3(64), block, 0, st, im0, flow, g1, ws, n, ic, ih, iw, flow_channels);
   INPAINT_HIP(hipGetLastError());
   return 0;
 }
@@ -337,7 +1154,10 @@ int medimax_forward(const float* vol, float* out, int n, int ih, int iw, int num
   if (n < 1 || ih < 1 || iw < 1 || num_disp < 1)
     return fail(INPAINT_ERR_ARG, "medimax_forward: bad shape %dx%dx%dx%d", n, ih, iw, num_disp);
   const long long HW = (long long)ih * iw, P = n * HW;
-  hipLaunchKernelGGL(median_forward_kernel, dim3((unsigned)((P + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, out, P,
+  if (num_disp <= kMaxRowBins)
+    launch_median_rows<false>(vol, nullptr, out, P, HW, num_disp, aligned16(vol), (hipStream_t)stream);
+  else
+    hipLaunchKernelGGL(median_forward_kernel, dim3((unsigned)((P + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, out, P,
                      HW, num_disp);
   INPAINT_HIP(hipGetLastError());
   return 0;
@@ -348,7 +1168,12 @@ int medimax_backward(const float* vol, const float* gin, float* gvol, int n, int
   if (n < 1 || ih < 1 || iw < 1 || num_disp < 1)
     return fail(INPAINT_ERR_ARG, "medimax_backward: bad shape %dx%dx%dx%d", n, ih, iw, num_disp);
   const long long HW = (long long)ih * iw, P = n * HW;
-  hipLaunchKernelGGL(median_backward_kernel, dim3((unsigned)((P + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, gin,
+  if (num_disp <= kMaxRowBins) {
+    g_timer.begin((hipStream_t)stream);
+    launch_median_rows<true>(vol, gin, gvol, P, HW, num_disp, aligned16(vol) && aligned16(gvol), (hipStream_t)stream);
+    g_timer.end((hipStream_t)stream, 1);
+  } else
+    hipLaunchKernelGGL(median_backward_kernel, dim3((unsigned)((P + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, gin,
                      gvol, P, HW, num_disp);
   INPAINT_HIP(hipGetLastError());
   return 0;

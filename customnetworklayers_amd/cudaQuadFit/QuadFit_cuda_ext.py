@@ -65,8 +65,9 @@ def forward(featureImage0, featureImage1, flow):
     return [flowUpdate]
 
 
-def backward(d_iGf, featureImage0, featureImage1, flow):
-    """d_iGf: (n,3,h,w) gradient wrt the result.  Returns [d_oFeat0, d_oFeat1]."""
+def backward(d_iGf, featureImage0, featureImage1, flow, use_atomics=False):
+    """d_iGf: (n,3,h,w) gradient wrt the result.  Returns [d_oFeat0, d_oFeat1].  `use_atomics` selects the
+    reference's scatter with float atomics instead of the gather through a scratch buffer."""
     for t, name in ((featureImage0, "featureImage0"), (featureImage1, "featureImage1"), (flow, "flow"),
                     (d_iGf, "d_iGf")):
         _check_input(t, name)
@@ -75,10 +76,12 @@ def backward(d_iGf, featureImage0, featureImage1, flow):
     if tuple(d_iGf.shape) != (n, 3, h, w):
         raise ValueError("d_iGf must have shape (%d, 3, %d, %d), got %s" % (n, h, w, tuple(d_iGf.shape)))
     d_oFeat0, d_oFeat1 = torch.empty_like(featureImage0), torch.empty_like(featureImage1)
+    ws_bytes = 0 if use_atomics else lib.quadfit_backward_workspace_bytes(n, h, w)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=flow.device) if ws_bytes else None
     with torch.cuda.device(flow.device):
         rc = lib.quadfit_backward(featureImage0.data_ptr(), featureImage1.data_ptr(), flow.data_ptr(),
                                   d_iGf.data_ptr(), d_oFeat0.data_ptr(), d_oFeat1.data_ptr(), n, c, h, w,
-                                  flow.shape[1], _stream(flow))
+                                  flow.shape[1], workspace.data_ptr() if ws_bytes else None, ws_bytes, _stream(flow))
     if rc:
         raise _ERRORS.get(rc, RuntimeError)("FlowQuadFitting::backward failed: %s" % _last_error())
     return [d_oFeat0, d_oFeat1]

@@ -5,7 +5,7 @@
  * device, contiguous float32 tensors, `stream` a hipStream_t passed as void* (NULL = the default
  * stream).  Return value 0 = ok; the error codes are the INPAINT_ERR_* values of tvinpaint.h and
  * flowaux_last_error() describes the failure.  The calls only enqueue work; they keep no state and
- * allocate nothing.
+ * allocate nothing (the one scratch buffer is the caller's).
  */
 #ifndef FLOWAUX_H_
 #define FLOWAUX_H_
@@ -32,12 +32,19 @@ int quadfit_forward(const float* im0, const float* im1, const float* flow, float
 /* Replaces FlowQuadFitting::backward (quadFit.h:30-32, quadFit.cu:145-300,338-369), bound by
  * QuadFit_cuda.cpp:83-114.
  *   gin    : (n,3,ih,iw) upstream gradient wrt `out`
- *   g0, g1 : (n,ic,ih,iw) gradients wrt im0 / im1 (overwritten).  g1 is a scatter with float
- *            atomics, as in the reference (quadFit.cu:279-283,296): its sums are order dependent at
- *            the rounding level.  There is no gradient wrt the flow (quadFit.h:11-12).
+ *   g0, g1 : (n,ic,ih,iw) gradients wrt im0 / im1 (overwritten).  There is no gradient wrt the flow
+ *            (quadFit.h:11-12).
+ *   workspace, workspace_bytes : device scratch of at least quadfit_backward_workspace_bytes(n,ih,iw)
+ *            bytes, 16-byte aligned, contents irrelevant on entry.  With it g1 is GATHERED through a
+ *            per-call inverse map (no float atomics unless more than 4 pixels land on one position).
+ *            workspace == NULL selects the reference's scatter with float atomics (quadFit.cu:279-283,
+ *            296), which this GPU executes far below memory speed.  Either way the sums that form g1 are
+ *            order dependent at the rounding level, as they are in the reference.
  */
+long long quadfit_backward_workspace_bytes(int n, int ih, int iw);
 int quadfit_backward(const float* im0, const float* im1, const float* flow, const float* gin, float* g0,
-                     float* g1, int n, int ic, int ih, int iw, int flow_channels, void* stream);
+                     float* g1, int n, int ic, int ih, int iw, int flow_channels, void* workspace,
+                     long long workspace_bytes, void* stream);
 
 /* Replaces MediMax::forward (cudaMedian/cudaCode/medimax.h:13, cudaMedian/cudaCode/medimax.cu:17-44,
  * 131-168), bound by cudaMedian/median_cuda.cpp:36-70.
@@ -54,6 +61,12 @@ int medimax_forward(const float* vol, float* out, int n, int ih, int iw, int num
  */
 int medimax_backward(const float* vol, const float* gin, float* gvol, int n, int ih, int iw, int num_disp,
                      void* stream);
+
+/* Measurement hooks, as tvinpaint_profile / tvinpaint_profile_read: with profiling on, every backward
+ * call brackets its dominant kernel (the per-source pass of the quadratic fit, the whole-histogram kernel of
+ * the median) with a HIP event pair on the caller's stream; _read waits for them and returns their total. */
+int flowaux_profile(int enable);
+int flowaux_profile_read(double* total_ms, int* launches);
 
 const char* flowaux_last_error(void);
 

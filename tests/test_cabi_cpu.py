@@ -61,3 +61,15 @@ def test_bad_arguments_are_rejected_before_any_gpu_work():
     assert "id" in last_error()
     assert lib.tvinpaint_backward(*([None] * 10), 1, 1, 4, 4, 4, -1, None) == 1
     assert lib.tvinpaint_slot_bytes(3) == 0
+
+
+def test_flow_layers_reject_bad_arguments_before_any_gpu_work():
+    from customnetworklayers_amd._lib import lib
+
+    assert lib.quadfit_forward(None, None, None, None, 1, 1, 4, 4, 2, None) == 2
+    assert lib.quadfit_backward(None, None, None, None, None, None, 1, 1, 4, 4, 2, None, 0, None) == 2
+    assert lib.medimax_forward(None, None, 1, 4, 4, 8, None) == 2
+    assert lib.medimax_backward(None, None, None, 1, 4, 4, 8, None) == 2
+    assert b"null pointer" in lib.flowaux_last_error()
+    assert lib.quadfit_backward_workspace_bytes(4, 384, 1248) >= 4 * 384 * 1248 * 4 * 11
+    assert lib.quadfit_backward_workspace_bytes(0, 384, 1248) == 0

@@ -46,17 +46,19 @@ def random_quadfit(n, c, h, w, seed, fc=2, amp=3.0):
 def check_quadfit(qf, o, d, name):
     print("case", name, flush=True)
     (out,) = qf.forward(dev(d["feat0"]), dev(d["feat1"]), dev(d["flow"]))
-    g0, g1 = qf.backward(dev(d["grad"]), dev(d["feat0"]), dev(d["feat1"]), dev(d["flow"]))
-    out, g0, g1 = out.cpu().numpy(), g0.cpu().numpy(), g1.cpu().numpy()
+    out = out.cpu().numpy()
     rout = o.quadfit_forward(d["feat0"], d["feat1"], d["flow"])
     r0, r1 = o.quadfit_backward(d["grad"], d["feat0"], d["feat1"], d["flow"])
-    e1 = np.abs(g1 - r1).max() / max(np.abs(r1).max(), 1e-30)
-    print("[%s] out bit-equal %.4f, g0 bit-equal %.4f, g1 rel err %.2e; valid x %.2f, outside %.2f"
-          % (name, (out == rout).mean(), (g0 == r0).mean(), e1, (rout[:, 0] != 0).mean(), (rout[:, 2] == 0).mean()),
-          flush=True)
     assert np.array_equal(out, rout)
-    assert np.array_equal(g0, r0)
-    assert e1 <= SCATTER_TOL
+    for path, atomics in (("gather", False), ("atomic scatter", True)):
+        g0, g1 = qf.backward(dev(d["grad"]), dev(d["feat0"]), dev(d["feat1"]), dev(d["flow"]), use_atomics=atomics)
+        g0, g1 = g0.cpu().numpy(), g1.cpu().numpy()
+        e1 = np.abs(g1 - r1).max() / max(np.abs(r1).max(), 1e-30)
+        print("[%s, %s] out bit-equal %.4f, g0 bit-equal %.4f, g1 rel err %.2e; valid x %.2f, outside %.2f"
+              % (name, path, (out == rout).mean(), (g0 == r0).mean(), e1, (rout[:, 0] != 0).mean(),
+                 (rout[:, 2] == 0).mean()), flush=True)
+        assert np.array_equal(g0, r0)
+        assert e1 <= SCATTER_TOL
     return out
 
 
@@ -82,12 +84,24 @@ def test_quadfit_warped_features_match_oracle(qf, flowaux_oracle, n, c, h, w):
 
 
 def test_quadfit_all_pixels_collide(qf, flowaux_oracle):
-    # every pixel is sent to one target: 5 addresses per channel take every atomic of the launch
+    # every pixel is sent to one target: its list overflows, and 5 addresses per channel take every atomic
     n, c, h, w = 1, 3, 40, 70
     d = random_quadfit(n, c, h, w, seed=5)
     ys, xs = np.mgrid[0:h, 0:w]
     d["flow"] = np.stack([30 - xs, 20 - ys])[None].astype(np.float32)
     check_quadfit(qf, flowaux_oracle, d, "collide")
+
+
+def test_quadfit_several_pixels_per_target(qf, flowaux_oracle):
+    # the flow folds the image onto itself: two to six pixels land on most targets (lists with several
+    # entries, some overflowing), none on others
+    n, c, h, w = 2, 5, 30, 64
+    d = random_quadfit(n, c, h, w, seed=6)
+    ys, xs = np.mgrid[0:h, 0:w]
+    fold_x = (xs // 3) * 1.0 + 10 - xs
+    fold_y = (ys // 2) * 1.0 + 5 - ys
+    d["flow"] = np.broadcast_to(np.stack([fold_x, fold_y])[None], (n, 2, h, w)).astype(np.float32).copy()
+    check_quadfit(qf, flowaux_oracle, d, "folded")
 
 
 def test_quadfit_outputs_are_overwritten_not_accumulated(qf, flowaux_oracle):
@@ -157,10 +171,26 @@ def check_median(med, o, vol, grad, name):
     (1, 7, 50, 100),     # four chunks, the last one ragged
     (3, 1, 1, 5),        # fewer pixels than one wavefront
     (1, 64, 65, 21),     # pixel count not a multiple of the block
+    (1, 6, 9, 255),      # the most bins the whole-histogram kernels take
+    (1, 6, 9, 300),      # beyond: the chunked kernels
+    (2, 5, 7, 2),
+    (1, 10, 13, 3),
 ])
 def test_median_matches_oracle(med, flowaux_oracle, n, h, w, d):
     m = workloads.median_inputs(n, h, w, d, seed=n + h + w + d, empty_fraction=0.1)
     check_median(med, flowaux_oracle, m["vol"], m["grad"], "%dx%dx%dx%d" % (n, h, w, d))
+
+
+def test_median_buffers_without_16_byte_alignment(med, flowaux_oracle):
+    m = workloads.median_inputs(1, 9, 14, 21, seed=9)
+    flat = torch.zeros(m["vol"].size + 3, dtype=torch.float32, device="cuda")
+    for shift in (1, 2, 3):
+        v = flat[shift:shift + m["vol"].size].view(m["vol"].shape)
+        v.copy_(dev(m["vol"]))
+        (out,) = med.forward(v)
+        (g,) = med.backward(dev(m["grad"]), v)
+        assert np.array_equal(out.cpu().numpy(), flowaux_oracle.median_forward(m["vol"]))
+        assert np.array_equal(g.cpu().numpy(), flowaux_oracle.median_backward(m["grad"], m["vol"]))
 
 
 def test_median_unnormalised_and_signed_histograms(med, flowaux_oracle):
