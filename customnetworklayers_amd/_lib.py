@@ -55,6 +55,9 @@ def _load():
     lib.medimax_forward.argtypes = [_f32p] * 2 + [_int] * 4 + [ctypes.c_void_p]
     lib.medimax_backward.argtypes = [_f32p] * 3 + [_int] * 4 + [ctypes.c_void_p]
     lib.flowaux_last_error.restype = ctypes.c_char_p
+    lib.hierarchy_next_level_forward.argtypes = [_f32p] * 5 + [_int] * 4 + [ctypes.c_float, ctypes.c_float, ctypes.c_void_p]
+    lib.hierarchy_next_level_backward.argtypes = [_f32p] * 3 + [_int] * 4 + [ctypes.c_float, ctypes.c_void_p]
+    lib.hierarchy_last_error.restype = ctypes.c_char_p
     lib.flowaux_profile.argtypes = [_int]
     lib.flowaux_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
     return lib

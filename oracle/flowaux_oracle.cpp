@@ -265,9 +265,157 @@ void median_backward(const R* vol, const R* gin, R* gvol, int N, int H, int W, i
       }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Glue between two levels of a coarse-to-fine hierarchy of inpainting layers (the reference's README.md:64-71
+// describes the hierarchy; it ships no code for the glue, so this is the build's own definition):
+//   up   = scale * bilinear x2 upsampling of the coarse solution -- the definition of bilinear resampling with
+//          half-pixel centres: source coordinate (dst + 0.5) / 2 - 0.5 clamped at 0, neighbours clamped at the border;
+//          flow vectors are measured in pixels, hence scale = 2;
+//   wx,wy = exp(-alpha |I(h, w+1) - I(h, w)|), exp(-alpha |I(h+1, w) - I(h, w)|), 1 in the last column / row --
+//          the edge weights of the fine level from its guidance image (single precision: exp_nonpos below).
+// Pins: torch.nn.functional.interpolate(mode="bilinear", align_corners=False) and its autograd adjoint.
+// ---------------------------------------------------------------------------------------------
+template <typename R>
+void axis_taps(int dst, int size, int& i0, int& i1, R& l0, R& l1) {
+  R src = (R)((dst + 0.5) * 0.5 - 0.5);
+  if (src < 0) src = 0;
+  i0 = (int)src;
+  i1 = std::min(i0 + 1, size - 1);
+  l1 = src - (R)i0;
+  l0 = (R)1 - l1;
+}
+
+template <typename R>
+void upsample2x(const R* in, R* out, int planes, int H, int W, R scale) {
+  const int H2 = 2 * H, W2 = 2 * W;
+#pragma omp parallel for num_threads(threads_for(planes))
+  for (int q = 0; q < planes; q++) {
+    const R* a = in + (size_t)q * H * W;
+    R* o = out + (size_t)q * H2 * W2;
+    for (int y = 0; y < H2; y++) {
+      int y0, y1;
+      R h0, h1;
+      axis_taps<R>(y, H, y0, y1, h0, h1);
+      for (int x = 0; x < W2; x++) {
+        int x0, x1;
+        R w0, w1;
+        axis_taps<R>(x, W, x0, x1, w0, w1);
+        const R v = h0 * (w0 * a[(size_t)y0 * W + x0] + w1 * a[(size_t)y0 * W + x1]) +
+                    h1 * (w0 * a[(size_t)y1 * W + x0] + w1 * a[(size_t)y1 * W + x1]);
+        o[(size_t)y * W2 + x] = scale * v;
+      }
+    }
+  }
+}
+
+// adjoint of upsample2x applied to ga (+ gb when given): every coarse pixel collects, in a fixed order (fine rows
+// ascending, then fine columns ascending), the fine pixels it was a tap of
+template <typename R>
+void upsample2x_adjoint(const R* ga, const R* gb, R* out, int planes, int H, int W, R scale) {
+  const int H2 = 2 * H, W2 = 2 * W;
+#pragma omp parallel for num_threads(threads_for(planes))
+  for (int q = 0; q < planes; q++) {
+    const R* g0 = ga + (size_t)q * H2 * W2;
+    const R* g1 = gb ? gb + (size_t)q * H2 * W2 : nullptr;
+    R* o = out + (size_t)q * H * W;
+    for (int cy = 0; cy < H; cy++)
+      for (int cx = 0; cx < W; cx++) {
+        R acc = 0;
+        for (int y = std::max(2 * cy - 1, 0); y <= std::min(2 * cy + 2, H2 - 1); y++) {
+          int y0, y1;
+          R h0, h1;
+          axis_taps<R>(y, H, y0, y1, h0, h1);
+          R wy = 0;  // weight of coarse row cy in fine row y (both taps can fall on the same clamped row)
+          if (y0 == cy) wy += h0;
+          if (y1 == cy) wy += h1;
+          if (wy == 0) continue;
+          for (int x = std::max(2 * cx - 1, 0); x <= std::min(2 * cx + 2, W2 - 1); x++) {
+            int x0, x1;
+            R w0, w1;
+            axis_taps<R>(x, W, x0, x1, w0, w1);
+            R wx = 0;
+            if (x0 == cx) wx += w0;
+            if (x1 == cx) wx += w1;
+            if (wx == 0) continue;
+            R g = g0[(size_t)y * W2 + x];
+            if (g1) g = g + g1[(size_t)y * W2 + x];
+            acc += (wy * wx) * g;
+          }
+        }
+        o[(size_t)cy * W + cx] = scale * acc;
+      }
+  }
+}
+
+// exp(x) for x <= 0 in single precision with a FIXED sequence of IEEE operations (Cody-Waite reduction by
+// ln 2, degree-7 Taylor polynomial in Horner form, exact scaling), so that a device and a host evaluation agree
+// bit for bit; about 1 ulp from the true value.  The double instantiation uses the library's exp.
+inline float exp_nonpos(float x) {
+  if (!(x > -87.0f)) return 0.0f;
+  const float n = std::rint(x * 1.44269504f);
+  float r = x - n * 0.693359375f;
+  r = r - n * -2.12194440e-4f;
+  float p = 1.98412698e-4f;
+  p = p * r + 1.38888889e-3f;
+  p = p * r + 8.33333333e-3f;
+  p = p * r + 4.16666667e-2f;
+  p = p * r + 1.66666667e-1f;
+  p = p * r + 0.5f;
+  p = p * r + 1.0f;
+  p = p * r + 1.0f;
+  return std::ldexp(p, (int)n);
+}
+inline double exp_nonpos(double x) { return std::exp(x); }
+
+template <typename R>
+void edge_weights(const R* img, R* wx, R* wy, int planes, int H, int W, R alpha) {
+  for (int q = 0; q < planes; q++) {
+    const R* a = img + (size_t)q * H * W;
+    for (int y = 0; y < H; y++)
+      for (int x = 0; x < W; x++) {
+        const size_t p = (size_t)q * H * W + (size_t)y * W + x;
+        wx[p] = x + 1 < W ? exp_nonpos(-alpha * std::fabs(a[(size_t)y * W + x + 1] - a[(size_t)y * W + x])) : (R)1;
+        wy[p] = y + 1 < H ? exp_nonpos(-alpha * std::fabs(a[(size_t)(y + 1) * W + x] - a[(size_t)y * W + x])) : (R)1;
+      }
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+int hierarchy_oracle_upsample2x(const float* in, float* out, int planes, int h, int w, float scale) {
+  if (planes < 1 || h < 1 || w < 1) return 1;
+  upsample2x<float>(in, out, planes, h, w, scale);
+  return 0;
+}
+int hierarchy_oracle_upsample2x_f64(const double* in, double* out, int planes, int h, int w, double scale) {
+  if (planes < 1 || h < 1 || w < 1) return 1;
+  upsample2x<double>(in, out, planes, h, w, scale);
+  return 0;
+}
+int hierarchy_oracle_upsample2x_adjoint(const float* ga, const float* gb, float* out, int planes, int h, int w, float scale) {
+  if (planes < 1 || h < 1 || w < 1) return 1;
+  upsample2x_adjoint<float>(ga, gb, out, planes, h, w, scale);
+  return 0;
+}
+int hierarchy_oracle_upsample2x_adjoint_f64(const double* ga, const double* gb, double* out, int planes, int h, int w,
+                                            double scale) {
+  if (planes < 1 || h < 1 || w < 1) return 1;
+  upsample2x_adjoint<double>(ga, gb, out, planes, h, w, scale);
+  return 0;
+}
+int hierarchy_oracle_edge_weights(const float* img, float* wx, float* wy, int planes, int h, int w, float alpha) {
+  if (planes < 1 || h < 1 || w < 1) return 1;
+  edge_weights<float>(img, wx, wy, planes, h, w, alpha);
+  return 0;
+}
+int hierarchy_oracle_edge_weights_f64(const double* img, double* wx, double* wy, int planes, int h, int w, double alpha) {
+  if (planes < 1 || h < 1 || w < 1) return 1;
+  edge_weights<double>(img, wx, wy, planes, h, w, alpha);
+  return 0;
+}
+
 
 void flowaux_oracle_set_threads(int t) { g_threads = t; }
 

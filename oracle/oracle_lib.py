@@ -306,6 +306,12 @@ class FlowAuxOracle:
         L.median_oracle_backward_f64.argtypes = [_f64p] * 3 + [_int] * 4
         L.flowaux_oracle_set_threads.argtypes = [_int]
         L.flowaux_oracle_set_threads.restype = None
+        L.hierarchy_oracle_upsample2x.argtypes = [_f32p] * 2 + [_int] * 3 + [ctypes.c_float]
+        L.hierarchy_oracle_upsample2x_f64.argtypes = [_f64p] * 2 + [_int] * 3 + [ctypes.c_double]
+        L.hierarchy_oracle_upsample2x_adjoint.argtypes = [_f32p] * 3 + [_int] * 3 + [ctypes.c_float]
+        L.hierarchy_oracle_upsample2x_adjoint_f64.argtypes = [_f64p] * 3 + [_int] * 3 + [ctypes.c_double]
+        L.hierarchy_oracle_edge_weights.argtypes = [_f32p] * 3 + [_int] * 3 + [ctypes.c_float]
+        L.hierarchy_oracle_edge_weights_f64.argtypes = [_f64p] * 3 + [_int] * 3 + [ctypes.c_double]
 
     def quadfit_forward(self, feat0, feat1, flow, f64=False):
         """feat0, feat1: (N,C,H,W); flow: (N,F,H,W) with F >= 2.  Returns (N,3,H,W) = (fx, fy, score)."""
@@ -361,3 +367,41 @@ class FlowAuxOracle:
 
     def set_threads(self, n):
         self.lib.flowaux_oracle_set_threads(int(n))
+
+    # -- glue between two levels of a hierarchy ----------------------------------------------------
+    def upsample2x(self, x, scale=2.0, f64=False):
+        """x: (N,C,H,W) -> scale * bilinear x2 upsampling, (N,C,2H,2W)."""
+        dt = np.float64 if f64 else np.float32
+        x = _c(x, dt)
+        n, c, h, w = x.shape
+        out = np.empty((n, c, 2 * h, 2 * w), dt)
+        P = _p64 if f64 else _p32
+        fn = self.lib.hierarchy_oracle_upsample2x_f64 if f64 else self.lib.hierarchy_oracle_upsample2x
+        if fn(P(x), P(out), n * c, h, w, scale):
+            raise RuntimeError("hierarchy_oracle_upsample2x failed")
+        return out
+
+    def upsample2x_adjoint(self, ga, gb=None, scale=2.0, f64=False):
+        """ga (and gb, summed): (N,C,2H,2W) -> the adjoint of upsample2x, (N,C,H,W)."""
+        dt = np.float64 if f64 else np.float32
+        ga = _c(ga, dt)
+        gb = None if gb is None else _c(gb, dt)
+        n, c, h2, w2 = ga.shape
+        out = np.empty((n, c, h2 // 2, w2 // 2), dt)
+        P = _p64 if f64 else _p32
+        fn = self.lib.hierarchy_oracle_upsample2x_adjoint_f64 if f64 else self.lib.hierarchy_oracle_upsample2x_adjoint
+        if fn(P(ga), None if gb is None else P(gb), P(out), n * c, h2 // 2, w2 // 2, scale):
+            raise RuntimeError("hierarchy_oracle_upsample2x_adjoint failed")
+        return out
+
+    def edge_weights(self, img, alpha=10.0, f64=False):
+        """img: (N,1,H,W) -> (wx, wy) = exp(-alpha |forward difference|), 1 in the last column / row."""
+        dt = np.float64 if f64 else np.float32
+        img = _c(img, dt)
+        n, c, h, w = img.shape
+        wx, wy = np.empty_like(img), np.empty_like(img)
+        P = _p64 if f64 else _p32
+        fn = self.lib.hierarchy_oracle_edge_weights_f64 if f64 else self.lib.hierarchy_oracle_edge_weights
+        if fn(P(img), P(wx), P(wy), n * c, h, w, alpha):
+            raise RuntimeError("hierarchy_oracle_edge_weights failed")
+        return wx, wy

@@ -1,0 +1,128 @@
+"""GPU parity of the glue between two levels of a hierarchy (scaled bilinear x2 upsampling, its
+adjoint, the edge weights) against the CPU oracle, and a three-level coarse-to-fine run in which
+the glue runs on the device between the layers.
+
+Bar: everything is BIT-EQUAL to the oracle (fixed operation order, including the exponential of the
+edge weights), and so is the whole three-level run."""
+import numpy as np
+import pytest
+import torch
+
+from customnetworklayers_amd import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+@pytest.mark.parametrize("n,c,h,w", [(1, 1, 1, 1), (2, 3, 5, 7), (1, 2, 16, 9), (1, 1, 1, 70), (1, 1, 40, 1), (2, 2, 112, 256),
+                                     (1, 2, 33, 129)])
+def test_next_level_matches_oracle(flowaux_oracle, n, c, h, w):
+    from customnetworklayers_amd import hierarchy
+
+    rng = np.random.default_rng(n + c + h + w)
+    sol = rng.standard_normal((n, c, h, w)).astype(np.float32) * 5
+    img = np.stack([workloads.smooth_image(rng, 2 * h, 2 * w, sigma=2.0) for _ in range(n)])[:, None].astype(np.float32)
+    ga = rng.standard_normal((n, c, 2 * h, 2 * w)).astype(np.float32)
+    gb = rng.standard_normal((n, c, 2 * h, 2 * w)).astype(np.float32)
+    up, wx, wy = hierarchy.next_level_forward(dev(sol), dev(img))
+    assert np.array_equal(up.cpu().numpy(), flowaux_oracle.upsample2x(sol, 2.0))
+    rx, ry = flowaux_oracle.edge_weights(img, 10.0)
+    assert np.array_equal(wx.cpu().numpy(), rx) and np.array_equal(wy.cpu().numpy(), ry)
+    up_only, none_x, none_y = hierarchy.next_level_forward(dev(sol), None, scale=1.0)
+    assert none_x is None and none_y is None
+    assert np.array_equal(up_only.cpu().numpy(), flowaux_oracle.upsample2x(sol, 1.0))
+    g2 = hierarchy.next_level_backward(dev(ga), dev(gb))
+    assert np.array_equal(g2.cpu().numpy(), flowaux_oracle.upsample2x_adjoint(ga, gb, 2.0))
+    g1 = hierarchy.next_level_backward(dev(ga))
+    assert np.array_equal(g1.cpu().numpy(), flowaux_oracle.upsample2x_adjoint(ga, None, 2.0))
+
+
+def test_next_level_autograd_and_errors(flowaux_oracle):
+    import torch.nn.functional as F
+
+    from customnetworklayers_amd import hierarchy
+
+    rng = np.random.default_rng(3)
+    sol = dev(rng.standard_normal((2, 2, 12, 20)).astype(np.float32)).requires_grad_(True)
+    img = dev(rng.random((2, 1, 24, 40)).astype(np.float32))
+    up, wx, wy = hierarchy.next_level(sol, img)
+    g = dev(rng.standard_normal((2, 2, 24, 40)).astype(np.float32))
+    (up * g).sum().backward()
+    ref = sol.detach().clone().requires_grad_(True)
+    (2.0 * F.interpolate(ref, scale_factor=2, mode="bilinear", align_corners=False) * g).sum().backward()
+    assert (sol.grad - ref.grad).abs().max().item() <= 1e-5 * ref.grad.abs().max().item()
+    assert not wx.requires_grad and not wy.requires_grad
+    with pytest.raises(RuntimeError):
+        hierarchy.next_level_forward(sol.detach().cpu())
+    with pytest.raises(ValueError):
+        hierarchy.next_level_forward(sol.detach(), img[:, :, :-2].contiguous())
+    with pytest.raises(TypeError):
+        hierarchy.next_level_forward(sol.detach().double())
+    with pytest.raises(ValueError):
+        hierarchy.next_level_backward(g[:, :, :-1].contiguous())
+
+
+def test_three_level_hierarchy_with_device_glue(tv_oracle, flowaux_oracle):
+    """Levels 28x64 -> 56x128 -> 112x256, ids 0,1,2 forward and 2,1,0 backward.  Device path: TV layers and glue
+    on the GPU, nothing leaves the device between levels.  Reference path: CPU oracles for both.  Bars: the layer's
+    tolerances, 1e-4 on solutions and 1e-3 on gradients (the printed errors are zero: every stage is bit-equal)."""
+    from customnetworklayers_amd import hierarchy
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+
+    n, c, its = 2, 2, 30
+    levels = [(28, 64), (56, 128), (112, 256)]
+    rng = np.random.default_rng(0)
+    imgs = [np.stack([workloads.smooth_image(rng, h, w, sigma=3.0) for _ in range(n)])[:, None].astype(np.float32)
+            for h, w in levels]
+    base = [workloads.tv_inputs(n, c, h, w, seed=20 + i, conf_density=0.25) for i, (h, w) in enumerate(levels)]
+
+    # --- reference path ---------------------------------------------------------------------
+    feeds, sols = [], []
+    wx, wy = flowaux_oracle.edge_weights(imgs[0], 10.0)
+    b = base[0]["db"]
+    for lvl in range(3):
+        feed = dict(dx=wx, dy=wy, dc=base[lvl]["dc"], db=b, di=b)
+        tv_oracle.reset_id(lvl)
+        sols.append(tv_oracle.forward(feed["dx"], feed["dy"], feed["dc"], feed["db"], feed["di"], its, lvl))
+        feeds.append(feed)
+        if lvl < 2:
+            b = flowaux_oracle.upsample2x(sols[-1], 2.0)
+            wx, wy = flowaux_oracle.edge_weights(imgs[lvl + 1], 10.0)
+    upstream = base[2]["grad"].copy()
+    ref_grads = [None] * 3
+    for lvl in (2, 1, 0):
+        f = feeds[lvl]
+        ref_grads[lvl] = tv_oracle.backward(upstream.copy(), f["dx"], f["dy"], f["dc"], f["db"], its, lvl)
+        if lvl > 0:
+            upstream = flowaux_oracle.upsample2x_adjoint(ref_grads[lvl][3], ref_grads[lvl][4], 2.0)
+
+    # --- device path -----------------------------------------------------------------------
+    dfeeds, dsols = [], []
+    ones = torch.zeros((n, c, levels[0][0] // 2, levels[0][1] // 2), device=DEV)
+    _, dwx, dwy = hierarchy.next_level_forward(ones, dev(imgs[0]))  # level 0's weights from its image
+    db = dev(base[0]["db"])
+    for lvl in range(3):
+        feed = dict(dx=dwx, dy=dwy, dc=dev(base[lvl]["dc"]), db=db)
+        ext.reset_id(lvl)
+        dsols.append(ext.forward(feed["dx"], feed["dy"], feed["dc"], feed["db"], feed["db"], its, lvl)[0])
+        dfeeds.append(feed)
+        if lvl < 2:
+            db, dwx, dwy = hierarchy.next_level_forward(dsols[-1], dev(imgs[lvl + 1]))
+    dup = dev(base[2]["grad"])
+    dev_grads = [None] * 3
+    for lvl in (2, 1, 0):
+        f = dfeeds[lvl]
+        dev_grads[lvl] = ext.backward(dup.clone(), f["dx"], f["dy"], f["dc"], f["db"], its, lvl)
+        if lvl > 0:
+            dup = hierarchy.next_level_backward(dev_grads[lvl][3], dev_grads[lvl][4])
+
+    rel = lambda a, r: float(np.abs(a - r).max() / max(np.abs(r).max(), 1e-30))
+    for lvl in range(3):
+        e_out = rel(dsols[lvl].cpu().numpy(), sols[lvl])
+        e_g = [rel(a.cpu().numpy(), r) for a, r in zip(dev_grads[lvl], ref_grads[lvl])]
+        print("[level %d] out %.2e grads %s" % (lvl, e_out, ["%.2e" % e for e in e_g]), flush=True)
+        assert e_out <= 1e-4 and max(e_g) <= 1e-3
