@@ -18,8 +18,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script
 # (headline workload: the two-step adjoint kernel fetches 2 x 87000 KiB, after the copy-kernel
 # calibration, and writes 68035 KiB; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
-# profiles/tgv_strip_config2_hbm_traffic.txt).  Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: (2 * 87000 + 68035) * 1024, 2: (2 * 142500 + 153510) * 1024}
+# profiles/tgv_strip_config2_hbm_traffic.txt; configs 5 and 6: profiles/quadfit_config5_*.txt, profiles/median_config6_*.txt).
+# Other workloads: not measured.
+MEASURED_TRAFFIC_BYTES = {1: (2 * 87000 + 68035) * 1024, 2: (2 * 174700 + 143820) * 1024,
+                          5: (2 * 408180 + 340500) * 1024, 6: (2 * 131080 + 247100) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):

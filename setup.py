@@ -2,9 +2,10 @@
 
 `python setup.py build_ext --inplace` (or `install`) compiles the HIP library for gfx950 with hipcc
 into customnetworklayers_amd/libinpaint_hip.so; the Python modules bind it through its C ABI
-(include/tvinpaint.h).  The reference builds one torch CUDAExtension per layer
-(cudaTV/setup.py:16-28, cudaTGV/setup.py:16-29 of the reference); the module names it produces,
-tvInpaint_cuda_ext and tgvInpaint_cuda_ext, are kept as importable top-level modules.
+(include/*.h).  The reference builds one torch CUDAExtension per layer
+(cudaTV/setup.py:16-28, cudaTGV/setup.py:16-29, cudaQuadFit/setup.py:16-28, cudaMedian/setup.py:16-27 of the
+reference); the module names it produces -- tvInpaint_cuda_ext, tgvInpaint_cuda_ext, QuadFit_cuda_ext,
+median_cuda_ext -- are kept as importable top-level modules.
 """
 import os
 import subprocess
@@ -39,9 +40,10 @@ class BuildPyWithHip(build_py):
 setup(
     name="customnetworklayers_amd",
     version="0.1.0",
-    description="TV / TGV FISTA inpainting layers for MI355X (gfx950)",
-    packages=["customnetworklayers_amd", "customnetworklayers_amd.cudaTV", "customnetworklayers_amd.cudaTGV"],
+    description="TV / TGV FISTA inpainting layers, quadratic fit and histogram median for MI355X (gfx950)",
+    packages=["customnetworklayers_amd", "customnetworklayers_amd.cudaTV", "customnetworklayers_amd.cudaTGV",
+              "customnetworklayers_amd.cudaQuadFit", "customnetworklayers_amd.cudaMedian"],
     package_data={"customnetworklayers_amd": ["libinpaint_hip.so"]},
-    py_modules=["tvInpaint_cuda_ext", "tgvInpaint_cuda_ext"],
+    py_modules=["tvInpaint_cuda_ext", "tgvInpaint_cuda_ext", "QuadFit_cuda_ext", "median_cuda_ext"],
     cmdclass={"build_ext": BuildHip, "build_py": BuildPyWithHip},
 )

@@ -102,7 +102,7 @@ def test_three_level_hierarchy_with_device_glue(tv_oracle, flowaux_oracle):
 
     # --- device path -----------------------------------------------------------------------
     dfeeds, dsols = [], []
-    ones = torch.zeros((n, c, levels[0][0] // 2, levels[0][1] // 2), device=DEV)
+    ones = torch.zeros((n, c, levels[0][0] // 2, levels[0][1] // 2), dtype=torch.float32, device=DEV)
     _, dwx, dwy = hierarchy.next_level_forward(ones, dev(imgs[0]))  # level 0's weights from its image
     db = dev(base[0]["db"])
     for lvl in range(3):
