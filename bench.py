@@ -40,7 +40,7 @@ def layer_of(kind):
     from customnetworklayers_amd import workloads
     if kind == "tgv":
         from customnetworklayers_amd.cudaTGV import tgvInpaint_cuda_ext as ext
-        return ext, "tgvinpaint", workloads.tgv_inputs, "TGVOracle", "tgvstrip::tgv_adjoint_strip2<2,false,false>"
+        return ext, "tgvinpaint", workloads.tgv_inputs, "TGVOracle", "tgvstrip::tgv_adjoint_strip2w<2,false,false>"
     from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
     return ext, "tvinpaint", workloads.tv_inputs, "TVOracle", "tvstrip::tv_adjoint_strip2<2,false,false>"
 

@@ -842,6 +842,37 @@ int strip_rows(int n, int ih, int iw, const char* env_name) {
   return 2;
 }
 
+// Rows per strip of the two-wavefront pair kernel.  Its workgroups (one strip each) are resident four per CU, so a
+// launch runs in ceil(workgroups / (4 * CUs)) rounds of (R + 3 pipeline rows + start-up) row steps each; the
+// strip height that minimises rounds x steps is taken (on 4 x 384 x 1248: 32 rows, 1008 workgroups, one round).
+int pair_split_rows(int n, int ih, int iw) {
+  if (const char* e = getenv("INPAINT_TGV_ADJ_ROWS")) {
+    const int v = atoi(e);
+    if (v >= 1 && v <= 4096) return v;
+  }
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+              ? prop.multiProcessorCount
+              : 256;
+  }
+  const long long cap = 4ll * cus;
+  const long long sx = (iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2;
+  int best = 16;
+  long long best_cost = -1;
+  for (int R = 8; R <= 64; R++) {
+    const long long wg = sx * ((ih + R - 1) / R) * n;
+    const long long cost = ((wg + cap - 1) / cap) * (R + 7);
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = R;
+    }
+  }
+  return best;
+}
+
 template <int C>
 void launch_forward_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                           float* xout, const float* yin, float* yout, float* x05, float t) {
@@ -951,20 +982,26 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
                                const float* xb, const float* xc, const float* g05_in, float* g05_out, const float* gxk,
                                float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
-  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
+  // two channels: the two steps run in two wavefronts of a workgroup (one strip per 128-thread workgroup);
+  // one channel: both steps fit one wavefront's registers (four strips per 256-thread workgroup)
+  const char* e = getenv("INPAINT_TGV_PAIR_WAVES");
+  const bool split = e ? strcmp(e, "2") == 0 : C >= 2;
+  const int R = split ? pair_split_rows(s.n, s.ih, s.iw) : strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
-  const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (gx_final)
-    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
-                       xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
-                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, tA, tB, R, sx,
-                       sy);
-  else
-    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
-                       xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
-                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, tA, tB, R, sx,
-                       sy);
+#define TGV_PAIR_ARGS                                                                                                      \
+  s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], \
+      s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, tA, tB, R, sx, sy
+  if (split) {
+    const dim3 grid((unsigned)((waves + 7) / 8 * 8)), block(128);
+    if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, true>), grid, block, 0, stream, TGV_PAIR_ARGS);
+    else hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, false>), grid, block, 0, stream, TGV_PAIR_ARGS);
+  } else {
+    const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
+    if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, TGV_PAIR_ARGS);
+    else hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, TGV_PAIR_ARGS);
+  }
+#undef TGV_PAIR_ARGS
 }
 
 template <bool BEND>

@@ -87,6 +87,31 @@ __device__ __forceinline__ bool strip_geometry(StripGeom& g, int cols, int R, in
   return true;
 }
 
+// The same numbering with ONE strip per workgroup (all wavefronts of the workgroup work on that strip).
+__device__ __forceinline__ bool strip_geometry_block(StripGeom& g, int cols, int R, int W, int strips_x, int strips_y,
+                                                     int N, int left_apron) {
+  const int per_xcd = gridDim.x >> 3;
+  const int strip = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  g.lane = threadIdx.x & 63;
+  const int sx = strip % strips_x;
+  const int rest = strip / strips_x;
+  const int sy = rest % strips_y;
+  g.n = rest / strips_y;
+  if (g.n >= N) return false;
+  g.w = sx * cols - left_apron + g.lane;
+  g.hs = sy * R;
+  g.col_ok = g.w >= 0 && g.w < W;
+  return true;
+}
+
+// Workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight (a full
+// __syncthreads() drains the one counter this GPU keeps for loads and stores alike).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // -------------------------------------------------------------------------------------------------
 // Forward iteration, TV.cu:1194-1319 (and 1321-1455 when x05 is given).
 //

@@ -155,6 +155,26 @@ def test_single_step_adjoint_strip_kernels(ext, tgv_oracle, n, c, h, w, its, mon
     compare("one adjoint step per launch c=%d" % c, run_gpu(ext, d, its, 2), ref)
 
 
+@pytest.mark.parametrize("waves", ["1", "2"])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 45, 130, 10), (1, 2, 3, 200, 6), (2, 2, 18, 121, 12),
+                                         (1, 2, 1, 70, 4), (1, 1, 33, 1, 4)])
+def test_adjoint_pairs_in_one_or_two_wavefronts(ext, tgv_oracle, n, c, h, w, its, waves, monkeypatch):
+    # the two steps of a pair run in one wavefront (default at one channel) or in the two wavefronts of a
+    # workgroup, handed over through LDS (default at two channels); force each layout for both channel counts
+    d = varying_inputs(n, c, h, w, seed=95 + c + h)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TGV_PAIR_WAVES", waves)
+    compare("pair in %s wavefront(s) c=%d %dx%d" % (waves, c, h, w), run_gpu(ext, d, its, 2), ref)
+
+
+@pytest.mark.parametrize("rows", ["8", "13", "64"])
+def test_adjoint_pair_strip_heights(ext, tgv_oracle, rows, monkeypatch):
+    d = varying_inputs(2, 2, 50, 140, seed=97)
+    ref = run_oracle(tgv_oracle, d, 12, 2)
+    monkeypatch.setenv("INPAINT_TGV_ADJ_ROWS", rows)
+    compare("strip height %s" % rows, run_gpu(ext, d, 12, 2), ref)
+
+
 @pytest.mark.parametrize("c", [1, 2])
 @pytest.mark.parametrize("its", [2, 3, 4, 5, 6, 8, 16, 17, 26])
 def test_every_pairing_of_the_reverse_sweep(ext, tgv_oracle, c, its):
