@@ -20,7 +20,7 @@ HBM_PEAK_GBS = 8000.0
 # calibration, and writes 68035 KiB; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
 # profiles/tgv_strip_config2_hbm_traffic.txt; configs 5 and 6: profiles/quadfit_config5_*.txt, profiles/median_config6_*.txt).
 # Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: (2 * 87000 + 68035) * 1024, 2: (2 * 174700 + 143820) * 1024,
+MEASURED_TRAFFIC_BYTES = {1: (2 * 87000 + 68035) * 1024, 2: (2 * 166450 + 147340) * 1024,
                           5: (2 * 408180 + 340500) * 1024, 6: (2 * 131080 + 247100) * 1024}
 
 

@@ -83,6 +83,20 @@ def test_quadfit_warped_features_match_oracle(qf, flowaux_oracle, n, c, h, w):
     assert (out[:, 0] != 0).mean() > 0.2  # a good share of valid fits
 
 
+@pytest.mark.parametrize("n,c,h,w", [(2, 6, 40, 90), (1, 3, 9, 200)])
+def test_quadfit_one_pixel_per_lane_kernels(qf, flowaux_oracle, n, c, h, w, monkeypatch):
+    # INPAINT_QUADFIT_PATH=px: the kernels without LDS windows (a lane reads its taps from memory)
+    monkeypatch.setenv("INPAINT_QUADFIT_PATH", "px")
+    check_quadfit(qf, flowaux_oracle, random_quadfit(n, c, h, w, seed=31 + c), "px path random %dx%dx%dx%d" % (n, c, h, w))
+    check_quadfit(qf, flowaux_oracle, workloads.quadfit_inputs(n, c, h, w, seed=32), "px path warped")
+
+
+def test_quadfit_flow_that_scatters_the_tile(qf, flowaux_oracle):
+    # a flow that varies by tens of pixels inside one 64 x 8 tile: most taps fall outside the LDS window
+    d = random_quadfit(1, 4, 64, 256, seed=33, amp=40.0)
+    check_quadfit(qf, flowaux_oracle, d, "scattered")
+
+
 def test_quadfit_all_pixels_collide(qf, flowaux_oracle):
     # every pixel is sent to one target: its list overflows, and 5 addresses per channel take every atomic
     n, c, h, w = 1, 3, 40, 70
