@@ -83,7 +83,7 @@ __device__ __forceinline__ Fit fit_pixel(const float* __restrict__ a, const floa
   const unsigned p = (unsigned)h * W + w;
   const float idx = w + fl[p];       // QF.cu:31-32
   const float idy = h + fl[HW + p];
-  f.inside = !(idx > W - 1 || idx < 0 || idy > H - 1 || idy < 0);  // QF.cu:35
+  f.inside = idx <= W - 1 && idx >= 0 && idy <= H - 1 && idy >= 0;  // QF.cu:35; a NaN displacement counts as outside
   f.validX = f.validY = 0;
   f.c00 = f.ax = f.ay = f.bx = f.by = f.fx = f.fy = 0.f;
   f.ix = f.iy = 0;
@@ -457,7 +457,7 @@ __device__ __forceinline__ void locate(TilePx& s, const float* __restrict__ fl, 
   if (!valid) return;
   const float idx = x + fl[s.p];
   const float idy = y + fl[HW + s.p];
-  if (idx > W - 1 || idx < 0 || idy > H - 1 || idy < 0) return;
+  if (!(idx <= W - 1 && idx >= 0 && idy <= H - 1 && idy >= 0)) return;  // QF.cu:35; NaN counts as outside
   s.inside = true;
   s.ix = (int)floor(idx + 0.5);
   s.iy = (int)floor(idy + 0.5);

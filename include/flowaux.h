@@ -23,7 +23,8 @@ extern "C" {
  *              (The reference kernel indexes a 2-channel tensor, quadFit.cu:314, while its Python module
  *              hands over 3 channels, cudaQuadFit/QuadFitting.py:53; the channel count is explicit here.)
  *   out      : (n,3,ih,iw) = (offset in x, offset in y, fitted score); all three are zero where
- *              the displaced pixel leaves the image.  The callee writes 3 channels as the reference
+ *              the displaced pixel leaves the image (a NaN displacement counts as leaving it; the reference
+ *              would index with an undefined integer).  The callee writes 3 channels as the reference
  *              kernel does (quadFit.cu:137,315; the reference binding allocates only 2, QuadFit_cuda.cpp:60).
  */
 int quadfit_forward(const float* im0, const float* im1, const float* flow, float* out, int n, int ic, int ih,

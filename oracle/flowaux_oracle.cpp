@@ -74,7 +74,9 @@ Fit<R> fit_pixel(const R* im0, const R* im1, const R* flow, int n, int d, int H,
   // QF.cu:31-38
   const R idx = w + fl[(size_t)h * W + w];
   const R idy = h + fl[HW + (size_t)h * W + w];
-  if (idx > W - 1 || idx < 0 || idy > H - 1 || idy < 0) {
+  // (written so that a NaN displacement counts as leaving the image; the reference's form of the test lets it
+  // through and then indexes with an undefined integer)
+  if (!(idx <= W - 1 && idx >= 0 && idy <= H - 1 && idy >= 0)) {
     f.inside = false;
     return f;
   }

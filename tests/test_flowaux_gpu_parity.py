@@ -97,6 +97,17 @@ def test_quadfit_flow_that_scatters_the_tile(qf, flowaux_oracle):
     check_quadfit(qf, flowaux_oracle, d, "scattered")
 
 
+def test_quadfit_non_finite_displacements_count_as_outside(qf, flowaux_oracle):
+    d = random_quadfit(1, 3, 20, 70, seed=34)
+    d["flow"][0, 0, 3, 5] = np.nan
+    d["flow"][0, 1, 4, 6] = np.nan
+    d["flow"][0, 0, 5, 7] = np.inf
+    d["flow"][0, 1, 6, 8] = -np.inf
+    out = check_quadfit(qf, flowaux_oracle, d, "non-finite flow")
+    for y, x in ((3, 5), (4, 6), (5, 7), (6, 8)):
+        assert (out[0, :, y, x] == 0).all()
+
+
 def test_quadfit_all_pixels_collide(qf, flowaux_oracle):
     # every pixel is sent to one target: its list overflows, and 5 addresses per channel take every atomic
     n, c, h, w = 1, 3, 40, 70
