@@ -182,6 +182,157 @@ def bench_flowaux(args, cfg, d):
     print(json.dumps(out))
 
 
+def hierarchy_inputs(cfg, n, seed=0):
+    """Config 3: per level the confidence / flow of tv_inputs, one guidance-image pyramid per sample."""
+    import numpy as np
+
+    from customnetworklayers_amd import workloads
+
+    rng = np.random.default_rng(seed)
+    top = cfg["levels"][-1]
+    imgs_top = [workloads.smooth_image(rng, *top) for _ in range(n)]
+    levels = []
+    for lvl, (h, w) in enumerate(cfg["levels"]):
+        d = workloads.tv_inputs(n, cfg["c"], h, w, seed=seed + 10 + lvl, **cfg["gen"])
+        f = top[0] // h
+        d["img"] = np.stack([im[::f, ::f] for im in imgs_top])[:, None].astype(np.float32)
+        levels.append(d)
+    return levels
+
+
+def bench_hierarchy(args, cfg):
+    """Config 3: three TV layers (ids 0,1,2) coarse to fine with the glue between the levels on the device, then the
+    backward passes fine to coarse.  One step = all of it."""
+    import torch
+
+    from customnetworklayers_amd import hierarchy
+    from customnetworklayers_amd._lib import lib
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+
+    dev = torch.device("cuda:0")
+    n, c, its = cfg["n"], cfg["c"], cfg["its"]
+    levels = hierarchy_inputs(cfg, n)
+    t = [{k: torch.from_numpy(v).to(dev) for k, v in d.items()} for d in levels]
+    nl = len(t)
+    h0, w0 = cfg["levels"][0]
+    _, wx0, wy0 = hierarchy.next_level_forward(torch.zeros((n, c, h0 // 2, w0 // 2), dtype=torch.float32, device=dev), t[0]["img"])
+    pxit = sum(n * h * w * 2 * (its // 2) for h, w in cfg["levels"])
+    glue_ev = []
+
+    def step(time_glue=False, per_level=None):
+        feeds, b, wx, wy = [], t[0]["db"], wx0, wy0
+        for lvl in range(nl):
+            feeds.append((wx, wy, b))
+            (sol,) = ext.forward(wx, wy, t[lvl]["dc"], b, b, its, lvl)
+            if lvl + 1 < nl:
+                if time_glue:
+                    e = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+                    e[0].record()
+                b, wx, wy = hierarchy.next_level_forward(sol, t[lvl + 1]["img"])
+                if time_glue:
+                    e[1].record()
+                    glue_ev.append(("fwd", lvl, e))
+        up = t[-1]["grad"]
+        for lvl in reversed(range(nl)):
+            wx, wy, b = feeds[lvl]
+            g = ext.backward(up, wx, wy, t[lvl]["dc"], b, its, lvl)
+            if per_level is not None:
+                ms, cnt = ctypes.c_double(0), ctypes.c_int(0)
+                lib.tvinpaint_profile_read(ctypes.byref(ms), ctypes.byref(cnt))
+                per_level[lvl] = (ms.value, cnt.value)
+            if lvl > 0:
+                if time_glue:
+                    e = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+                    e[0].record()
+                up = hierarchy.next_level_backward(g[3], g[4])
+                if time_glue:
+                    e[1].record()
+                    glue_ev.append(("bwd", lvl, e))
+        return g
+
+    for lvl in range(nl):
+        ext.reset_id(lvl)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    # one more, untimed step with event pairs around the glue launches and around each level's adjoint pair launches
+    per_level = {}
+    lib.tvinpaint_profile(1)
+    step(time_glue=True, per_level=per_level)
+    torch.cuda.synchronize()
+    lib.tvinpaint_profile(0)
+    glue_ms = {"fwd": 0.0, "bwd": 0.0}
+    for kind, lvl, e in glue_ev:
+        glue_ms[kind] += e[0].elapsed_time(e[1])
+    # glue bytes: forward reads sol and the fine image, writes up, wx, wy; backward reads two fine gradients, writes one coarse
+    fine = [n * h * w for h, w in cfg["levels"][1:]]
+    glue_bytes = {"fwd": sum(4 * (p // 4 * c + p + p * c + 2 * p) for p in fine), "bwd": sum(4 * (2 * p * c + p // 4 * c) for p in fine)}
+    bpp = algorithmic_bytes_per_pixel(c, "tv")
+    top_ms, top_cnt = per_level[nl - 1]
+    h, w = cfg["levels"][-1]
+    k_ms = top_ms / max(top_cnt, 1)
+    k_bytes = 2 * bpp["adjoint"] * n * h * w
+    achieved = k_bytes / (k_ms * 1e-3) / 1e9 if k_ms > 0 else 0.0
+    sec = elapsed / args.steps
+    out = {
+        "metric": "TV-FISTA hierarchy fwd+bwd Mpixel-iter/s, %d levels up to %dx%dx%dx%d; achieved HBM GB/s vs peak" % (nl, n, c, h, w),
+        "value": round(pxit / sec / 1e6, 2), "unit": "Mpixel-iter/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "three TV layers coarse to fine with device glue, N=%d, C=%d, levels %s, %d iterations each (config 3)"
+                               % (n, c, "/".join("%dx%d" % l for l in cfg["levels"]), its), "pixel_iterations_per_step": pxit},
+        "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(bpp["total"] * pxit / sec / 1e9, 1),
+                      "frac_of_hbm_peak": round(bpp["total"] * pxit / sec / 1e9 / HBM_PEAK_GBS, 4),
+                      "glue_forward_ms": round(glue_ms["fwd"], 4), "glue_backward_ms": round(glue_ms["bwd"], 4),
+                      "glue_forward_GBps": round(glue_bytes["fwd"] / (glue_ms["fwd"] * 1e-3) / 1e9, 1),
+                      "glue_backward_GBps": round(glue_bytes["bwd"] / (glue_ms["bwd"] * 1e-3) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "kernel": "tvstrip::tv_adjoint_strip2<2,false,false> at the finest level", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": k_bytes, "adjoint_steps_per_launch": 2, "avg_launch_ms": round(k_ms, 5), "launches_timed": top_cnt},
+    }
+    if not args.no_cpu_baseline:
+        import oracle.oracle_lib as oracle_lib
+
+        tv, aux = oracle_lib.TVOracle(), oracle_lib.FlowAuxOracle()
+        tv.set_quirks()
+        one = [{k: v[:1] for k, v in d.items()} for d in levels]
+
+        def once():
+            t1 = time.perf_counter()
+            feeds, b = [], one[0]["db"]
+            wx, wy = aux.edge_weights(one[0]["img"], 10.0)
+            for lvl in range(nl):
+                feeds.append((wx, wy, b))
+                tv.reset_id(lvl)
+                sol = tv.forward(wx, wy, one[lvl]["dc"], b, b, its, lvl)
+                if lvl + 1 < nl:
+                    b = aux.upsample2x(sol, 2.0)
+                    wx, wy = aux.edge_weights(one[lvl + 1]["img"], 10.0)
+            up = one[-1]["grad"].copy()
+            for lvl in reversed(range(nl)):
+                wx, wy, b = feeds[lvl]
+                g = tv.backward(up.copy(), wx, wy, one[lvl]["dc"], b, its, lvl)
+                if lvl > 0:
+                    up = aux.upsample2x_adjoint(g[3], g[4], 2.0)
+            return time.perf_counter() - t1
+
+        import multiprocessing
+        avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else multiprocessing.cpu_count()
+        cores = min(avail, int(os.environ.get("OMP_NUM_THREADS", "0") or avail))
+        tv.set_threads(cores)
+        aux.set_threads(cores)
+        once()
+        t_all = min(once(), once())
+        out["cpu_baseline"] = dict(value=round(pxit / n / t_all / 1e6, 3), unit="Mpixel-iter/s", cores=cores, kind="port",
+                                   sample="1 of %d samples, all levels, fwd+bwd, best of 2" % n, host_cpu_count=os.cpu_count())
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -189,7 +340,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", type=int, default=1,
-                    help="workload index (1 = headline TV layer, 2 = TGV layer, 5 = quadratic fit, 6 = median)")
+                    help="workload index (1 = headline TV layer, 2 = TGV layer, 3 = three-level TV hierarchy, 5 = quadratic fit, 6 = median)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
@@ -202,6 +353,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    from customnetworklayers_amd.workloads import CONFIGS
+    if CONFIGS[args.config]["kind"] == "tv_hierarchy":
+        return bench_hierarchy(args, CONFIGS[args.config])
     cfg, d = config_inputs(args.config, seed=0)
     if cfg["kind"] in ("quadfit", "median"):
         return bench_flowaux(args, cfg, d)
