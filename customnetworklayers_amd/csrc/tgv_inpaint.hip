@@ -701,6 +701,7 @@ struct Slot {
   int run = 0;
   int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
   bool forward_done = false;
+  bool x05_last_valid = false;  // the forward left the last segment's x05 rows in the ring: the backward need not recompute it
   std::vector<int> iterations;
   std::vector<float> steps;
   int max_inter_its = 0;
@@ -1031,6 +1032,7 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   hipStream_t stream = (hipStream_t)stream_;
   Slot& s = g_slots[id];
   s.forward_done = false;
+  s.x05_last_valid = false;
   rc = prepare_slot(s, n, ic, ih, iw, its, stream);
   if (rc) return rc;
   const size_t S3 = state_count(s), SB = S3 * sizeof(float);
@@ -1056,6 +1058,9 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
     scale_weights(s, stream, dx, dy);
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, SB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, SB, hipMemcpyDeviceToDevice, stream));
+    const char* keep_env = getenv("INPAINT_KEEP_LAST");  // =0: the backward pass recomputes every segment, as the reference does
+    const bool keep_last = !(keep_env && strcmp(keep_env, "0") == 0) && !s.iterations.empty();
+    const int kl = keep_last ? s.iterations.back() : K;  // first iteration of the last segment
     if (forward_pairs(s)) {
       // two iterations per launch; K and every checkpoint index are even, the ping-pong alternates per pair
       auto Yp = [&](int k) { int i = ck_index(k); return (i >= 0 && k < K) ? s.ckpt_y + (size_t)i * S3 : s.ypp[(k >> 1) & 1]; };
@@ -1064,13 +1069,19 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
         int i = ck_index(k);
         return i >= 0 ? s.ckpt_x + (size_t)i * S3 : s.xpp[(k >> 1) & 1];
       };
-      for (int k = 0; k < K; k += 2)
-        launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), nullptr, nullptr, s.steps[k],
+      // the iterations of the last segment also store their x05 rows: the backward pass starts with that segment
+      // and would otherwise recompute exactly these values (TGV.cu:2775-2814) first
+      for (int k = 0; k < K; k += 2) {
+        float* h0 = k >= kl ? s.x05 + (size_t)(k - kl) * S3 : nullptr;
+        launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + S3 : nullptr, s.steps[k],
                             s.steps[k + 1]);
+      }
     } else {
       for (int k = 0; k < K; k++)
-        launch_forward(s, stream, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
+        launch_forward(s, stream, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1),
+                       k >= kl ? s.x05 + (size_t)(k - kl) * S3 : nullptr, s.steps[k]);
     }
+    s.x05_last_valid = keep_last;
   }
   INPAINT_HIP(hipGetLastError());
   s.forward_done = true;
@@ -1149,8 +1160,12 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     const int len = 2 * ((lastIt - k0) / 2);
     const float* cky = s.ckpt_y + (size_t)outer * S3;
     const float* ckx = s.ckpt_x + (size_t)outer * S3;
-    // recompute the segment, keeping x05 (TGV.cu:2775-2814)
-    if (forward_pairs(s)) {
+    // recompute the segment, keeping x05 (TGV.cu:2775-2814) -- unless it is the last segment and the forward pass
+    // left its x05 rows in the ring
+    const bool have_x05 = outer == nseg - 1 && s.x05_last_valid;
+    s.x05_last_valid = false;
+    if (have_x05) {
+    } else if (forward_pairs(s)) {
       for (int j = 0; j < len; j += 2) {  // segments have even length
         const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
         const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];

@@ -388,6 +388,7 @@ struct Slot {
   int run = 0;
   int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
   bool forward_done = false;
+  bool x05_last_valid = false;  // the forward left the last segment's x05 rows in the ring: the backward need not recompute it
   std::vector<int> iterations;
   std::vector<float> steps;
   int max_inter_its = 0;
@@ -489,6 +490,10 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
 bool force_tile_path() {
   const char* e = getenv("INPAINT_TV_PATH");
   return e && strcmp(e, "tile") == 0;
+}
+bool keep_last_segment() {  // INPAINT_KEEP_LAST=0: the backward pass recomputes every segment, as the reference does
+  const char* e = getenv("INPAINT_KEEP_LAST");
+  return !(e && strcmp(e, "0") == 0);
 }
 int strip_rows(int n, int ih, int iw, int cols, const char* env_name) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap
@@ -674,6 +679,7 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   hipStream_t stream = (hipStream_t)stream_;
   Slot& s = g_slots[id];
   s.forward_done = false;
+  s.x05_last_valid = false;
   rc = prepare_slot(s, n, ic, ih, iw, its, stream);
   if (rc) return rc;
   const size_t F = field_count(s), FB = F * sizeof(float);
@@ -700,6 +706,8 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   } else {
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, FB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, FB, hipMemcpyDeviceToDevice, stream));
+    const bool keep_last = keep_last_segment() && !s.iterations.empty();
+    const int kl = keep_last ? s.iterations.back() : K;  // first iteration of the last segment
     if (forward_pairs(s)) {
       // two iterations per launch; K is even and so is every checkpoint index.  The intermediate
       // iterate k+1 stays in registers, so the ping-pong alternates per pair.
@@ -709,13 +717,19 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
         int i = ck_index(k);
         return i >= 0 ? s.ckpt_x + (size_t)i * F : s.xpp[(k >> 1) & 1];
       };
-      for (int k = 0; k < K; k += 2)
-        launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), nullptr, nullptr, s.steps[k],
+      // the iterations of the last segment also store their x05 rows: the backward pass starts with that segment
+      // and would otherwise recompute exactly these values (TV.cu:1678-1687) first
+      for (int k = 0; k < K; k += 2) {
+        float* h0 = k >= kl ? s.x05 + (size_t)(k - kl) * F : nullptr;
+        launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + F : nullptr, s.steps[k],
                             s.steps[k + 1]);
+      }
     } else {
       for (int k = 0; k < K; k++)
-        launch_forward(s, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1), nullptr, s.steps[k]);
+        launch_forward(s, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1),
+                       k >= kl ? s.x05 + (size_t)(k - kl) * F : nullptr, s.steps[k]);
     }
+    s.x05_last_valid = keep_last;
   }
   INPAINT_HIP(hipGetLastError());
   s.forward_done = true;
@@ -761,8 +775,12 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     bool flushed = false;
     const float* cky = s.ckpt_y + (size_t)outer * F;
     const float* ckx = s.ckpt_x + (size_t)outer * F;
-    // recompute the segment, keeping x05 (TV.cu:1678-1687)
-    if (forward_pairs(s)) {
+    // recompute the segment, keeping x05 (TV.cu:1678-1687) -- unless it is the last segment and the forward pass
+    // left its x05 rows in the ring
+    const bool have_x05 = outer == nseg - 1 && s.x05_last_valid;
+    s.x05_last_valid = false;
+    if (have_x05) {
+    } else if (forward_pairs(s)) {
       for (int j = 0; j < len; j += 2) {  // segments have even length
         const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
         const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];

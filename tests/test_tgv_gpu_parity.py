@@ -328,3 +328,34 @@ def test_module_surface_and_autograd(ext, tgv_oracle):
     ref = run_oracle(tgv_oracle, d, 14, 3)
     got_grads = [t.grad.permute(2, 0, 1).unsqueeze(0).cpu().numpy() for t in (tx, ty, tc, tb, ti)]
     compare("module", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 40, 130, 20), (1, 1, 30, 70, 9), (1, 3, 20, 64, 6)])
+def test_last_segment_kept_by_the_forward_or_recomputed(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
+    # the forward pass leaves the last segment's x05 rows in the ring and the backward pass uses them once; a second
+    # backward on the same forward, and INPAINT_KEEP_LAST=0, take the recompute path -- all three give the same bits
+    d = varying_inputs(n, c, h, w, seed=55)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    ext.reset_id(2)
+    (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+    first = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+    state = ext.get_state(2)
+    ext.reset_id(2)
+    (sol2,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+    ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+    ext.reset_id(2)  # fresh guard state, then a forward whose backward runs twice
+    (sol3,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+    ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+    ext.set_state(2, [0.0] * 6)
+    again = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+    for a, b in zip(first, again):
+        assert torch.equal(a, b)
+    compare("kept", (sol.cpu().numpy(), [g.cpu().numpy() for g in first], None), ref)
+    monkeypatch.setenv("INPAINT_KEEP_LAST", "0")
+    got = run_gpu(ext, d, its, 2)
+    compare("recomputed", got, ref)
+    for a, b in zip(first, got[1]):
+        assert np.array_equal(a.cpu().numpy(), b)
+    assert state is not None
