@@ -992,7 +992,8 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const long long waves = (long long)sx * sy * s.n;
 #define TGV_PAIR_ARGS                                                                                                      \
   s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], \
-      s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, tA, tB, R, sx, sy
+      s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih,  \
+      s.iw, tA, tB, R, sx, sy
   if (split) {
     const dim3 grid((unsigned)((waves + 7) / 8 * 8)), block(128);
     if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, true>), grid, block, 0, stream, TGV_PAIR_ARGS);
@@ -1181,6 +1182,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       }
     }
     int timed_run = 0;
+    bool flushed = false;  // the pair that ends the segment adds the segment sums to the totals itself
     if (adjoint_pairs(s)) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
       // `pp_src` = the g05 / g_x buffer the next launch reads; it flips once per launch
       int j = len - 1;
@@ -1216,6 +1218,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
           launch_adjoint_pair<true>(s, stream, c, b, xa, xb, cky, s.g05[pp_src], s.g05[1 - pp_src], s.gxk[pp_src],
                                     s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr, s.steps[k0 + j],
                                     s.steps[k0 + j - 1]);
+          flushed = true;
         }
         pp_src = 1 - pp_src;
       }
@@ -1241,11 +1244,13 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       }
     }
     // fp32 segment sums into the fp64 totals (TGV.cu:2944)
-    const int a = s.acc_cur;
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[a], s.tot_gc, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
-    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
-    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[a], s.tot_gb, (long long)F);
+    if (!flushed) {
+      const int a = s.acc_cur;
+      hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[a], s.tot_gc, (long long)P);
+      hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
+      hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
+      hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[a], s.tot_gb, (long long)F);
+    }
     lastIt = k0;
   }
 
