@@ -1170,8 +1170,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       for (int j = 0; j < len; j += 2) {  // segments have even length
         const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
         const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];
-        launch_forward_pair(s, stream, c, b, xin, s.xpp[((j >> 1) + 1) & 1], yin, s.ypp[((j >> 1) + 1) & 1],
-                            s.x05 + (size_t)j * S3, s.x05 + (size_t)(j + 1) * S3, s.steps[k0 + j], s.steps[k0 + j + 1]);
+        const bool last = j + 2 >= len;  // nobody reads the iterates the segment's last pair would write
+        launch_forward_pair(s, stream, c, b, xin, last ? nullptr : s.xpp[((j >> 1) + 1) & 1], yin,
+                            last ? nullptr : s.ypp[((j >> 1) + 1) & 1], s.x05 + (size_t)j * S3, s.x05 + (size_t)(j + 1) * S3,
+                            s.steps[k0 + j], s.steps[k0 + j + 1]);
       }
     } else {
       for (int j = 0; j < len; j++) {

@@ -256,6 +256,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     float tB, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
+  const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
   const size_t HW = (size_t)H * W, CHW = HW * C;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
@@ -426,12 +427,14 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
           const Upd u = update(pyB[0][ch], pyB[1][ch], pyB[2][ch], t, aFa, aG1y, aG2y, pc, rc1B, pbb[ch], pxB[0][ch],
                                pxB[1][ch], pxB[2][ch], tB);
           if (store_lane) {
-            stg(yo_p[0][ch], roffB, u.yn);
-            stg(yo_p[1][ch], roffB, u.y1o);
-            stg(yo_p[2][ch], roffB, u.y2o);
-            stg(xo_p[0][ch], roffB, u.x_loc);
-            stg(xo_p[1][ch], roffB, u.y1n);
-            stg(xo_p[2][ch], roffB, u.y2n);
+            if (store_xy) {
+              stg(yo_p[0][ch], roffB, u.yn);
+              stg(yo_p[1][ch], roffB, u.y1o);
+              stg(yo_p[2][ch], roffB, u.y2o);
+              stg(xo_p[0][ch], roffB, u.x_loc);
+              stg(xo_p[1][ch], roffB, u.y1n);
+              stg(xo_p[2][ch], roffB, u.y2n);
+            }
             if (X05) {
               stg(xb_p[0][ch], roffB, u.xh);
               stg(xb_p[1][ch], roffB, u.y1n);

@@ -290,6 +290,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     int N, int H, int W, float tA, float tB, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
+  const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
   const size_t HW = (size_t)H * W;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
@@ -407,8 +408,10 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
           float xh, x_loc, yn;
           update(pyB[ch], e1_above, from_left_lane(e2), e1, e2, pc, rc1B, pbb[ch], pxB[ch], tB, xh, x_loc, yn);
           if (store_lane) {
-            stg(yo_p[ch], roffB, yn);
-            stg(xo_p[ch], roffB, x_loc);
+            if (store_xy) {
+              stg(yo_p[ch], roffB, yn);
+              stg(xo_p[ch], roffB, x_loc);
+            }
             if (X05) stg(xb_p[ch], roffB, xh);
           }
         }
