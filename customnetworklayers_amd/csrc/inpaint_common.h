@@ -169,13 +169,20 @@ __device__ inline unsigned int wave_sum_u(unsigned int v) {
   return v;
 }
 
-// pass 1: sum, max, counts, position of the last non-finite entry.  One set of atomics per block.
-// With clamp_mean (TGV) an entry above max_tol enters the mean as max_tol; the TV layer's mean
-// takes it as it is.
+// pass 1: sum, max, counts, position of the last non-finite entry (one set of atomics per block); with clamp_mean
+// (TGV) an entry above max_tol enters the mean as max_tol, the TV layer's mean takes it as it is.
+// pass 2 (does nothing unless pass 1 saw a non-finite entry): sum of |g| behind the last one.
+// The five tensors of one backward in one launch each for pass 1, pass 2 and the final scaling (blockIdx.y picks
+// the tensor; blocks beyond a tensor's own grid find nothing to do).
+struct GuardJobs {
+  const void* ptr[5];
+  long long n[5];
+  int is_f32[5];
+};
+
 template <class T>
-__global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__ g, long long n,
-                                                           GuardStats* __restrict__ st, double max_tol,
-                                                           bool clamp_mean = false) {
+__device__ __forceinline__ void guard_reduce_body(const T* __restrict__ g, long long n, GuardStats* __restrict__ st,
+                                                  double max_tol, bool clamp_mean) {
   __shared__ double s_sum[4];
   __shared__ unsigned long long s_mx[4], s_last[4];
   __shared__ unsigned int s_above[4], s_invalid[4];
@@ -222,11 +229,16 @@ __global__ __launch_bounds__(256) void guard_reduce_kernel(const T* __restrict__
   }
 }
 
-// pass 2 (does nothing unless pass 1 saw a non-finite entry): sum of |g| behind the last one
+static __global__ __launch_bounds__(256) void guard_reduce_many(GuardJobs jobs, GuardStats* __restrict__ st, double max_tol,
+                                                                bool clamp_mean) {
+  const int k = blockIdx.y;
+  if (jobs.is_f32[k]) guard_reduce_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
+  else guard_reduce_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
+}
+
 template <class T>
-__global__ __launch_bounds__(256) void guard_tail_kernel(const T* __restrict__ g, long long n,
-                                                         GuardStats* __restrict__ st, double max_tol = 0,
-                                                         bool clamp_mean = false) {
+__device__ __forceinline__ void guard_tail_body(const T* __restrict__ g, long long n, GuardStats* __restrict__ st,
+                                                double max_tol, bool clamp_mean) {
   if (st->num_invalid == 0) return;
   const long long start = (long long)st->last_invalid1;
   double s = 0;
@@ -237,6 +249,13 @@ __global__ __launch_bounds__(256) void guard_tail_kernel(const T* __restrict__ g
   }
   s = wave_sum(s);
   if ((threadIdx.x & 63) == 0 && s != 0) atomicAdd(&st->tail_sum, s);
+}
+
+static __global__ __launch_bounds__(256) void guard_tail_many(GuardJobs jobs, GuardStats* __restrict__ st, double max_tol,
+                                                              bool clamp_mean) {
+  const int k = blockIdx.y;
+  if (jobs.is_f32[k]) guard_tail_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
+  else guard_tail_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
 }
 
 struct GuardCounts {
@@ -338,25 +357,6 @@ __device__ inline T guard_limit(T v, const GuardParams& p) {
   return v;
 }
 
-// Guarded fp64 total -> fp32 output: limit, kill / rescale, global multiplier, then the chain
-// factor of the weight scaling (TVInpaintFista.cu:1795-1818; TGVInpaintFistaBetas.cu:3024-3050).
-// The chain factor is chain_const, or chain_per_sample[i / per_sample] when that pointer is given.
-static __global__ __launch_bounds__(256) void finalize_f64(const double* __restrict__ total, float* __restrict__ out,
-                                                           long long n, const GuardState* __restrict__ gs, int k,
-                                                           GuardParams p, float global_mult, double chain_const,
-                                                           const double* __restrict__ chain_per_sample,
-                                                           long long per_sample) {
-  const double mult = gs->scale[k];
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    double v = guard_limit(total[i], p);
-    if (mult != 1.0) v = (mult == 0.0) ? 0.0 : v * mult;
-    const float f = (float)(v * global_mult);
-    const double chain = chain_per_sample ? chain_per_sample[i / per_sample] : chain_const;
-    out[i] = (chain == 1.0) ? f : (float)(chain * (double)f);
-  }
-}
-
 // Gradient wrt the starting point, guarded as a float tensor (TVInpaintFista.cu:1784-1791,1816).
 static __global__ __launch_bounds__(256) void finalize_f32(const float* __restrict__ src, float* __restrict__ out,
                                                            long long n, const GuardState* __restrict__ gs, int k,
@@ -367,6 +367,37 @@ static __global__ __launch_bounds__(256) void finalize_f32(const float* __restri
     float v = guard_limit(src[i], p);
     if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
     out[i] = 0.0f + v;
+  }
+}
+
+// Guarded fp64 totals -> fp32 outputs, the four tensors of one backward in one launch (blockIdx.y picks the tensor):
+// limit, kill / rescale, global multiplier, then the chain factor of the weight scaling (TVInpaintFista.cu:1795-1818;
+// TGVInpaintFistaBetas.cu:3024-3050).  The chain factor is chain_const, or chain_per_sample[i / per_sample] when that
+// pointer is given.
+struct FinalizeJobs {
+  const double* total[4];
+  float* out[4];
+  long long n[4];
+  double chain_const[4];
+  const double* chain_per_sample[4];
+  long long per_sample[4];
+};
+static __global__ __launch_bounds__(256) void finalize_many(FinalizeJobs jobs, const GuardState* __restrict__ gs, GuardParams p,
+                                                            float global_mult) {
+  const int k = blockIdx.y;
+  const double mult = gs->scale[k];
+  const double* __restrict__ total = jobs.total[k];
+  float* __restrict__ out = jobs.out[k];
+  const double* __restrict__ chain_per_sample = jobs.chain_per_sample[k];
+  const double chain_const = jobs.chain_const[k];
+  const long long n = jobs.n[k], per_sample = jobs.per_sample[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x) {
+    double v = guard_limit(total[i], p);
+    if (mult != 1.0) v = (mult == 0.0) ? 0.0 : v * mult;
+    const float f = (float)(v * global_mult);
+    const double chain = chain_per_sample ? chain_per_sample[i / per_sample] : chain_const;
+    out[i] = (chain == 1.0) ? f : (float)(chain * (double)f);
   }
 }
 

@@ -1263,29 +1263,32 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
   const long long cnts[5] = {(long long)P, (long long)(2 * P), (long long)(2 * P), (long long)F, (long long)F};
-  for (int k = 0; k < 4; k++) {
-    hipLaunchKernelGGL(guard_reduce_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k],
-                       cnts[k], st + k, kGuard.max_tolerance, true);
-    hipLaunchKernelGGL(guard_tail_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k], cnts[k],
-                       st + k, kGuard.max_tolerance, true);
+  GuardJobs jobs;
+  long long longest = 0;
+  for (int k = 0; k < 5; k++) {
+    jobs.ptr[k] = k < 4 ? (const void*)tots[k] : (const void*)s.gi_u;
+    jobs.n[k] = cnts[k];
+    jobs.is_f32[k] = k == 4;
+    longest = std::max(longest, cnts[k]);
   }
-  hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gi_u, cnts[4],
-                     st + 4, kGuard.max_tolerance, true);
-  hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gi_u, cnts[4],
-                     st + 4, kGuard.max_tolerance, true);
+  hipLaunchKernelGGL(guard_reduce_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, kGuard.max_tolerance, true);
+  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, kGuard.max_tolerance, true);
   GuardCounts gcnt;
   for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
   hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
-  const double* no_chain = nullptr;
   const long long HW2 = 2LL * ih * iw;
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gc, gc, (long long)P, s.guard, 0, kGuard,
-                     kGlobalGMult, 1.0, no_chain, 1LL);
-  hipLaunchKernelGGL(finalize_f64, dim3(g2P), dim3(256), 0, stream, s.tot_gx, gx, (long long)(2 * P), s.guard, 1, kGuard,
-                     kGlobalGMult, 0.0, (const double*)s.Ls, HW2);
-  hipLaunchKernelGGL(finalize_f64, dim3(g2P), dim3(256), 0, stream, s.tot_gy, gy, (long long)(2 * P), s.guard, 2, kGuard,
-                     kGlobalGMult, 0.0, (const double*)s.Ls, HW2);
-  hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, kGuard,
-                     kGlobalGMult, 1.0, no_chain, 1LL);
+  FinalizeJobs fin;
+  float* outs[4] = {gc, gx, gy, gb};
+  for (int k = 0; k < 4; k++) {
+    const bool weights = k == 1 || k == 2;  // gx, gy carry the per-sample weight scaling (TGV.cu:3027-3046)
+    fin.total[k] = tots[k];
+    fin.out[k] = outs[k];
+    fin.n[k] = cnts[k];
+    fin.chain_const[k] = weights ? 0.0 : 1.0;
+    fin.chain_per_sample[k] = weights ? (const double*)s.Ls : nullptr;
+    fin.per_sample[k] = weights ? HW2 : 1;
+  }
+  hipLaunchKernelGGL(finalize_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, kGlobalGMult);
   hipLaunchKernelGGL(tgv_finalize_init, dim3(grid1d((long long)S3)), dim3(256), 0, stream, gi_src, gi,
                      (long long)ic * ih * iw, (long long)S3, s.guard, kGuard);
   INPAINT_HIP(hipGetLastError());

@@ -879,28 +879,30 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
   const long long cnts[5] = {(long long)P, (long long)P, (long long)P, (long long)F, (long long)F};
-  for (int k = 0; k < 4; k++) {
-    hipLaunchKernelGGL(guard_reduce_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k],
-                       cnts[k], st + k, kGuard.max_tolerance, false);
-    hipLaunchKernelGGL(guard_tail_kernel<double>, dim3(guard_grid(cnts[k])), dim3(256), 0, stream, tots[k], cnts[k],
-                       st + k, 0.0, false);
+  GuardJobs jobs;
+  long long longest = 0;
+  for (int k = 0; k < 5; k++) {
+    jobs.ptr[k] = k < 4 ? (const void*)tots[k] : (const void*)s.gx_final;
+    jobs.n[k] = cnts[k];
+    jobs.is_f32[k] = k == 4;
+    longest = std::max(longest, cnts[k]);
   }
-  hipLaunchKernelGGL(guard_reduce_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gx_final, cnts[4],
-                     st + 4, kGuard.max_tolerance, false);
-  hipLaunchKernelGGL(guard_tail_kernel<float>, dim3(guard_grid(cnts[4])), dim3(256), 0, stream, s.gx_final, cnts[4],
-                     st + 4, 0.0, false);
+  hipLaunchKernelGGL(guard_reduce_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, kGuard.max_tolerance, false);
+  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, 0.0, false);
   GuardCounts gcnt;
   for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
   hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
-  const double* no_chain = nullptr;
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gc, gc, (long long)P, s.guard, 0, kGuard,
-                     kGlobalGMult, 1.0, no_chain, 1LL);
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gx, gx, (long long)P, s.guard, 1, kGuard,
-                     kGlobalGMult, (double)kL, no_chain, 1LL);
-  hipLaunchKernelGGL(finalize_f64, dim3(gP), dim3(256), 0, stream, s.tot_gy, gy, (long long)P, s.guard, 2, kGuard,
-                     kGlobalGMult, (double)kL, no_chain, 1LL);
-  hipLaunchKernelGGL(finalize_f64, dim3(gF), dim3(256), 0, stream, s.tot_gb, gb, (long long)F, s.guard, 3, kGuard,
-                     kGlobalGMult, 1.0, no_chain, 1LL);
+  FinalizeJobs fin;
+  float* outs[4] = {gc, gx, gy, gb};
+  for (int k = 0; k < 4; k++) {
+    fin.total[k] = tots[k];
+    fin.out[k] = outs[k];
+    fin.n[k] = cnts[k];
+    fin.chain_const[k] = (k == 1 || k == 2) ? (double)kL : 1.0;  // gx, gy carry the weight scaling (TV.cu:1797-1818)
+    fin.chain_per_sample[k] = nullptr;
+    fin.per_sample[k] = 1;
+  }
+  hipLaunchKernelGGL(finalize_many, dim3(gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, kGlobalGMult);
   hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gx_final, gi, (long long)F, s.guard, 4, kGuard);
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TV.cu:1829
