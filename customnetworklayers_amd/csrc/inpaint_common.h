@@ -121,12 +121,18 @@ struct GuardStats {
   unsigned int num_above, num_invalid;
 };
 
+constexpr int kGuardBlocks = 256;  // blocks per tensor in pass 1, each leaves one partial record
+
 struct GuardState {  // lives in device memory, one per id
   double av[5];      // running means: C, X, Y, B, I
   double scale[5];   // multiplier chosen for the current backward (1, mult, or 0)
   double report[25]; // per tensor: mean |g|, max |g|, num_above, num_invalid, action
   GuardStats stats[5];
+  // pass 1 leaves per-block records here; they are combined in a fixed order (no atomics on one address, which
+  // this GPU serialises at the memory side, and a mean that does not depend on the order of arrival)
+  GuardStats partial[5][kGuardBlocks];
 };
+constexpr size_t kGuardHeaderBytes = offsetof(GuardState, partial);  // what the host reads back
 
 // The decision rule, shared by the device kernel and the host-side test hook.
 // Returns 0 plain / 1 rescaled / 2 killed.
@@ -189,6 +195,7 @@ __device__ __forceinline__ void guard_reduce_body(const T* __restrict__ g, long 
   double s = 0;
   unsigned long long mx = 0, last = 0;
   unsigned int above = 0, invalid = 0;
+#pragma unroll 4
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (long long)gridDim.x * blockDim.x) {
     T v = g[i];
@@ -221,26 +228,69 @@ __device__ __forceinline__ void guard_reduce_body(const T* __restrict__ g, long 
       above += s_above[k];
       invalid += s_invalid[k];
     }
-    if (s != 0) atomicAdd(&st->sum, s);
-    if (mx) atomicMax(&st->max_bits, mx);
-    if (last) atomicMax(&st->last_invalid1, last);
-    if (above) atomicAdd(&st->num_above, above);
-    if (invalid) atomicAdd(&st->num_invalid, invalid);
+    GuardStats r;
+    r.sum = s; r.tail_sum = 0; r.max_bits = mx; r.last_invalid1 = last; r.num_above = above; r.num_invalid = invalid;
+    *st = r;
   }
 }
 
-static __global__ __launch_bounds__(256) void guard_reduce_many(GuardJobs jobs, GuardStats* __restrict__ st, double max_tol,
+// launch with grid (kGuardBlocks, 5)
+static __global__ __launch_bounds__(256) void guard_reduce_many(GuardJobs jobs, GuardState* __restrict__ gs, double max_tol,
                                                                 bool clamp_mean) {
   const int k = blockIdx.y;
-  if (jobs.is_f32[k]) guard_reduce_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
-  else guard_reduce_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
+  GuardStats* st = &gs->partial[k][blockIdx.x];
+  if (jobs.is_f32[k]) guard_reduce_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], st, max_tol, clamp_mean);
+  else guard_reduce_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], st, max_tol, clamp_mean);
+}
+
+// the partial records of one tensor, combined by one wavefront in a fixed order (lane l takes records l, l+64, ...)
+__device__ __forceinline__ GuardStats guard_combine(const GuardStats* __restrict__ part, int lane) {
+  double s = 0;
+  unsigned long long mx = 0, last = 0;
+  unsigned int above = 0, invalid = 0;
+  for (int i = lane; i < kGuardBlocks; i += 64) {
+    s += part[i].sum;
+    mx = part[i].max_bits > mx ? part[i].max_bits : mx;
+    last = part[i].last_invalid1 > last ? part[i].last_invalid1 : last;
+    above += part[i].num_above;
+    invalid += part[i].num_invalid;
+  }
+  GuardStats r;
+  r.sum = wave_sum(s);
+  r.tail_sum = 0;
+  r.max_bits = wave_max(mx);
+  r.last_invalid1 = wave_max(last);
+  r.num_above = wave_sum_u(above);
+  r.num_invalid = wave_sum_u(invalid);
+  r.sum = __shfl(r.sum, 0, 64);
+  r.max_bits = __shfl(r.max_bits, 0, 64);
+  r.last_invalid1 = __shfl(r.last_invalid1, 0, 64);
+  r.num_above = __shfl(r.num_above, 0, 64);
+  r.num_invalid = __shfl(r.num_invalid, 0, 64);
+  return r;
 }
 
 template <class T>
-__device__ __forceinline__ void guard_tail_body(const T* __restrict__ g, long long n, GuardStats* __restrict__ st,
-                                                double max_tol, bool clamp_mean) {
-  if (st->num_invalid == 0) return;
-  const long long start = (long long)st->last_invalid1;
+__device__ __forceinline__ void guard_tail_body(const T* __restrict__ g, long long n, const GuardStats* __restrict__ part,
+                                                GuardStats* __restrict__ st, double max_tol, bool clamp_mean) {
+  __shared__ unsigned long long s_last[4];
+  __shared__ unsigned int s_invalid[4];
+  {
+    unsigned long long last = 0;
+    unsigned int invalid = 0;
+    for (int i = threadIdx.x; i < kGuardBlocks; i += blockDim.x) {
+      last = part[i].last_invalid1 > last ? part[i].last_invalid1 : last;
+      invalid += part[i].num_invalid;
+    }
+    last = wave_max(last);
+    invalid = wave_sum_u(invalid);
+    if ((threadIdx.x & 63) == 0) { s_last[threadIdx.x >> 6] = last; s_invalid[threadIdx.x >> 6] = invalid; }
+    __syncthreads();
+  }
+  if (s_invalid[0] + s_invalid[1] + s_invalid[2] + s_invalid[3] == 0) return;
+  unsigned long long last1 = s_last[0];
+  for (int k = 1; k < 4; k++) last1 = s_last[k] > last1 ? s_last[k] : last1;
+  const long long start = (long long)last1;
   double s = 0;
   for (long long i = start + (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (long long)gridDim.x * blockDim.x) {
@@ -251,42 +301,46 @@ __device__ __forceinline__ void guard_tail_body(const T* __restrict__ g, long lo
   if ((threadIdx.x & 63) == 0 && s != 0) atomicAdd(&st->tail_sum, s);
 }
 
-static __global__ __launch_bounds__(256) void guard_tail_many(GuardJobs jobs, GuardStats* __restrict__ st, double max_tol,
+static __global__ __launch_bounds__(256) void guard_tail_many(GuardJobs jobs, GuardState* __restrict__ gs, double max_tol,
                                                               bool clamp_mean) {
   const int k = blockIdx.y;
-  if (jobs.is_f32[k]) guard_tail_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
-  else guard_tail_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], st + k, max_tol, clamp_mean);
+  if (jobs.is_f32[k])
+    guard_tail_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], gs->partial[k], &gs->stats[k], max_tol, clamp_mean);
+  else
+    guard_tail_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], gs->partial[k], &gs->stats[k], max_tol, clamp_mean);
 }
 
 struct GuardCounts {
   long long n[5];
 };
 
-// single thread: turn the statistics into per-tensor multipliers and update the running means.
-// Sequential running mean of the reference, av_{i+1} = (|g_i| + i av_i)/(i+1) with a reset to
-// 1000*running mean at every non-finite entry, in closed form.
-static __global__ void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, GuardParams p) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  for (int k = 0; k < 5; k++) {
-    GuardStats& s = gs->stats[k];
-    const double n = (double)cnt.n[k];
-    double av_gc;
-    if (cnt.n[k] <= 0) {
-      av_gc = 0;
-    } else if (s.num_invalid == 0) {
-      av_gc = s.sum / n;
-    } else {
-      av_gc = ((double)s.last_invalid1 * (gs->av[k] * 1000.) + s.tail_sum) / n;
-    }
-    double mult = 1.0;
-    int action = guard_decide_rule(run, av_gc, gs->av[k], mult, p);
-    gs->scale[k] = mult;
-    gs->report[5 * k + 0] = av_gc;
-    gs->report[5 * k + 1] = __longlong_as_double((long long)s.max_bits);
-    gs->report[5 * k + 2] = s.num_above;
-    gs->report[5 * k + 3] = s.num_invalid;
-    gs->report[5 * k + 4] = action;
+// One wavefront per tensor (launch with 320 threads): combine the partial records, then lane 0 turns the
+// statistics into the tensor's multiplier and updates its running mean.  Sequential running mean of the reference,
+// av_{i+1} = (|g_i| + i av_i)/(i+1) with a reset to 1000*running mean at every non-finite entry, in closed form.
+static __global__ __launch_bounds__(320) void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, GuardParams p) {
+  const int k = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (k >= 5 || blockIdx.x != 0) return;
+  GuardStats s = guard_combine(gs->partial[k], lane);
+  if (lane != 0) return;
+  s.tail_sum = gs->stats[k].tail_sum;  // pass 2 adds into it (cleared before pass 1)
+  gs->stats[k] = s;
+  const double n = (double)cnt.n[k];
+  double av_gc;
+  if (cnt.n[k] <= 0) {
+    av_gc = 0;
+  } else if (s.num_invalid == 0) {
+    av_gc = s.sum / n;
+  } else {
+    av_gc = ((double)s.last_invalid1 * (gs->av[k] * 1000.) + s.tail_sum) / n;
   }
+  double mult = 1.0;
+  int action = guard_decide_rule(run, av_gc, gs->av[k], mult, p);
+  gs->scale[k] = mult;
+  gs->report[5 * k + 0] = av_gc;
+  gs->report[5 * k + 1] = __longlong_as_double((long long)s.max_bits);
+  gs->report[5 * k + 2] = s.num_above;
+  gs->report[5 * k + 3] = s.num_invalid;
+  gs->report[5 * k + 4] = action;
 }
 
 static __global__ void guard_clear_kernel(GuardState* gs) {

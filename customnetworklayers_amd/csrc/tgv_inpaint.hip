@@ -734,7 +734,7 @@ int fetch_running_means(Slot& s) {
   if (s.guard) {
     GuardState host;
     INPAINT_HIP(hipStreamSynchronize(s.stream));
-    INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+    INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
     for (int k = 0; k < 5; k++) s.pending_av[k] = host.av[k];
   }
   return 0;
@@ -1260,7 +1260,6 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
   hipLaunchKernelGGL(tgv_gather_u, dim3(grid1d((long long)F)), dim3(256), 0, stream, gi_src, s.gi_u,
                      (long long)ic * ih * iw, (long long)F);
-  GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
   const long long cnts[5] = {(long long)P, (long long)(2 * P), (long long)(2 * P), (long long)F, (long long)F};
   GuardJobs jobs;
@@ -1271,11 +1270,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     jobs.is_f32[k] = k == 4;
     longest = std::max(longest, cnts[k]);
   }
-  hipLaunchKernelGGL(guard_reduce_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, kGuard.max_tolerance, true);
-  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, kGuard.max_tolerance, true);
+  hipLaunchKernelGGL(guard_reduce_many, dim3(kGuardBlocks, 5), dim3(256), 0, stream, jobs, s.guard, kGuard.max_tolerance, true);
+  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, s.guard, kGuard.max_tolerance, true);
   GuardCounts gcnt;
   for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
-  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
+  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(320), 0, stream, s.guard, gcnt, s.run, kGuard);
   const long long HW2 = 2LL * ih * iw;
   FinalizeJobs fin;
   float* outs[4] = {gc, gx, gy, gb};
@@ -1334,7 +1333,7 @@ int tgvinpaint_guard_stats(int id, double* stats25) {
   if (!s.guard) return fail(INPAINT_ERR_PAIRING, "id %d holds no state", id);
   GuardState host;
   INPAINT_HIP(hipStreamSynchronize(s.stream));
-  INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+  INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
   memcpy(stats25, host.report, sizeof(host.report));
   return 0;
 }

@@ -418,7 +418,7 @@ int fetch_running_means(Slot& s) {
   if (s.guard) {
     GuardState host;
     INPAINT_HIP(hipStreamSynchronize(s.stream));
-    INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+    INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
     for (int k = 0; k < 5; k++) s.pending_av[k] = host.av[k];
   }
   return 0;
@@ -876,7 +876,6 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
 
   // output guard on the device (TV.cu:1760-1791), then scale and store (TV.cu:1795-1818)
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
-  GuardStats* st = reinterpret_cast<GuardStats*>(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, stats));
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
   const long long cnts[5] = {(long long)P, (long long)P, (long long)P, (long long)F, (long long)F};
   GuardJobs jobs;
@@ -887,11 +886,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     jobs.is_f32[k] = k == 4;
     longest = std::max(longest, cnts[k]);
   }
-  hipLaunchKernelGGL(guard_reduce_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, kGuard.max_tolerance, false);
-  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, st, 0.0, false);
+  hipLaunchKernelGGL(guard_reduce_many, dim3(kGuardBlocks, 5), dim3(256), 0, stream, jobs, s.guard, kGuard.max_tolerance, false);
+  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, s.guard, 0.0, false);
   GuardCounts gcnt;
   for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
-  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(1), 0, stream, s.guard, gcnt, s.run, kGuard);
+  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(320), 0, stream, s.guard, gcnt, s.run, kGuard);
   FinalizeJobs fin;
   float* outs[4] = {gc, gx, gy, gb};
   for (int k = 0; k < 4; k++) {
@@ -947,7 +946,7 @@ int tvinpaint_guard_stats(int id, double* stats25) {
   if (!s.guard) return fail(INPAINT_ERR_PAIRING, "id %d holds no state", id);
   GuardState host;
   INPAINT_HIP(hipStreamSynchronize(s.stream));
-  INPAINT_HIP(hipMemcpy(&host, s.guard, sizeof(GuardState), hipMemcpyDeviceToHost));
+  INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
   memcpy(stats25, host.report, sizeof(host.report));
   return 0;
 }
