@@ -251,9 +251,9 @@ template <int C, bool X05>
 __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
-    const float* __restrict__ xin, float* __restrict__ xout, const float* __restrict__ yin,
-    float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b, int N, int H, int W, float tA,
-    float tB, int R, int strips_x, int strips_y) {
+    const float* __restrict__ xin, const float* __restrict__ xin_aux, float* __restrict__ xout,
+    const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
+    int store_x_aux, int N, int H, int W, float tA, float tB, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
@@ -275,7 +275,9 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
 #pragma unroll
     for (int v = 0; v < 3; v++) {
       const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
-      y_p[v][ch] = yin + q; x_p[v][ch] = xin + q;
+      // v1, v2 of an iterate equal the x05 rows of the iteration that made it (no prox on them): a recompute launch
+      // reads them from the ring (xin_aux) instead of a second copy, and does not write that copy (store_x_aux == 0)
+      y_p[v][ch] = yin + q; x_p[v][ch] = ((v > 0 && xin_aux) ? xin_aux : xin) + q;
       yo_p[v][ch] = yout + q; xo_p[v][ch] = xout + q;
       xa_p[v][ch] = X05 ? x05a + q : nullptr; xb_p[v][ch] = X05 ? x05b + q : nullptr;
     }
@@ -432,8 +434,10 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
               stg(yo_p[1][ch], roffB, u.y1o);
               stg(yo_p[2][ch], roffB, u.y2o);
               stg(xo_p[0][ch], roffB, u.x_loc);
-              stg(xo_p[1][ch], roffB, u.y1n);
-              stg(xo_p[2][ch], roffB, u.y2n);
+              if (store_x_aux) {
+                stg(xo_p[1][ch], roffB, u.y1n);
+                stg(xo_p[2][ch], roffB, u.y2n);
+              }
             }
             if (X05) {
               stg(xb_p[0][ch], roffB, u.xh);
