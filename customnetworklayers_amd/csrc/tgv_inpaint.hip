@@ -906,17 +906,21 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* c, const flo
 template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                                const float* xin_aux, float* xout, const float* yin, float* yout, float* x05a, float* x05b,
-                               bool store_x_aux, float tA, float tB) {
+                               bool store_x_aux, float tA, float tB, bool ring, float tP) {
   const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_FWD_ROWS");
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (x05a)
+  if (x05a && ring)
+    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, true, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+                       xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, tP, R, sx,
+                       sy);
+  else if (x05a)
     hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
-                       xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+                       xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
   else
     hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
-                       xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+                       xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
 }
 
 bool forward_pairs(const Slot& s) {
@@ -925,12 +929,16 @@ bool forward_pairs(const Slot& s) {
   return use_strip(s);
 }
 
-// xin_aux (optional): where v1, v2 of the input iterate are read from instead of xin; store_x_aux: write v1, v2 of xout
+// xin_aux (optional): where v1, v2 of the input iterate are read from instead of xin; store_x_aux: write v1, v2 of xout.
+// ring: xin / yin are the x05 rows of the two iterations before this pair and the iterate is rebuilt from them (tP:
+// extrapolation factor of the iteration that made it); such a launch writes x05 rows only.
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                          const float* yin, float* yout, float* x05a, float* x05b, float tA, float tB,
-                         const float* xin_aux = nullptr, bool store_x_aux = true) {
-  if (s.ic == 1) launch_forward_pair_strip<1>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB);
-  else launch_forward_pair_strip<2>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB);
+                         const float* xin_aux = nullptr, bool store_x_aux = true, bool ring = false, float tP = 0.f) {
+  if (s.ic == 1)
+    launch_forward_pair_strip<1>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP);
+  else
+    launch_forward_pair_strip<2>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP);
 }
 
 template <int C, bool END>
@@ -1170,14 +1178,16 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     s.x05_last_valid = false;
     if (have_x05) {
     } else if (forward_pairs(s)) {
+      // Only the x05 rows are kept.  The first pair starts from the checkpoint; every later pair rebuilds its input
+      // iterate from the two x05 rows before it (the forward pass's own expressions), so no iterate travels
+      // through memory.
       for (int j = 0; j < len; j += 2) {  // segments have even length
-        const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
-        const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];
-        const bool last = j + 2 >= len;  // nobody reads the iterates the segment's last pair would write
-        // v1, v2 of the input iterate are the x05 rows of iteration j-1, already in the ring
-        launch_forward_pair(s, stream, c, b, xin, last ? nullptr : s.xpp[((j >> 1) + 1) & 1], yin,
-                            last ? nullptr : s.ypp[((j >> 1) + 1) & 1], s.x05 + (size_t)j * S3, s.x05 + (size_t)(j + 1) * S3,
-                            s.steps[k0 + j], s.steps[k0 + j + 1], j == 0 ? nullptr : s.x05 + (size_t)(j - 1) * S3, false);
+        if (j == 0)
+          launch_forward_pair(s, stream, c, b, ckx, nullptr, cky, nullptr, s.x05, s.x05 + S3, s.steps[k0], s.steps[k0 + 1]);
+        else
+          launch_forward_pair(s, stream, c, b, s.x05 + (size_t)(j - 2) * S3, nullptr, s.x05 + (size_t)(j - 1) * S3, nullptr,
+                              s.x05 + (size_t)j * S3, s.x05 + (size_t)(j + 1) * S3, s.steps[k0 + j], s.steps[k0 + j + 1],
+                              nullptr, false, true, s.steps[k0 + j - 1]);
       }
     } else {
       for (int j = 0; j < len; j++) {

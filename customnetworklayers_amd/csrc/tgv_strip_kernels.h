@@ -247,13 +247,17 @@ struct Fwd2Row {
   float y[3][C], x[3][C], bb[C], c, wxs, wys, bxs, bys;
 };
 
-template <int C, bool X05>
+// RING (recompute launches after a segment's first): the input iterate is not read but rebuilt from the x05 rows of
+// the two iterations before it, which the ring holds anyway -- u: x = prox(x05[j-1]), y = x + tP (x - prox(x05[j-2]));
+// v1, v2: x = x05[j-1], y = x + tP (x - x05[j-2]), the forward pass's own expressions -- and no iterate is written.
+// yin / xin then point at those two rows.
+template <int C, bool X05, bool RING = false>
 __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
     const float* __restrict__ xin, const float* __restrict__ xin_aux, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int store_x_aux, int N, int H, int W, float tA, float tB, int R, int strips_x, int strips_y) {
+    int store_x_aux, int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
@@ -290,24 +294,49 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const unsigned row = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4;
     const unsigned row_w = (unsigned)min(max(h, 0), h_hi) * W4;
     const unsigned row_p = (unsigned)min(max(h, h_lo), h_hi) * W4;
-    in.c = ldg(cf_p, row_p + wc);
+    const unsigned row_c = RING ? row : row_p;  // rebuilding y needs c and b wherever y is read
+    in.c = ldg(cf_p, row_c + wc);
     in.wxs = ldg(wx_p, row_w + wc);
     in.wys = ldg(wy_p, row_w + wc);
     in.bxs = ldg(bx_p, row_w + wc);
     in.bys = ldg(by_p, row_w + wc);
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      in.bb[ch] = ldg(b_p[ch], row_p + wc);
+      in.bb[ch] = ldg(b_p[ch], row_c + wc);
 #pragma unroll
       for (int v = 0; v < 3; v++) {
         in.y[v][ch] = ldg(y_p[v][ch], row + wc);
-        in.x[v][ch] = ldg(x_p[v][ch], row_p + wc);
+        in.x[v][ch] = ldg(x_p[v][ch], row_c + wc);
       }
     }
+  };
+  // Huber-1 prox of the data term (TGV.cu:1740-1744)
+  auto prox = [&](float yt, float c, float rc1, float bv) {
+    float x_loc = div_by(c * bv + yt, 1.f + c, rc1);
+    const float lo = yt - c, hi = yt + c;
+    if (lo > 1.f + bv) x_loc = lo;
+    if (hi < bv - 1.f) x_loc = hi;
+    return x_loc;
   };
   auto absorb = [&](int k, Fwd2Row<C>& o) {
     const int h = g.hs - 2 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
+    if (RING) {  // o.y holds x05[j-1], o.x holds x05[j-2]
+      const float rc1 = rcp_refined(1.f + o.c);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xj = prox(o.y[0][ch], o.c, rc1, o.bb[ch]);
+        const float xm = prox(o.x[0][ch], o.c, rc1, o.bb[ch]);
+        o.x[0][ch] = xj;
+        o.y[0][ch] = xj + tP * (xj - xm);  // TGV.cu:1773
+#pragma unroll
+        for (int v = 1; v < 3; v++) {
+          const float xv = o.y[v][ch], xmv = o.x[v][ch];
+          o.x[v][ch] = xv;
+          o.y[v][ch] = xv + tP * (xv - xmv);  // TGV.cu:1686-1690
+        }
+      }
+    }
     o.wxs = (ok && rmask) ? o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? o.wys : 0.f;
     o.bxs = ok ? o.bxs : 0.f;
@@ -368,10 +397,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     u.xh = yt;
     u.y1n = y1n;
     u.y2n = y2n;
-    float x_loc = div_by(c * bv + yt, 1.f + c, rc1);
-    const float lo = yt - c, hi = yt + c;
-    if (lo > 1.f + bv) x_loc = lo;
-    if (hi < bv - 1.f) x_loc = hi;
+    const float x_loc = prox(yt, c, rc1, bv);
     u.x_loc = x_loc;
     u.yn = x_loc + tm * (x_loc - x0);
     return u;

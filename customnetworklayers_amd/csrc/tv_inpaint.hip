@@ -532,17 +532,20 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, co
 template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                                const float* b, const float* xin, float* xout, const float* yin, float* yout,
-                               float* x05a, float* x05b, float tA, float tB) {
+                               float* x05a, float* x05b, float tA, float tB, bool ring, float tP) {
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_FWD_ROWS");
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (x05a)
+  if (x05a && ring)
+    hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, true, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin,
+                       yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB, tP, R, sx, sy);
+  else if (x05a)
     hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
-                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
   else
     hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, false>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
-                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
 }
 
 bool forward_pairs(const Slot& s) {
@@ -551,14 +554,16 @@ bool forward_pairs(const Slot& s) {
   return !force_tile_path() && s.ic >= 1 && s.ic <= 4;
 }
 
+// ring: xin / yin are the x05 rows of the two iterations before this pair and the iterate is rebuilt from them
+// (tP: extrapolation factor of the iteration that made it); such a launch writes x05 rows only
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                          const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05a,
-                         float* x05b, float tA, float tB) {
+                         float* x05b, float tA, float tB, bool ring = false, float tP = 0.f) {
   switch (s.ic) {
-    case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
-    case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
-    case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
-    default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB); break;
+    case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
+    case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
+    case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
+    default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
   }
 }
 
@@ -781,13 +786,17 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     s.x05_last_valid = false;
     if (have_x05) {
     } else if (forward_pairs(s)) {
+      // Only the x05 rows are kept.  The first pair starts from the checkpoint; every later pair rebuilds its input
+      // iterate from the two x05 rows before it (x_j = prox(x05[j-1]), y_j = x_j + s_{j-1} (x_j - prox(x05[j-2])),
+      // the forward pass's own expressions), so no iterate travels through memory.
       for (int j = 0; j < len; j += 2) {  // segments have even length
-        const float* yin = (j == 0) ? cky : s.ypp[(j >> 1) & 1];
-        const float* xin = (j == 0) ? ckx : s.xpp[(j >> 1) & 1];
-        const bool last = j + 2 >= len;  // nobody reads the iterates the segment's last pair would write
-        launch_forward_pair(s, stream, dx, dy, c, b, xin, last ? nullptr : s.xpp[((j >> 1) + 1) & 1], yin,
-                            last ? nullptr : s.ypp[((j >> 1) + 1) & 1], s.x05 + (size_t)j * F, s.x05 + (size_t)(j + 1) * F,
-                            s.steps[k0 + j], s.steps[k0 + j + 1]);
+        if (j == 0)
+          launch_forward_pair(s, stream, dx, dy, c, b, ckx, nullptr, cky, nullptr, s.x05, s.x05 + F, s.steps[k0],
+                              s.steps[k0 + 1]);
+        else
+          launch_forward_pair(s, stream, dx, dy, c, b, s.x05 + (size_t)(j - 2) * F, nullptr, s.x05 + (size_t)(j - 1) * F,
+                              nullptr, s.x05 + (size_t)j * F, s.x05 + (size_t)(j + 1) * F, s.steps[k0 + j],
+                              s.steps[k0 + j + 1], true, s.steps[k0 + j - 1]);
       }
     } else {
       for (int j = 0; j < len; j++) {

@@ -282,12 +282,15 @@ struct Fwd2Row {
   float y[C], x[C], bb[C], c, wxs, wys;
 };
 
-template <int C, bool X05>
+// RING (recompute launches after a segment's first): the input iterate is not read but rebuilt from the x05 rows of
+// the two iterations before it, which the ring holds anyway -- x = prox(x05[j-1]), y = x + tP (x - prox(x05[j-2])),
+// the forward pass's own expressions -- and no iterate is written.  yin / xin then point at those two rows.
+template <int C, bool X05, bool RING = false>
 __global__ __launch_bounds__(256) void tv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int N, int H, int W, float tA, float tB, int R, int strips_x, int strips_y) {
+    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
@@ -320,19 +323,38 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     // read from a row the strip needs anyway, so that no cache line is fetched for nothing
     const unsigned row_w = (unsigned)min(max(h, 0), h_hi) * W4;
     const unsigned row_p = (unsigned)min(max(h, h_lo), h_hi) * W4;
-    in.c = ldg(cf_p, row_p + wc);
+    const unsigned row_c = RING ? row : row_p;  // rebuilding y needs c and b wherever y is read
+    in.c = ldg(cf_p, row_c + wc);
     in.wxs = ldg(wx_p, row_w + wc);
     in.wys = ldg(wy_p, row_w + wc);
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       in.y[ch] = ldg(y_p[ch], row + wc);
-      in.x[ch] = ldg(x_p[ch], row_p + wc);
-      in.bb[ch] = ldg(b_p[ch], row_p + wc);
+      in.x[ch] = ldg(x_p[ch], row_c + wc);
+      in.bb[ch] = ldg(b_p[ch], row_c + wc);
     }
+  };
+  // Huber-1 prox of the data term (TV.cu:1286-1292)
+  auto prox = [&](float yt, float c, float rc1, float bv) {
+    float x_loc = div_by(c * bv + yt, 1.f + c, rc1);
+    const float lo = yt - c, hi = yt + c;
+    if (lo > 1.f + bv) x_loc = lo;
+    if (hi < bv - 1.f) x_loc = hi;
+    return x_loc;
   };
   auto absorb = [&](int k, Fwd2Row<C>& o) {
     const int h = g.hs - 2 + k;
     const bool rok = h >= 0 && h < H;
+    if (RING) {  // o.y holds x05[j-1], o.x holds x05[j-2]
+      const float rc1 = rcp_refined(1.f + o.c);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xj = prox(o.y[ch], o.c, rc1, o.bb[ch]);
+        const float xm = prox(o.x[ch], o.c, rc1, o.bb[ch]);
+        o.x[ch] = xj;
+        o.y[ch] = xj + tP * (xj - xm);  // TV.cu:1315
+      }
+    }
     o.wxs = (rok && wx_ok) ? kL * o.wxs : 0.f;
     o.wys = (rok && g.col_ok && h < H - 1) ? kL * o.wys : 0.f;
 #pragma unroll
@@ -358,10 +380,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     yt -= e1;
     yt -= e2;
     xh = yt;
-    x_loc = div_by(c * bv + yt, 1.f + c, rc1);
-    const float lo = yt - c, hi = yt + c;
-    if (lo > 1.f + bv) x_loc = lo;
-    if (hi < bv - 1.f) x_loc = hi;
+    x_loc = prox(yt, c, rc1, bv);
     yn = x_loc + t * (x_loc - xold);
   };
 
