@@ -22,6 +22,7 @@ def _load():
     lib.tvinpaint_set_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_reset_id.argtypes = [_int]
     lib.tvinpaint_guard_stats.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tvinpaint_keep_iterates.argtypes = [_int, _int]
     lib.tvinpaint_slot_bytes.argtypes = [_int]
     lib.tvinpaint_slot_bytes.restype = ctypes.c_longlong
     lib.tvinpaint_schedule.argtypes = [_int, ctypes.POINTER(_int), ctypes.POINTER(_int)]
@@ -39,6 +40,7 @@ def _load():
     lib.tgvinpaint_set_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
     lib.tgvinpaint_reset_id.argtypes = [_int]
     lib.tgvinpaint_guard_stats.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
+    lib.tgvinpaint_keep_iterates.argtypes = [_int, _int]
     lib.tgvinpaint_slot_bytes.argtypes = [_int]
     lib.tgvinpaint_slot_bytes.restype = ctypes.c_longlong
     lib.tgvinpaint_lipschitz.argtypes = [_int, ctypes.POINTER(ctypes.c_double), _int]

@@ -701,7 +701,14 @@ struct Slot {
   int run = 0;
   int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
   bool forward_done = false;
-  bool x05_last_valid = false;  // the forward left the last segment's x05 rows in the ring: the backward need not recompute it
+  // Which x05 rows the forward pass keeps for the backward pass (tgvinpaint_keep_iterates): 0 none (every segment is
+  // recomputed from its checkpoint, the reference's order of work), 1 those of the last segment, 2 all of them (no
+  // recompute at all; the ring then has one row per iteration).
+  int keep_mode = 2;
+  int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
+  int x05_mode = 0;     // how the last forward laid its rows out: 2 row = iteration, else row = iteration - first kept
+  int x05_from = 0;     // first iteration whose x05 row the last forward kept
+  bool x05_valid = false;
   std::vector<int> iterations;
   std::vector<float> steps;
   int max_inter_its = 0;
@@ -740,11 +747,15 @@ int fetch_running_means(Slot& s) {
   return 0;
 }
 
-int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t stream) {
+int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode, hipStream_t stream) {
   int dev = -1;
   INPAINT_HIP(hipGetDevice(&dev));
+  std::vector<int> iterations;
+  int max_inter_its = 0;
+  make_schedule(its, iterations, max_inter_its);
+  const int ring_rows = keep_mode == 2 ? std::max(its, 1) : std::max(max_inter_its, 1);
   const bool same = s.arena.base && s.arena.device == dev && s.n == n && s.ic == ic && s.ih == ih &&
-                    s.iw == iw && s.its == its;
+                    s.iw == iw && s.its == its && s.ring_rows >= ring_rows;  // the ring only grows
   s.stream = stream;
   if (same) return 0;
   int rc = fetch_running_means(s);
@@ -753,7 +764,8 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   make_schedule(its, s.iterations, s.max_inter_its);
   make_step_sizes(its, s.steps);
   const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
-  const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)std::max(s.max_inter_its, 1);
+  s.ring_rows = ring_rows;
+  const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)ring_rows;
   size_t need = 0;
   need += Arena::padded(S3, 4) * (2 + 2 + 2 + 2 + 1 + 1) + Arena::padded(S3 * nck, 4) * 2 + Arena::padded(S3 * ring, 4);
   need += Arena::padded(F, 4) * 3 + Arena::padded(F, 8);
@@ -791,6 +803,25 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   INPAINT_HIP(hipMemcpyAsync(s.guard, &init, sizeof(init), hipMemcpyHostToDevice, stream));
   INPAINT_HIP(hipStreamSynchronize(stream));
   return 0;
+}
+
+// The x05 rows the forward pass keeps.  INPAINT_KEEP=0|1|2 overrides the id's setting (INPAINT_KEEP_LAST=0 is the
+// older spelling of INPAINT_KEEP=0); keeping all rows needs its * state bytes, at most INPAINT_KEEP_GB (default 32).
+int resolve_keep_mode(const Slot& s, int n, int ic, int ih, int iw, int its) {
+  int mode = s.keep_mode;
+  if (const char* e = getenv("INPAINT_KEEP_LAST"))
+    if (strcmp(e, "0") == 0) mode = 0;
+  if (const char* e = getenv("INPAINT_KEEP")) {
+    const int v = atoi(e);
+    if (v >= 0 && v <= 2) mode = v;
+  }
+  if (mode == 2) {
+    double gb = 32.0;
+    if (const char* e = getenv("INPAINT_KEEP_GB")) gb = atof(e);
+    const double bytes = 4.0 * 3 * n * ic * (double)ih * iw * its;
+    if (bytes > gb * 1073741824.0) mode = 1;
+  }
+  return mode;
 }
 
 int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int iw, int its, int id) {
@@ -1044,8 +1075,9 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   hipStream_t stream = (hipStream_t)stream_;
   Slot& s = g_slots[id];
   s.forward_done = false;
-  s.x05_last_valid = false;
-  rc = prepare_slot(s, n, ic, ih, iw, its, stream);
+  s.x05_valid = false;
+  const int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
+  rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
   if (rc) return rc;
   const size_t S3 = state_count(s), SB = S3 * sizeof(float);
   const int K = 2 * (its / 2);
@@ -1070,9 +1102,9 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
     scale_weights(s, stream, dx, dy);
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, SB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, SB, hipMemcpyDeviceToDevice, stream));
-    const char* keep_env = getenv("INPAINT_KEEP_LAST");  // =0: the backward pass recomputes every segment, as the reference does
-    const bool keep_last = !(keep_env && strcmp(keep_env, "0") == 0) && !s.iterations.empty();
-    const int kl = keep_last ? s.iterations.back() : K;  // first iteration of the last segment
+    // first iteration whose x05 row is kept, and the ring row of iteration k
+    const int kl = s.iterations.empty() ? K : (keep == 2 ? 0 : (keep == 1 ? s.iterations.back() : K));
+    auto ring_row = [&](int k) { return s.x05 + (size_t)(keep == 2 ? k : k - kl) * S3; };
     if (forward_pairs(s)) {
       // two iterations per launch; K and every checkpoint index are even, the ping-pong alternates per pair
       auto Yp = [&](int k) { int i = ck_index(k); return (i >= 0 && k < K) ? s.ckpt_y + (size_t)i * S3 : s.ypp[(k >> 1) & 1]; };
@@ -1081,19 +1113,21 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
         int i = ck_index(k);
         return i >= 0 ? s.ckpt_x + (size_t)i * S3 : s.xpp[(k >> 1) & 1];
       };
-      // the iterations of the last segment also store their x05 rows: the backward pass starts with that segment
-      // and would otherwise recompute exactly these values (TGV.cu:2775-2814) first
+      // kept iterations also store their x05 rows: the backward pass would otherwise recompute exactly these values
+      // from the checkpoints (TGV.cu:2775-2814)
       for (int k = 0; k < K; k += 2) {
-        float* h0 = k >= kl ? s.x05 + (size_t)(k - kl) * S3 : nullptr;
+        float* h0 = k >= kl ? ring_row(k) : nullptr;
         launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + S3 : nullptr, s.steps[k],
                             s.steps[k + 1]);
       }
     } else {
       for (int k = 0; k < K; k++)
         launch_forward(s, stream, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1),
-                       k >= kl ? s.x05 + (size_t)(k - kl) * S3 : nullptr, s.steps[k]);
+                       k >= kl ? ring_row(k) : nullptr, s.steps[k]);
     }
-    s.x05_last_valid = keep_last;
+    s.x05_valid = kl < K;
+    s.x05_from = kl;
+    s.x05_mode = keep;
   }
   INPAINT_HIP(hipGetLastError());
   s.forward_done = true;
@@ -1174,8 +1208,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     const float* ckx = s.ckpt_x + (size_t)outer * S3;
     // recompute the segment, keeping x05 (TGV.cu:2775-2814) -- unless it is the last segment and the forward pass
     // left its x05 rows in the ring
-    const bool have_x05 = outer == nseg - 1 && s.x05_last_valid;
-    s.x05_last_valid = false;
+    const bool have_x05 = s.x05_valid && k0 >= s.x05_from;
+    // rows of this segment: one per iteration of the whole run when all were kept, else the segment's own ring
+    float* const ring = s.x05 + (s.x05_valid && s.x05_mode == 2 ? (size_t)k0 * S3 : 0);
+    if (!have_x05 || s.x05_mode != 2) s.x05_valid = false;  // a recomputed (or a shared) ring is overwritten below
     if (have_x05) {
     } else if (forward_pairs(s)) {
       // Only the x05 rows are kept.  The first pair starts from the checkpoint; every later pair rebuilds its input
@@ -1183,17 +1219,17 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       // through memory.
       for (int j = 0; j < len; j += 2) {  // segments have even length
         if (j == 0)
-          launch_forward_pair(s, stream, c, b, ckx, nullptr, cky, nullptr, s.x05, s.x05 + S3, s.steps[k0], s.steps[k0 + 1]);
+          launch_forward_pair(s, stream, c, b, ckx, nullptr, cky, nullptr, ring, ring + S3, s.steps[k0], s.steps[k0 + 1]);
         else
-          launch_forward_pair(s, stream, c, b, s.x05 + (size_t)(j - 2) * S3, nullptr, s.x05 + (size_t)(j - 1) * S3, nullptr,
-                              s.x05 + (size_t)j * S3, s.x05 + (size_t)(j + 1) * S3, s.steps[k0 + j], s.steps[k0 + j + 1],
+          launch_forward_pair(s, stream, c, b, ring + (size_t)(j - 2) * S3, nullptr, ring + (size_t)(j - 1) * S3, nullptr,
+                              ring + (size_t)j * S3, ring + (size_t)(j + 1) * S3, s.steps[k0 + j], s.steps[k0 + j + 1],
                               nullptr, false, true, s.steps[k0 + j - 1]);
       }
     } else {
       for (int j = 0; j < len; j++) {
         const float* yin = (j == 0) ? cky : s.ypp[j & 1];
         const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
-        launch_forward(s, stream, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], s.x05 + (size_t)j * S3,
+        launch_forward(s, stream, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1], ring + (size_t)j * S3,
                        s.steps[k0 + j]);
       }
     }
@@ -1204,15 +1240,15 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       int j = len - 1;
       if (outer == nseg - 1 && j >= 0) {
         hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                           s.x05 + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                           ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
                            (long long)ih * iw, (long long)P);
         pp_src = 1;
         j--;
       }
       if (j >= 0 && ((j + 1) & 1)) {  // an odd number of steps is left: one single step, then pairs
-        const float* xa = s.x05 + (size_t)j * S3;
+        const float* xa = ring + (size_t)j * S3;
         if (j > 0)
-          launch_adjoint<false>(s, stream, c, b, xa, s.x05 + (size_t)(j - 1) * S3, nullptr, s.g05[pp_src],
+          launch_adjoint<false>(s, stream, c, b, xa, ring + (size_t)(j - 1) * S3, nullptr, s.g05[pp_src],
                                 s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j]);
         else
           launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[pp_src], s.g05[1 - pp_src], s.gxk[pp_src],
@@ -1221,11 +1257,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
         j--;
       }
       for (; j >= 1; j -= 2) {
-        const float* xa = s.x05 + (size_t)j * S3;
-        const float* xb = s.x05 + (size_t)(j - 1) * S3;
+        const float* xa = ring + (size_t)j * S3;
+        const float* xb = ring + (size_t)(j - 1) * S3;
         if (j - 1 > 0) {
           if (timed_run == 0) g_timer.begin(stream);
-          launch_adjoint_pair<false>(s, stream, c, b, xa, xb, s.x05 + (size_t)(j - 2) * S3, s.g05[pp_src],
+          launch_adjoint_pair<false>(s, stream, c, b, xa, xb, ring + (size_t)(j - 2) * S3, s.g05[pp_src],
                                      s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j],
                                      s.steps[k0 + j - 1]);
           timed_run++;
@@ -1241,13 +1277,13 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     } else
     for (int j = len - 1; j >= 0; j--) {  // reverse sweep (TGV.cu:2851-2933)
       const float t = s.steps[k0 + j];
-      const float* xa = s.x05 + (size_t)j * S3;
+      const float* xa = ring + (size_t)j * S3;
       const int odd = j & 1;
       if (outer == nseg - 1 && j == len - 1) {
         hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
                            s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
-        const float* xb = s.x05 + (size_t)(j - 1) * S3;
+        const float* xb = ring + (size_t)(j - 1) * S3;
         if (timed_run == 0) g_timer.begin(stream);
         launch_adjoint<false>(s, stream, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
                               s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
@@ -1349,6 +1385,13 @@ int tgvinpaint_guard_stats(int id, double* stats25) {
   INPAINT_HIP(hipStreamSynchronize(s.stream));
   INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
   memcpy(stats25, host.report, sizeof(host.report));
+  return 0;
+}
+
+int tgvinpaint_keep_iterates(int id, int mode) {
+  if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  if (mode < 0 || mode > 2) return fail(INPAINT_ERR_ARG, "keep mode %d is not 0, 1 or 2", mode);
+  g_slots[id].keep_mode = mode;
   return 0;
 }
 

@@ -388,7 +388,14 @@ struct Slot {
   int run = 0;
   int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
   bool forward_done = false;
-  bool x05_last_valid = false;  // the forward left the last segment's x05 rows in the ring: the backward need not recompute it
+  // Which x05 rows the forward pass keeps for the backward pass (tvinpaint_keep_iterates): 0 none (every segment is
+  // recomputed from its checkpoint, the reference's order of work), 1 those of the last segment, 2 all of them (no
+  // recompute at all; the ring then has one row per iteration).
+  int keep_mode = 2;
+  int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
+  int x05_mode = 0;     // how the last forward laid its rows out: 2 row = iteration, else row = iteration - first kept
+  int x05_from = 0;     // first iteration whose x05 row the last forward kept
+  bool x05_valid = false;
   std::vector<int> iterations;
   std::vector<float> steps;
   int max_inter_its = 0;
@@ -424,11 +431,15 @@ int fetch_running_means(Slot& s) {
   return 0;
 }
 
-int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t stream) {
+int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode, hipStream_t stream) {
   int dev = -1;
   INPAINT_HIP(hipGetDevice(&dev));
+  std::vector<int> iterations;
+  int max_inter_its = 0;
+  make_schedule(its, iterations, max_inter_its);
+  const int ring_rows = keep_mode == 2 ? std::max(its, 1) : std::max(max_inter_its, 1);
   const bool same = s.arena.base && s.arena.device == dev && s.n == n && s.ic == ic && s.ih == ih &&
-                    s.iw == iw && s.its == its;
+                    s.iw == iw && s.its == its && s.ring_rows >= ring_rows;  // the ring only grows
   s.stream = stream;
   if (same) return 0;
   int rc = fetch_running_means(s);  // the running means survive a change of shape
@@ -437,7 +448,8 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, hipStream_t st
   make_schedule(its, s.iterations, s.max_inter_its);
   make_step_sizes(its, s.steps);
   const size_t F = field_count(s), P = plane_count(s);
-  const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)std::max(s.max_inter_its, 1);
+  s.ring_rows = ring_rows;
+  const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)ring_rows;
   size_t need = 0;
   need += Arena::padded(F, 4) * (2 + 2 + 2 * nck + ring + 2 + 2 + 1 + 2);
   need += Arena::padded(P, 4) * 6;
@@ -491,9 +503,23 @@ bool force_tile_path() {
   const char* e = getenv("INPAINT_TV_PATH");
   return e && strcmp(e, "tile") == 0;
 }
-bool keep_last_segment() {  // INPAINT_KEEP_LAST=0: the backward pass recomputes every segment, as the reference does
-  const char* e = getenv("INPAINT_KEEP_LAST");
-  return !(e && strcmp(e, "0") == 0);
+// The x05 rows the forward pass keeps.  INPAINT_KEEP=0|1|2 overrides the id's setting (INPAINT_KEEP_LAST=0 is the
+// older spelling of INPAINT_KEEP=0); keeping all rows needs its * field bytes, at most INPAINT_KEEP_GB (default 32).
+int resolve_keep_mode(const Slot& s, int n, int ic, int ih, int iw, int its) {
+  int mode = s.keep_mode;
+  if (const char* e = getenv("INPAINT_KEEP_LAST"))
+    if (strcmp(e, "0") == 0) mode = 0;
+  if (const char* e = getenv("INPAINT_KEEP")) {
+    const int v = atoi(e);
+    if (v >= 0 && v <= 2) mode = v;
+  }
+  if (mode == 2) {
+    double gb = 32.0;
+    if (const char* e = getenv("INPAINT_KEEP_GB")) gb = atof(e);
+    const double bytes = 4.0 * n * ic * (double)ih * iw * its;
+    if (bytes > gb * 1073741824.0) mode = 1;
+  }
+  return mode;
 }
 int strip_rows(int n, int ih, int iw, int cols, const char* env_name) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap
@@ -684,8 +710,9 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   hipStream_t stream = (hipStream_t)stream_;
   Slot& s = g_slots[id];
   s.forward_done = false;
-  s.x05_last_valid = false;
-  rc = prepare_slot(s, n, ic, ih, iw, its, stream);
+  s.x05_valid = false;
+  const int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
+  rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
   if (rc) return rc;
   const size_t F = field_count(s), FB = F * sizeof(float);
   const int K = 2 * (its / 2);
@@ -711,8 +738,9 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   } else {
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, FB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
     INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, FB, hipMemcpyDeviceToDevice, stream));
-    const bool keep_last = keep_last_segment() && !s.iterations.empty();
-    const int kl = keep_last ? s.iterations.back() : K;  // first iteration of the last segment
+    // first iteration whose x05 row is kept, and the ring row of iteration k
+    const int kl = s.iterations.empty() ? K : (keep == 2 ? 0 : (keep == 1 ? s.iterations.back() : K));
+    auto ring_row = [&](int k) { return s.x05 + (size_t)(keep == 2 ? k : k - kl) * F; };
     if (forward_pairs(s)) {
       // two iterations per launch; K is even and so is every checkpoint index.  The intermediate
       // iterate k+1 stays in registers, so the ping-pong alternates per pair.
@@ -722,19 +750,21 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
         int i = ck_index(k);
         return i >= 0 ? s.ckpt_x + (size_t)i * F : s.xpp[(k >> 1) & 1];
       };
-      // the iterations of the last segment also store their x05 rows: the backward pass starts with that segment
-      // and would otherwise recompute exactly these values (TV.cu:1678-1687) first
+      // kept iterations also store their x05 rows: the backward pass would otherwise recompute exactly these values
+      // from the checkpoints (TV.cu:1678-1687)
       for (int k = 0; k < K; k += 2) {
-        float* h0 = k >= kl ? s.x05 + (size_t)(k - kl) * F : nullptr;
+        float* h0 = k >= kl ? ring_row(k) : nullptr;
         launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + F : nullptr, s.steps[k],
                             s.steps[k + 1]);
       }
     } else {
       for (int k = 0; k < K; k++)
         launch_forward(s, stream, dx, dy, c, b, Xbuf(k), Xbuf(k + 1), Ybuf(k), Ybuf(k + 1),
-                       k >= kl ? s.x05 + (size_t)(k - kl) * F : nullptr, s.steps[k]);
+                       k >= kl ? ring_row(k) : nullptr, s.steps[k]);
     }
-    s.x05_last_valid = keep_last;
+    s.x05_valid = kl < K;
+    s.x05_from = kl;
+    s.x05_mode = keep;
   }
   INPAINT_HIP(hipGetLastError());
   s.forward_done = true;
@@ -782,8 +812,10 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     const float* ckx = s.ckpt_x + (size_t)outer * F;
     // recompute the segment, keeping x05 (TV.cu:1678-1687) -- unless it is the last segment and the forward pass
     // left its x05 rows in the ring
-    const bool have_x05 = outer == nseg - 1 && s.x05_last_valid;
-    s.x05_last_valid = false;
+    const bool have_x05 = s.x05_valid && k0 >= s.x05_from;
+    // rows of this segment: one per iteration of the whole run when all were kept, else the segment's own ring
+    float* const ring = s.x05 + (s.x05_valid && s.x05_mode == 2 ? (size_t)k0 * F : 0);
+    if (!have_x05 || s.x05_mode != 2) s.x05_valid = false;  // a recomputed (or a shared) ring is overwritten below
     if (have_x05) {
     } else if (forward_pairs(s)) {
       // Only the x05 rows are kept.  The first pair starts from the checkpoint; every later pair rebuilds its input
@@ -791,11 +823,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       // the forward pass's own expressions), so no iterate travels through memory.
       for (int j = 0; j < len; j += 2) {  // segments have even length
         if (j == 0)
-          launch_forward_pair(s, stream, dx, dy, c, b, ckx, nullptr, cky, nullptr, s.x05, s.x05 + F, s.steps[k0],
+          launch_forward_pair(s, stream, dx, dy, c, b, ckx, nullptr, cky, nullptr, ring, ring + F, s.steps[k0],
                               s.steps[k0 + 1]);
         else
-          launch_forward_pair(s, stream, dx, dy, c, b, s.x05 + (size_t)(j - 2) * F, nullptr, s.x05 + (size_t)(j - 1) * F,
-                              nullptr, s.x05 + (size_t)j * F, s.x05 + (size_t)(j + 1) * F, s.steps[k0 + j],
+          launch_forward_pair(s, stream, dx, dy, c, b, ring + (size_t)(j - 2) * F, nullptr, ring + (size_t)(j - 1) * F,
+                              nullptr, ring + (size_t)j * F, ring + (size_t)(j + 1) * F, s.steps[k0 + j],
                               s.steps[k0 + j + 1], true, s.steps[k0 + j - 1]);
       }
     } else {
@@ -803,7 +835,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
         const float* yin = (j == 0) ? cky : s.ypp[j & 1];
         const float* xin = (j == 0) ? ckx : s.xpp[j & 1];
         launch_forward(s, stream, dx, dy, c, b, xin, s.xpp[(j + 1) & 1], yin, s.ypp[(j + 1) & 1],
-                       s.x05 + (size_t)j * F, s.steps[k0 + j]);
+                       ring + (size_t)j * F, s.steps[k0 + j]);
       }
     }
     // reverse sweep (TV.cu:1696-1729)
@@ -815,15 +847,15 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       int j = len - 1;
       if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
         hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                           s.x05 + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                           ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
                            (long long)ih * iw, (long long)P);
         pp_src = 1;
         j--;
       }
       if (j >= 0 && ((j + 1) & 1)) {  // an odd number of steps is left: one single step, then pairs
-        const float* xa = s.x05 + (size_t)j * F;
+        const float* xa = ring + (size_t)j * F;
         if (j > 0)
-          launch_adjoint<false>(s, stream, dx, dy, c, b, xa, s.x05 + (size_t)(j - 1) * F, nullptr, s.g05[pp_src],
+          launch_adjoint<false>(s, stream, dx, dy, c, b, xa, ring + (size_t)(j - 1) * F, nullptr, s.g05[pp_src],
                                 s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j]);
         else
           flushed = launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[pp_src], s.g05[1 - pp_src],
@@ -833,11 +865,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
         j--;
       }
       for (; j >= 1; j -= 2) {
-        const float* xa = s.x05 + (size_t)j * F;
-        const float* xb = s.x05 + (size_t)(j - 1) * F;
+        const float* xa = ring + (size_t)j * F;
+        const float* xb = ring + (size_t)(j - 1) * F;
         if (j - 1 > 0) {
           if (timed_run == 0) g_timer.begin(stream);
-          launch_adjoint_pair<false>(s, stream, dx, dy, c, b, xa, xb, s.x05 + (size_t)(j - 2) * F, s.g05[pp_src],
+          launch_adjoint_pair<false>(s, stream, dx, dy, c, b, xa, xb, ring + (size_t)(j - 2) * F, s.g05[pp_src],
                                      s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j],
                                      s.steps[k0 + j - 1]);
           timed_run++;
@@ -854,13 +886,13 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     } else
     for (int j = len - 1; j >= 0; j--) {
       const float t = s.steps[k0 + j];
-      const float* xa = s.x05 + (size_t)j * F;
+      const float* xa = ring + (size_t)j * F;
       const int odd = j & 1;
       if (outer == nseg - 1 && j == len - 1) {
         hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
                            s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
-        const float* xb = s.x05 + (size_t)(j - 1) * F;
+        const float* xb = ring + (size_t)(j - 1) * F;
         if (timed_run == 0) g_timer.begin(stream);
         launch_adjoint<false>(s, stream, dx, dy, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
                               s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
@@ -957,6 +989,13 @@ int tvinpaint_guard_stats(int id, double* stats25) {
   INPAINT_HIP(hipStreamSynchronize(s.stream));
   INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
   memcpy(stats25, host.report, sizeof(host.report));
+  return 0;
+}
+
+int tvinpaint_keep_iterates(int id, int mode) {
+  if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  if (mode < 0 || mode > 2) return fail(INPAINT_ERR_ARG, "keep mode %d is not 0, 1 or 2", mode);
+  g_slots[id].keep_mode = mode;
   return 0;
 }
 

@@ -15,8 +15,10 @@ class TGVInpaintingFunction(Function):
 
     @staticmethod
     def forward(ctx, dx, dy, dc, db, di, its, pid):
+        # a forward nobody differentiates keeps no intermediate iterates
         outputs = tgvInpaint_cuda_ext.forward(dx.contiguous(), dy.contiguous(), dc.contiguous(),
-                                              db.contiguous(), di.contiguous(), its, pid)
+                                              db.contiguous(), di.contiguous(), its, pid,
+                                              keep=None if any(ctx.needs_input_grad[:5]) else 0)
         sol = outputs[0]
         variables = [dx, dy, dc, db, torch.from_numpy(np.array([its, pid]))]
         ctx.save_for_backward(*variables)

@@ -51,17 +51,22 @@ def _check_shapes(d_x, d_y, d_c, d_b, others):
         raise RuntimeError("all tensors must live on one device")
 
 
-def forward(d_x, d_y, d_c, d_b, d_i, its, id):  # noqa: A002 - the reference's argument name
+def forward(d_x, d_y, d_c, d_b, d_i, its, id, keep=None):  # noqa: A002 - the reference's argument name
     """d_x, d_y: edge weights along W / H, d_c: confidence, (n,1,h,w); d_b: right-hand side and d_i:
-    starting point, (n,c,h,w).  Returns [solution] after 2*floor(its/2) iterations."""
+    starting point, (n,c,h,w).  Returns [solution] after 2*floor(its/2) iterations.
+    keep (not in the reference): keep mode for this one call, see keep_iterates; None = the id's own."""
     for t, name in ((d_x, "d_x"), (d_y, "d_y"), (d_c, "d_c"), (d_b, "d_b"), (d_i, "d_i")):
         _check_input(t, name)
     _check_shapes(d_x, d_y, d_c, d_b, ((d_i, "d_i"),))
     n, c, h, w = d_b.shape
     solution = torch.empty_like(d_b)
+    if keep is not None:
+        _set_keep(id, keep)
     with torch.cuda.device(d_b.device):
         rc = lib.tvinpaint_forward(d_x.data_ptr(), d_y.data_ptr(), d_c.data_ptr(), d_b.data_ptr(), d_i.data_ptr(),
                                    solution.data_ptr(), n, c, h, w, int(its), int(id), _stream(d_b))
+    if keep is not None:
+        _set_keep(id, _keep_modes.get(int(id), 2))
     if rc:
         _raise(rc, "TVInpaint::forward")
     return [solution]
@@ -115,6 +120,29 @@ def reset_id(id):  # noqa: A002
     rc = lib.tvinpaint_reset_id(int(id))
     if rc:
         _raise(rc, "reset_id")
+    _keep_modes.pop(int(id), None)
+
+
+def slot_bytes(id):  # noqa: A002
+    """Bytes of device memory the id's slot owns."""
+    return int(lib.tvinpaint_slot_bytes(int(id)))
+
+
+_keep_modes = {}  # id -> mode set through keep_iterates (the library's default is 2)
+
+
+def _set_keep(id, mode):  # noqa: A002
+    rc = lib.tvinpaint_keep_iterates(int(id), int(mode))
+    if rc:
+        _raise(rc, "keep_iterates")
+
+
+def keep_iterates(id, mode):  # noqa: A002
+    """Which intermediate iterates the forwards on `id` keep for the backward: 0 none (the backward recomputes every
+    segment from its checkpoint, as the reference does), 1 the last segment's, 2 all (default: no recompute, `its`
+    more fields of memory).  The gradients are the same bits in every mode."""
+    _set_keep(id, mode)
+    _keep_modes[int(id)] = int(mode)
 
 
 def guard_stats(id):  # noqa: A002

@@ -46,6 +46,15 @@ int tgvinpaint_get_state(int id, double* state6);
 int tgvinpaint_set_state(int id, const double* state6);
 int tgvinpaint_reset_id(int id);
 
+/* Which intermediate iterates (the x05 rows of TGVInpaintFista.cu:2775-2814) the next forwards on `id` keep for
+ * the backward pass.  0: none -- the backward recomputes every segment from its checkpoint, the reference's order
+ * of work and its memory footprint.  1: those of the last segment.  2 (default): all of them -- its states
+ * (3 fields each) of memory, no recompute, and the fastest backward.  The gradients are the same bits in every
+ * mode.  A forward whose gradients are never asked for is fastest with 0.  Mode 2 falls back to 1 when the rows
+ * would need more than INPAINT_KEEP_GB (default 32) GiB; INPAINT_KEEP=0|1|2 overrides this call.
+ * No counterpart in the reference, which always recomputes. */
+int tgvinpaint_keep_iterates(int id, int mode);
+
 /* Statistics of the last backward's output guard (check_gradUpdate, TGVInpaintFistaHelp.cu:155-177):
  * 5 tensors (C, X, Y, B, I) x {mean |g|, max |g|, count above 5e6, count non-finite, action}.  The
  * guard on I looks at the u block only (TGVInpaintFistaBetas.cu:3014-3021). */

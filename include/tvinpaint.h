@@ -52,6 +52,15 @@ int tvinpaint_reset_id(int id);
  * action (0 plain, 1 rescaled, 2 killed)}.  Waits for the slot's stream. */
 int tvinpaint_guard_stats(int id, double* stats25);
 
+/* Which intermediate iterates (the x05 rows of TVInpaintFista.cu:1678-1687) the next forwards on `id` keep for
+ * the backward pass.  0: none -- the backward recomputes every segment from its checkpoint, the reference's order
+ * of work and its memory footprint (2 sqrt(its) + sqrt(its) fields).  1: those of the last segment.  2 (default):
+ * all of them -- its fields of memory, no recompute, and the fastest backward.  The gradients are the same bits
+ * in every mode.  A forward whose gradients are never asked for is fastest with 0.  Mode 2 falls back to 1 when
+ * the rows would need more than INPAINT_KEEP_GB (default 32) GiB; INPAINT_KEEP=0|1|2 overrides this call.
+ * No counterpart in the reference, which always recomputes. */
+int tvinpaint_keep_iterates(int id, int mode);
+
 /* Bytes of device memory the slot currently owns (0 if none). */
 long long tvinpaint_slot_bytes(int id);
 

@@ -257,31 +257,47 @@ def test_module_surface_and_autograd(ext, tv_oracle):
 
 
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 40, 130, 20), (1, 1, 30, 70, 9), (1, 3, 20, 64, 6)])
-def test_last_segment_kept_by_the_forward_or_recomputed(ext, tv_oracle, n, c, h, w, its, monkeypatch):
-    # the forward pass leaves the last segment's x05 rows in the ring and the backward pass uses them once; a second
-    # backward on the same forward, and INPAINT_KEEP_LAST=0, take the recompute path -- all three give the same bits
+def test_kept_iterates_or_recomputed_segments_give_the_same_bits(ext, tv_oracle, n, c, h, w, its, monkeypatch):
+    # keep mode 2 (default) stores every x05 row in the forward and recomputes nothing; mode 1 keeps the last
+    # segment's rows, which serve one backward; mode 0 recomputes every segment as the reference does.  A second
+    # backward on one forward, a too-small memory budget and the per-call `keep` argument are covered as well.
     d = tv_inputs(n, c, h, w, seed=55, conf_density=0.3)
     ref = run_oracle(tv_oracle, d, its, 2)
     dev = torch.device("cuda:0")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
-    ext.reset_id(2)
-    (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
-    first = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
-    state = ext.get_state(2)
-    ext.reset_id(2)
-    (sol2,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
-    ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
-    ext.reset_id(2)  # fresh guard state, then a forward whose backward runs twice
-    (sol3,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
-    ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
-    ext.set_state(2, [0.0] * 6)
-    again = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
-    for a, b in zip(first, again):
-        assert torch.equal(a, b)
-    compare("kept", (sol.cpu().numpy(), [g.cpu().numpy() for g in first], None), ref)
+
+    def fwd_bwd(twice=False, **kw):
+        ext.reset_id(2)
+        if "mode" in kw:
+            ext.keep_iterates(2, kw["mode"])
+        (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2, **{k: v for k, v in kw.items() if k == "keep"})
+        grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+        if twice:
+            ext.set_state(2, [0.0] * 6)
+            again = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+            for a, b in zip(grads, again):
+                assert torch.equal(a, b)
+        nbytes = ext.slot_bytes(2) if hasattr(ext, "slot_bytes") else 0
+        return sol, grads, nbytes
+
+    sol, first, bytes_all = fwd_bwd(twice=True)
+    compare("all kept", (sol.cpu().numpy(), [g.cpu().numpy() for g in first], None), ref)
+    runs = {"mode 2": fwd_bwd(mode=2, twice=True), "mode 1": fwd_bwd(mode=1, twice=True),
+            "mode 0": fwd_bwd(mode=0, twice=True), "keep=0 once": fwd_bwd(keep=0), "after keep=0": fwd_bwd()}
+    monkeypatch.setenv("INPAINT_KEEP_GB", "0.000001")  # the rows do not fit: the last segment's are kept instead
+    runs["budget"] = fwd_bwd(twice=True)
+    monkeypatch.delenv("INPAINT_KEEP_GB")
+    monkeypatch.setenv("INPAINT_KEEP", "0")
+    runs["env 0"] = fwd_bwd()
+    monkeypatch.delenv("INPAINT_KEEP")
     monkeypatch.setenv("INPAINT_KEEP_LAST", "0")
-    got = run_gpu(ext, d, its, 2)
-    compare("recomputed", got, ref)
-    for a, b in zip(first, got[1]):
-        assert np.array_equal(a.cpu().numpy(), b)
-    assert state is not None
+    runs["env last 0"] = fwd_bwd()
+    for name, (s2, grads, _) in runs.items():
+        assert torch.equal(sol, s2), name
+        for a, b in zip(first, grads):
+            assert torch.equal(a, b), name
+    if bytes_all:  # a slot that recomputes is smaller than one that keeps every row
+        assert runs["mode 0"][2] < bytes_all
+    with pytest.raises(ValueError):
+        ext.keep_iterates(2, 3)
+    ext.reset_id(2)
