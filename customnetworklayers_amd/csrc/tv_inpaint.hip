@@ -754,8 +754,16 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
       // from the checkpoints (TV.cu:1678-1687)
       for (int k = 0; k < K; k += 2) {
         float* h0 = k >= kl ? ring_row(k) : nullptr;
-        launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + F : nullptr, s.steps[k],
-                            s.steps[k + 1]);
+        if (keep == 2 && k >= 2) {
+          // With every x05 row kept the iterate need not travel through memory either: the pair rebuilds it from the
+          // two rows before it, as the recompute launches of the backward pass do, and stores it only where somebody
+          // reads it -- at a checkpoint and at the end.
+          const bool wanted = k + 2 == K || ck_index(k + 2) >= 0;
+          launch_forward_pair(s, stream, dx, dy, c, b, ring_row(k - 2), wanted ? Xp(k + 2) : nullptr, ring_row(k - 1),
+                              wanted ? Yp(k + 2) : nullptr, h0, h0 + F, s.steps[k], s.steps[k + 1], true, s.steps[k - 1]);
+        } else
+          launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + F : nullptr,
+                              s.steps[k], s.steps[k + 1]);
       }
     } else {
       for (int k = 0; k < K; k++)
