@@ -20,8 +20,12 @@ HBM_PEAK_GBS = 8000.0
 # calibration, and writes 68035 KiB; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
 # profiles/tgv_strip_config2_hbm_traffic.txt; configs 5 and 6: profiles/quadfit_config5_*.txt, profiles/median_config6_*.txt).
 # Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: (2 * 87000 + 68035) * 1024, 2: (2 * 166450 + 147340) * 1024,
+MEASURED_TRAFFIC_BYTES = {1: (2 * 86992 + 67886) * 1024, 2: (2 * 165999 + 147003) * 1024,
                           5: (2 * 408180 + 340500) * 1024, 6: (2 * 131080 + 247100) * 1024}
+# HBM bytes of one whole forward+backward (every kernel and copy of a step), from the same two counter runs: the job
+# moves far fewer bytes than the one-round-trip-per-iteration model because two iterations share a launch, the
+# backward recomputes nothing and iterates are rebuilt from the kept x05 rows instead of being stored.
+MEASURED_STEP_BYTES = {1: (2 * 6932008 + 6307040) * 1024, 2: (2 * 13564395 + 14853807) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):
@@ -407,7 +411,11 @@ def main():
         "config": {"workload": cfg["kind"].upper() + " inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
                                % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
         "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
-                      "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4)},
+                      "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4),
+                      "effective_bytes_per_pixel_iteration": (round(MEASURED_STEP_BYTES[args.config] / pxit, 1)
+                                                              if args.config in MEASURED_STEP_BYTES else None),
+                      "effective_GBps": (round(MEASURED_STEP_BYTES[args.config] / (elapsed / args.steps) / 1e9, 1)
+                                         if args.config in MEASURED_STEP_BYTES else None)},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.config), "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
