@@ -23,6 +23,7 @@ def _load():
     lib.tvinpaint_reset_id.argtypes = [_int]
     lib.tvinpaint_guard_stats.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_keep_iterates.argtypes = [_int, _int]
+    lib.tvinpaint_gradient_mode.argtypes = [_int, _int]
     lib.tvinpaint_slot_bytes.argtypes = [_int]
     lib.tvinpaint_slot_bytes.restype = ctypes.c_longlong
     lib.tvinpaint_schedule.argtypes = [_int, ctypes.POINTER(_int), ctypes.POINTER(_int)]

@@ -171,29 +171,31 @@ __global__ __launch_bounds__(NT) void tv_forward_iter(
 
 // Prox adjoint + confidence / rhs gradient: TV.cu:806-828 (and 240-255 for the first step).
 // Only g05 continues down the chain; none of these values reaches a switch.
-template <bool FIRST>
+template <bool FIRST, bool TRUE_ADJ = false>
 __device__ __forceinline__ void prox_adjoint(float df_dxk, float bb, float x05v, float conf, float& g05,
                                              float& gc, float& gb) {
+  constexpr float kGC = TRUE_ADJ ? 1.f : kLocalGCMult, kGB = TRUE_ADJ ? 1.f : kLocalGBMult;
   const float diff = bb - x05v;
   const float sign = (diff < 0) ? -1.f : 1.f;
   if (1. + (double)conf >= (double)(sign * diff)) {
-    gc += df_dxk * (bb / (1.f + conf) - (conf * bb + x05v) / ((1.f + conf) * (1.f + conf))) * kLocalGCMult;
+    gc += df_dxk * (bb / (1.f + conf) - (conf * bb + x05v) / ((1.f + conf) * (1.f + conf))) * kGC;
     g05 = df_dxk / (1.f + conf);
-    gb += df_dxk * conf / (1.f + conf) * kLocalGBMult;
+    gb += df_dxk * conf / (1.f + conf) * kGB;
   } else if (FIRST) {
     g05 = df_dxk;
-    gc += sign * df_dxk * kLocalGCMult;
+    gc += sign * df_dxk * kGC;
     gb = 0.f;  // TV.cu:254
   } else if (conf >= sign * diff) {  // TV.cu:818-822, unreachable for conf >= 0
     g05 = 0.f;
-    gb += df_dxk * kLocalGBMult;
+    gb += df_dxk * kGB;
   } else {
     g05 = df_dxk;
-    gc += sign * df_dxk * kLocalGCMult;
+    gc += sign * df_dxk * kGC;
   }
 }
 
-// First adjoint step: TV.cu:222-287.
+// First adjoint step: TV.cu:222-287.  TRUE_ADJ: multipliers 1 (the corrected gradient).
+template <bool TRUE_ADJ>
 __global__ __launch_bounds__(256) void tv_adjoint_first(const float* __restrict__ cf, const float* __restrict__ b,
                                                         const float* __restrict__ x05, float* __restrict__ gc,
                                                         float* __restrict__ gb, float* __restrict__ g05,
@@ -207,11 +209,106 @@ __global__ __launch_bounds__(256) void tv_adjoint_first(const float* __restrict_
   for (int ch = 0; ch < C; ch++) {
     const long long q = (s * C + ch) * HW + p;
     float g05v, gbv = gb[q];
-    prox_adjoint<true>(gin[q], b[q], x05[q], conf, g05v, gcv, gbv);
+    prox_adjoint<true, TRUE_ADJ>(gin[q], b[q], x05[q], conf, g05v, gcv, gbv);
     g05[q] = g05v;
     gb[q] = gbv;
   }
   gc[i] = gcv;
+}
+
+// Corrected gradient only: the gradient step of iteration 0, which the reference never back-propagates
+// (TV.cu:1696-1729 ends after producing g05[0]; TV.cu:1816 returns g_x[1] as the gradient wrt the start).
+// gi = J^T(y_0) g05[0] + g_x[0] with the transposed Jacobian of TV.cu:651-771 at the starting point y_0, and
+// the weight gradients of iteration 0 (multiplier 1) are added to the fp64 totals.  One thread per pixel; each
+// of the three triangles a pixel belongs to is evaluated here, as the reference's kernels do.
+__global__ __launch_bounds__(256) void tv_adjoint_iter0(const float* __restrict__ wx_, const float* __restrict__ wy_,
+                                                        const float* __restrict__ y0, const float* __restrict__ g05,
+                                                        const float* __restrict__ gx0, float* __restrict__ gi,
+                                                        double* __restrict__ tot_gx, double* __restrict__ tot_gy, int C,
+                                                        int H, int W, long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // over n*HW pixels
+  if (i >= total) return;
+  const long long HW = (long long)H * W;
+  const long long smp = i / HW, p = i - smp * HW;
+  const int h = (int)(p / W), w = (int)(p - (long long)h * W);
+  const float* wx = wx_ + smp * HW;
+  const float* wy = wy_ + smp * HW;
+  const float wx_0 = (w > 0) ? kL * wx[p - 1] : 0.f;
+  const float wx_1 = (w < W - 1) ? kL * wx[p] : 0.f;
+  const float wy_0 = (h > 0) ? kL * wy[p - W] : 0.f;
+  const float wy_1 = (h < H - 1) ? kL * wy[p] : 0.f;
+  const float wx_2 = (h > 0 && w < W - 1) ? kL * wx[p - W] : 0.f;
+  const float wy_2 = (w > 0 && h < H - 1) ? kL * wy[p - 1] : 0.f;
+  float gwx = 0.f, gwy = 0.f;
+  for (int ch = 0; ch < C; ch++) {
+    const long long q = (smp * C + ch) * HW;
+    const float* y = y0 + q;
+    const float* g = g05 + q;
+    auto at = [&](const float* f, int hh, int ww) {
+      return (hh >= 0 && hh < H && ww >= 0 && ww < W) ? f[(long long)hh * W + ww] : 0.f;
+    };
+    const float yk = y[p], df_dy = g[p];
+    float t = df_dy;
+    if (h > 0) {  // triangle owned by the pixel above, TV.cu:655-686
+      const float yu = at(y, h - 1, w), yur = at(y, h - 1, w + 1), gu = at(g, h - 1, w), gur = at(g, h - 1, w + 1);
+      const float a_y = (yk - yu) * (yk - yu) * wy_0;
+      const float a_x = (yu - yur) * (yu - yur) * wx_2;
+      const float hub = sqrtf(a_x + a_y);
+      if (hub > kDelta) {
+        const float nom = kDelta / hub;
+        const float denom = nom / (2.f * hub * hub);
+        t -= (df_dy - gu) * (wy_0 * nom);
+        const float temp = -denom * 2.f * (yk - yu) * wy_0;
+        t -= (df_dy - gu) * wy_0 * (yk - yu) * temp;
+        t -= (gur - gu) * wx_2 * (yur - yu) * temp;
+      } else {
+        t -= (df_dy - gu) * wy_0;
+      }
+    }
+    if (w > 0) {  // triangle owned by the pixel to the left, TV.cu:687-720
+      const float yl = at(y, h, w - 1), yld = at(y, h + 1, w - 1), gl = at(g, h, w - 1), gld = at(g, h + 1, w - 1);
+      const float a_x = (yk - yl) * (yk - yl) * wx_0;
+      const float a_y = (yl - yld) * (yl - yld) * wy_2;
+      const float hub = sqrtf(a_x + a_y);
+      if (hub > kDelta) {
+        const float nom = kDelta / hub;
+        const float denom = nom / (2.f * hub * hub);
+        t -= (df_dy - gl) * (wx_0 * nom);
+        const float temp = -denom * 2.f * (yk - yl) * wx_0;
+        t -= (df_dy - gl) * wx_0 * (yk - yl) * temp;
+        t -= (gld - gl) * wy_2 * (yld - yl) * temp;
+      } else {
+        t -= (df_dy - gl) * wx_0;
+      }
+    }
+    {  // the pixel's own triangle, TV.cu:722-771
+      const float yr = at(y, h, w + 1), yd = at(y, h + 1, w), gr = at(g, h, w + 1), gd = at(g, h + 1, w);
+      const float a_x = (yk - yr) * (yk - yr) * wx_1;
+      const float a_y = (yk - yd) * (yk - yd) * wy_1;
+      const float hub = sqrtf(a_x + a_y);
+      if (hub > kDelta) {
+        const float nom = kDelta / hub;
+        const float denom = nom / (2.f * hub * hub);
+        t -= (df_dy - gd) * (wy_1 * nom);
+        t -= (df_dy - gr) * (wx_1 * nom);
+        const float temp = denom * 2.f * ((yd - yk) * wy_1 + (yr - yk) * wx_1);
+        t -= (df_dy - gd) * wy_1 * (yk - yd) * temp;
+        t -= (df_dy - gr) * wx_1 * (yk - yr) * temp;
+        if (w < W - 1)
+          gwx = gwx - (yk - yr) * ((df_dy - gr) * (nom - a_x * denom) - (df_dy - gd) * (yk - yr) * (yk - yd) * denom * wy_1);
+        if (h < H - 1)
+          gwy = gwy - (yk - yd) * ((df_dy - gd) * (nom - a_y * denom) - (df_dy - gr) * (yk - yd) * (yk - yr) * denom * wx_1);
+      } else {
+        t -= (df_dy - gd) * wy_1;
+        t -= (df_dy - gr) * wx_1;
+        if (w < W - 1) gwx = gwx - (yk - yr) * (df_dy - gr);
+        if (h < H - 1) gwy = gwy - (yk - yd) * (df_dy - gd);
+      }
+    }
+    gi[q + p] = t + gx0[q + p];
+  }
+  tot_gx[i] += (double)gwx;
+  tot_gy[i] += (double)gwy;
 }
 
 // Main adjoint step with the y rebuild fused in: TV.cu:586-859 (+1130-1189), and, with END, the
@@ -392,6 +489,7 @@ struct Slot {
   // recomputed from its checkpoint, the reference's order of work), 1 those of the last segment, 2 all of them (no
   // recompute at all; the ring then has one row per iteration).
   int keep_mode = 2;
+  int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
   int x05_mode = 0;     // how the last forward laid its rows out: 2 row = iteration, else row = iteration - first kept
   int x05_from = 0;     // first iteration whose x05 row the last forward kept
@@ -611,7 +709,7 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const fl
   }
 }
 
-template <int C, bool END>
+template <int C, bool END, bool TRUE_ADJ>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                           const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
                           float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
@@ -621,29 +719,30 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, co
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
   if (gx_final)
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, true>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
                        s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih, s.iw, t, R, sx,
                        sy);
   else
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, false>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
                        s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih, s.iw, t, R, sx,
                        sy);
 }
 
 // One adjoint step: reads accumulator set acc_cur, writes the other one, then flips acc_cur.
-template <bool END>
+// TRUE_ADJ (strip path only, the caller checks): the corrected gradient; with END, yck is the checkpointed x.
+template <bool END, bool TRUE_ADJ = false>
 bool launch_adjoint(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
                     float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
   const bool strip = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
   if (strip) {
     switch (s.ic) {
-      case 1: launch_adjoint_strip<1, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
-      case 2: launch_adjoint_strip<2, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
-      case 3: launch_adjoint_strip<3, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
-      default: launch_adjoint_strip<4, END>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      case 1: launch_adjoint_strip<1, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      case 2: launch_adjoint_strip<2, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      case 3: launch_adjoint_strip<3, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+      default: launch_adjoint_strip<4, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
     }
   } else {
     const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
@@ -789,6 +888,9 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   Slot& s = g_slots[id];
   if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
+  const bool corr = s.grad_mode == 1;
+  if (corr && (force_tile_path() || s.ic > 4))
+    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (1..4 channels), got %d", s.ic);
   s.stream = stream;
   const size_t F = field_count(s), P = plane_count(s);
   const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
@@ -848,13 +950,13 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     }
     // reverse sweep (TV.cu:1696-1729)
     int timed_run = 0;
-    if (adjoint_pairs(s)) {
+    if (adjoint_pairs(s) && !corr) {
       // The g05 / g_x ping-pong flips once per launch: `src` holds what the next launch reads.  The
       // first step of the whole backward writes g05[1]; a segment's last launch leaves its result
       // where the next segment picks it up.
       int j = len - 1;
       if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
-        hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+        hipLaunchKernelGGL(tv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
                            ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
                            (long long)ih * iw, (long long)P);
         pp_src = 1;
@@ -897,15 +999,27 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       const float* xa = ring + (size_t)j * F;
       const int odd = j & 1;
       if (outer == nseg - 1 && j == len - 1) {
-        hipLaunchKernelGGL(tv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
-                           s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+        if (corr)
+          hipLaunchKernelGGL(tv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+        else
+          hipLaunchKernelGGL(tv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = ring + (size_t)(j - 1) * F;
         if (timed_run == 0) g_timer.begin(stream);
-        launch_adjoint<false>(s, stream, dx, dy, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
-                              s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
+        if (corr)
+          launch_adjoint<false, true>(s, stream, dx, dy, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
+                                      s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
+        else
+          launch_adjoint<false>(s, stream, dx, dy, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
+                                s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
         timed_run++;
         if (j == 1) g_timer.end(stream, timed_run);  // one event pair around the sweep's run of launches
+      } else if (corr) {
+        // corrected gradient: linearise at the true y_{k0+1}, rebuilt from x05[k0] and the checkpointed x_{k0}
+        flushed = launch_adjoint<true, true>(s, stream, dx, dy, c, b, xa, xa, ckx, s.g05[1], s.g05[0], s.gxk[1],
+                                             s.gxk[0], outer == 0 ? s.gx_final : nullptr, t);
       } else {
         // the very last step's g_x[k+1] is the gradient wrt the starting point (TV.cu:1785,1816)
         flushed = launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
@@ -923,6 +1037,12 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     lastIt = k0;
   }
 
+  if (corr && 2 * (its / 2) > 0) {
+    // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it); the last
+    // step above left g05[0] and the partial g_x[0] in the `0` halves of the ping-pongs, checkpoint 0 is y_0
+    hipLaunchKernelGGL(tv_adjoint_iter0, dim3(grid1d((long long)P)), dim3(256), 0, stream, dx, dy, s.ckpt_y, s.g05[0],
+                       s.gxk[0], s.gx_final, s.tot_gx, s.tot_gy, ic, ih, iw, (long long)P);
+  }
   // output guard on the device (TV.cu:1760-1791), then scale and store (TV.cu:1795-1818)
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
@@ -950,7 +1070,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     fin.chain_per_sample[k] = nullptr;
     fin.per_sample[k] = 1;
   }
-  hipLaunchKernelGGL(finalize_many, dim3(gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, kGlobalGMult);
+  hipLaunchKernelGGL(finalize_many, dim3(gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, corr ? 1.f : kGlobalGMult);
   hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gx_final, gi, (long long)F, s.guard, 4, kGuard);
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TV.cu:1829
@@ -997,6 +1117,13 @@ int tvinpaint_guard_stats(int id, double* stats25) {
   INPAINT_HIP(hipStreamSynchronize(s.stream));
   INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
   memcpy(stats25, host.report, sizeof(host.report));
+  return 0;
+}
+
+int tvinpaint_gradient_mode(int id, int mode) {
+  if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  if (mode < 0 || mode > 1) return fail(INPAINT_ERR_ARG, "gradient mode %d is not 0 or 1", mode);
+  g_slots[id].grad_mode = mode;
   return 0;
 }
 

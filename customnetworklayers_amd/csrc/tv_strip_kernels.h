@@ -511,6 +511,16 @@ __device__ __forceinline__ float rebuild_y_fast(float bb, float xa, float xb, fl
   return quad ? y_q : y_l;
 }
 
+// y_{k+1} exactly as the forward pass made it: x_{k+1} = prox(x05[k]) (TV.cu:1286-1292), y_{k+1} = x_{k+1} +
+// t (x_{k+1} - x_k) (TV.cu:1315); x_k is prox(x05[k-1]) or, at a segment start, the checkpointed iterate itself.
+__device__ __forceinline__ float prox_huber1(float yt, float c, float rc1, float bv) {
+  float x_loc = div_by(c * bv + yt, 1.f + c, rc1);
+  const float lo = yt - c, hi = yt + c;
+  if (lo > 1.f + bv) x_loc = lo;
+  if (hi < bv - 1.f) x_loc = hi;
+  return x_loc;
+}
+
 template <int C>
 struct AdjRow {
   float c, rc1, wxs, wys, xa[C], y[C], bb[C], g[C];  // y is loaded as x05[k-1] (or the checkpoint y) and rebuilt in place
@@ -518,7 +528,10 @@ struct AdjRow {
   double opc_d;                                      // 1. + (double)c, the left side of the prox regime test
 };
 
-template <int C, bool END, bool FINAL>
+// TRUE_ADJ selects the corrected gradient (not the reference's): y is the forward pass's own y (see prox_huber1;
+// with END the y slot carries the checkpointed x of the segment start, not the checkpointed y), the segment-start
+// step uses the main kernel's weight-gradient form, and the per-step multipliers are 1.
+template <int C, bool END, bool FINAL, bool TRUE_ADJ = false>
 __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
@@ -538,6 +551,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
   const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
   const bool wx_ok = g.col_ok && g.w < W - 1;
   const double opt = 1. + (double)t;
+  constexpr float kGX = TRUE_ADJ ? 1.f : kLocalGXMult, kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
   // wave-uniform plane pointers + 32-bit element offsets (SGPR base, VGPR offset)
   const size_t poff = (size_t)g.n * HW;
   const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
@@ -590,7 +604,13 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.y[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
-      o.y[ch] = END ? xb : rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
+      if (TRUE_ADJ) {
+        const float xn = prox_huber1(xa, o.c, o.rc1, bv);
+        const float xo = END ? xb : prox_huber1(xb, o.c, o.rc1, bv);
+        o.y[ch] = xn + t * (xn - xo);
+      } else {
+        o.y[ch] = END ? xb : rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
+      }
       o.g[ch] = ok ? o.g[ch] : 0.f;
       o.xa[ch] = xa;
       o.bb[ch] = bv;
@@ -642,14 +662,14 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
       if (!first.value) {
         // weight gradients of the pixel's own triangle, TV.cu:749-769 / 1019-1037
         float ux, uy;
-        if (!END) {
-          ux = kLocalGXMult * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
-          uy = kLocalGXMult * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
+        if (!END || TRUE_ADJ) {
+          ux = kGX * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
+          uy = kGX * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
         } else {
-          const float ux_a = kLocalGXMult * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
-          const float uy_a = kLocalGXMult * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
-          ux = act ? ux_a : kLocalGXMult * d2 * gpr;
-          uy = act ? uy_a : kLocalGXMult * d1 * gpd;
+          const float ux_a = kGX * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
+          const float uy_a = kGX * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
+          ux = act ? ux_a : kGX * d2 * gpr;
+          uy = act ? uy_a : kGX * d1 * gpd;
         }
         if (g.w < W - 1) gwxv = gwxv - ux;
         if (h < H - 1) gwyv = gwyv - uy;
@@ -675,14 +695,14 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
         const float sign = (diff < 0) ? -1.f : 1.f;
         const bool quad = (cur.opc_d >= (double)(sign * diff));
         const float opc = 1.f + conf;
-        const float gc_q = df * (div_by(bv, opc, cur.rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kLocalGCMult;
+        const float gc_q = df * (div_by(bv, opc, cur.rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
         const float g05_q = div_by(df, opc, cur.rc1);
         const float gb_q = div_by(df * conf, opc, cur.rc1) * 1.0f;
         // three regimes (quadratic / TV.cu:818-822, unreachable for c >= 0 / linear) as selects;
         // adding +0 where the reference adds nothing leaves the accumulators unchanged
         const bool mid = !quad && (conf >= sign * diff);
         const float g05v = quad ? g05_q : (mid ? 0.f : df);
-        gcv += quad ? gc_q : (mid ? 0.f : sign * df * kLocalGCMult);
+        gcv += quad ? gc_q : (mid ? 0.f : sign * df * kGC);
         gbv += quad ? gb_q : (mid ? df * 1.0f : 0.f);
         if (store_lane) {  // a block this small is predicated, not branched around
           if (FINAL) stg(gxf_p[ch], roff, df);  // only the last step's g_x is read again (TV.cu:800,1785)

@@ -52,6 +52,17 @@ int tvinpaint_reset_id(int id);
  * action (0 plain, 1 rescaled, 2 killed)}.  Waits for the slot's stream. */
 int tvinpaint_guard_stats(int id, double* stats25);
 
+/* Which gradient the next backwards on `id` return.  0 (default): the reference's, bit for bit, with everything
+ * its hand-derived backward does differently from the chain rule.  1: the corrected gradient -- the adjoint is
+ * linearised at the y the forward pass really used (the reference rebuilds y from the half-step iterates with a
+ * simplified prox, TVInpaintFista.cu:1130-1189, and uses the checkpoint y_k0 for y_k0+1 at every segment start,
+ * 1724-1727), iteration 0 is back-propagated too (the reference stops before it and returns g_x[1] as the gradient
+ * wrt the start, 1696-1729, 1816), and the multipliers 0.1 / 0.1 / 1.0 and the global 0.1 (63-69) are 1.  The
+ * clamp of the adjoint iterates (797-799), the upstream scrub and the output guard stay.  With them inactive the
+ * result is the gradient of the forward pass (tests compare it with automatic differentiation).  Strip kernels
+ * only (1..4 channels); one adjoint step per launch, so a backward takes about 1.3x the default's time. */
+int tvinpaint_gradient_mode(int id, int mode);
+
 /* Which intermediate iterates (the x05 rows of TVInpaintFista.cu:1678-1687) the next forwards on `id` keep for
  * the backward pass.  0: none -- the backward recomputes every segment from its checkpoint, the reference's order
  * of work and its memory footprint (2 sqrt(its) + sqrt(its) fields).  1: those of the last segment.  2 (default):

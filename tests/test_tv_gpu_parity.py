@@ -301,3 +301,88 @@ def test_kept_iterates_or_recomputed_segments_give_the_same_bits(ext, tv_oracle,
     with pytest.raises(ValueError):
         ext.keep_iterates(2, 3)
     ext.reset_id(2)
+
+
+# the quirk toggles of the oracle that the corrected gradient switches off (clamp and guard stay)
+CORRECTED = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale_factors=0, clamp=1, guard=1)
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 2, 64, 128, 20), (2, 3, 37, 101, 9), (1, 1, 16, 64, 2), (1, 4, 19, 126, 6), (1, 2, 1, 70, 4),
+    (1, 1, 33, 1, 4), (3, 2, 130, 200, 50), (1, 2, 21, 64, 3),
+])
+def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tv_oracle, n, c, h, w, its, monkeypatch):
+    # gradient_mode 1: y as the forward pass made it, no checkpoint stand-in at segment starts, iteration 0
+    # back-propagated, multipliers 1 -- the oracle with exactly these toggles off is the checker; every keep mode
+    d = tv_inputs(n, c, h, w, seed=n * 100 + h + w + its, conf_density=0.3)
+    try:
+        tv_oracle.set_quirks(**CORRECTED)
+        ref = run_oracle(tv_oracle, d, its, 2)
+    finally:
+        tv_oracle.set_quirks()
+    plain = run_oracle(tv_oracle, d, its, 2)
+    assert any(not np.array_equal(a, b) for a, b in zip(ref[1], plain[1]))  # the toggles do something
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        for keep in (2, 1, 0):
+            ext.reset_id(2)
+            ext.gradient_mode(2, 1)
+            ext.keep_iterates(2, keep)
+            (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+            grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+            got = (sol.cpu().numpy(), [g.cpu().numpy() for g in grads], None)
+            compare("corrected, keep %d" % keep, got, ref)
+            for a, b in zip(got[1], ref[1]):
+                assert np.array_equal(a, b)
+    finally:
+        ext.reset_id(2)  # back to the reference's gradient
+    compare("plain again", run_gpu(ext, d, its, 2), plain)
+
+
+def test_corrected_gradient_is_the_gradient_of_the_forward_pass(ext, tv_oracle):
+    # with the clamp and the guard idle the corrected gradient is the true one: the float64 oracle with every quirk
+    # off (which the CPU pins equate with automatic differentiation of an independent forward pass) agrees to
+    # float32 accuracy, and a directional finite difference of the GPU forward pass agrees as well
+    n, c, h, w, its = 1, 2, 24, 40, 12
+    d = tv_inputs(n, c, h, w, seed=5, conf_density=0.4)
+    d64 = {k: v.astype(np.float64) for k, v in d.items()}
+    try:
+        tv_oracle.set_quirks(0, 0, 0, 0, 0, 0)
+        tv_oracle.reset_id(3)
+        tv_oracle.forward(d64["dx"], d64["dy"], d64["dc"], d64["db"], d64["di"], its, 3, f64=True)
+        true = tv_oracle.backward(d64["grad"].copy(), d64["dx"], d64["dy"], d64["dc"], d64["db"], its, 3, f64=True)
+    finally:
+        tv_oracle.set_quirks()
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        ext.reset_id(2)
+        ext.gradient_mode(2, 1)
+        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+        grads = [g.cpu().numpy() for g in ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)]
+    finally:
+        ext.reset_id(2)
+    errs = [rel_err(g, r) for g, r in zip(grads, true)]
+    print("\ncorrected gradient vs float64 true gradient: gx %.2e gy %.2e gc %.2e gb %.2e gi %.2e" % tuple(errs), flush=True)
+    for e in errs:
+        assert e <= 1e-3
+    # the reference's gradient is a different vector: scale factors alone put it a factor 10..100 away
+    plain = run_gpu(ext, d, its, 2)[1]
+    assert rel_err(plain[3], true[3]) > 0.5
+
+
+def test_corrected_gradient_needs_the_strip_kernels(ext, monkeypatch):
+    d = tv_inputs(1, 5, 12, 20, seed=1, conf_density=0.3)
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        ext.reset_id(2)
+        ext.gradient_mode(2, 1)
+        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 4, 2)
+        with pytest.raises(ValueError):
+            ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], 4, 2)
+        with pytest.raises(ValueError):
+            ext.gradient_mode(2, 2)
+    finally:
+        ext.reset_id(2)
