@@ -345,6 +345,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", type=int, default=1,
                     help="workload index (1 = headline TV layer, 2 = TGV layer, 3 = three-level TV hierarchy, 5 = quadratic fit, 6 = median)")
+    ap.add_argument("--corrected-gradient", action="store_true",
+                    help="configs 1 and 2: time the opt-in corrected gradient instead of the reference's (not the headline)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
@@ -369,6 +371,9 @@ def main():
         kernel_name = "tvstrip::tv_adjoint_strip<2,false,false>"
     if cfg["kind"] == "tgv" and (os.environ.get("INPAINT_TGV_FUSE", "1") == "0" or os.environ.get("INPAINT_TGV_FUSE_ADJ", "1") == "0"):
         kernel_name = "tgvstrip::tgv_adjoint_strip<2,false,false>"
+    if args.corrected_gradient:  # one adjoint step per launch
+        kernel_name = ("tvstrip::tv_adjoint_strip<2,false,false,true>" if cfg["kind"] == "tv"
+                       else "tgvstrip::tgv_adjoint_strip<2,false,false,1>")
     profile, profile_read = getattr(lib, prefix + "_profile"), getattr(lib, prefix + "_profile_read")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     its, pid = cfg["its"], 0
@@ -380,6 +385,8 @@ def main():
         return ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, pid)
 
     ext.reset_id(pid)
+    if args.corrected_gradient:
+        ext.gradient_mode(pid, 1)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -399,6 +406,8 @@ def main():
     kernel_ms = tot_ms.value / max(launches.value, 1)
     # the dominant kernel runs two adjoint steps per launch
     steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2
+    if args.corrected_gradient:
+        cfg = dict(cfg, kind=cfg["kind"] + " (corrected gradient)")
     kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9

@@ -42,6 +42,7 @@ def _load():
     lib.tgvinpaint_reset_id.argtypes = [_int]
     lib.tgvinpaint_guard_stats.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
     lib.tgvinpaint_keep_iterates.argtypes = [_int, _int]
+    lib.tgvinpaint_gradient_mode.argtypes = [_int, _int]
     lib.tgvinpaint_slot_bytes.argtypes = [_int]
     lib.tgvinpaint_slot_bytes.restype = ctypes.c_longlong
     lib.tgvinpaint_lipschitz.argtypes = [_int, ctypes.POINTER(ctypes.c_double), _int]

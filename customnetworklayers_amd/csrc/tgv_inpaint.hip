@@ -272,29 +272,31 @@ __global__ __launch_bounds__(256) void tgv_getyk_kernel(const float* __restrict_
 }
 
 // Prox adjoint + confidence / rhs gradient: TGV.cu:592-612, 1418-1442 (and 166-182 for the first step).
-template <bool FIRST>
+template <bool FIRST, bool TRUE_ADJ = false>
 __device__ __forceinline__ void prox_adjoint(float df_dxk, float bb, float x05v, float conf, float& g05,
                                              float& gc, float& gb) {
+  constexpr float kGC = TRUE_ADJ ? 1.f : kLocalGCMult, kGB = TRUE_ADJ ? 1.f : kLocalGBMult;
   const float diff = bb - x05v;
   const float sign = (diff < 0) ? -1.f : 1.f;
   if (1. + (double)conf >= (double)(sign * diff)) {
-    gc += df_dxk * (bb / (1.f + conf) - (conf * bb + x05v) / ((1.f + conf) * (1.f + conf))) * kLocalGCMult;
+    gc += df_dxk * (bb / (1.f + conf) - (conf * bb + x05v) / ((1.f + conf) * (1.f + conf))) * kGC;
     g05 = df_dxk / (1.f + conf);
-    gb += df_dxk * conf / (1.f + conf) * kLocalGBMult;
+    gb += df_dxk * conf / (1.f + conf) * kGB;
   } else if (FIRST) {
     g05 = df_dxk;
-    gc += sign * df_dxk * kLocalGCMult;
+    gc += sign * df_dxk * kGC;
     gb = 0.f;  // TGV.cu:181
   } else if (conf >= sign * diff) {
     g05 = 0.f;
-    gb += df_dxk * kLocalGBMult;
+    gb += df_dxk * kGB;
   } else {
     g05 = df_dxk;
-    gc += sign * df_dxk * kLocalGCMult;
+    gc += sign * df_dxk * kGC;
   }
 }
 
-// First adjoint step: TGV.cu:151-218.
+// First adjoint step: TGV.cu:151-218.  TRUE_ADJ: multipliers 1 (the corrected gradient).
+template <bool TRUE_ADJ>
 __global__ __launch_bounds__(256) void tgv_adjoint_first(const float* __restrict__ cf, const float* __restrict__ b,
                                                          const float* __restrict__ x05, float* __restrict__ gc,
                                                          float* __restrict__ gb, float* __restrict__ g05,
@@ -310,7 +312,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_first(const float* __restrict
     const long long q = s * 3 * CHW + ch * HW + p;
     const long long qb = s * CHW + ch * HW + p;
     float g05v, gbv = gb[qb];
-    prox_adjoint<true>(gin[q], b[qb], x05[q], conf, g05v, gcv, gbv);
+    prox_adjoint<true, TRUE_ADJ>(gin[q], b[qb], x05[q], conf, g05v, gcv, gbv);
     g05[q] = g05v;
     gb[qb] = gbv;
     g05[q + CHW] = gin[q + CHW];          // TGV.cu:215
@@ -328,7 +330,12 @@ __device__ __forceinline__ float huber_w_end(float hub, float delta) { return 1.
 // Main adjoint step (TGV.cu:224-644) and, with END, the segment-start variant (TGV.cu:1061-1472)
 // that linearises at the checkpoint y and writes the same Jacobian with sqrt and divisions.
 // y is y_{k+1} rebuilt by tgv_getyk_kernel, or the checkpoint y.
-template <bool END>
+// JT0 (corrected gradient only): the gradient step of iteration 0, which the reference never back-propagates
+// (TGV.cu:2851-2933 ends after producing g05[0]; TGV.cu:3047 returns g_x[1]).  Only the transposed Jacobian is applied,
+// in the main kernel's form with the v2 block's division (TGV.cu:355) replaced by its siblings' product and
+// multiplier 1: g05_out receives J^T g05_in + gxk (the gradient wrt the start), the weight gradients are added to
+// gwx / gwy; gc, gb, gxk, gxk_m1 are left alone and y is the starting point.
+template <bool END, bool JT0 = false>
 __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
     const float* __restrict__ wx_, const float* __restrict__ wy_, const float* __restrict__ bx_,
     const float* __restrict__ by_, const float* __restrict__ cf_, const float* __restrict__ b_,
@@ -352,7 +359,7 @@ __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
   const float bX_l = (w > 0) ? bx[p - 1] : 0.f, bY_l = (w > 0) ? by[p - 1] : 0.f;
   const float bX_c = bx[p], bY_c = by[p];
   const float oneL = 1.0f;
-  const float gxm = kLocalGXMult;
+  const float gxm = JT0 ? 1.f : kLocalGXMult;
   float gcv = gc_[smp * HW + p];
   float gwx0 = gwx_[smp * 2 * HW + p], gwx1 = gwx_[smp * 2 * HW + HW + p];
   float gwy0 = gwy_[smp * 2 * HW + p], gwy1 = gwy_[smp * 2 * HW + HW + p];
@@ -428,7 +435,7 @@ __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
           const float hub = rsq(B);
           W_TIJ = fminf(1.f, hub * kD2);
           active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ / (hub * hub);  // TGV.cu:355: a division where every sibling block multiplies
+          dW_TIJ = JT0 ? W_TIJ * (hub * hub) : W_TIJ / (hub * hub);  // TGV.cu:355: a division where every sibling block multiplies
         }
         df_dy2_t -= betaTY * oneL * W_TIJ * (df_dy2 - QY(G2, -1, 0));
         if (active)
@@ -618,6 +625,12 @@ __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
     // aux variables: momentum adjoint only (TGV.cu:560-577 / 1383-1399); the literal 1. makes the
     // product double
     const size_t q = o + p;
+    if (JT0) {
+      g05_out_[q] = df_dy_t + gxk_[q];
+      g05_out_[q + CHW] = df_dy1_t + gxk_[q + CHW];
+      g05_out_[q + 2 * CHW] = df_dy2_t + gxk_[q + 2 * CHW];
+      continue;
+    }
     gxk_m1_[q + CHW] = -t * df_dy1_t;
     df_dy1_t = (float)((double)gxk_[q + CHW] + (1. + (double)t) * (double)df_dy1_t);
     df_dy1_t = fmaxf(-kClipLocalGrad, fminf(df_dy1_t, kClipLocalGrad));
@@ -639,7 +652,7 @@ __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
     g05_out_[q] = g05v;
     gb_[qb] = gbv;
   }
-  gc_[smp * HW + p] = gcv;
+  if (!JT0) gc_[smp * HW + p] = gcv;
   gwx_[smp * 2 * HW + p] = gwx0;
   gwx_[smp * 2 * HW + HW + p] = gwx1;
   gwy_[smp * 2 * HW + p] = gwy0;
@@ -705,6 +718,7 @@ struct Slot {
   // recomputed from its checkpoint, the reference's order of work), 1 those of the last segment, 2 all of them (no
   // recompute at all; the ring then has one row per iteration).
   int keep_mode = 2;
+  int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tgvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
   int x05_mode = 0;     // how the last forward laid its rows out: 2 row = iteration, else row = iteration - first kept
   int x05_from = 0;     // first iteration whose x05 row the last forward kept
@@ -972,7 +986,7 @@ void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, cons
     launch_forward_pair_strip<2>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP);
 }
 
-template <int C, bool END>
+template <int C, bool END, int ADJ>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
                           const float* xb, const float* yck, const float* g05_in, float* g05_out, const float* gxk,
                           float* gxk_m1, float* gx_final, float t) {
@@ -982,11 +996,11 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, con
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   if (gx_final)
-    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, true, ADJ>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
                        xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
                        s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
   else
-    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
+    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, false, ADJ>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
                        xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
                        s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
 }
@@ -995,13 +1009,14 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, con
 // read from the checkpoint yck); accumulator set acc_cur is read, the other one written, then
 // acc_cur flips; g_x is stored (to gx_final) only when asked.  Per-pixel path: y comes from the yk
 // buffer (or yck), accumulators and g_x are updated in place.
-template <bool END>
+// ADJ > 0 (strip path only, the caller checks): the corrected gradient; ADJ == 2: xb is the checkpointed x.
+template <bool END, int ADJ = 0>
 void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa, const float* xb,
                     const float* yck, const float* g05_in, float* g05_out, float* gxk, float* gxk_m1, float* gx_final,
                     float t) {
   if (use_strip(s)) {
-    if (s.ic == 1) launch_adjoint_strip<1, END>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
-    else launch_adjoint_strip<2, END>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
+    if (s.ic == 1) launch_adjoint_strip<1, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
+    else launch_adjoint_strip<2, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
     s.acc_cur = 1 - s.acc_cur;
     return;
   }
@@ -1153,6 +1168,9 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   Slot& s = g_slots[id];
   if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
+  const bool corr = s.grad_mode == 1;
+  if (corr && !use_strip(s))
+    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (1 or 2 channels), got %d", s.ic);
   s.stream = stream;
   const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
   const int gS = grid_stride((long long)S3), gF = grid_stride((long long)F), gP = grid_stride((long long)P),
@@ -1244,11 +1262,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     }
     int timed_run = 0;
     bool flushed = false;  // the pair that ends the segment adds the segment sums to the totals itself
-    if (adjoint_pairs(s)) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
+    if (adjoint_pairs(s) && !corr) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
       // `pp_src` = the g05 / g_x buffer the next launch reads; it flips once per launch
       int j = len - 1;
       if (outer == nseg - 1 && j >= 0) {
-        hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+        hipLaunchKernelGGL(tgv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
                            ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
                            (long long)ih * iw, (long long)P);
         pp_src = 1;
@@ -1289,15 +1307,27 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       const float* xa = ring + (size_t)j * S3;
       const int odd = j & 1;
       if (outer == nseg - 1 && j == len - 1) {
-        hipLaunchKernelGGL(tgv_adjoint_first, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
-                           s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+        if (corr)
+          hipLaunchKernelGGL(tgv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+        else
+          hipLaunchKernelGGL(tgv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = ring + (size_t)(j - 1) * S3;
         if (timed_run == 0) g_timer.begin(stream);
-        launch_adjoint<false>(s, stream, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
-                              s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
+        if (corr)
+          launch_adjoint<false, 1>(s, stream, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
+                                   s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
+        else
+          launch_adjoint<false>(s, stream, c, b, xa, xb, nullptr, s.g05[odd ? 0 : 1], s.g05[odd ? 1 : 0],
+                                s.gxk[odd ? 0 : 1], s.gxk[odd ? 1 : 0], nullptr, t);
         timed_run++;
         if (j == 1) g_timer.end(stream, timed_run);  // one event pair around the sweep's run of launches
+      } else if (corr) {
+        // corrected gradient: linearise at the true y_{k0+1}, rebuilt from x05[k0] and the checkpointed x_{k0}
+        launch_adjoint<false, 2>(s, stream, c, b, xa, ckx, nullptr, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
+                                 outer == 0 ? s.gx_final : nullptr, t);
       } else {
         // the very last step's g_x is the gradient wrt the starting point (TGV.cu:3047)
         launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
@@ -1315,6 +1345,18 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     lastIt = k0;
   }
 
+  if (corr && 2 * (its / 2) > 0) {
+    // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it).  The last
+    // step above left g05[0] and the partial g_x[0] in the `0` halves of the ping-pongs; checkpoint 0 is y_0; the
+    // accumulators are zero after the flush and take iteration 0's weight gradients, which a second flush adds.
+    const int a = s.acc_cur;
+    const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
+    hipLaunchKernelGGL((tgv_adjoint_px<false, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, s.ckpt_y,
+                       s.acc_gc[a], s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], s.g05[0], s.gx_final, s.gxk[0], s.gxk[1],
+                       s.ckpt_y, s.ic, s.ih, s.iw, 0.f);
+    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
+    hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
+  }
   // output guard on the device (TGV.cu:2990-3021), then scale and store (TGV.cu:3024-3050)
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
   hipLaunchKernelGGL(tgv_gather_u, dim3(grid1d((long long)F)), dim3(256), 0, stream, gi_src, s.gi_u,
@@ -1346,7 +1388,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     fin.chain_per_sample[k] = weights ? (const double*)s.Ls : nullptr;
     fin.per_sample[k] = weights ? HW2 : 1;
   }
-  hipLaunchKernelGGL(finalize_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, kGlobalGMult);
+  hipLaunchKernelGGL(finalize_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, corr ? 1.f : kGlobalGMult);
   hipLaunchKernelGGL(tgv_finalize_init, dim3(grid1d((long long)S3)), dim3(256), 0, stream, gi_src, gi,
                      (long long)ic * ih * iw, (long long)S3, s.guard, kGuard);
   INPAINT_HIP(hipGetLastError());
@@ -1394,6 +1436,13 @@ int tgvinpaint_guard_stats(int id, double* stats25) {
   INPAINT_HIP(hipStreamSynchronize(s.stream));
   INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
   memcpy(stats25, host.report, sizeof(host.report));
+  return 0;
+}
+
+int tgvinpaint_gradient_mode(int id, int mode) {
+  if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  if (mode < 0 || mode > 1) return fail(INPAINT_ERR_ARG, "gradient mode %d is not 0 or 1", mode);
+  g_slots[id].grad_mode = mode;
   return 0;
 }
 

@@ -538,12 +538,17 @@ struct AdjRow {
   float c, rc1, wxs, wys, bxs, bys;
   float y[3][C];   // y[0]: loaded as x05[k-1] (or the checkpoint y) and rebuilt in place; y[1], y[2]: x05[k] aux (or checkpoint)
   float xa[C];     // x05[k] of u, for the prox regime
+  float yp[2][C];  // corrected gradient only: aux of x05[k-1] (or of the checkpointed x), for the momentum of aux y
   float bb[C], g[3][C];
   float gx_i[3][C], gb_i[C], gc_i, gwx0_i, gwx1_i, gwy0_i, gwy1_i;
   double opc_d;
 };
 
-template <int C, bool END, bool FINAL>
+// ADJ > 0 selects the corrected gradient (not the reference's): y is the forward pass's own y -- u: x+ + t (x+ - x-)
+// with x+ = prox(x05[k]) and x- = prox(x05[k-1]) (ADJ == 1) or the checkpointed x of a segment start passed as
+// x05b (ADJ == 2); aux: x05[k] + t (x05[k] - x05[k-1]), momentum included (TGV.cu:1686-1690) --, the upper-triangle
+// v2 block multiplies by hub^2 like its siblings, and the per-step multipliers are 1.  END must be false then.
+template <int C, bool END, bool FINAL, int ADJ = 0>
 __global__ __launch_bounds__(256) void tgv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
@@ -562,7 +567,9 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
   const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
   const bool rmask = g.col_ok && g.w < W - 1;
   const double opt = 1. + (double)t;
-  const float gxm = kLocalGXMult;
+  static_assert(!(END && ADJ), "the corrected gradient has no segment-start form");
+  const float gxm = ADJ ? 1.f : kLocalGXMult;
+  constexpr float kGC = ADJ ? 1.f : kLocalGCMult;
   const size_t poff = (size_t)g.n * HW;
   const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
                      *const cf_p = cf + poff;
@@ -570,7 +577,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
                      *const gwy0i_p = gwy_in + 2 * poff, *const gwy1i_p = gwy_in + 2 * poff + HW;
   float *const gco_p = gc + poff, *const gwx0o_p = gwx + 2 * poff, *const gwx1o_p = gwx + 2 * poff + HW,
                *const gwy0o_p = gwy + 2 * poff, *const gwy1o_p = gwy + 2 * poff + HW;
-  const float *ys_p[3][C], *xa_p[C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
+  const float *ys_p[3][C], *yp_p[2][C], *xa_p[C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
   float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
@@ -582,6 +589,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
       // y sources: u from x05[k-1] (rebuilt with x05[k]), aux straight from x05[k] (TGV.cu:1536-1537);
       // END: all three from the checkpoint y
       ys_p[v][ch] = (END ? yck : (v == 0 ? x05b : x05a)) + q;
+      if (v > 0) yp_p[v - 1][ch] = x05b + q;
       g_p[v][ch] = g05_in + q; gxi_p[v][ch] = gxk + q;
       g05o_p[v][ch] = g05_out + q; gxm_p[v][ch] = gxk_m1 + q; gxf_p[v][ch] = FINAL ? gx_final + q : nullptr;
     }
@@ -608,6 +616,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
 #pragma unroll
       for (int v = 0; v < 3; v++) {
         in.y[v][ch] = ldg(ys_p[v][ch], off);
+        if (ADJ && v > 0) in.yp[v - 1][ch] = ldg(yp_p[v - 1][ch], off);
         in.g[v][ch] = ldg(g_p[v][ch], off);
         in.gx_i[v][ch] = ldg(gxi_p[v][ch], off_p);
       }
@@ -631,9 +640,20 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.y[0][ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
-      o.y[0][ch] = END ? xb : tvstrip::rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
-      o.y[1][ch] = ok ? o.y[1][ch] : 0.f;
-      o.y[2][ch] = ok ? o.y[2][ch] : 0.f;
+      if (ADJ) {
+        const float xn = tvstrip::prox_huber1(xa, o.c, o.rc1, bv);
+        const float xo = ADJ == 2 ? xb : tvstrip::prox_huber1(xb, o.c, o.rc1, bv);
+        o.y[0][ch] = xn + t * (xn - xo);  // TGV.cu:1773
+#pragma unroll
+        for (int v = 1; v < 3; v++) {
+          const float xv = ok ? o.y[v][ch] : 0.f, xp = ok ? o.yp[v - 1][ch] : 0.f;
+          o.y[v][ch] = xv + t * (xv - xp);  // TGV.cu:1686-1690
+        }
+      } else {
+        o.y[0][ch] = END ? xb : tvstrip::rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
+        o.y[1][ch] = ok ? o.y[1][ch] : 0.f;
+        o.y[2][ch] = ok ? o.y[2][ch] : 0.f;
+      }
       o.xa[ch] = xa;
       o.bb[ch] = bv;
 #pragma unroll
@@ -722,7 +742,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
       const float dv2 = dg2x * u21 * bY + dg2y * u22 * bY;
       const float R2 = act2 ? bY * dW2 * (u21 + u22) * dv2 : 0.f;
       // the main kernel's upper-triangle v2 block divides by hub^2 where every sibling multiplies (TGV.cu:355)
-      const float dW2_below = END ? dW2 : exact_div(W2, h2sq);
+      const float dW2_below = (END || ADJ) ? dW2 : exact_div(W2, h2sq);
       const float N2y = act2 ? bY * (dW2_below * bY * u22) * S2 : 0.f;
       const float N2x = act2 ? bY * (dW2 * bY * u21) * S2 : 0.f;
 
@@ -817,12 +837,12 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
         const float sign = (diff < 0) ? -1.f : 1.f;
         const bool quad = (cur.opc_d >= (double)(sign * diff));
         const float opc = 1.f + conf;
-        const float gc_q = df * (div_by(bv, opc, cur.rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kLocalGCMult;
+        const float gc_q = df * (div_by(bv, opc, cur.rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
         const float g05_q = div_by(df, opc, cur.rc1);
         const float gb_q = div_by(df * conf, opc, cur.rc1) * 1.0f;
         const bool mid = !quad && (conf >= sign * diff);
         const float g05v = quad ? g05_q : (mid ? 0.f : df);
-        gcv += quad ? gc_q : (mid ? 0.f : sign * df * kLocalGCMult);
+        gcv += quad ? gc_q : (mid ? 0.f : sign * df * kGC);
         float gbv = cur.gb_i[ch];
         gbv += quad ? gb_q : (mid ? df * 1.0f : 0.f);
         if (store_lane) {

@@ -38,13 +38,16 @@ class TGVInpaint(nn.Module):
     """Unbatched H x W x C interface of the reference module (cudaTGV/TGVInpainting.py:46-74).
     pid is a unique number between 0 and 9."""
 
-    def __init__(self, device, its, pid=3):
+    def __init__(self, device, its, pid=3, corrected_gradient=False):
         super(TGVInpaint, self).__init__()
         self.its = its
         self.id = pid
         self.device = device
+        # not in the reference: back-propagate the corrected gradient instead of the reference's (gradient_mode)
+        self.corrected_gradient = bool(corrected_gradient)
 
     def forward(self, t_dx, t_dy, t_dc, t_db, t_di):
+        tgvInpaint_cuda_ext.gradient_mode(self.id, 1 if self.corrected_gradient else 0)
         Yx, Xx, Lx = t_dx.shape  # no batches here
         assert Lx == 2, "tensors should have 2 channels\n"
         Yi, Xi, Li = t_di.shape

@@ -110,6 +110,14 @@ def reset_id(id):  # noqa: A002
     _keep_modes.pop(int(id), None)
 
 
+def gradient_mode(id, mode):  # noqa: A002
+    """0 (default): the reference's backward, bit for bit.  1: the corrected gradient -- the adjoint linearised at
+    the forward pass's own y, iteration 0 back-propagated, all multipliers 1 (see include/tgvinpaint.h)."""
+    rc = lib.tgvinpaint_gradient_mode(int(id), int(mode))
+    if rc:
+        _raise(rc, "gradient_mode")
+
+
 def slot_bytes(id):  # noqa: A002
     """Bytes of device memory the id's slot owns."""
     return int(lib.tgvinpaint_slot_bytes(int(id)))

@@ -46,6 +46,16 @@ int tgvinpaint_get_state(int id, double* state6);
 int tgvinpaint_set_state(int id, const double* state6);
 int tgvinpaint_reset_id(int id);
 
+/* Which gradient the next backwards on `id` return.  0 (default): the reference's, bit for bit.  1: the corrected
+ * gradient -- the adjoint is linearised at the y the forward pass really used (the reference rebuilds u with a
+ * simplified prox and the auxiliary variables without their momentum, TGVInpaintFistaBetas.cu:1478-1541, and uses the
+ * checkpoint y_k0 for y_k0+1 at every segment start, 2914-2917), the upper-triangle v2 block multiplies by hub^2 like
+ * its siblings (355), iteration 0 is back-propagated too (2851-2933, 3047), and the multipliers (87-93) are 1.  The
+ * clamp of the adjoint iterates (562-583), the upstream check and the output guard stay.  With them inactive the
+ * result is the gradient of the forward pass (tests compare it with the float64 oracle that automatic differentiation
+ * pins).  Strip kernels only (1 or 2 channels); one adjoint step per launch. */
+int tgvinpaint_gradient_mode(int id, int mode);
+
 /* Which intermediate iterates (the x05 rows of TGVInpaintFista.cu:2775-2814) the next forwards on `id` keep for
  * the backward pass.  0: none -- the backward recomputes every segment from its checkpoint, the reference's order
  * of work and its memory footprint.  1: those of the last segment.  2 (default): all of them -- its states

@@ -375,3 +375,88 @@ def test_kept_iterates_or_recomputed_segments_give_the_same_bits(ext, tgv_oracle
     with pytest.raises(ValueError):
         ext.keep_iterates(2, 3)
     ext.reset_id(2)
+
+
+# the quirk toggles of the oracle that the corrected gradient switches off (clamp and guard stay)
+CORRECTED = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale_factors=0, clamp=1, guard=1, dw_div=0)
+
+
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 2, 64, 128, 20), (2, 1, 37, 101, 9), (1, 1, 16, 64, 2), (1, 2, 1, 70, 4), (1, 1, 33, 1, 4),
+    (2, 2, 90, 200, 30), (1, 2, 21, 63, 3),
+])
+def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tgv_oracle, n, c, h, w, its):
+    # gradient_mode 1: y (all three variables) as the forward pass made it, no checkpoint stand-in at segment starts,
+    # the v2 block's division replaced by the product, iteration 0 back-propagated, multipliers 1 -- the oracle with
+    # exactly these toggles off is the checker; every keep mode
+    d = varying_inputs(n, c, h, w, seed=n * 100 + h + w + its)
+    try:
+        tgv_oracle.set_quirks(**CORRECTED)
+        ref = run_oracle(tgv_oracle, d, its, 2)
+    finally:
+        tgv_oracle.set_quirks()
+    plain = run_oracle(tgv_oracle, d, its, 2)
+    assert any(not np.array_equal(a, b) for a, b in zip(ref[1], plain[1]))  # the toggles do something
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        for keep in (2, 1, 0):
+            ext.reset_id(2)
+            ext.gradient_mode(2, 1)
+            ext.keep_iterates(2, keep)
+            (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+            grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+            got = (sol.cpu().numpy(), [g.cpu().numpy() for g in grads], None)
+            compare("corrected, keep %d" % keep, got, ref)
+            for a, b in zip(got[1], ref[1]):
+                assert np.array_equal(a, b)
+    finally:
+        ext.reset_id(2)  # back to the reference's gradient
+    compare("plain again", run_gpu(ext, d, its, 2), plain)
+
+
+def test_corrected_gradient_is_the_gradient_of_the_forward_pass(ext, tgv_oracle):
+    # with the clamp and the guard idle the corrected gradient is the true one: the float64 oracle with every quirk
+    # off (which the CPU pins equate with automatic differentiation of an independent forward pass) agrees to
+    # float32 accuracy
+    n, c, h, w, its = 1, 2, 24, 40, 12
+    d = varying_inputs(n, c, h, w, seed=5)
+    d64 = {k: v.astype(np.float64) for k, v in d.items()}
+    try:
+        tgv_oracle.set_quirks(0, 0, 0, 0, 0, 0, 0)
+        tgv_oracle.reset_id(3)
+        tgv_oracle.forward(d64["dx"], d64["dy"], d64["dc"], d64["db"], d64["di"], its, 3, f64=True)
+        true = tgv_oracle.backward(d64["grad"].copy(), d64["dx"], d64["dy"], d64["dc"], d64["db"], its, 3, f64=True)
+    finally:
+        tgv_oracle.set_quirks()
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        ext.reset_id(2)
+        ext.gradient_mode(2, 1)
+        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+        grads = [g.cpu().numpy() for g in ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)]
+    finally:
+        ext.reset_id(2)
+    errs = [rel_err(g, r) for g, r in zip(grads, true)]
+    print("\ncorrected gradient vs float64 true gradient: gx %.2e gy %.2e gc %.2e gb %.2e gi %.2e" % tuple(errs), flush=True)
+    for e in errs:
+        assert e <= 1e-3
+    plain = run_gpu(ext, d, its, 2)[1]
+    assert rel_err(plain[3], true[3]) > 0.5  # the reference's gradient is a different vector
+
+
+def test_corrected_gradient_needs_the_strip_kernels(ext):
+    d = varying_inputs(1, 3, 12, 20, seed=1)
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        ext.reset_id(2)
+        ext.gradient_mode(2, 1)
+        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 4, 2)
+        with pytest.raises(ValueError):
+            ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], 4, 2)
+        with pytest.raises(ValueError):
+            ext.gradient_mode(2, 2)
+    finally:
+        ext.reset_id(2)

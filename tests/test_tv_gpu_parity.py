@@ -386,3 +386,29 @@ def test_corrected_gradient_needs_the_strip_kernels(ext, monkeypatch):
             ext.gradient_mode(2, 2)
     finally:
         ext.reset_id(2)
+
+
+def test_module_with_the_corrected_gradient(ext, tv_oracle):
+    from customnetworklayers_amd import TVInpaint
+
+    dev = torch.device("cuda:0")
+    d = tv_inputs(1, 2, 30, 44, seed=9)
+    hwc = lambda a: torch.from_numpy(np.ascontiguousarray(a[0].transpose(1, 2, 0))).to(dev).requires_grad_(True)
+    tx, ty, tc, tb, ti = (hwc(d[k]) for k in ("dx", "dy", "dc", "db", "di"))
+    try:
+        ext.reset_id(6)
+        layer = TVInpaint(dev, 14, pid=6, corrected_gradient=True)
+        sol = layer(tx, ty, tc, tb, ti)
+        up = torch.from_numpy(np.ascontiguousarray(d["grad"][0].transpose(1, 2, 0))).to(dev)
+        sol.backward(up)
+    finally:
+        ext.reset_id(6)
+    try:
+        tv_oracle.set_quirks(**CORRECTED)
+        ref = run_oracle(tv_oracle, d, 14, 6)
+    finally:
+        tv_oracle.set_quirks()
+    got_grads = [t.grad.permute(2, 0, 1).unsqueeze(0).cpu().numpy() for t in (tx, ty, tc, tb, ti)]
+    compare("module, corrected", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
+    for a, b in zip(got_grads, ref[1]):
+        assert np.array_equal(a, b)
