@@ -406,8 +406,10 @@ def main():
     kernel_ms = tot_ms.value / max(launches.value, 1)
     # the dominant kernel runs two adjoint steps per launch
     steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2
-    if args.corrected_gradient:
+    measured_cfg = args.config
+    if args.corrected_gradient:  # the counters were read on the default gradient
         cfg = dict(cfg, kind=cfg["kind"] + " (corrected gradient)")
+        measured_cfg = None
     kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9
@@ -421,13 +423,13 @@ def main():
                                % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
         "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
                       "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4),
-                      "effective_bytes_per_pixel_iteration": (round(MEASURED_STEP_BYTES[args.config] / pxit, 1)
-                                                              if args.config in MEASURED_STEP_BYTES else None),
-                      "effective_GBps": (round(MEASURED_STEP_BYTES[args.config] / (elapsed / args.steps) / 1e9, 1)
-                                         if args.config in MEASURED_STEP_BYTES else None)},
+                      "effective_bytes_per_pixel_iteration": (round(MEASURED_STEP_BYTES[measured_cfg] / pxit, 1)
+                                                              if measured_cfg in MEASURED_STEP_BYTES else None),
+                      "effective_GBps": (round(MEASURED_STEP_BYTES[measured_cfg] / (elapsed / args.steps) / 1e9, 1)
+                                         if measured_cfg in MEASURED_STEP_BYTES else None)},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config), "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(measured_cfg), "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
                      "avg_launch_ms": round(kernel_ms, 5), "launches_timed": launches.value},
     }
     if not args.no_cpu_baseline:
