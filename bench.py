@@ -22,6 +22,12 @@ HBM_PEAK_GBS = 8000.0
 # Other workloads: not measured.
 MEASURED_TRAFFIC_BYTES = {1: (2 * 86992 + 67886) * 1024, 2: (2 * 165999 + 147003) * 1024,
                           5: (2 * 408180 + 340500) * 1024, 6: (2 * 131080 + 247100) * 1024}
+# LDS bytes per launch of the dominant kernel (rocprofv3 --pmc SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT: the TV strip kernels
+# issue no LDS instruction at all -- neighbours are exchanged through DPP in registers; the two-wavefront TGV pair kernel
+# hands 7C+5 = 19 floats per lane and row from step A to step B: 688460 two-dword instructions, no bank conflicts).
+# Peak: 128 B per clock and CU x 256 CUs x 2.4 GHz.
+LDS_PEAK_GBS = 128 * 256 * 2.4
+MEASURED_LDS_BYTES = {1: 0, 2: 688460 * 64 * 8}
 # HBM bytes of one whole forward+backward (every kernel and copy of a step), from the same two counter runs: the job
 # moves far fewer bytes than the one-round-trip-per-iteration model because two iterations share a launch, the
 # backward recomputes nothing and iterates are rebuilt from the kept x05 rows instead of being stored.
@@ -407,19 +413,20 @@ def main():
     # the dominant kernel runs two adjoint steps per launch
     steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2
     measured_cfg = args.config
+    label = cfg["kind"].upper()
     if args.corrected_gradient:  # the counters were read on the default gradient
-        cfg = dict(cfg, kind=cfg["kind"] + " (corrected gradient)")
+        label += " (corrected gradient)"
         measured_cfg = None
     kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9
     out = {
         "metric": "%s-FISTA fwd+bwd Mpixel-iter/s at %dx%dx%dx%d; achieved HBM GB/s vs peak"
-                  % (cfg["kind"].upper(), n, c, h, w),
+                  % (label, n, c, h, w),
         "value": round(value, 2), "unit": "Mpixel-iter/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": cfg["kind"].upper() + " inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
+        "config": {"workload": label + " inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
                                % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
         "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
                       "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4),
@@ -432,6 +439,10 @@ def main():
                      "traffic": MEASURED_TRAFFIC_BYTES.get(measured_cfg), "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
                      "avg_launch_ms": round(kernel_ms, 5), "launches_timed": launches.value},
     }
+    if measured_cfg in MEASURED_LDS_BYTES and kernel_ms > 0:
+        lds_gbs = MEASURED_LDS_BYTES[measured_cfg] / (kernel_ms * 1e-3) / 1e9
+        out["roofline"]["lds"] = {"bytes_per_launch": MEASURED_LDS_BYTES[measured_cfg], "achieved_GBps": round(lds_gbs, 1),
+                                  "peak_GBps": round(LDS_PEAK_GBS, 1), "frac": round(lds_gbs / LDS_PEAK_GBS, 4)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))
