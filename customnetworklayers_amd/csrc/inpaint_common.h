@@ -374,6 +374,39 @@ static __global__ __launch_bounds__(256) void flush_kernel(float* __restrict__ a
   }
 }
 
+// The same flush in two halves, for the paths that keep one fp32 record per segment: segment_store_many moves the
+// accumulators of a finished segment into its record and zeroes them; combine_segments_many, after the last segment,
+// adds the records into the fp64 totals in the order the reference flushes them (last segment first), with the
+// reference's expression.  The totals then hold the bits they would after per-segment flushes, and nobody has read
+// and rewritten them once per segment.
+struct SegmentJobs {
+  float* acc[4];     // accumulators (segment_store_many) -- unused by combine_segments_many
+  float* seg[4];     // segment_store_many: this segment's record; combine_segments_many: record of segment 0
+  double* total[4];  // combine_segments_many only
+  long long n[4];    // elements per record
+};
+static __global__ __launch_bounds__(256) void segment_store_many(SegmentJobs jobs) {
+  const int k = blockIdx.y;
+  float* __restrict__ acc = jobs.acc[k];
+  float* __restrict__ seg = jobs.seg[k];
+  const long long n = jobs.n[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    seg[i] = acc[i];
+    acc[i] = 0.f;
+  }
+}
+static __global__ __launch_bounds__(256) void combine_segments_many(SegmentJobs jobs, int nseg) {
+  const int k = blockIdx.y;
+  const float* __restrict__ seg = jobs.seg[k];
+  double* __restrict__ total = jobs.total[k];
+  const long long n = jobs.n[k];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    double t = 0.;
+    for (int o = nseg - 1; o >= 0; o--) t = (double)seg[(long long)o * n + i] + t / 1.;
+    total[i] = t;
+  }
+}
+
 static __global__ __launch_bounds__(256) void fill_zero_f32(float* __restrict__ p, long long n) {
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (long long)gridDim.x * blockDim.x)

@@ -740,6 +740,9 @@ struct Slot {
         *acc_gb[2] = {nullptr, nullptr};
   int acc_cur = 0;
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
+  // strip path: one fp32 record per segment and tensor, added into the totals after the last segment
+  float *seg_gc = nullptr, *seg_gx = nullptr, *seg_gy = nullptr, *seg_gb = nullptr;
+  int seg_cur = 0;  // segment the backward pass is in
   GuardState* guard = nullptr;
   double pending_av[5] = {0, 0, 0, 0, 0};
 };
@@ -785,6 +788,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   need += Arena::padded(F, 4) * 3 + Arena::padded(F, 8);
   need += Arena::padded(P, 4) * (4 + 2) + Arena::padded(2 * P, 4) * 4;
   need += Arena::padded(P, 8) + Arena::padded(2 * P, 8) * 2;
+  need += Arena::padded(P * nck, 4) + Arena::padded(2 * P * nck, 4) * 2 + Arena::padded(F * nck, 4);
   need += Arena::padded((size_t)n, 8) + Arena::padded((size_t)n, 4) + Arena::padded(2, 4);
   need += Arena::padded(1, sizeof(GuardState));
   rc = s.arena.reserve(need);
@@ -809,6 +813,8 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   }
   s.tot_gc = a.take<double>(P); s.tot_gx = a.take<double>(2 * P); s.tot_gy = a.take<double>(2 * P);
   s.tot_gb = a.take<double>(F);
+  s.seg_gc = a.take<float>(P * nck); s.seg_gx = a.take<float>(2 * P * nck); s.seg_gy = a.take<float>(2 * P * nck);
+  s.seg_gb = a.take<float>(F * nck);
   s.guard = a.take<GuardState>(1);
   if (!s.guard) return fail(INPAINT_ERR_HIP, "arena layout overflow");
   GuardState init;
@@ -1047,9 +1053,10 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const int R = split ? pair_split_rows(s.n, s.ih, s.iw) : strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
 #define TGV_PAIR_ARGS                                                                                                      \
   s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], \
-      s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih,  \
+      s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + 2 * sP, s.seg_gy + 2 * sP, s.n, s.ih,  \
       s.iw, tA, tB, R, sx, sy
   if (split) {
     const dim3 grid((unsigned)((waves + 7) / 8 * 8)), block(128);
@@ -1202,6 +1209,22 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   }
 
   scale_weights(s, stream, dx, dy);
+  // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
+  // totals after the last segment, in the reference's order (TGV.cu:2944 flushes after every segment: same bits,
+  // but the totals are not read and rewritten once per segment).
+  const bool seg_mode = use_strip(s);
+  SegmentJobs sj;
+  {
+    float* segs[4] = {s.seg_gc, s.seg_gx, s.seg_gy, s.seg_gb};
+    double* tots_[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
+    const long long ns[4] = {(long long)P, (long long)(2 * P), (long long)(2 * P), (long long)F};
+    for (int k = 0; k < 4; k++) {
+      sj.acc[k] = nullptr;
+      sj.seg[k] = segs[k];
+      sj.total[k] = tots_[k];
+      sj.n[k] = ns[k];
+    }
+  }
   {
     ZeroList z;
     int k = 0;
@@ -1211,10 +1234,12 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     z.ptr[k] = s.acc_gc[0]; z.bytes[k++] = (long long)P * 4;
     z.ptr[k] = s.acc_gx[0]; z.bytes[k++] = (long long)P * 8;
     z.ptr[k] = s.acc_gy[0]; z.bytes[k++] = (long long)P * 8;
-    z.ptr[k] = s.tot_gc; z.bytes[k++] = (long long)P * 8;
-    z.ptr[k] = s.tot_gx; z.bytes[k++] = (long long)P * 16;
-    z.ptr[k] = s.tot_gy; z.bytes[k++] = (long long)P * 16;
-    z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
+    if (!seg_mode) {  // (the strip path writes every total when it adds up the segment records)
+      z.ptr[k] = s.tot_gc; z.bytes[k++] = (long long)P * 8;
+      z.ptr[k] = s.tot_gx; z.bytes[k++] = (long long)P * 16;
+      z.ptr[k] = s.tot_gy; z.bytes[k++] = (long long)P * 16;
+      z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
+    }
     hipLaunchKernelGGL(fill_zero_many, dim3(gS, k), dim3(256), 0, stream, z);
   }
 
@@ -1231,6 +1256,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   for (int outer = nseg - 1; outer >= 0; outer--) {
     const int k0 = s.iterations[outer];
     const int len = 2 * ((lastIt - k0) / 2);
+    s.seg_cur = outer;
     const float* cky = s.ckpt_y + (size_t)outer * S3;
     const float* ckx = s.ckpt_x + (size_t)outer * S3;
     // recompute the segment, keeping x05 (TGV.cu:2775-2814) -- unless it is the last segment and the forward pass
@@ -1335,7 +1361,16 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       }
     }
     // fp32 segment sums into the fp64 totals (TGV.cu:2944)
-    if (!flushed) {
+    if (!flushed && seg_mode) {
+      SegmentJobs st = sj;
+      const int a = s.acc_cur;
+      float* accs[4] = {s.acc_gc[a], s.acc_gx[a], s.acc_gy[a], s.acc_gb[a]};
+      for (int k = 0; k < 4; k++) {
+        st.acc[k] = accs[k];
+        st.seg[k] = sj.seg[k] + (size_t)outer * sj.n[k];
+      }
+      hipLaunchKernelGGL(segment_store_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, st);
+    } else if (!flushed) {
       const int a = s.acc_cur;
       hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[a], s.tot_gc, (long long)P);
       hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
@@ -1345,6 +1380,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     lastIt = k0;
   }
 
+  if (seg_mode) hipLaunchKernelGGL(combine_segments_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, sj, nseg);
   if (corr && 2 * (its / 2) > 0) {
     // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it).  The last
     // step above left g05[0] and the partial g_x[0] in the `0` halves of the ping-pongs; checkpoint 0 is y_0; the

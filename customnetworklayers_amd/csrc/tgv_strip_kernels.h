@@ -901,7 +901,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
 // tvstrip::tv_adjoint_strip2).  A's g05[j] and partial g_x[j] stay in registers; the seven
 // accumulators are read and written once for both steps.  BEND: B is the segment's first iteration
 // (checkpoint y, segment-start arithmetic) and the segment flush is fused: the fp32 segment sums go into the
-// fp64 totals and the accumulators are left at zero.  FINAL: B's completed g_x is stored.
+// segment's record (added into the fp64 totals after the last segment) and the accumulators are left at zero.  FINAL: B's completed g_x is stored.
 // To fit two wavefronts per SIMD the row buffers hold only what a row's neighbours need; the fields
 // that only the pixel's own update reads (partial g_x, accumulators) are loaded one step ahead into a
 // single set of registers.
@@ -926,8 +926,8 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
     const float* __restrict__ gc_in, float* __restrict__ gc, const float* __restrict__ gb_in, float* __restrict__ gb,
     const float* __restrict__ gwx_in, float* __restrict__ gwx, const float* __restrict__ gwy_in,
     float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
-    const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, double* __restrict__ tot_gc,
-    double* __restrict__ tot_gb, double* __restrict__ tot_gwx, double* __restrict__ tot_gwy, int N, int H, int W,
+    const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float tA, float tB, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
@@ -1280,9 +1280,8 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
             stg(g05o_p[0][ch], roffB, o.g05v);
             stg(g05o_p[1][ch], roffB, o.d1);
             stg(g05o_p[2][ch], roffB, o.d2);
-            if (BEND) {  // segment flush, fused: fp32 segment sum into its fp64 total, then zero (TGVH.cu:178-216)
-              double* tb = tot_gb + ((size_t)g.n * C + ch) * HW + (roffB >> 2);
-              *tb = (double)gbv + *tb / 1.;
+            if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
+              seg_gb[((size_t)g.n * C + ch) * HW + (roffB >> 2)] = gbv;
               stg(gbo_p[ch], roffB, 0.f);
             } else {
               stg(gbo_p[ch], roffB, gbv);
@@ -1293,11 +1292,11 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
       if (do_b.value && store_lane) {
         if (BEND) {
           const size_t e1 = poff + (roffB >> 2), e2 = 2 * poff + (roffB >> 2);
-          tot_gc[e1] = (double)gcB + tot_gc[e1] / 1.;
-          tot_gwx[e2] = (double)accB.gwx0 + tot_gwx[e2] / 1.;
-          tot_gwx[e2 + HW] = (double)accB.gwx1 + tot_gwx[e2 + HW] / 1.;
-          tot_gwy[e2] = (double)accB.gwy0 + tot_gwy[e2] / 1.;
-          tot_gwy[e2 + HW] = (double)accB.gwy1 + tot_gwy[e2 + HW] / 1.;
+          seg_gc[e1] = gcB;
+          seg_gwx[e2] = accB.gwx0;
+          seg_gwx[e2 + HW] = accB.gwx1;
+          seg_gwy[e2] = accB.gwy0;
+          seg_gwy[e2 + HW] = accB.gwy1;
           stg(gco_p, roffB, 0.f);
           stg(gwx0o_p, roffB, 0.f);
           stg(gwx1o_p, roffB, 0.f);
@@ -1388,8 +1387,8 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     const float* __restrict__ gc_in, float* __restrict__ gc, const float* __restrict__ gb_in, float* __restrict__ gb,
     const float* __restrict__ gwx_in, float* __restrict__ gwx, const float* __restrict__ gwy_in,
     float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
-    const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, double* __restrict__ tot_gc,
-    double* __restrict__ tot_gb, double* __restrict__ tot_gwx, double* __restrict__ tot_gwy, int N, int H, int W,
+    const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float tA, float tB, int R, int strips_x, int strips_y) {
   constexpr int kHand = 7 * C + 5;  // floats step A hands to step B per row and lane
   __shared__ float hand[2][kHand][64];
@@ -1857,9 +1856,8 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
               stg(g05o_p[0][ch], roffB, o.g05v);
               stg(g05o_p[1][ch], roffB, o.d1);
               stg(g05o_p[2][ch], roffB, o.d2);
-              if (BEND) {  // segment flush, fused: fp32 segment sum into its fp64 total, then zero (TGVH.cu:178-216)
-                double* tb = tot_gb + ((size_t)g.n * C + ch) * HW + (roffB >> 2);
-                *tb = (double)gbv + *tb / 1.;
+              if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
+                seg_gb[((size_t)g.n * C + ch) * HW + (roffB >> 2)] = gbv;
                 stg(gbo_p[ch], roffB, 0.f);
               } else {
                 stg(gbo_p[ch], roffB, gbv);
@@ -1870,11 +1868,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
         if (do_b.value && store_lane) {
           if (BEND) {
             const size_t e1 = poff + (roffB >> 2), e2 = 2 * poff + (roffB >> 2);
-            tot_gc[e1] = (double)gcB + tot_gc[e1] / 1.;
-            tot_gwx[e2] = (double)accB.gwx0 + tot_gwx[e2] / 1.;
-            tot_gwx[e2 + HW] = (double)accB.gwx1 + tot_gwx[e2 + HW] / 1.;
-            tot_gwy[e2] = (double)accB.gwy0 + tot_gwy[e2] / 1.;
-            tot_gwy[e2 + HW] = (double)accB.gwy1 + tot_gwy[e2 + HW] / 1.;
+            seg_gc[e1] = gcB;
+            seg_gwx[e2] = accB.gwx0;
+            seg_gwx[e2 + HW] = accB.gwx1;
+            seg_gwy[e2] = accB.gwy0;
+            seg_gwy[e2 + HW] = accB.gwy1;
             stg(gco_p, roffB, 0.f);
             stg(gwx0o_p, roffB, 0.f);
             stg(gwx1o_p, roffB, 0.f);

@@ -507,6 +507,9 @@ struct Slot {
         *acc_gb[2] = {nullptr, nullptr};
   int acc_cur = 0;
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
+  // strip path: one fp32 record per segment and tensor, added into the totals after the last segment
+  float *seg_gc = nullptr, *seg_gx = nullptr, *seg_gy = nullptr, *seg_gb = nullptr;
+  int seg_cur = 0;  // segment the backward pass is in
   GuardState* guard = nullptr;      // device
   double pending_av[5] = {0, 0, 0, 0, 0};  // running means to upload when the arena is (re)made
   bool have_guard_state = false;
@@ -552,6 +555,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   need += Arena::padded(F, 4) * (2 + 2 + 2 * nck + ring + 2 + 2 + 1 + 2);
   need += Arena::padded(P, 4) * 6;
   need += Arena::padded(P, 8) * 3 + Arena::padded(F, 8);
+  need += Arena::padded(P * nck, 4) * 3 + Arena::padded(F * nck, 4);
   need += Arena::padded(1, sizeof(GuardState));
   rc = s.arena.reserve(need);
   if (rc) return rc;
@@ -568,6 +572,8 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   }
   s.tot_gc = a.take<double>(P); s.tot_gx = a.take<double>(P); s.tot_gy = a.take<double>(P);
   s.tot_gb = a.take<double>(F);
+  s.seg_gc = a.take<float>(P * nck); s.seg_gx = a.take<float>(P * nck); s.seg_gy = a.take<float>(P * nck);
+  s.seg_gb = a.take<float>(F * nck);
   s.guard = a.take<GuardState>(1);
   if (!s.guard) return fail(INPAINT_ERR_HIP, "arena layout overflow");
   GuardState init;
@@ -714,6 +720,7 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, co
                           const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
                           float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, "INPAINT_TV_ADJ_ROWS");
   const int sx = (s.iw + tvstrip::kAdjCols - 1) / tvstrip::kAdjCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
@@ -721,12 +728,12 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, co
   if (gx_final)
     hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih, s.iw, t, R, sx,
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, t, R, sx,
                        sy);
   else
     hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n, s.ih, s.iw, t, R, sx,
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, t, R, sx,
                        sy);
 }
 
@@ -762,6 +769,7 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
                                const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                                float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_ADJ_ROWS");
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
@@ -769,12 +777,12 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
   if (gx_final)
     hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n,
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n,
                        s.ih, s.iw, tA, tB, R, sx, sy);
   else
     hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.tot_gc, s.tot_gb, s.tot_gx, s.tot_gy, s.n,
+                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n,
                        s.ih, s.iw, tA, tB, R, sx, sy);
 }
 
@@ -897,13 +905,30 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
 
   hipLaunchKernelGGL(scrub_kernel, dim3(gF), dim3(256), 0, stream, gin, (long long)F);
   s.acc_cur = 0;
+  // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
+  // totals after the last segment, in the reference's order (TV.cu:1730 flushes after every segment: same bits,
+  // but the totals are not read and rewritten ten times).
+  const bool seg_mode = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
+  SegmentJobs sj;
+  {
+    float* segs[4] = {s.seg_gc, s.seg_gx, s.seg_gy, s.seg_gb};
+    double* tots_[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
+    for (int k = 0; k < 4; k++) {
+      sj.acc[k] = nullptr;
+      sj.seg[k] = segs[k];
+      sj.total[k] = tots_[k];
+      sj.n[k] = k < 3 ? (long long)P : (long long)F;
+    }
+  }
   {
     ZeroList z;
     int k = 0;
     for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.gx_final, s.acc_gb[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)F * 4; }
     for (float* p : {s.acc_gc[0], s.acc_gx[0], s.acc_gy[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 4; }
-    for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 8; }
-    z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
+    if (!seg_mode) {  // (the strip path writes every total when it adds up the segment records)
+      for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 8; }
+      z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
+    }
     hipLaunchKernelGGL(fill_zero_many, dim3(gF, k), dim3(256), 0, stream, z);
   }
 
@@ -918,6 +943,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     const int k0 = s.iterations[outer];
     const int len = 2 * ((lastIt - k0) / 2);
     bool flushed = false;
+    s.seg_cur = outer;
     const float* cky = s.ckpt_y + (size_t)outer * F;
     const float* ckx = s.ckpt_x + (size_t)outer * F;
     // recompute the segment, keeping x05 (TV.cu:1678-1687) -- unless it is the last segment and the forward pass
@@ -1028,7 +1054,15 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     }
     // fp32 segment sums into the fp64 totals (TV.cu:1730); the strip kernel of the segment's first
     // iteration has already done it
-    if (!flushed) {
+    if (!flushed && seg_mode) {
+      SegmentJobs st = sj;
+      float* accs[4] = {s.acc_gc[s.acc_cur], s.acc_gx[s.acc_cur], s.acc_gy[s.acc_cur], s.acc_gb[s.acc_cur]};
+      for (int k = 0; k < 4; k++) {
+        st.acc[k] = accs[k];
+        st.seg[k] = sj.seg[k] + (size_t)outer * sj.n[k];
+      }
+      hipLaunchKernelGGL(segment_store_many, dim3(gF, 4), dim3(256), 0, stream, st);
+    } else if (!flushed) {
     hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[s.acc_cur], s.tot_gc, (long long)P);
     hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gx[s.acc_cur], s.tot_gx, (long long)P);
     hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gy[s.acc_cur], s.tot_gy, (long long)P);
@@ -1037,6 +1071,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     lastIt = k0;
   }
 
+  if (seg_mode) hipLaunchKernelGGL(combine_segments_many, dim3(gF, 4), dim3(256), 0, stream, sj, nseg);
   if (corr && 2 * (its / 2) > 0) {
     // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it); the last
     // step above left g05[0] and the partial g_x[0] in the `0` halves of the ping-pongs, checkpoint 0 is y_0

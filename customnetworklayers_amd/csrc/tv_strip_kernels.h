@@ -480,8 +480,9 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
 // -------------------------------------------------------------------------------------------------
 // Adjoint iteration with the y rebuild fused in: TV.cu:586-859 (+1130-1189); END = the
 // segment-start variant TV.cu:862-1126 that reads y from the checkpoint.  END is the last step of
-// its segment, so it also performs the segment flush (copy_and_set_to_0, TV.cu:178-218): the fp32
-// segment sums go into the fp64 totals and the accumulators are left at zero.
+// its segment, so it also performs the first half of the segment flush (copy_and_set_to_0, TV.cu:178-218): the
+// fp32 segment sums are stored into the segment's own record (seg_*) and the accumulators are left at zero.  The
+// records are added up into the fp64 totals in the reference's order after the last segment.
 //
 // Per triangle (owner q) the kernel forms, once, every term that the reference evaluates at q,
 // at the pixel below q and at the pixel right of q:
@@ -539,8 +540,8 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ gb_in, float* __restrict__ gb, const float* __restrict__ gwx_in,
     float* __restrict__ gwx, const float* __restrict__ gwy_in, float* __restrict__ gwy,
     const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
-    float* __restrict__ gxk_m1, float* __restrict__ gx_final, double* __restrict__ tot_gc,
-    double* __restrict__ tot_gb, double* __restrict__ tot_gwx, double* __restrict__ tot_gwy, int N, int H, int W,
+    float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float t, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kAdjCols, R, W, strips_x, strips_y, N)) return;
@@ -708,9 +709,8 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
           if (FINAL) stg(gxf_p[ch], roff, df);  // only the last step's g_x is read again (TV.cu:800,1785)
           stg(gxm_p[ch], roff, gxm);
           stg(g05o_p[ch], roff, g05v);
-          if (END) {  // segment flush, fused: fp32 segment sum into its fp64 total, then zero (TV.cu:178-218)
-            double* tb = tot_gb + ((size_t)g.n * C + ch) * HW + (roff >> 2);
-            *tb = (double)gbv + *tb / 1.;
+          if (END) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TV.cu:178-218)
+            seg_gb[((size_t)g.n * C + ch) * HW + (roff >> 2)] = gbv;
             stg(gbo_p[ch], roff, 0.f);
           } else {
             stg(gbo_p[ch], roff, gbv);
@@ -724,9 +724,9 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
     if (!first.value && store_lane) {
       if (END) {
         const size_t e = poff + (roff >> 2);
-        tot_gc[e] = (double)gcv + tot_gc[e] / 1.;
-        tot_gwx[e] = (double)gwxv + tot_gwx[e] / 1.;
-        tot_gwy[e] = (double)gwyv + tot_gwy[e] / 1.;
+        seg_gc[e] = gcv;
+        seg_gwx[e] = gwxv;
+        seg_gwy[e] = gwyv;
         stg(gco_p, roff, 0.f);
         stg(gwxo_p, roff, 0.f);
         stg(gwyo_p, roff, 0.f);
@@ -798,8 +798,8 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     const float* __restrict__ gb_in, float* __restrict__ gb, const float* __restrict__ gwx_in,
     float* __restrict__ gwx, const float* __restrict__ gwy_in, float* __restrict__ gwy,
     const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
-    float* __restrict__ gxk_m1, float* __restrict__ gx_final, double* __restrict__ tot_gc,
-    double* __restrict__ tot_gb, double* __restrict__ tot_gwx, double* __restrict__ tot_gwy, int N, int H, int W,
+    float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float tA, float tB, int R, int strips_x, int strips_y) {
   StripGeom g;
   if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
@@ -1007,8 +1007,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
             stg(gxm_p[ch], roffB, gxm);
             stg(g05o_p[ch], roffB, g05v);
             if (BEND) {  // segment flush, fused (TV.cu:178-218)
-              double* tb = tot_gb + ((size_t)g.n * C + ch) * HW + (roffB >> 2);
-              *tb = (double)gbv + *tb / 1.;
+              seg_gb[((size_t)g.n * C + ch) * HW + (roffB >> 2)] = gbv;
               stg(gbo_p[ch], roffB, 0.f);
             } else {
               stg(gbo_p[ch], roffB, gbv);
@@ -1019,9 +1018,9 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
       if (do_b.value && store_lane) {
         if (BEND) {
           const size_t e = poff + (roffB >> 2);
-          tot_gc[e] = (double)gcB + tot_gc[e] / 1.;
-          tot_gwx[e] = (double)gwxB + tot_gwx[e] / 1.;
-          tot_gwy[e] = (double)gwyB + tot_gwy[e] / 1.;
+          seg_gc[e] = gcB;
+          seg_gwx[e] = gwxB;
+          seg_gwy[e] = gwyB;
           stg(gco_p, roffB, 0.f);
           stg(gwxo_p, roffB, 0.f);
           stg(gwyo_p, roffB, 0.f);
