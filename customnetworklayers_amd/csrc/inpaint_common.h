@@ -402,7 +402,16 @@ static __global__ __launch_bounds__(256) void combine_segments_many(SegmentJobs 
   const long long n = jobs.n[k];
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
     double t = 0.;
-    for (int o = nseg - 1; o >= 0; o--) t = (double)seg[(long long)o * n + i] + t / 1.;
+    int o = nseg - 1;
+    for (; o >= 3; o -= 4) {  // four records in flight at a time; the additions keep their order
+      const float v0 = seg[(long long)o * n + i], v1 = seg[(long long)(o - 1) * n + i];
+      const float v2 = seg[(long long)(o - 2) * n + i], v3 = seg[(long long)(o - 3) * n + i];
+      t = (double)v0 + t / 1.;
+      t = (double)v1 + t / 1.;
+      t = (double)v2 + t / 1.;
+      t = (double)v3 + t / 1.;
+    }
+    for (; o >= 0; o--) t = (double)seg[(long long)o * n + i] + t / 1.;
     total[i] = t;
   }
 }
