@@ -31,7 +31,7 @@ MEASURED_LDS_BYTES = {1: 0, 2: 688460 * 64 * 8}
 # HBM bytes of one whole forward+backward (every kernel and copy of a step), from the same two counter runs: the job
 # moves far fewer bytes than the one-round-trip-per-iteration model because two iterations share a launch, the
 # backward recomputes nothing and iterates are rebuilt from the kept x05 rows instead of being stored.
-MEASURED_STEP_BYTES = {1: (2 * 6932008 + 6307040) * 1024, 2: (2 * 13564395 + 14853807) * 1024}
+MEASURED_STEP_BYTES = {1: (2 * 6743452 + 5939935) * 1024, 2: (2 * 13282875 + 14329346) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):
