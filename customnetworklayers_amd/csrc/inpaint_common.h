@@ -89,7 +89,11 @@ struct Arena {
     int rc = release();
     if (rc) return rc;
     INPAINT_HIP(hipGetDevice(&device));
-    INPAINT_HIP(hipMalloc((void**)&base, need));
+    const hipError_t e = hipMalloc((void**)&base, need);
+    if (e != hipSuccess) {
+      base = nullptr;
+      return fail(INPAINT_ERR_HIP, "hipMalloc of %zu bytes failed: %s", need, hipGetErrorString(e));
+    }
     bytes = need;
     used = 0;
     return 0;

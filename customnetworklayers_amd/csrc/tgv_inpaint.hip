@@ -777,6 +777,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   if (same) return 0;
   int rc = fetch_running_means(s);
   if (rc) return rc;
+  s.guard = nullptr;  // the arena is about to be released; the means live in pending_av until the new one exists
   s.n = n; s.ic = ic; s.ih = ih; s.iw = iw; s.its = its;
   make_schedule(its, s.iterations, s.max_inter_its);
   make_step_sizes(its, s.steps);
@@ -1098,8 +1099,13 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   Slot& s = g_slots[id];
   s.forward_done = false;
   s.x05_valid = false;
-  const int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
+  int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
   rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
+  if (rc && keep == 2) {  // no room for every x05 row: keep the last segment's instead and recompute the others
+    (void)hipGetLastError();
+    keep = 1;
+    rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
+  }
   if (rc) return rc;
   const size_t S3 = state_count(s), SB = S3 * sizeof(float);
   const int K = 2 * (its / 2);

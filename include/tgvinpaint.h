@@ -61,7 +61,7 @@ int tgvinpaint_gradient_mode(int id, int mode);
  * of work and its memory footprint.  1: those of the last segment.  2 (default): all of them -- its states
  * (3 fields each) of memory, no recompute, and the fastest backward.  The gradients are the same bits in every
  * mode.  A forward whose gradients are never asked for is fastest with 0.  Mode 2 falls back to 1 when the rows
- * would need more than INPAINT_KEEP_GB (default 32) GiB; INPAINT_KEEP=0|1|2 overrides this call.
+ * would need more than INPAINT_KEEP_GB (default 32) GiB or the device cannot allocate them; INPAINT_KEEP=0|1|2 overrides this call.
  * No counterpart in the reference, which always recomputes. */
 int tgvinpaint_keep_iterates(int id, int mode);
 

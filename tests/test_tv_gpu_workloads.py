@@ -136,3 +136,35 @@ def test_three_level_hierarchy_matches_oracle(ext, tv_oracle):
         print("\n[hierarchy level %d %s] out %.2e grads %s" % (lvl, cfg["levels"][lvl], e_out, ["%.2e" % e for e in e_g]),
               flush=True)
         assert e_out <= 1e-4 and max(e_g) <= 1e-3
+
+
+def test_keep_all_falls_back_when_the_rows_do_not_fit_the_device(monkeypatch):
+    # 10000 iterations of a 2 x 2 x 1024 x 2048 problem: every x05 row would take 335 GB, more than the device has, so
+    # the allocation fails and the layer keeps the last segment's rows instead (keep mode 1) -- same bits as asking
+    # for mode 1, and a slot of ordinary size
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+
+    n, c, h, w, its = 2, 2, 1024, 2048, 10000
+    d = tv_inputs(n, c, h, w, seed=3, conf_density=0.2)
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    monkeypatch.setenv("INPAINT_KEEP_GB", "100000")  # lift the budget so that mode 2 is really attempted
+    try:
+        ext.reset_id(4)
+        (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 4)
+        grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+        torch.cuda.synchronize()
+        fallback_bytes = ext.slot_bytes(4)
+        assert 0 < fallback_bytes < 40e9
+        ext.reset_id(4)
+        ext.keep_iterates(4, 1)
+        (sol1,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 4)
+        grads1 = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+        torch.cuda.synchronize()
+        assert ext.slot_bytes(4) == fallback_bytes
+        assert torch.equal(sol, sol1)
+        for a, b in zip(grads, grads1):
+            assert torch.equal(a, b)
+        assert bool(torch.isfinite(sol).all())
+    finally:
+        ext.reset_id(4)
