@@ -765,7 +765,7 @@ bool launch_adjoint(Slot& s, hipStream_t stream, const float* dx, const float* d
 
 // Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
 // (third y source xc = slot j-2, or the checkpoint y when B is the segment's first iteration).
-template <int C, bool BEND>
+template <int C, bool BEND, bool TRUE_ADJ>
 void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                                const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                                float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
@@ -776,25 +776,25 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   if (gx_final)
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, true, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
                        s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n,
                        s.ih, s.iw, tA, tB, R, sx, sy);
   else
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
+    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, false, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
                        s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
                        s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n,
                        s.ih, s.iw, tA, tB, R, sx, sy);
 }
 
-template <bool BEND>
+template <bool BEND, bool TRUE_ADJ = false>
 void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c, const float* b,
                          const float* xa, const float* xb, const float* xc, const float* g05_in, float* g05_out,
                          const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   if (s.ic == 1)
-    launch_adjoint_pair_strip<1, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+    launch_adjoint_pair_strip<1, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   else
-    launch_adjoint_pair_strip<2, BEND>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+    launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
 }
 
@@ -982,45 +982,57 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     }
     // reverse sweep (TV.cu:1696-1729)
     int timed_run = 0;
-    if (adjoint_pairs(s) && !corr) {
+    if (adjoint_pairs(s)) {
       // The g05 / g_x ping-pong flips once per launch: `src` holds what the next launch reads.  The
       // first step of the whole backward writes g05[1]; a segment's last launch leaves its result
       // where the next segment picks it up.
       int j = len - 1;
       if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
-        hipLaunchKernelGGL(tv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                           ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
-                           (long long)ih * iw, (long long)P);
+        if (corr)
+          hipLaunchKernelGGL(tv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+                             ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             (long long)ih * iw, (long long)P);
+        else
+          hipLaunchKernelGGL(tv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+                             ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             (long long)ih * iw, (long long)P);
         pp_src = 1;
         j--;
       }
+      // corrected gradient: the same launches with the TRUE_ADJ kernels; a segment's first iteration takes the
+      // checkpointed x (to rebuild the true y_{k0+1}) where the reference's takes the checkpoint y
+      const float* ck = corr ? ckx : cky;
       if (j >= 0 && ((j + 1) & 1)) {  // an odd number of steps is left: one single step, then pairs
         const float* xa = ring + (size_t)j * F;
-        if (j > 0)
-          launch_adjoint<false>(s, stream, dx, dy, c, b, xa, ring + (size_t)(j - 1) * F, nullptr, s.g05[pp_src],
-                                s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j]);
-        else
-          flushed = launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, cky, s.g05[pp_src], s.g05[1 - pp_src],
-                                         s.gxk[pp_src], s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr,
-                                         s.steps[k0 + j]);
+        float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
+        if (j > 0) {
+          const float* xb = ring + (size_t)(j - 1) * F;
+          if (corr) launch_adjoint<false, true>(s, stream, dx, dy, c, b, xa, xb, nullptr, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j]);
+          else launch_adjoint<false>(s, stream, dx, dy, c, b, xa, xb, nullptr, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j]);
+        } else {
+          float* gf = outer == 0 ? s.gx_final : nullptr;
+          if (corr) flushed = launch_adjoint<true, true>(s, stream, dx, dy, c, b, xa, xa, ck, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j]);
+          else flushed = launch_adjoint<true>(s, stream, dx, dy, c, b, xa, xa, ck, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j]);
+        }
         pp_src = 1 - pp_src;
         j--;
       }
       for (; j >= 1; j -= 2) {
         const float* xa = ring + (size_t)j * F;
         const float* xb = ring + (size_t)(j - 1) * F;
+        float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
         if (j - 1 > 0) {
+          const float* xc = ring + (size_t)(j - 2) * F;
           if (timed_run == 0) g_timer.begin(stream);
-          launch_adjoint_pair<false>(s, stream, dx, dy, c, b, xa, xb, ring + (size_t)(j - 2) * F, s.g05[pp_src],
-                                     s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j],
-                                     s.steps[k0 + j - 1]);
+          if (corr) launch_adjoint_pair<false, true>(s, stream, dx, dy, c, b, xa, xb, xc, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j], s.steps[k0 + j - 1]);
+          else launch_adjoint_pair<false>(s, stream, dx, dy, c, b, xa, xb, xc, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j], s.steps[k0 + j - 1]);
           timed_run++;
           if (j - 2 <= 1) g_timer.end(stream, timed_run);  // one event pair around the sweep's run of launches
         } else {
           // B is the segment's first iteration; the very last one's g_x is the gradient wrt the start
-          launch_adjoint_pair<true>(s, stream, dx, dy, c, b, xa, xb, cky, s.g05[pp_src], s.g05[1 - pp_src],
-                                    s.gxk[pp_src], s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr,
-                                    s.steps[k0 + j], s.steps[k0 + j - 1]);
+          float* gf = outer == 0 ? s.gx_final : nullptr;
+          if (corr) launch_adjoint_pair<true, true>(s, stream, dx, dy, c, b, xa, xb, ck, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j], s.steps[k0 + j - 1]);
+          else launch_adjoint_pair<true>(s, stream, dx, dy, c, b, xa, xb, ck, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j], s.steps[k0 + j - 1]);
           flushed = true;
         }
         pp_src = 1 - pp_src;
@@ -1080,9 +1092,10 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   if (seg_mode) hipLaunchKernelGGL(combine_segments_many, dim3(gF, 4), dim3(256), 0, stream, sj, nseg);
   if (corr && 2 * (its / 2) > 0) {
     // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it); the last
-    // step above left g05[0] and the partial g_x[0] in the `0` halves of the ping-pongs, checkpoint 0 is y_0
-    hipLaunchKernelGGL(tv_adjoint_iter0, dim3(grid1d((long long)P)), dim3(256), 0, stream, dx, dy, s.ckpt_y, s.g05[0],
-                       s.gxk[0], s.gx_final, s.tot_gx, s.tot_gy, ic, ih, iw, (long long)P);
+    // step above left g05[0] and the partial g_x[0] in the halves of the ping-pongs it wrote, checkpoint 0 is y_0
+    const int last = adjoint_pairs(s) ? pp_src : 0;
+    hipLaunchKernelGGL(tv_adjoint_iter0, dim3(grid1d((long long)P)), dim3(256), 0, stream, dx, dy, s.ckpt_y, s.g05[last],
+                       s.gxk[last], s.gx_final, s.tot_gx, s.tot_gy, ic, ih, iw, (long long)P);
   }
   // output guard on the device (TV.cu:1760-1791), then scale and store (TV.cu:1795-1818)
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);

@@ -790,7 +790,8 @@ struct Adj2Row {
   double opc_d;
 };
 
-template <int C, bool BEND, bool FINAL>
+// TRUE_ADJ: the corrected gradient, as in tv_adjoint_strip (with BEND, x05c is the checkpointed x of the segment start).
+template <int C, bool BEND, bool FINAL, bool TRUE_ADJ = false>
 __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
@@ -864,8 +865,15 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.xb[ch] : 0.f, xc = ok ? o.yB[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
-      o.yA[ch] = rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, tA);
-      o.yB[ch] = BEND ? xc : rebuild_y_fast(bv, xb, xc, o.c, o.rc1, o.opc_d, tB);
+      if (TRUE_ADJ) {
+        const float pa = prox_huber1(xa, o.c, o.rc1, bv), pb = prox_huber1(xb, o.c, o.rc1, bv);
+        const float pc = BEND ? xc : prox_huber1(xc, o.c, o.rc1, bv);
+        o.yA[ch] = pa + tA * (pa - pb);
+        o.yB[ch] = pb + tB * (pb - pc);
+      } else {
+        o.yA[ch] = rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, tA);
+        o.yB[ch] = BEND ? xc : rebuild_y_fast(bv, xb, xc, o.c, o.rc1, o.opc_d, tB);
+      }
       o.g[ch] = ok ? o.g[ch] : 0.f;
       o.xa[ch] = xa;
       o.xb[ch] = xb;
@@ -873,6 +881,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     }
   };
 
+  constexpr float kGX = TRUE_ADJ ? 1.f : kLocalGXMult, kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
   struct Tri {  // everything one triangle contributes (see tv_adjoint_strip)
     float O1, O2, O3, O4, n3, n4, l1, l3, l4, ux, uy;
   };
@@ -906,13 +915,13 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     r.l3 = from_left_lane(P2 * tl);
     r.l4 = from_left_lane(P1 * tl);
     if (!end_form.value) {  // TV.cu:749-769
-      r.ux = kLocalGXMult * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
-      r.uy = kLocalGXMult * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
+      r.ux = kGX * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
+      r.uy = kGX * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
     } else {  // TV.cu:1019-1037
-      const float ux_a = kLocalGXMult * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
-      const float uy_a = kLocalGXMult * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
-      r.ux = act ? ux_a : kLocalGXMult * d2 * gpr;
-      r.uy = act ? uy_a : kLocalGXMult * d1 * gpd;
+      const float ux_a = kGX * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
+      const float uy_a = kGX * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
+      r.ux = act ? ux_a : kGX * d2 * gpr;
+      r.uy = act ? uy_a : kGX * d1 * gpd;
     }
     return r;
   };
@@ -938,12 +947,12 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     const float sign = (diff < 0) ? -1.f : 1.f;
     const bool quad = (opc_d >= (double)(sign * diff));
     const float opc = 1.f + conf;
-    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kLocalGCMult;
+    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
     const float g05_q = div_by(df, opc, rc1);
     const float gb_q = div_by(df * conf, opc, rc1) * 1.0f;
     const bool mid = !quad && (conf >= sign * diff);
     g05v = quad ? g05_q : (mid ? 0.f : df);
-    gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kLocalGCMult);
+    gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kGC);
     gb_add = quad ? gb_q : (mid ? df * 1.0f : 0.f);
   };
 
@@ -959,7 +968,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
   }
   const std::true_type kYes{};
   const std::false_type kNo{};
-  const std::integral_constant<bool, BEND> kBEnd{};
+  const std::integral_constant<bool, BEND && !TRUE_ADJ> kBEnd{};  // the corrected gradient has one arithmetic form
 
   auto step = [&](int k, const Adj2Row<C>& cur, const Adj2Row<C>& nxt, auto do_a, auto tri_b, auto do_b) {
     const int h = g.hs - 2 + k;  // A's row; B's row is h - 1
