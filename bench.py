@@ -377,9 +377,8 @@ def main():
         kernel_name = "tvstrip::tv_adjoint_strip<2,false,false>"
     if cfg["kind"] == "tgv" and (os.environ.get("INPAINT_TGV_FUSE", "1") == "0" or os.environ.get("INPAINT_TGV_FUSE_ADJ", "1") == "0"):
         kernel_name = "tgvstrip::tgv_adjoint_strip<2,false,false>"
-    if args.corrected_gradient:  # (the TGV layer's corrected gradient runs one adjoint step per launch)
-        kernel_name = ("tvstrip::tv_adjoint_strip2<2,false,false,true>" if cfg["kind"] == "tv"
-                       else "tgvstrip::tgv_adjoint_strip<2,false,false,1>")
+    if args.corrected_gradient:
+        kernel_name = kernel_name.replace(">", ",true>")
     profile, profile_read = getattr(lib, prefix + "_profile"), getattr(lib, prefix + "_profile_read")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     its, pid = cfg["its"], 0

@@ -1042,15 +1042,21 @@ void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b,
 
 // Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
 // (xc = slot j-2, or the checkpoint y when B is the segment's first iteration).
-template <int C, bool BEND>
+// Whether the pair kernel runs its two steps in two wavefronts (the default with two channels).
+bool pair_split(int channels) {
+  const char* e = getenv("INPAINT_TGV_PAIR_WAVES");
+  return e ? strcmp(e, "2") == 0 : channels >= 2;
+}
+
+// TRUE_ADJ (the corrected gradient) exists for the two-wavefront kernel only; the caller checks pair_split().
+template <int C, bool BEND, bool TRUE_ADJ>
 void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
                                const float* xb, const float* xc, const float* g05_in, float* g05_out, const float* gxk,
                                float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
   // two channels: the two steps run in two wavefronts of a workgroup (one strip per 128-thread workgroup);
   // one channel: both steps fit one wavefront's registers (four strips per 256-thread workgroup)
-  const char* e = getenv("INPAINT_TGV_PAIR_WAVES");
-  const bool split = e ? strcmp(e, "2") == 0 : C >= 2;
+  const bool split = pair_split(C);
   const int R = split ? pair_split_rows(s.n, s.ih, s.iw) : strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
@@ -1061,8 +1067,8 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
       s.iw, tA, tB, R, sx, sy
   if (split) {
     const dim3 grid((unsigned)((waves + 7) / 8 * 8)), block(128);
-    if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, true>), grid, block, 0, stream, TGV_PAIR_ARGS);
-    else hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, false>), grid, block, 0, stream, TGV_PAIR_ARGS);
+    if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, true, TRUE_ADJ>), grid, block, 0, stream, TGV_PAIR_ARGS);
+    else hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, false, TRUE_ADJ>), grid, block, 0, stream, TGV_PAIR_ARGS);
   } else {
     const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
     if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, TGV_PAIR_ARGS);
@@ -1071,12 +1077,12 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
 #undef TGV_PAIR_ARGS
 }
 
-template <bool BEND>
+template <bool BEND, bool TRUE_ADJ = false>
 void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa, const float* xb,
                          const float* xc, const float* g05_in, float* g05_out, const float* gxk, float* gxk_m1,
                          float* gx_final, float tA, float tB) {
-  if (s.ic == 1) launch_adjoint_pair_strip<1, BEND>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
-  else launch_adjoint_pair_strip<2, BEND>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  if (s.ic == 1) launch_adjoint_pair_strip<1, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
 }
 
@@ -1256,6 +1262,8 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   // keep it in gxk[1] as the reference does.
   const bool strip = use_strip(s);
   const float* gi_src = strip ? s.gx_final : s.gxk[1];
+  // the corrected gradient has a pair kernel in the two-wavefront form only
+  const bool pairs = adjoint_pairs(s) && (!corr || pair_split(s.ic));
   int lastIt = its;
   int pp_src = 1;
   const int nseg = (int)s.iterations.size();
@@ -1294,41 +1302,54 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     }
     int timed_run = 0;
     bool flushed = false;  // the pair that ends the segment adds the segment sums to the totals itself
-    if (adjoint_pairs(s) && !corr) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
+    if (pairs) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
       // `pp_src` = the g05 / g_x buffer the next launch reads; it flips once per launch
       int j = len - 1;
       if (outer == nseg - 1 && j >= 0) {
-        hipLaunchKernelGGL(tgv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                           ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
-                           (long long)ih * iw, (long long)P);
+        if (corr)
+          hipLaunchKernelGGL(tgv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+                             ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             (long long)ih * iw, (long long)P);
+        else
+          hipLaunchKernelGGL(tgv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
+                             ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             (long long)ih * iw, (long long)P);
         pp_src = 1;
         j--;
       }
       if (j >= 0 && ((j + 1) & 1)) {  // an odd number of steps is left: one single step, then pairs
         const float* xa = ring + (size_t)j * S3;
-        if (j > 0)
-          launch_adjoint<false>(s, stream, c, b, xa, ring + (size_t)(j - 1) * S3, nullptr, s.g05[pp_src],
-                                s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j]);
-        else
-          launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[pp_src], s.g05[1 - pp_src], s.gxk[pp_src],
-                               s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr, s.steps[k0 + j]);
+        float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
+        float* gf = outer == 0 ? s.gx_final : nullptr;
+        if (j > 0) {
+          const float* xb = ring + (size_t)(j - 1) * S3;
+          if (corr) launch_adjoint<false, 1>(s, stream, c, b, xa, xb, nullptr, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j]);
+          else launch_adjoint<false>(s, stream, c, b, xa, xb, nullptr, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j]);
+        } else if (corr) {
+          launch_adjoint<false, 2>(s, stream, c, b, xa, ckx, nullptr, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j]);
+        } else {
+          launch_adjoint<true>(s, stream, c, b, xa, xa, cky, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j]);
+        }
         pp_src = 1 - pp_src;
         j--;
       }
       for (; j >= 1; j -= 2) {
         const float* xa = ring + (size_t)j * S3;
         const float* xb = ring + (size_t)(j - 1) * S3;
+        float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
         if (j - 1 > 0) {
+          const float* xc = ring + (size_t)(j - 2) * S3;
           if (timed_run == 0) g_timer.begin(stream);
-          launch_adjoint_pair<false>(s, stream, c, b, xa, xb, ring + (size_t)(j - 2) * S3, s.g05[pp_src],
-                                     s.g05[1 - pp_src], s.gxk[pp_src], s.gxk[1 - pp_src], nullptr, s.steps[k0 + j],
-                                     s.steps[k0 + j - 1]);
+          if (corr) launch_adjoint_pair<false, true>(s, stream, c, b, xa, xb, xc, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j], s.steps[k0 + j - 1]);
+          else launch_adjoint_pair<false>(s, stream, c, b, xa, xb, xc, g_in, g_out, x_in, x_out, nullptr, s.steps[k0 + j], s.steps[k0 + j - 1]);
           timed_run++;
           if (j - 2 <= 1) g_timer.end(stream, timed_run);
         } else {
-          launch_adjoint_pair<true>(s, stream, c, b, xa, xb, cky, s.g05[pp_src], s.g05[1 - pp_src], s.gxk[pp_src],
-                                    s.gxk[1 - pp_src], outer == 0 ? s.gx_final : nullptr, s.steps[k0 + j],
-                                    s.steps[k0 + j - 1]);
+          // B is the segment's first iteration: the checkpoint y (the corrected gradient: the checkpointed x, from
+          // which the true y_{k0+1} is rebuilt) stands where x05[j-2] does otherwise
+          float* gf = outer == 0 ? s.gx_final : nullptr;
+          if (corr) launch_adjoint_pair<true, true>(s, stream, c, b, xa, xb, ckx, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j], s.steps[k0 + j - 1]);
+          else launch_adjoint_pair<true>(s, stream, c, b, xa, xb, cky, g_in, g_out, x_in, x_out, gf, s.steps[k0 + j], s.steps[k0 + j - 1]);
           flushed = true;
         }
         pp_src = 1 - pp_src;
@@ -1389,13 +1410,14 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   if (seg_mode) hipLaunchKernelGGL(combine_segments_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, sj, nseg);
   if (corr && 2 * (its / 2) > 0) {
     // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it).  The last
-    // step above left g05[0] and the partial g_x[0] in the `0` halves of the ping-pongs; checkpoint 0 is y_0; the
+    // step above left g05[0] and the partial g_x[0] in the halves of the ping-pongs it wrote; checkpoint 0 is y_0; the
     // accumulators are zero after the flush and take iteration 0's weight gradients, which a second flush adds.
     const int a = s.acc_cur;
     const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
+    const int last = pairs ? pp_src : 0;
     hipLaunchKernelGGL((tgv_adjoint_px<false, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, s.ckpt_y,
-                       s.acc_gc[a], s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], s.g05[0], s.gx_final, s.gxk[0], s.gxk[1],
-                       s.ckpt_y, s.ic, s.ih, s.iw, 0.f);
+                       s.acc_gc[a], s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], s.g05[last], s.gx_final, s.gxk[last],
+                       s.gxk[1 - last], s.ckpt_y, s.ic, s.ih, s.iw, 0.f);
     hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
     hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
   }

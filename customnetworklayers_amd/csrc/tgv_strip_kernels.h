@@ -912,6 +912,7 @@ struct Adj2Row {
   float yA[3][C];  // yA[0] rebuilt from x05[j], x05[j-1]; yA[1], yA[2] = aux of x05[j]
   float yB[3][C];  // yB[0] rebuilt from x05[j-1], x05[j-2] (loaded there); yB[1], yB[2] = aux of x05[j-1]; BEND: checkpoint y
   float xa0[C], xb0[C], bb[C], g[3][C];
+  float pv[2][C];  // corrected gradient only: aux of x05[j-1]
 };
 template <int C>
 struct Adj2Late {
@@ -1371,15 +1372,18 @@ struct Adj2ARow {
   float c, wxs, wys, bxs, bys;
   float yA[3][C];  // yA[0] rebuilt from x05[j], x05[j-1]; yA[1], yA[2] = aux of x05[j]
   float xa0[C], xb0[C], bb[C], g[3][C];
+  float pv[2][C];  // corrected gradient only: aux of x05[j-1]
 };
 template <int C>
 struct Adj2BRow {
   float c, wxs, wys, bxs, bys;
   float yB[3][C];  // yB[0] rebuilt from x05[j-1], x05[j-2] (loaded there); yB[1], yB[2] = aux of x05[j-1]; BEND: checkpoint y
   float xb0[C], bb[C];
+  float pv[2][C];  // corrected gradient only: aux of x05[j-2] (BEND: of the checkpointed x)
 };
 
-template <int C, bool BEND, bool FINAL>
+// TRUE_ADJ: the corrected gradient, as in tgv_adjoint_strip (with BEND, x05c is the checkpointed x of the segment start).
+template <int C, bool BEND, bool FINAL, bool TRUE_ADJ = false>
 __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
@@ -1403,7 +1407,8 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
   const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
   const bool rmask = g.col_ok && g.w < W - 1;
   const double optA = 1. + (double)tA, optB = 1. + (double)tB;
-  const float gxm = kLocalGXMult;
+  const float gxm = TRUE_ADJ ? 1.f : kLocalGXMult;
+  constexpr float kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
   const size_t poff = (size_t)g.n * HW;
   const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
                      *const cf_p = cf + poff;
@@ -1411,7 +1416,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
                      *const gwy0i_p = gwy_in + 2 * poff, *const gwy1i_p = gwy_in + 2 * poff + HW;
   float *const gco_p = gc + poff, *const gwx0o_p = gwx + 2 * poff, *const gwx1o_p = gwx + 2 * poff + HW,
                *const gwy0o_p = gwy + 2 * poff, *const gwy1o_p = gwy + 2 * poff + HW;
-  const float *xa_p[3][C], *xb_p[3][C], *xc_p[C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
+  const float *xa_p[3][C], *xb_p[3][C], *xc_p[C], *pv_p[2][2][C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
   float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
@@ -1422,7 +1427,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     for (int v = 0; v < 3; v++) {
       const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
       xa_p[v][ch] = x05a + q;
-      xb_p[v][ch] = ((BEND && v > 0) ? x05c : x05b) + q;  // B's aux y: x05[j-1], or the checkpoint when BEND
+      xb_p[v][ch] = ((BEND && v > 0 && !TRUE_ADJ) ? x05c : x05b) + q;  // B's aux y: x05[j-1], or the checkpoint when BEND
+      if (v > 0) {  // corrected gradient: the aux rows before A's and B's, for the momentum of aux y
+        pv_p[0][v - 1][ch] = x05b + q;
+        pv_p[1][v - 1][ch] = x05c + q;
+      }
       g_p[v][ch] = g05_in + q; gxi_p[v][ch] = gxk + q;
       g05o_p[v][ch] = g05_out + q; gxm_p[v][ch] = gxk_m1 + q; gxf_p[v][ch] = FINAL ? gx_final + q : nullptr;
     }
@@ -1507,7 +1516,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     const float S2 = dg2x * u21 + dg2y * u22;
     const float dv2 = dg2x * u21 * bY + dg2y * u22 * bY;
     const float R2 = act2 ? bY * dW2 * (u21 + u22) * dv2 : 0.f;
-    const float dW2_below = end_form.value ? dW2 : exact_div(W2, h2sq);  // TGV.cu:355
+    const float dW2_below = (end_form.value || TRUE_ADJ) ? dW2 : exact_div(W2, h2sq);  // TGV.cu:355
     const float N2y = act2 ? bY * (dW2_below * bY * u22) * S2 : 0.f;
     const float N2x = act2 ? bY * (dW2 * bY * u21) * S2 : 0.f;
 
@@ -1605,19 +1614,19 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     const float sign = (diff < 0) ? -1.f : 1.f;
     const bool quad = (opc_d >= (double)(sign * diff));
     const float opc = 1.f + conf;
-    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kLocalGCMult;
+    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
     const float g05_q = div_by(df, opc, rc1);
     const float gb_q = div_by(df * conf, opc, rc1) * 1.0f;
     const bool mid = !quad && (conf >= sign * diff);
     o.g05v = quad ? g05_q : (mid ? 0.f : df);
-    o.gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kLocalGCMult);
+    o.gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kGC);
     o.gb_add = quad ? gb_q : (mid ? df * 1.0f : 0.f);
     return o;
   };
 
   const std::true_type kYes{};
   const std::false_type kNo{};
-  const std::integral_constant<bool, BEND> kBEnd{};
+  const std::integral_constant<bool, BEND && !TRUE_ADJ> kBEnd{};  // the corrected gradient has one arithmetic form
 
   if (role == 0) {
     // ---------------------------------- step A ----------------------------------
@@ -1635,6 +1644,10 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
         in.yA[1][ch] = ldg(xa_p[1][ch], off);
         in.yA[2][ch] = ldg(xa_p[2][ch], off);
         in.xb0[ch] = ldg(xb_p[0][ch], off);
+        if (TRUE_ADJ) {
+          in.pv[0][ch] = ldg(pv_p[0][0][ch], off);
+          in.pv[1][ch] = ldg(pv_p[0][1][ch], off);
+        }
         in.bb[ch] = ldg(b_p[ch], off);
 #pragma unroll
         for (int v = 0; v < 3; v++) in.g[v][ch] = ldg(g_p[v][ch], off);
@@ -1669,11 +1682,19 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
         const float xa = ok ? o.xa0[ch] : 0.f, xb = ok ? o.xb0[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
-        o.yA[0][ch] = tvstrip::rebuild_y_fast(bv, xa, xb, o.c, rc1, opc_d, tA);
+        if (TRUE_ADJ) {
+          const float pa = tvstrip::prox_huber1(xa, o.c, rc1, bv), pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
+          o.yA[0][ch] = pa + tA * (pa - pb);  // TGV.cu:1773
+        } else {
+          o.yA[0][ch] = tvstrip::rebuild_y_fast(bv, xa, xb, o.c, rc1, opc_d, tA);
+        }
         o.xa0[ch] = xa;
         o.bb[ch] = bv;
 #pragma unroll
-        for (int v = 1; v < 3; v++) o.yA[v][ch] = ok ? o.yA[v][ch] : 0.f;
+        for (int v = 1; v < 3; v++) {
+          const float xv = ok ? o.yA[v][ch] : 0.f;
+          o.yA[v][ch] = TRUE_ADJ ? xv + tA * (xv - (ok ? o.pv[v - 1][ch] : 0.f)) : xv;  // TGV.cu:1686-1690
+        }
 #pragma unroll
         for (int v = 0; v < 3; v++) o.g[v][ch] = ok ? o.g[v][ch] : 0.f;
       }
@@ -1778,6 +1799,10 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
         in.yB[1][ch] = ldg(xb_p[1][ch], off);
         in.yB[2][ch] = ldg(xb_p[2][ch], off);
         in.yB[0][ch] = ldg(xc_p[ch], off);
+        if (TRUE_ADJ) {
+          in.pv[0][ch] = ldg(pv_p[1][0][ch], off);
+          in.pv[1][ch] = ldg(pv_p[1][1][ch], off);
+        }
         in.bb[ch] = ldg(b_p[ch], off);
       }
     };
@@ -1794,11 +1819,20 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
         const float xb = ok ? o.xb0[ch] : 0.f, xc = ok ? o.yB[0][ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
-        o.yB[0][ch] = BEND ? xc : tvstrip::rebuild_y_fast(bv, xb, xc, o.c, rc1, opc_d, tB);
+        if (TRUE_ADJ) {
+          const float pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
+          const float pc = BEND ? xc : tvstrip::prox_huber1(xc, o.c, rc1, bv);
+          o.yB[0][ch] = pb + tB * (pb - pc);
+        } else {
+          o.yB[0][ch] = BEND ? xc : tvstrip::rebuild_y_fast(bv, xb, xc, o.c, rc1, opc_d, tB);
+        }
         o.xb0[ch] = xb;
         o.bb[ch] = bv;
 #pragma unroll
-        for (int v = 1; v < 3; v++) o.yB[v][ch] = ok ? o.yB[v][ch] : 0.f;
+        for (int v = 1; v < 3; v++) {
+          const float xv = ok ? o.yB[v][ch] : 0.f;
+          o.yB[v][ch] = TRUE_ADJ ? xv + tB * (xv - (ok ? o.pv[v - 1][ch] : 0.f)) : xv;
+        }
       }
     };
     float dnB[C][6];

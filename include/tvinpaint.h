@@ -60,7 +60,7 @@ int tvinpaint_guard_stats(int id, double* stats25);
  * wrt the start, 1696-1729, 1816), and the multipliers 0.1 / 0.1 / 1.0 and the global 0.1 (63-69) are 1.  The
  * clamp of the adjoint iterates (797-799), the upstream scrub and the output guard stay.  With them inactive the
  * result is the gradient of the forward pass (tests compare it with automatic differentiation).  Strip kernels
- * only (1..4 channels); one adjoint step per launch, so a backward takes about 1.3x the default's time. */
+ * only (1..4 channels); same speed as the default. */
 int tvinpaint_gradient_mode(int id, int mode);
 
 /* Which intermediate iterates (the x05 rows of TVInpaintFista.cu:1678-1687) the next forwards on `id` keep for
