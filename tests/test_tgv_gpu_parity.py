@@ -460,3 +460,32 @@ def test_corrected_gradient_needs_the_strip_kernels(ext):
             ext.gradient_mode(2, 2)
     finally:
         ext.reset_id(2)
+
+
+@pytest.mark.parametrize("env,c", [({"INPAINT_TGV_PAIR_WAVES": "2"}, 1), ({"INPAINT_TGV_FUSE_ADJ": "0"}, 2),
+                                   ({"INPAINT_TGV_PAIR_WAVES": "1"}, 2)])
+def test_corrected_gradient_on_the_other_kernel_selections(ext, tgv_oracle, env, c, monkeypatch):
+    # one channel in the two-wavefront pair kernel, two channels one step per launch, and two channels with the
+    # one-wavefront pair kernel selected (which has no corrected form: the layer must fall back to single steps)
+    n, h, w, its = 2, 45, 130, 12
+    d = varying_inputs(n, c, h, w, seed=17 + c)
+    try:
+        tgv_oracle.set_quirks(**CORRECTED)
+        ref = run_oracle(tgv_oracle, d, its, 2)
+    finally:
+        tgv_oracle.set_quirks()
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        ext.reset_id(2)
+        ext.gradient_mode(2, 1)
+        (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+        grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+        got = (sol.cpu().numpy(), [g.cpu().numpy() for g in grads], None)
+    finally:
+        ext.reset_id(2)
+    compare("corrected, %s" % env, got, ref)
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)

@@ -412,3 +412,28 @@ def test_module_with_the_corrected_gradient(ext, tv_oracle):
     compare("module, corrected", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
     for a, b in zip(got_grads, ref[1]):
         assert np.array_equal(a, b)
+
+
+def test_corrected_gradient_one_step_per_launch(ext, tv_oracle, monkeypatch):
+    # two channels normally take the pair kernels; INPAINT_TV_FUSE_ADJ=0 keeps the one-step corrected kernels covered
+    n, c, h, w, its = 2, 2, 45, 130, 12
+    d = tv_inputs(n, c, h, w, seed=23, conf_density=0.3)
+    try:
+        tv_oracle.set_quirks(**CORRECTED)
+        ref = run_oracle(tv_oracle, d, its, 2)
+    finally:
+        tv_oracle.set_quirks()
+    monkeypatch.setenv("INPAINT_TV_FUSE_ADJ", "0")
+    dev = torch.device("cuda:0")
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    try:
+        ext.reset_id(2)
+        ext.gradient_mode(2, 1)
+        (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+        grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+        got = (sol.cpu().numpy(), [g.cpu().numpy() for g in grads], None)
+    finally:
+        ext.reset_id(2)
+    compare("corrected, one step per launch", got, ref)
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
