@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+
 #include <algorithm>
 #include <cmath>
 #include <cstdarg>
@@ -106,6 +107,46 @@ struct Arena {
   }
   static size_t padded(size_t count, size_t elem) { return ((count * elem + 255) & ~size_t(255)) + 256; }
 };
+
+// ---------------------------------------------------------------------------------------------
+// strip height
+// ---------------------------------------------------------------------------------------------
+inline int compute_unit_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+              ? prop.multiProcessorCount
+              : 256;
+  }
+  return cus;
+}
+
+// Rows per strip (one wavefront per strip, `waves_per_block` of them in a workgroup; `strips` = strips across the
+// image width x samples).  Taller strips re-read fewer halo rows, but the launch should still put about two
+// wavefronts on every SIMD (>= 1792 of them), and the workgroups are dealt to the CUs in whole numbers: the CU with
+// one workgroup more than the others sets the time.  Among the heights that keep the device full, take the one that
+// minimises (workgroups on the fullest CU) x (rows a wavefront walks: R + `lag` halo, pipeline and start-up rows).
+// Measured: 4 x 2 x 384 x 1248, pair kernels: 16 rows (504 workgroups, two per CU) beat 8, 12, 17, 18 and 24;
+// 16 x 2 x 256 x 512: 19 rows (504 workgroups) 9.8 ms, 16 rows (576: three on some CUs) 12.0 ms.
+inline int choose_strip_rows(long long strips, int ih, int waves_per_block, int lag) {
+  const long long cus = compute_unit_count();
+  int best = 0;
+  long long best_cost = 0;
+  for (int R = 3; R <= 32; R++) {
+    const long long waves = strips * ((ih + R - 1) / R);
+    if (waves < 1792) break;  // (waves fall as R grows)
+    const long long blocks = (waves + waves_per_block - 1) / waves_per_block;
+    const long long cost = ((blocks + cus - 1) / cus) * (R + lag);
+    const bool even = ih % R == 0, best_even = best > 0 && ih % best == 0;
+    if (best == 0 || cost < best_cost || (cost == best_cost && (even || !best_even))) {
+      best = R;
+      best_cost = cost;
+    }
+  }
+  return best > 0 ? best : 2;
+}
 
 // ---------------------------------------------------------------------------------------------
 // output guard (reference: check_gradUpdate + update_correct_av_step_host,

@@ -880,19 +880,15 @@ bool use_strip(const Slot& s) {
   if (e && strcmp(e, "px") == 0) return false;
   return s.ic >= 1 && s.ic <= 2;
 }
-int strip_rows(int n, int ih, int iw, const char* env_name) {
+int strip_rows(int n, int ih, int iw, int cols, const char* env_name, int lag) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap between
   // strips, but the launch should still keep every SIMD of the chip busy.
   if (const char* e = getenv(env_name)) {
     const int v = atoi(e);
     if (v >= 1 && v <= 4096) return v;
   }
-  const long long sx = (iw + tgvstrip::kCols - 1) / tgvstrip::kCols;
-  for (int R : {16, 12, 8, 6, 4, 3}) {
-    const long long waves = sx * ((ih + R - 1) / R) * n;
-    if (waves >= 1792) return R;
-  }
-  return 2;
+  const long long sx = (iw + cols - 1) / cols;
+  return choose_strip_rows(sx * n, ih, 4, lag);
 }
 
 // Rows per strip of the two-wavefront pair kernel.  Its workgroups (one strip each) are resident four per CU, so a
@@ -929,16 +925,13 @@ int pair_split_rows(int n, int ih, int iw) {
 template <int C>
 void launch_forward_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                           float* xout, const float* yin, float* yout, float* x05, float t) {
-  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_FWD_ROWS");
+  auto kern = x05 ? tgvstrip::tgv_forward_strip<C, true> : tgvstrip::tgv_forward_strip<C, false>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, "INPAINT_TGV_FWD_ROWS", 6);
   const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
-  if (x05)
-    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip<C, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
-                       xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
-  else
-    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip<C, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
-                       xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xout, yin, yout, x05, s.n, s.ih, s.iw, t,
+                     R, sx, sy);
 }
 
 void launch_forward(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
@@ -959,20 +952,15 @@ template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                                const float* xin_aux, float* xout, const float* yin, float* yout, float* x05a, float* x05b,
                                bool store_x_aux, float tA, float tB, bool ring, float tP) {
-  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_FWD_ROWS");
+  auto kern = tgvstrip::tgv_forward_strip2<C, false>;
+  if (x05a && ring) kern = tgvstrip::tgv_forward_strip2<C, true, true>;
+  else if (x05a) kern = tgvstrip::tgv_forward_strip2<C, true>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, "INPAINT_TGV_FWD_ROWS", 8);
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (x05a && ring)
-    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, true, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
-                       xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, tP, R, sx,
-                       sy);
-  else if (x05a)
-    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
-                       xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
-  else
-    hipLaunchKernelGGL((tgvstrip::tgv_forward_strip2<C, false>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin,
-                       xin_aux, xout, yin, yout, x05a, x05b, store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b,
+                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy);
 }
 
 bool forward_pairs(const Slot& s) {
@@ -998,18 +986,14 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, con
                           const float* xb, const float* yck, const float* g05_in, float* g05_out, const float* gxk,
                           float* gxk_m1, float* gx_final, float t) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
-  const int R = strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
+  auto kern = gx_final ? tgvstrip::tgv_adjoint_strip<C, END, true, ADJ> : tgvstrip::tgv_adjoint_strip<C, END, false, ADJ>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, "INPAINT_TGV_ADJ_ROWS", 6);
   const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (gx_final)
-    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, true, ADJ>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
-                       xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
-                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
-  else
-    hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip<C, END, false, ADJ>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b,
-                       xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o],
-                       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, xb, yck, s.acc_gc[i], s.acc_gc[o],
+                     s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1,
+                     gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
 }
 
 // One adjoint step.  Strip path: y is rebuilt inside the kernel from xa = x05[k], xb = x05[k-1] (END:
@@ -1057,7 +1041,9 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
   // two channels: the two steps run in two wavefronts of a workgroup (one strip per 128-thread workgroup);
   // one channel: both steps fit one wavefront's registers (four strips per 256-thread workgroup)
   const bool split = pair_split(C);
-  const int R = split ? pair_split_rows(s.n, s.ih, s.iw) : strip_rows(s.n, s.ih, s.iw, "INPAINT_TGV_ADJ_ROWS");
+  auto kern1 = gx_final ? tgvstrip::tgv_adjoint_strip2<C, BEND, true> : tgvstrip::tgv_adjoint_strip2<C, BEND, false>;
+  const int R = split ? pair_split_rows(s.n, s.ih, s.iw)
+                      : strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, "INPAINT_TGV_ADJ_ROWS", 8);
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
@@ -1071,8 +1057,7 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
     else hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, false, TRUE_ADJ>), grid, block, 0, stream, TGV_PAIR_ARGS);
   } else {
     const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-    if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, true>), grid, block, 0, stream, TGV_PAIR_ARGS);
-    else hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2<C, BEND, false>), grid, block, 0, stream, TGV_PAIR_ARGS);
+    hipLaunchKernelGGL(kern1, grid, block, 0, stream, TGV_PAIR_ARGS);
   }
 #undef TGV_PAIR_ARGS
 }

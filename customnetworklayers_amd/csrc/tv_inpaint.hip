@@ -626,7 +626,7 @@ int resolve_keep_mode(const Slot& s, int n, int ic, int ih, int iw, int its) {
   }
   return mode;
 }
-int strip_rows(int n, int ih, int iw, int cols, const char* env_name) {
+int strip_rows(int n, int ih, int iw, int cols, const char* env_name, int lag) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap
   // between strips, but the launch should still put about two wavefronts on each of the 1024 SIMDs
   // (measured on the 4 x 2 x 384 x 1248 workload: 16 rows beat 8 and 24).
@@ -635,27 +635,19 @@ int strip_rows(int n, int ih, int iw, int cols, const char* env_name) {
     if (v >= 1 && v <= 4096) return v;
   }
   const long long sx = (iw + cols - 1) / cols;
-  for (int R : {16, 12, 8, 6, 4, 3}) {
-    const long long waves = sx * ((ih + R - 1) / R) * n;
-    if (waves >= 1792) return R;
-  }
-  return 2;
+  return choose_strip_rows(sx * n, ih, 4, lag);
 }
 
 template <int C>
 void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                           const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
                           float t) {
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwdCols, "INPAINT_TV_FWD_ROWS");
+  auto kern = x05 ? tvstrip::tv_forward_strip<C, true> : tvstrip::tv_forward_strip<C, false>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwdCols, "INPAINT_TV_FWD_ROWS", 6);
   const int sx = (s.iw + tvstrip::kFwdCols - 1) / tvstrip::kFwdCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
-  if (x05)
-    hipLaunchKernelGGL((tvstrip::tv_forward_strip<C, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
-                       x05, s.n, s.ih, s.iw, t, R, sx, sy);
-  else
-    hipLaunchKernelGGL((tvstrip::tv_forward_strip<C, false>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin,
-                       yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
 }
 
 // Two forward iterations in one launch (strip path only): (xin, yin) = iterate k, (xout, yout) = iterate k+2;
@@ -664,19 +656,15 @@ template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                                const float* b, const float* xin, float* xout, const float* yin, float* yout,
                                float* x05a, float* x05b, float tA, float tB, bool ring, float tP) {
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_FWD_ROWS");
+  auto kern = tvstrip::tv_forward_strip2<C, false>;
+  if (x05a && ring) kern = tvstrip::tv_forward_strip2<C, true, true>;
+  else if (x05a) kern = tvstrip::tv_forward_strip2<C, true>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_FWD_ROWS", 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (x05a && ring)
-    hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, true, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin,
-                       yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB, tP, R, sx, sy);
-  else if (x05a)
-    hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, true>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
-                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
-  else
-    hipLaunchKernelGGL((tvstrip::tv_forward_strip2<C, false>), grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout,
-                       x05a, x05b, s.n, s.ih, s.iw, tA, tB, 0.f, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB,
+                     (x05a && ring) ? tP : 0.f, R, sx, sy);
 }
 
 bool forward_pairs(const Slot& s) {
@@ -722,20 +710,14 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, co
                           float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, "INPAINT_TV_ADJ_ROWS");
+  auto kern = gx_final ? tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, "INPAINT_TV_ADJ_ROWS", 6);
   const int sx = (s.iw + tvstrip::kAdjCols - 1) / tvstrip::kAdjCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
-  if (gx_final)
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
-                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, t, R, sx,
-                       sy);
-  else
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, yck,
-                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, t, R, sx,
-                       sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i],
+                     s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final,
+                     s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, t, R, sx, sy);
 }
 
 // One adjoint step: reads accumulator set acc_cur, writes the other one, then flips acc_cur.
@@ -771,20 +753,14 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
                                float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_ADJ_ROWS");
+  auto kern = gx_final ? tvstrip::tv_adjoint_strip2<C, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2<C, BEND, false, TRUE_ADJ>;
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_ADJ_ROWS", 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  if (gx_final)
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, true, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
-                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n,
-                       s.ih, s.iw, tA, tB, R, sx, sy);
-  else
-    hipLaunchKernelGGL((tvstrip::tv_adjoint_strip2<C, BEND, false, TRUE_ADJ>), grid, block, 0, stream, dx, dy, c, b, xa, xb, xc,
-                       s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i],
-                       s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n,
-                       s.ih, s.iw, tA, tB, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o],
+                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+                     s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
 }
 
 template <bool BEND, bool TRUE_ADJ = false>
