@@ -128,7 +128,7 @@ inline int compute_unit_count() {
 // wavefronts on every SIMD (>= 1792 of them), and the workgroups are dealt to the CUs in whole numbers: the CU with
 // one workgroup more than the others sets the time.  Among the heights that keep the device full, take the one that
 // minimises (workgroups on the fullest CU) x (rows a wavefront walks: R + `lag` halo, pipeline and start-up rows).
-// Measured: 4 x 2 x 384 x 1248, pair kernels: 16 rows (504 workgroups, two per CU) beat 8, 12, 17, 18 and 24;
+// Measured: 4 x 2 x 384 x 1248, pair kernels: 16 rows (504 workgroups, two per CU) beat 8, 17, 18 and 24;
 // 16 x 2 x 256 x 512: 19 rows (504 workgroups) 9.8 ms, 16 rows (576: three on some CUs) 12.0 ms.
 inline int choose_strip_rows(long long strips, int ih, int waves_per_block, int lag) {
   const long long cus = compute_unit_count();
