@@ -31,13 +31,26 @@ def main():
     tv.reset_id(0)
     sol = tv.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 8, 0)
     gx, gy, gc, gb, gi = tv.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], 8, 0)
-    np.savez_compressed(os.path.join(HERE, "tv_1x2x12x16_its8.npz"), its=8, sol=sol, gx=gx, gy=gy, gc=gc, gb=gb, gi=gi, **d)
+    # the corrected gradient (gradient_mode 1): same forward, the oracle's adjoint with these quirks off
+    tv.set_quirks(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale_factors=0, clamp=1, guard=1)
+    tv.reset_id(0)
+    tv.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 8, 0)
+    cx, cy, cc, cb, ci = tv.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], 8, 0)
+    tv.set_quirks()
+    np.savez_compressed(os.path.join(HERE, "tv_1x2x12x16_its8.npz"), its=8, sol=sol, gx=gx, gy=gy, gc=gc, gb=gb, gi=gi,
+                        corrected_gx=cx, corrected_gy=cy, corrected_gc=cc, corrected_gb=cb, corrected_gi=ci, **d)
 
     d = workloads.tgv_inputs(1, 1, 10, 14, seed=42, conf_density=0.3)
     tgv.reset_id(0)
     sol = tgv.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 6, 0)
     gx, gy, gc, gb, gi = tgv.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], 6, 0)
-    np.savez_compressed(os.path.join(HERE, "tgv_1x1x10x14_its6.npz"), its=6, sol=sol, gx=gx, gy=gy, gc=gc, gb=gb, gi=gi, **d)
+    tgv.set_quirks(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale_factors=0, clamp=1, guard=1, dw_div=0)
+    tgv.reset_id(0)
+    tgv.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 6, 0)
+    cx, cy, cc, cb, ci = tgv.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], 6, 0)
+    tgv.set_quirks()
+    np.savez_compressed(os.path.join(HERE, "tgv_1x1x10x14_its6.npz"), its=6, sol=sol, gx=gx, gy=gy, gc=gc, gb=gb, gi=gi,
+                        corrected_gx=cx, corrected_gy=cy, corrected_gc=cc, corrected_gb=cb, corrected_gi=ci, **d)
 
     d = workloads.quadfit_inputs(1, 4, 12, 18, seed=43, flow_channels=3, amplitude=3.0)
     out = aux.quadfit_forward(d["feat0"], d["feat1"], d["flow"])

@@ -58,6 +58,55 @@ def test_flow_layer_oracles_reproduce_fixtures(flowaux_oracle):
     assert np.array_equal(o.upsample2x_adjoint(v["ga"], v["gb"], 2.0), v["g_sol"])
 
 
+CORRECTED_KEYS = ("corrected_gx", "corrected_gy", "corrected_gc", "corrected_gb", "corrected_gi")
+
+
+@pytest.mark.parametrize("layer,name", [("tv", "tv_1x2x12x16_its8.npz"), ("tgv", "tgv_1x1x10x14_its6.npz")])
+def test_oracles_reproduce_the_corrected_gradient_fixtures(layer, name):
+    from oracle.oracle_lib import TGVOracle, TVOracle
+
+    o = TVOracle() if layer == "tv" else TGVOracle()
+    v = load(name)
+    its = int(v["its"])
+    quirks = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale_factors=0, clamp=1, guard=1)
+    if layer == "tgv":
+        quirks["dw_div"] = 0
+    try:
+        o.set_quirks(**quirks)
+        o.reset_id(0)
+        o.forward(v["dx"], v["dy"], v["dc"], v["db"], v["di"], its, 0)
+        grads = o.backward(v["grad"].copy(), v["dx"], v["dy"], v["dc"], v["db"], its, 0)
+    finally:
+        o.set_quirks()
+    for k, a in zip(CORRECTED_KEYS, grads):
+        assert np.array_equal(a, v[k]), k
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layer,name", [("tv", "tv_1x2x12x16_its8.npz"), ("tgv", "tgv_1x1x10x14_its6.npz")])
+def test_inpainting_layers_reproduce_the_corrected_gradient_fixtures_on_the_gpu(layer, name):
+    import torch
+
+    if layer == "tv":
+        from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+    else:
+        from customnetworklayers_amd.cudaTGV import tgvInpaint_cuda_ext as ext
+    v = load(name)
+    its = int(v["its"])
+    t = {k: torch.from_numpy(v[k]).cuda() for k in ("dx", "dy", "dc", "db", "di", "grad")}
+    try:
+        ext.reset_id(0)
+        ext.gradient_mode(0, 1)
+        (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 0)
+        grads = ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, 0)
+        got = [g.cpu().numpy() for g in grads]
+    finally:
+        ext.reset_id(0)
+    assert np.array_equal(sol.cpu().numpy(), v["sol"])
+    for k, a in zip(CORRECTED_KEYS, got):
+        assert np.array_equal(a, v[k]), k
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("layer,name", [("tv", "tv_1x2x12x16_its8.npz"), ("tgv", "tgv_1x1x10x14_its6.npz")])
 def test_inpainting_layers_reproduce_fixtures_on_the_gpu(layer, name):
