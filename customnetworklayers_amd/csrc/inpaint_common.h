@@ -166,7 +166,7 @@ struct GuardStats {
   unsigned int num_above, num_invalid;
 };
 
-constexpr int kGuardBlocks = 256;  // blocks per tensor in pass 1, each leaves one partial record
+constexpr int kGuardBlocks = 512;  // blocks per tensor in pass 1, each leaves one partial record
 
 struct GuardState {  // lives in device memory, one per id
   double av[5];      // running means: C, X, Y, B, I
