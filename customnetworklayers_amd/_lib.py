@@ -18,6 +18,8 @@ def _load():
     lib = ctypes.CDLL(LIB_PATH)
     lib.tvinpaint_forward.argtypes = [_f32p] * 6 + [_int] * 6 + [ctypes.c_void_p]
     lib.tvinpaint_backward.argtypes = [_f32p] * 10 + [_int] * 6 + [ctypes.c_void_p]
+    lib.tvinpaint_forward_noalloc.argtypes = [_f32p] * 6 + [_int] * 5 + [ctypes.c_void_p]
+    lib.tvinpaint_forward_noalloc_max_floats.restype = ctypes.c_longlong
     lib.tvinpaint_get_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_set_state.argtypes = [_int, ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_reset_id.argtypes = [_int]

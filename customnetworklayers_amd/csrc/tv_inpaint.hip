@@ -782,6 +782,32 @@ bool adjoint_pairs(const Slot& s) {
   return forward_pairs(s) && s.ic <= 2;
 }
 
+// -------------------------------------------------------------------------------------------------
+// Fixed scratch of tvinpaint_forward_noalloc: the y and x ping-pongs of a forward pass (4 fields) in a
+// device array that is part of the code object, so that the call allocates nothing.  Every GPU the
+// library is loaded on holds its own copy (64 MiB) at its own address until the process ends; the
+// name `scratch` is only a host-side handle of it, the address comes from hipGetSymbolAddress, once
+// per device.
+// -------------------------------------------------------------------------------------------------
+constexpr size_t kNoAllocMaxField = size_t(1) << 22;  // floats per field (n*ic*ih*iw), 16 MiB
+constexpr int kNoAllocMaxDevices = 64;
+static __device__ __align__(256) float scratch[4 * kNoAllocMaxField];
+float* g_scratch_ptr[kNoAllocMaxDevices] = {nullptr};
+
+int scratch_of_current_device(float** out) {
+  int dev = -1;
+  INPAINT_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kNoAllocMaxDevices) return fail(INPAINT_ERR_ARG, "device index %d is beyond %d", dev, kNoAllocMaxDevices);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    INPAINT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(INPAINT_ERR_HIP, "hipGetSymbolAddress returned no address for the scratch array");
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -867,6 +893,61 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   s.forward_done = true;
   return 0;
 }
+
+// The forward pass of tvinpaint_forward for callers that cannot allocate (code under graph capture, serving loops):
+// same kernels and launch order, no id, no checkpoints and no x05 rows (nothing is kept for a backward pass), the
+// two iterate ping-pongs in the library's fixed scratch.  Calls no hipMalloc / hipFree.  Nothing in the scratch has
+// to start at zero: every launch writes all pixels of the buffers the next one reads.  Calls that overlap on one
+// GPU (two streams, two threads) share the scratch and race.
+int tvinpaint_forward_noalloc(const float* dx, const float* dy, const float* c, const float* b, const float* init,
+                              float* out, int n, int ic, int ih, int iw, int its, void* stream_) {
+  const void* ptrs[] = {dx, dy, c, b, init, out};
+  int rc = check_common(ptrs, 6, n, ic, ih, iw, its, 0);
+  if (rc) return rc;
+  const unsigned long long F64 = (unsigned long long)n * ic * (unsigned long long)ih * iw;
+  if (F64 > kNoAllocMaxField)
+    return fail(INPAINT_ERR_ARG, "tvinpaint_forward_noalloc: n*ic*ih*iw = %llu floats exceeds the fixed scratch (%zu per field)",
+                F64, kNoAllocMaxField);
+  float* base = nullptr;
+  rc = scratch_of_current_device(&base);
+  if (rc) return rc;
+  hipStream_t stream = (hipStream_t)stream_;
+  Slot s;  // shape only: the launch helpers read n, ic, ih, iw
+  s.n = n; s.ic = ic; s.ih = ih; s.iw = iw; s.its = its;
+  const size_t F = (size_t)F64;
+  float* ypp[2] = {base, base + kNoAllocMaxField};
+  float* xpp[2] = {base + 2 * kNoAllocMaxField, base + 3 * kNoAllocMaxField};
+  const int K = 2 * (its / 2);
+  if (K == 0) {
+    INPAINT_HIP(hipMemcpyAsync(out, init, F * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    return 0;
+  }
+  // extrapolation factors as make_step_sizes produces them (TV.cu:1525-1532), one at a time
+  double t = 1, t_prev = 1;
+  auto next_step = [&]() {
+    t_prev = t;
+    t = (1. + std::sqrt(1. + 4. * t * t)) / 2.;
+    return (float)std::max(0.0, (t_prev - 1.) / t);
+  };
+  if (forward_pairs(s)) {
+    for (int k = 0; k < K; k += 2) {
+      const float tA = next_step(), tB = next_step();
+      const int i = (k >> 1) & 1;
+      launch_forward_pair(s, stream, dx, dy, c, b, k == 0 ? init : xpp[i], k + 2 == K ? out : xpp[1 - i],
+                          k == 0 ? init : ypp[i], ypp[1 - i], nullptr, nullptr, tA, tB);
+    }
+  } else {
+    for (int k = 0; k < K; k++) {
+      const int i = k & 1;
+      launch_forward(s, stream, dx, dy, c, b, k == 0 ? init : xpp[i], k + 1 == K ? out : xpp[1 - i],
+                     k == 0 ? init : ypp[i], ypp[1 - i], nullptr, next_step());
+    }
+  }
+  INPAINT_HIP(hipGetLastError());
+  return 0;
+}
+
+long long tvinpaint_forward_noalloc_max_floats(void) { return (long long)kNoAllocMaxField; }
 
 int tvinpaint_backward(const float* dx, const float* dy, const float* c, const float* b, float* gin, float* gx,
                        float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih, int iw, int its, int id,

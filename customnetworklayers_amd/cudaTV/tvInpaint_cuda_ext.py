@@ -90,6 +90,28 @@ def backward(d_iGf, d_x, d_y, d_c, d_b, its, id):  # noqa: A002
     return [d_oGx, d_oGy, d_oGc, d_oGb, d_oGi]
 
 
+def forward_noalloc(d_x, d_y, d_c, d_b, d_i, its, out):
+    """The forward pass without an id and without any device allocation (not in the reference): the caller passes
+    the output tensor, the iterates live in a fixed array inside the library.  For inference under graph capture or
+    in loops that must not allocate; no backward can follow.  Raises ValueError when d_b holds more than
+    noalloc_max_floats() values.  Calls that overlap on one GPU share the array and race."""
+    for t, name in ((d_x, "d_x"), (d_y, "d_y"), (d_c, "d_c"), (d_b, "d_b"), (d_i, "d_i"), (out, "out")):
+        _check_input(t, name)
+    _check_shapes(d_x, d_y, d_c, d_b, ((d_i, "d_i"), (out, "out")))
+    n, c, h, w = d_b.shape
+    with torch.cuda.device(d_b.device):
+        rc = lib.tvinpaint_forward_noalloc(d_x.data_ptr(), d_y.data_ptr(), d_c.data_ptr(), d_b.data_ptr(), d_i.data_ptr(),
+                                           out.data_ptr(), n, c, h, w, int(its), _stream(d_b))
+    if rc:
+        _raise(rc, "TVInpaint::forward_noalloc")
+    return out
+
+
+def noalloc_max_floats():
+    """Largest n*c*h*w forward_noalloc accepts."""
+    return int(lib.tvinpaint_forward_noalloc_max_floats())
+
+
 def dummy():
     print("Input: not present just dummy:")
     return []

@@ -41,6 +41,19 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
                        float* gx, float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih,
                        int iw, int its, int id, void* stream);
 
+/* The forward pass of tvinpaint_forward for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * Same arguments, kernels and result (bit for bit) as tvinpaint_forward, without an id: nothing is kept for a
+ * backward pass, so there is no matching backward.  The iterate ping-pongs live in a fixed device array inside
+ * the library (64 MiB per GPU, held until the process ends), so the call makes no hipMalloc / hipFree; it returns
+ * INPAINT_ERR_ARG when n*ic*ih*iw exceeds tvinpaint_forward_noalloc_max_floats() (4,194,304 floats = one field of
+ * 16 x 2 x 256 x 512).  All calls on one GPU share that array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls ordered on one stream do not.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make that call outside a graph capture. */
+int tvinpaint_forward_noalloc(const float* dx, const float* dy, const float* c, const float* b, const float* init,
+                              float* out, int n, int ic, int ih, int iw, int its, void* stream);
+long long tvinpaint_forward_noalloc_max_floats(void);
+
 /* Per-id state (idStruct, TVInpaintFista.h:7-50).  state6 (host) = {run, av_GC, av_GX, av_GY, av_GB,
  * av_GI}.  get waits for the slot's stream; reset frees the slot's device buffers as well. */
 int tvinpaint_get_state(int id, double* state6);
