@@ -69,6 +69,10 @@ class TVOracle:
         L.tv_oracle_forward_iter_f64.restype = None
         L.tv_oracle_guard_f64.argtypes = [_f64p, ctypes.c_long, _int, _f64p, _f64p]
         L.tv_oracle_guard_f32.argtypes = [_f32p, ctypes.c_long, _int, _f64p, _f64p]
+        L.tv_oracle_get_yk.argtypes = [_f32p] * 5 + [_int] * 3 + [ctypes.c_float]
+        L.tv_oracle_get_yk.restype = None
+        L.tv_oracle_get_yk_f64.argtypes = [_f64p] * 5 + [_int] * 3 + [ctypes.c_double]
+        L.tv_oracle_get_yk_f64.restype = None
         L.tv_oracle_set_threads.argtypes = [_int]
         L.tv_oracle_set_threads.restype = None
 
@@ -144,6 +148,17 @@ class TVOracle:
         fn = self.lib.tv_oracle_forward_iter_f64 if f64 else self.lib.tv_oracle_forward_iter
         fn(P(wx), P(wy), P(c), P(b), P(x), P(y), P(yout), P(x05) if want_x05 else None, ic, ih, iw, t)
         return (x, yout, x05) if want_x05 else (x, yout)
+
+    def get_yk(self, c, b, x05_it, x05_itm1, t, f64=False):
+        """The backward pass's rebuild of y_{k+1} from x05[k], x05[k-1] on one sample: c (H,W), the rest (C,H,W)."""
+        dt = np.float64 if f64 else np.float32
+        c, b, xa, xb = (_c(a, dt) for a in (c, b, x05_it, x05_itm1))
+        ic, ih, iw = b.shape
+        out = np.empty_like(b)
+        P = _p64 if f64 else _p32
+        fn = self.lib.tv_oracle_get_yk_f64 if f64 else self.lib.tv_oracle_get_yk
+        fn(P(c), P(b), P(xa), P(xb), P(out), ic, ih, iw, t)
+        return out
 
     def guard(self, g, run, av, f32=False):
         """Output guard on one gradient tensor.  Returns (g_new, av_new, action, stats4)."""

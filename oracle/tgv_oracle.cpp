@@ -25,9 +25,16 @@
 //       independently written TGV energy, closed forms, brute-force Lipschitz on small images)
 //   adjoint chain with all quirk toggles OFF ....................... pinned (autograd of an
 //       independently written forward, finite differences)
-//   quirks (segment-start linearisation, skipped iteration 0, dW division in one v2 block, aux y
-//   without momentum, guard on u only, early return on bad upstream), clamp and guard constants:
-//       source reading only -- "parity unpinned".
+//   what the backward pass does differently from the chain rule -- y rebuilt from the half-step
+//   values (aux variables without their extrapolation), the checkpointed y at segment starts, the
+//   skipped Jacobian of iteration 0, the division in one v2 block, the clamp -- and the crossed
+//   beta reads of the Lipschitz kernel .............................. pinned one at a time
+//       (tests/test_tgv_quirk_pins.py: the exact adjoint recursion with autograd Jacobian products
+//       and that one deviation; c = 0 and no-rebuild special cases; a sub-run started at x_1;
+//       a brute-force bound with explicit [row, col] reads); guard on u only, early return on a
+//       bad upstream gradient, multipliers: table / ratio tests in tests/test_tgv_oracle_pins.py.
+//   The numeric constants themselves (0.2, 2000, 0.1, 35, 10, 0.95, 5e6, beta = 4) are values
+//   read off the reference source; nothing else can fix them.
 //
 // The batch dimension n is an extension (the reference accepts n == 1 only, TGV.cpp:77-81):
 // samples are independent problems, each with its own Lipschitz constant; guard statistics run

@@ -13,16 +13,23 @@
 //   * no fused multiply-add contraction (build with -ffp-contract=off); division and sqrt are
 //     the correctly rounded IEEE ones.
 // The reference's own build lets nvcc contract a*b+c into FMAs; that choice is not recoverable
-// from the sources, so results agree with a CUDA run only to rounding (parity unpinned at the
-// ulp level, see the header of tests/test_tv_oracle_pins.py for what *is* pinned).
+// from the sources, so results agree with a CUDA run only to rounding (see the headers of
+// tests/test_tv_oracle_pins.py and tests/test_tv_quirk_pins.py for what is pinned and how).
 //
 // Pin status of the functions below:
 //   forward iteration / schedule / step sizes / prox ......... pinned (closed forms, sparse
 //       Laplacian, convex fixed point, invariants)
 //   adjoint chain with all quirk toggles OFF .................. pinned (autograd of an
 //       independently written forward, finite differences)
-//   quirks Q2, Q3, Q13, clamp and guard constants ............. source reading only:
-//       "parity unpinned" -- nothing but the reference text fixes them.
+//   what the backward pass does differently from the chain rule -- y rebuilt by the get_yk rule,
+//   the checkpointed y at segment starts, the skipped Jacobian of iteration 0, the clamp
+//       ............................................................ pinned one at a time
+//       (tests/test_tv_quirk_pins.py: the exact adjoint recursion with autograd Jacobian products
+//       and that one deviation; c = 0, regimes that never change, a fixed point and a sub-run
+//       started at x_1 as model-free special cases); multipliers and the guard: ratio / table
+//       tests in tests/test_tv_oracle_pins.py.
+//   The numeric constants themselves (0.1, 1e4, 0.1 / 0.1 / 1.0 / 0.1, 50, 10, 0.975, 1e7) are
+//   values read off the reference source; nothing else can fix them.
 //
 // The batch dimension n is an extension (the reference accepts n == 1 only, TV.cpp:61-65):
 // samples are independent problems; guard statistics run over the whole batch tensor.
@@ -727,6 +734,16 @@ void tv_oracle_forward_iter_f64(const double* wx, const double* wy, const double
                                 double* x, const double* y, double* yout, double* x05, int ic, int ih,
                                 int iw, double t) {
   forward_iter<double>(wx, wy, c, b, x, y, yout, x05, ic, ih, iw, t);
+}
+
+// the y rebuild of the backward pass on one sample: y_{k+1} from x05[k] (x05_it) and x05[k-1] (x05_itm1)
+void tv_oracle_get_yk_f64(const double* c, const double* b, const double* x05_it, const double* x05_itm1,
+                          double* yk_out, int ic, int ih, int iw, double t) {
+  get_yk<double>(c, b, x05_it, x05_itm1, yk_out, ic, ih, iw, t);
+}
+void tv_oracle_get_yk(const float* c, const float* b, const float* x05_it, const float* x05_itm1, float* yk_out,
+                      int ic, int ih, int iw, float t) {
+  get_yk<float>(c, b, x05_it, x05_itm1, yk_out, ic, ih, iw, t);
 }
 
 // guard on a double vector (tensors C, X, Y, B) or a float vector (tensor I); `av` is the

@@ -13,11 +13,12 @@ cannot be built here, so each check below is something mathematics fixes:
              through the independent forward, and central finite differences;
   guard      table-driven with this layer's constants (clamp at 5e6, memory 0.95, kill 35x).
 
-What only the reference text fixes (segment-start linearisation and its different arithmetic
-form, skipped iteration-0 adjoint, the y rebuild rule with aux variables taken without momentum,
-the division in one v2 block, guard on u only, early return on a bad upstream gradient, swapped
-beta offsets in the Lipschitz kernel, clamp and guard constants, scale factors) is "parity
-unpinned": the last tests measure each quirk's effect so that a change is visible.
+What the reference's backward does differently from the chain rule (segment-start linearisation,
+skipped iteration-0 adjoint, the y rebuild rule with aux variables taken without momentum, the
+division in one v2 block, the clamp) and the crossed beta reads of the Lipschitz kernel are
+pinned one at a time in tests/test_tgv_quirk_pins.py; the segment-start kernel's different
+arithmetic form, the guard on u only and the early return on a bad upstream gradient are pinned
+below.  The test before the last only records the size of each effect.
 """
 import numpy as np
 import pytest
@@ -387,7 +388,7 @@ def test_bad_id_and_mismatched_backward_are_errors(tgv_oracle):
 
 
 # ------------------------------------------------------------------------------------------------
-# quirks: fixed by the reference text only -- record the size of each effect
+# deviations from the chain rule (pinned in test_tgv_quirk_pins.py): the size of each effect on a realistic input
 # ------------------------------------------------------------------------------------------------
 def test_quirk_effect_sizes_are_visible(tgv_oracle):
     from customnetworklayers_amd.workloads import tgv_inputs

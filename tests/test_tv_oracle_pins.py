@@ -11,9 +11,9 @@ here, so each check below is something mathematics fixes:
             through an independently written forward, and central finite differences;
   guard     table-driven (NaN, > 1e7, 20x and 60x the running mean after 10 calls).
 
-What only the reference text fixes (segment-start linearisation point, skipped iteration-0
-adjoint, the y rebuild rule, clamp and guard constants, gradient scale factors) is "parity
-unpinned": the last test measures each quirk's effect so that a change is visible.
+What the reference's backward does differently from the chain rule (segment-start linearisation
+point, skipped iteration-0 adjoint, the y rebuild rule, the clamp) is pinned one deviation at a
+time in tests/test_tv_quirk_pins.py; the last test here only records the size of each effect.
 """
 import numpy as np
 import pytest
@@ -352,7 +352,7 @@ def test_bad_id_and_mismatched_backward_are_errors(tv_oracle):
 
 
 # ------------------------------------------------------------------------------------------------
-# quirks: fixed by the reference text only -- record the size of each effect
+# deviations from the chain rule (pinned in test_tv_quirk_pins.py): the size of each effect on a realistic input
 # ------------------------------------------------------------------------------------------------
 def test_quirk_effect_sizes_are_visible(tv_oracle):
     from customnetworklayers_amd.workloads import tv_inputs
