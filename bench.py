@@ -15,23 +15,25 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script
-# (headline workload: the two-step adjoint kernel fetches 2 x 87000 KiB, after the copy-kernel
-# calibration, and writes 68035 KiB; profiles/tv_strip_headline_hbm_traffic.txt; config 2, the TGV layer:
-# profiles/tgv_strip_config2_hbm_traffic.txt; configs 5 and 6: profiles/quadfit_config5_*.txt, profiles/median_config6_*.txt).
-# Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: (2 * 86992 + 67886) * 1024, 2: (2 * 165999 + 147003) * 1024,
-                          5: (2 * 408180 + 340500) * 1024, 6: (2 * 131080 + 247100) * 1024}
-# LDS bytes per launch of the dominant kernel (rocprofv3 --pmc SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT: the TV strip kernels
-# issue no LDS instruction at all -- neighbours are exchanged through DPP in registers; the two-wavefront TGV pair kernel
-# hands 7C+5 = 19 floats per lane and row from step A to step B: 688460 two-dword instructions, no bank conflicts).
-# Peak: 128 B per clock and CU x 256 CUs x 2.4 GHz.
+# Counter figures that no bench run can take itself (rocprofv3 --pmc needs a run of its own); each names the file under
+# profiles/ that holds it and the commit of the library it was read at.
+#   traffic   HBM bytes per launch of the dominant kernel: FETCH_SIZE (scaled by the copy-kernel calibration of the
+#             same run) + WRITE_SIZE
+#   step      HBM bytes of one whole forward+backward (every kernel and copy)
+#   lds       LDS bytes per launch of the dominant kernel (SQ_INSTS_LDS x 64 lanes x 8 B; the TV strip kernels issue
+#             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
+#   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
+COUNTERS = {
+    1: dict(traffic=(2 * 86992 + 67886) * 1024, step=(2 * 6743452 + 5939935) * 1024, lds=0, rocprof_ms=0.06121,
+            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="a48ee64"),
+    2: dict(traffic=(2 * 165999 + 147003) * 1024, step=(2 * 13282875 + 14329346) * 1024, lds=688460 * 64 * 8, rocprof_ms=0.13565,
+            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="a48ee64"),
+    5: dict(traffic=(2 * 408180 + 340500) * 1024, files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
+    6: dict(traffic=(2 * 131080 + 247100) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
+}
+MEASURED_TRAFFIC_BYTES = {k: v["traffic"] for k, v in COUNTERS.items()}
+# Peak LDS rate: 128 B per clock and CU x 256 CUs x 2.4 GHz.
 LDS_PEAK_GBS = 128 * 256 * 2.4
-MEASURED_LDS_BYTES = {1: 0, 2: 688460 * 64 * 8}
-# HBM bytes of one whole forward+backward (every kernel and copy of a step), from the same two counter runs: the job
-# moves far fewer bytes than the one-round-trip-per-iteration model because two iterations share a launch, the
-# backward recomputes nothing and iterates are rebuilt from the kept x05 rows instead of being stored.
-MEASURED_STEP_BYTES = {1: (2 * 6743452 + 5939935) * 1024, 2: (2 * 13282875 + 14329346) * 1024}
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):
@@ -340,44 +342,39 @@ def bench_hierarchy(args, cfg):
         t_all = min(once(), once())
         out["cpu_baseline"] = dict(value=round(pxit / n / t_all / 1e6, 3), unit="Mpixel-iter/s", cores=cores, kind="port",
                                    sample="1 of %d samples, all levels, fwd+bwd, best of 2" % n, host_cpu_count=os.cpu_count())
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--config", type=int, default=1,
-                    help="workload index (1 = headline TV layer, 2 = TGV layer, 3 = three-level TV hierarchy, 5 = quadratic fit, 6 = median)")
-    ap.add_argument("--corrected-gradient", action="store_true",
-                    help="configs 1 and 2: time the opt-in corrected gradient instead of the reference's (not the headline)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
-              "see DESIGN.md)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-
+def event_median_ms(step, steps):
+    """Median duration of `steps` more calls of step(), each bracketed by its own pair of HIP events on the stream
+    the layers launch on (torch's current stream)."""
     import torch
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    ms = sorted(a.elapsed_time(b) for a, b in ev)
+    return ms[len(ms) // 2]
+
+
+def bench_layer(config, steps, warmup, corrected=False, keep=None, detail=True):
+    """Configs 0, 1, 2, 4: one TV or TGV layer, forward + backward per step.  Returns the result dict."""
+    import torch
+
     from customnetworklayers_amd._lib import lib
     from customnetworklayers_amd.workloads import config_inputs
 
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
-    from customnetworklayers_amd.workloads import CONFIGS
-    if CONFIGS[args.config]["kind"] == "tv_hierarchy":
-        return bench_hierarchy(args, CONFIGS[args.config])
-    cfg, d = config_inputs(args.config, seed=0)
-    if cfg["kind"] in ("quadfit", "median"):
-        return bench_flowaux(args, cfg, d)
-    assert cfg["kind"] in ("tv", "tgv")
+    cfg, d = config_inputs(config, seed=0)
     ext, prefix, _, _, kernel_name = layer_of(cfg["kind"])
     if cfg["kind"] == "tv" and (os.environ.get("INPAINT_TV_FUSE", "1") == "0" or os.environ.get("INPAINT_TV_FUSE_ADJ", "1") == "0"):
         kernel_name = "tvstrip::tv_adjoint_strip<2,false,false>"
     if cfg["kind"] == "tgv" and (os.environ.get("INPAINT_TGV_FUSE", "1") == "0" or os.environ.get("INPAINT_TGV_FUSE_ADJ", "1") == "0"):
         kernel_name = "tgvstrip::tgv_adjoint_strip<2,false,false>"
-    if args.corrected_gradient:
+    if corrected:
         kernel_name = kernel_name.replace(">", ",true>")
     profile, profile_read = getattr(lib, prefix + "_profile"), getattr(lib, prefix + "_profile_read")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
@@ -390,58 +387,138 @@ def main():
         return ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, pid)
 
     ext.reset_id(pid)
-    if args.corrected_gradient:
+    if corrected:
         ext.gradient_mode(pid, 1)
-    for _ in range(args.warmup):
+    if keep is not None:
+        ext.keep_iterates(pid, keep)
+    for _ in range(warmup):
         step()
+    # the timed region: exactly `steps` steps between two synchronisations, nothing else inside
     torch.cuda.synchronize()
-    profile(1)  # HIP events around every launch of the main adjoint kernel
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    sec = elapsed / steps
+    med_ms = event_median_ms(step, steps)
+    slot_bytes = int(getattr(lib, prefix + "_slot_bytes")(pid))
+    label = cfg["kind"].upper() + (" (corrected gradient)" if corrected else "")
+    out = {
+        "metric": "%s-FISTA fwd+bwd Mpixel-iter/s at %dx%dx%dx%d; achieved HBM GB/s vs peak" % (label, n, c, h, w),
+        "value": round(pxit / sec / 1e6, 2), "unit": "Mpixel-iter/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(sec * 1e3, 4), "ms_per_step_event_median": round(med_ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": label + " inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
+                               % (n, c, h, w, its, config), "pixel_iterations_per_step": pxit,
+                   "keep_mode": 2 if keep is None else keep, "slot_bytes": slot_bytes},
+    }
+    if not detail:
+        ext.reset_id(pid)
+        return out, cfg
+    # one more, untimed run of steps with event pairs around each reverse sweep's launches of the dominant kernel
+    profile(1)
+    for _ in range(min(steps, 5)):
+        step()
+    torch.cuda.synchronize()
     tot_ms, launches = ctypes.c_double(0), ctypes.c_int(0)
     profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
     profile(0)
-
-    ms_per_step = elapsed * 1e3 / args.steps
-    value = pxit / (elapsed / args.steps) / 1e6
+    ext.reset_id(pid)
     bpp = algorithmic_bytes_per_pixel(c, cfg["kind"])
     kernel_ms = tot_ms.value / max(launches.value, 1)
-    # the dominant kernel runs two adjoint steps per launch
-    steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2
-    measured_cfg = args.config
-    label = cfg["kind"].upper()
-    if args.corrected_gradient:  # the counters were read on the default gradient
-        label += " (corrected gradient)"
-        measured_cfg = None
+    steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2  # the pair kernels run two adjoint steps
+    cnt = COUNTERS.get(config) if not corrected and keep is None else None  # the counters were read on the default path
     kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
-    whole_gbs = bpp["total"] * pxit / (elapsed / args.steps) / 1e9
-    out = {
-        "metric": "%s-FISTA fwd+bwd Mpixel-iter/s at %dx%dx%dx%d; achieved HBM GB/s vs peak"
-                  % (label, n, c, h, w),
-        "value": round(value, 2), "unit": "Mpixel-iter/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": label + " inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations (config %d)"
-                               % (n, c, h, w, its, args.config), "pixel_iterations_per_step": pxit},
-        "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(whole_gbs, 1),
-                      "frac_of_hbm_peak": round(whole_gbs / HBM_PEAK_GBS, 4),
-                      "effective_bytes_per_pixel_iteration": (round(MEASURED_STEP_BYTES[measured_cfg] / pxit, 1)
-                                                              if measured_cfg in MEASURED_STEP_BYTES else None),
-                      "effective_GBps": (round(MEASURED_STEP_BYTES[measured_cfg] / (elapsed / args.steps) / 1e9, 1)
-                                         if measured_cfg in MEASURED_STEP_BYTES else None)},
-        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(measured_cfg), "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
-                     "avg_launch_ms": round(kernel_ms, 5), "launches_timed": launches.value},
-    }
-    if measured_cfg in MEASURED_LDS_BYTES and kernel_ms > 0:
-        lds_gbs = MEASURED_LDS_BYTES[measured_cfg] / (kernel_ms * 1e-3) / 1e9
-        out["roofline"]["lds"] = {"bytes_per_launch": MEASURED_LDS_BYTES[measured_cfg], "achieved_GBps": round(lds_gbs, 1),
-                                  "peak_GBps": round(LDS_PEAK_GBS, 1), "frac": round(lds_gbs / LDS_PEAK_GBS, 4)}
+    model_gbs = bpp["total"] * pxit / sec / 1e9
+    out["whole_job"] = {
+        # the one-round-trip-per-iteration model counts a recompute this build does not execute (keep mode 2) and one
+        # round trip per iteration where a pair launch makes one per two, so its rate may exceed the HBM peak
+        "model_bytes_per_pixel_iteration": bpp["total"], "model_GBps": round(model_gbs, 1),
+        "model_frac_of_hbm_peak": round(model_gbs / HBM_PEAK_GBS, 4),
+        "effective_bytes_per_pixel_iteration": round(cnt["step"] / pxit, 1) if cnt and "step" in cnt else None,
+        "effective_GBps": round(cnt["step"] / sec / 1e9, 1) if cnt and "step" in cnt else None,
+        "effective_frac_of_hbm_peak": round(cnt["step"] / sec / 1e9 / HBM_PEAK_GBS, 4) if cnt and "step" in cnt else None}
+    roof = {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": cnt["traffic"] if cnt else None,
+            "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
+            "avg_launch_ms_events": round(kernel_ms, 5), "launches_timed": launches.value}
+    if cnt:
+        roof["traffic_GBps"] = round(cnt["traffic"] / (kernel_ms * 1e-3) / 1e9, 1) if kernel_ms > 0 else None
+        roof["traffic_frac"] = round(cnt["traffic"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if kernel_ms > 0 else None
+        roof["counters_from"] = {"files": cnt["files"], "library_commit": cnt["commit"]}
+        if "rocprof_ms" in cnt:
+            r_gbs = kernel_bytes / (cnt["rocprof_ms"] * 1e-3) / 1e9
+            roof["rocprof"] = {"avg_launch_ms": cnt["rocprof_ms"], "achieved": round(r_gbs, 1), "frac": round(r_gbs / HBM_PEAK_GBS, 4)}
+        if "lds" in cnt and kernel_ms > 0:
+            lds_gbs = cnt["lds"] / (kernel_ms * 1e-3) / 1e9
+            roof["lds"] = {"bytes_per_launch": cnt["lds"], "achieved_GBps": round(lds_gbs, 1), "peak_GBps": round(LDS_PEAK_GBS, 1),
+                           "frac": round(lds_gbs / LDS_PEAK_GBS, 4)}
+    out["roofline"] = roof
+    return out, cfg
+
+
+def copy_ceiling():
+    """What a plain copy kernel over 1 GiB reaches on this GPU (read + written bytes per second)."""
+    import torch
+
+    from customnetworklayers_amd._lib import lib
+
+    g = ctypes.c_double(0)
+    rc = lib.inpaint_copy_bandwidth(1 << 30, 10, ctypes.byref(g), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return round(g.value, 1) if rc == 0 else None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="config 1 only: skip the short legs of configs 2, 3, 4 and of keep mode 0 after the headline's timed region")
+    ap.add_argument("--config", type=int, default=1,
+                    help="workload index (1 = headline TV layer, 2 = TGV layer, 3 = three-level TV hierarchy, 4 = stress shape, "
+                         "5 = quadratic fit, 6 = median)")
+    ap.add_argument("--keep", type=int, default=None, choices=[0, 1, 2],
+                    help="configs 1, 2, 4: which half-step iterates the forward pass keeps (default 2 = all; 0 = the reference's footprint)")
+    ap.add_argument("--corrected-gradient", action="store_true",
+                    help="configs 1 and 2: time the opt-in corrected gradient instead of the reference's (not the headline)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
+              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from customnetworklayers_amd.workloads import CONFIGS, config_inputs
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    kind = CONFIGS[args.config]["kind"]
+    if kind == "tv_hierarchy":
+        print(json.dumps(bench_hierarchy(args, CONFIGS[args.config])))
+        return
+    if kind in ("quadfit", "median"):
+        cfg, d = config_inputs(args.config, seed=0)
+        return bench_flowaux(args, cfg, d)
+    out, cfg = bench_layer(args.config, args.steps, args.warmup, corrected=args.corrected_gradient, keep=args.keep)
+    out["roofline"]["hbm_copy_ceiling_GBps"] = copy_ceiling()
+    if args.config == 1 and not args.no_other_configs and not args.corrected_gradient and args.keep is None:
+        # after the headline's timed region: short legs of the other workloads, so that one run witnesses them all
+        other = {}
+        leg = lambda o: {k: o[k] for k in ("value", "unit", "ms_per_step", "ms_per_step_event_median", "steps", "warmup")}  # noqa: E731
+        o, _ = bench_layer(1, 5, 2, keep=0, detail=False)
+        other["config1_keep_mode_0"] = dict(leg(o), workload=o["config"]["workload"] + ", nothing kept: every segment recomputed (the reference's footprint)",
+                                            slot_bytes=o["config"]["slot_bytes"])
+        o, _ = bench_layer(2, 4, 2, detail=False)
+        other["config2_tgv"] = dict(leg(o), workload=o["config"]["workload"], slot_bytes=o["config"]["slot_bytes"])
+        hargs = argparse.Namespace(steps=5, warmup=2, no_cpu_baseline=True)
+        o = bench_hierarchy(hargs, CONFIGS[3])
+        other["config3_hierarchy"] = dict({k: o[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup")}, workload=o["config"]["workload"])
+        o, _ = bench_layer(4, 3, 1, detail=False)
+        other["config4_stress"] = dict(leg(o), workload=o["config"]["workload"], slot_bytes=o["config"]["slot_bytes"])
+        out["other_configs"] = other
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))

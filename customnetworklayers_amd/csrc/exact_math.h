@@ -45,9 +45,11 @@ __device__ __forceinline__ float exact_sqrt(float x) {
   const float s_up = __int_as_float(__float_as_int(s) + 1);
   const float r_dn = __builtin_fmaf(-s_dn, s, x);
   const float r_up = __builtin_fmaf(-s_up, s, x);
+  // x = 0 and x = +inf need no case of their own: their residuals are 0 or NaN, both tests fail and s itself
+  // (0 or +inf) is returned
   float out = (r_dn <= 0.0f) ? s_dn : s;
   out = (r_up > 0.0f) ? s_up : out;
-  return (x == 0.0f || x == __builtin_inff()) ? x : out;
+  return out;
 }
 
 }  // namespace inpaint

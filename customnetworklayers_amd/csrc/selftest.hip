@@ -17,7 +17,7 @@ __device__ inline unsigned int mix(unsigned int x) {  // integer hash, good enou
   return x;
 }
 
-// counts[0]: sqrt over every float in [2^-96, FLT_MAX] plus 0
+// counts[0]: sqrt over every float in [2^-96, FLT_MAX] plus 0 and +inf
 // counts[1]: x / 0.1f over 0 and every float in [2^-96, 2^96]
 // counts[2]: n / d on hashed pairs, d in [2^-6, 2^40), |n| in [2^-60, 2^60) or 0, plus structured
 //            denominators (all-ones and single-bit mantissas)
@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* count
   const unsigned int tid = blockIdx.x * blockDim.x + threadIdx.x;
   const unsigned int stride = gridDim.x * blockDim.x;
   unsigned int bad0 = 0, bad1 = 0, bad2 = 0, bad3 = 0;
-  for (unsigned long long i = tid; i < 0x7f800000ULL; i += stride) {
+  for (unsigned long long i = tid; i <= 0x7f800000ULL; i += stride) {
     const float x = __uint_as_float((unsigned int)i);
     if (x == 0.f || x >= 1.2621774e-29f) bad0 += !same_bits(exact_sqrt(x), sqrtf(x));
     if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) bad1 += !same_bits(exact_div(x, 0.1f), x / 0.1f);
@@ -84,6 +84,12 @@ __global__ __launch_bounds__(256) void selftest_rsqrt_kernel(unsigned long long*
   if (bad3) atomicAdd(&counts[3], (unsigned long long)bad3);
 }
 
+// plain streaming copy, 16 bytes per lane and trip
+__global__ __launch_bounds__(256) void copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, long long n16) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (long long)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 int run_selftest(void (*kernel)(unsigned long long*, unsigned int), unsigned long long* host4, unsigned int rounds) {
   unsigned long long* dev = nullptr;
   INPAINT_HIP(hipMalloc((void**)&dev, 4 * sizeof(unsigned long long)));
@@ -109,5 +115,39 @@ extern "C" int inpaint_selftest_math(unsigned long long* mismatches4_host, unsig
   INPAINT_HIP(hipGetLastError());
   INPAINT_HIP(hipMemcpy(mismatches4_host, dev, 4 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
   INPAINT_HIP(hipFree(dev));
+  return 0;
+}
+
+// Diagnostic: what a plain device-to-device copy kernel reaches on this GPU, as a practical ceiling to quote beside
+// the published HBM peak.  Copies `bytes` (rounded down to 16) from one fresh buffer to another `repeats` times after
+// one warm-up launch and returns (bytes read + bytes written) / time in GB/s, timed with HIP events on `stream`.
+extern "C" int inpaint_copy_bandwidth(long long bytes, int repeats, double* gbps_host, void* stream_) {
+  if (bytes < 16 || repeats < 1 || !gbps_host) return inpaint::fail(INPAINT_ERR_ARG, "bad arguments");
+  hipStream_t stream = (hipStream_t)stream_;
+  const long long n16 = bytes / 16;
+  float4 *src = nullptr, *dst = nullptr;
+  INPAINT_HIP(hipMalloc((void**)&src, (size_t)n16 * 16));
+  if (hipMalloc((void**)&dst, (size_t)n16 * 16) != hipSuccess) {
+    (void)hipFree(src);
+    return inpaint::fail(INPAINT_ERR_HIP, "hipMalloc of the copy target failed");
+  }
+  INPAINT_HIP(hipMemsetAsync(src, 0x3c, (size_t)n16 * 16, stream));
+  hipEvent_t e0, e1;
+  INPAINT_HIP(hipEventCreate(&e0));
+  INPAINT_HIP(hipEventCreate(&e1));
+  const int grid = (int)std::min<long long>((n16 + 255) / 256, 256LL * 32);
+  hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, stream, src, dst, n16);
+  INPAINT_HIP(hipEventRecord(e0, stream));
+  for (int r = 0; r < repeats; r++) hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, stream, src, dst, n16);
+  INPAINT_HIP(hipEventRecord(e1, stream));
+  INPAINT_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  INPAINT_HIP(hipEventElapsedTime(&ms, e0, e1));
+  INPAINT_HIP(hipGetLastError());
+  *gbps_host = ms > 0 ? 2.0 * (double)n16 * 16 * repeats / (ms * 1e-3) / 1e9 : 0.0;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  (void)hipFree(src);
+  (void)hipFree(dst);
   return 0;
 }

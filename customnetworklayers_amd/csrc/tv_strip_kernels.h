@@ -512,6 +512,29 @@ __device__ __forceinline__ float rebuild_y_fast(float bb, float xa, float xb, fl
   return quad ? y_q : y_l;
 }
 
+// The pieces of that rebuild for one half-step value v: q = the quadratic branch's iterate (TV.cu:1156-1157),
+// l = the other branch's (TV.cu:1162-1164), quad = the regime test on v (TV.cu:1154).  rebuild_y_fast(bb, xa, xb, ...)
+// is quad(xa) ? q(xa) + t (q(xa) - q(xb)) : l(xa) + t (l(xa) - l(xb)); a kernel that rebuilds two consecutive y
+// evaluates the pieces of the shared middle value once.
+struct RebuildPieces {
+  float q, l;
+  bool quad;
+};
+__device__ __forceinline__ RebuildPieces rebuild_pieces(float bb, float v, float conf, float rc, double opc_d) {
+  RebuildPieces r;
+  const float diff = bb - v;
+  const float sign = (diff < 0) ? -1.f : 1.f;
+  r.quad = (opc_d >= (double)(sign * diff));
+  r.q = div_by(conf * bb + v, 1.f + conf, rc);
+  r.l = (conf <= sign * diff) ? bb - diff + sign * conf : bb;
+  return r;
+}
+__device__ __forceinline__ float rebuild_from(const RebuildPieces& a, const RebuildPieces& b, float t) {
+  const float y_q = a.q + t * (a.q - b.q);
+  const float y_l = a.l + t * (a.l - b.l);
+  return a.quad ? y_q : y_l;
+}
+
 // y_{k+1} exactly as the forward pass made it: x_{k+1} = prox(x05[k]) (TV.cu:1286-1292), y_{k+1} = x_{k+1} +
 // t (x_{k+1} - x_k) (TV.cu:1315); x_k is prox(x05[k-1]) or, at a segment start, the checkpointed iterate itself.
 __device__ __forceinline__ float prox_huber1(float yt, float c, float rc1, float bv) {
@@ -871,8 +894,10 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
         o.yA[ch] = pa + tA * (pa - pb);
         o.yB[ch] = pb + tB * (pb - pc);
       } else {
-        o.yA[ch] = rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, tA);
-        o.yB[ch] = BEND ? xc : rebuild_y_fast(bv, xb, xc, o.c, o.rc1, o.opc_d, tB);
+        // rebuild_y_fast(bv, xa, xb, ..., tA) and rebuild_y_fast(bv, xb, xc, ..., tB) with the pieces of xb formed once
+        const RebuildPieces ra = rebuild_pieces(bv, xa, o.c, o.rc1, o.opc_d), rb = rebuild_pieces(bv, xb, o.c, o.rc1, o.opc_d);
+        o.yA[ch] = rebuild_from(ra, rb, tA);
+        o.yB[ch] = BEND ? xc : rebuild_from(rb, rebuild_pieces(bv, xc, o.c, o.rc1, o.opc_d), tB);
       }
       o.g[ch] = ok ? o.g[ch] : 0.f;
       o.xa[ch] = xa;
@@ -904,11 +929,13 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     const float P1 = gpd * wyv * d1;
     const float P2 = gpr * wxv * d2;
     const float dd = denom * 2.0f;
-    const float tp = dd * ((yd - yk) * wyv + (yrt - yk) * wxv);
+    // the reference's factor dd * ((yd - yk) * wyv + (yrt - yk) * wxv) is minus this one, exactly: a - b = -(b - a),
+    // (-a) * w = -(a * w) and (-a) + (-b) = -(a + b) in IEEE arithmetic; O3, O4 carry the sign
+    const float tp = dd * (d1 * wyv + d2 * wxv);
     const float tu = dd * d1 * wyv;
     const float tl = dd * d2 * wxv;
-    r.O3 = P1 * tp;
-    r.O4 = P2 * tp;
+    r.O3 = -(P1 * tp);
+    r.O4 = -(P2 * tp);
     r.n3 = P1 * tu;
     r.n4 = P2 * tu;
     r.l1 = from_left_lane(r.O2);

@@ -108,6 +108,11 @@ int tvinpaint_profile_read(double* total_ms, int* launches);
  * pairs per thread otherwise) and returns the four mismatch counts (host array).  All must be 0. */
 int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds);
 
+/* Diagnostic: the rate a plain device-to-device copy kernel reaches on the current GPU (bytes read + bytes written per
+ * second, in GB/s, host pointer), to quote beside the published HBM peak.  Allocates and frees two buffers of `bytes`,
+ * copies `repeats` times after a warm-up launch, timed with HIP events on `stream`; waits for the result. */
+int inpaint_copy_bandwidth(long long bytes, int repeats, double* gbps_host, void* stream);
+
 /* Text of the last error on the calling thread ("" if none). */
 const char* tvinpaint_last_error(void);
 
