@@ -1,0 +1,85 @@
+// Compiled PyTorch binding of the TGV inpainting layer over the C ABI in include/tgvinpaint.h: the functions of the
+// reference's pybind module tgvInpaint_cuda_ext (cudaTGV/TGVInpaintFista_cuda.cpp:47-180 of the reference) with its
+// two static calls (lines 94-97 and 160-165 there) replaced by tgvinpaint_forward / tgvinpaint_backward.  Host C++
+// only; links libinpaint_hip.so.  Differences from the reference binding: batches n >= 1 are accepted (77-81 refuses
+// them), failures throw, the solution and the gradient wrt the starting point have the 3 * channel channels the callee
+// writes (the reference allocates `channel`, lines 91 and 157), and the work is enqueued on PyTorch's current stream.
+#include <torch/extension.h>
+
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <vector>
+
+#include "tgvinpaint.h"
+
+namespace {
+
+void check_input(const at::Tensor& x, const char* name) {  // CHECK_INPUT, TGVInpaintFista_cuda.cpp:24-26, and the type test of 87
+  TORCH_CHECK(x.is_cuda(), name, " must be a CUDA tensor");
+  TORCH_CHECK(x.is_contiguous(), name, " must be contiguous");
+  TORCH_CHECK(x.scalar_type() == at::kFloat, "Input/Output type to the operator must be single/float (", name, ")");
+}
+
+// channel counts of TGVInpaintFista_cuda.cpp:65-83: two weight channels, three variables per channel of b
+void check_shapes(const at::Tensor& d_x, const at::Tensor& d_y, const at::Tensor& d_c, const at::Tensor& d_b,
+                  const at::Tensor& state, const char* state_name) {
+  TORCH_CHECK(d_b.dim() == 4, "d_b must be (n, c, h, w)");
+  const auto n = d_b.size(0), c = d_b.size(1), h = d_b.size(2), w = d_b.size(3);
+  for (const at::Tensor* t : {&d_x, &d_y})
+    TORCH_CHECK(t->dim() == 4 && t->size(0) == n && t->size(1) == 2 && t->size(2) == h && t->size(3) == w,
+                "d_x and d_y must have shape (n, 2, h, w): edge weight and beta");
+  TORCH_CHECK(d_c.dim() == 4 && d_c.size(0) == n && d_c.size(1) == 1 && d_c.size(2) == h && d_c.size(3) == w,
+              "d_c must have shape (n, 1, h, w)");
+  TORCH_CHECK(state.dim() == 4 && state.size(0) == n && state.size(1) == 3 * c && state.size(2) == h && state.size(3) == w,
+              state_name, " must have shape (n, 3 * channels of d_b, h, w): u, v1, v2");
+  for (const at::Tensor* t : {&d_x, &d_y, &d_c, &state})
+    TORCH_CHECK(t->device() == d_b.device(), "all tensors must live on one device");
+}
+
+void* current_stream(const at::Tensor& t) { return c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
+
+}  // namespace
+
+std::vector<at::Tensor> tgvInpaint_dummy() {
+  std::cout << "Input: not present just dummy:\n";
+  return {};
+}
+
+void tgvInpaint_dummy_only() { std::cout << "Dummy call:\n"; }
+
+std::vector<at::Tensor> tgvInpaint_forward(at::Tensor d_x, at::Tensor d_y, at::Tensor d_c, at::Tensor d_b, at::Tensor d_i,
+                                           int its, int id) {
+  check_input(d_x, "d_x"); check_input(d_y, "d_y"); check_input(d_c, "d_c"); check_input(d_b, "d_b"); check_input(d_i, "d_i");
+  check_shapes(d_x, d_y, d_c, d_b, d_i, "d_i");
+  const c10::hip::HIPGuard guard(d_b.device());
+  at::Tensor solution = at::empty_like(d_i);
+  const int rc = tgvinpaint_forward(d_x.data_ptr<float>(), d_y.data_ptr<float>(), d_c.data_ptr<float>(), d_b.data_ptr<float>(),
+                                    d_i.data_ptr<float>(), solution.data_ptr<float>(), (int)d_b.size(0), (int)d_b.size(1),
+                                    (int)d_b.size(2), (int)d_b.size(3), its, id, current_stream(d_b));
+  TORCH_CHECK(rc == 0, "TGVInpaint::forward failed: ", tgvinpaint_last_error());
+  return {solution};
+}
+
+std::vector<at::Tensor> tgvInpaint_backward(at::Tensor d_iGf, at::Tensor d_x, at::Tensor d_y, at::Tensor d_c, at::Tensor d_b,
+                                            int its, int id) {
+  check_input(d_x, "d_x"); check_input(d_y, "d_y"); check_input(d_c, "d_c"); check_input(d_b, "d_b"); check_input(d_iGf, "d_iGf");
+  check_shapes(d_x, d_y, d_c, d_b, d_iGf, "d_iGf");
+  const c10::hip::HIPGuard guard(d_b.device());
+  at::Tensor d_oGx = at::empty_like(d_x), d_oGy = at::empty_like(d_y), d_oGc = at::empty_like(d_c);
+  at::Tensor d_oGb = at::empty_like(d_b), d_oGi = at::empty_like(d_iGf);
+  const int rc = tgvinpaint_backward(d_x.data_ptr<float>(), d_y.data_ptr<float>(), d_c.data_ptr<float>(), d_b.data_ptr<float>(),
+                                     d_iGf.data_ptr<float>(), d_oGx.data_ptr<float>(), d_oGy.data_ptr<float>(),
+                                     d_oGc.data_ptr<float>(), d_oGb.data_ptr<float>(), d_oGi.data_ptr<float>(), (int)d_b.size(0),
+                                     (int)d_b.size(1), (int)d_b.size(2), (int)d_b.size(3), its, id, current_stream(d_b));
+  TORCH_CHECK(rc == 0, "TGVInpaint::backward failed: ", tgvinpaint_last_error());
+  return {d_oGx, d_oGy, d_oGc, d_oGb, d_oGi};
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("forward", &tgvInpaint_forward, "tgvInpaint forward (HIP)");
+  m.def("backward", &tgvInpaint_backward, "tgvInpaint backward (HIP)");
+  m.def("dummy", &tgvInpaint_dummy, "tgvInpaint dummy");
+  m.def("dummy_only", &tgvInpaint_dummy_only, "tgvInpaint dummy2");
+  m.def("reset_id", [](int id) { TORCH_CHECK(tgvinpaint_reset_id(id) == 0, tgvinpaint_last_error()); }, "free the id's state");
+}

@@ -1087,7 +1087,7 @@ int quadfit_forward(const float* im0, const float* im1, const float* flow, float
   const int tiles_x = (iw + kTW - 1) / kTW, tiles_y = (ih + TileCfg<kPxForward>::TH - 1) / TileCfg<kPxForward>::TH;
   const long long tiles = (long long)n * tiles_x * tiles_y;
   if (tiles >= (1ll << 31) - 8) return fail(INPAINT_ERR_ARG, "quadfit_forward: too many tiles");
-  if (getenv("INPAINT_QUADFIT_PATH") && strcmp(getenv("INPAINT_QUADFIT_PATH"), "px") == 0)
+  if (inpaint::knobs().quadfit_px_path)
     hipLaunchKernelGGL(quadfit_forward_kernel, banded_grid(P), dim3(256), 0, (hipStream_t)stream, im0, im1, flow, out, n,
                        ic, ih, iw, flow_channels);
   else
@@ -1127,7 +1127,7 @@ int quadfit_backward(const float* im0, const float* im1, const float* flow, cons
                      reinterpret_cast<float*>(ws.count), P + 64);
   const int tiles_x = (iw + kTW - 1) / kTW, tiles_y = (ih + TileCfg<kPxSources>::TH - 1) / TileCfg<kPxSources>::TH;
   const long long tiles = (long long)n * tiles_x * tiles_y;
-  const bool px_path = getenv("INPAINT_QUADFIT_PATH") && strcmp(getenv("INPAINT_QUADFIT_PATH"), "px") == 0;
+  const bool px_path = inpaint::knobs().quadfit_px_path;
   if (px_path)
     hipLaunchKernelGGL(quadfit_backward_sources, grid, block, 0, st, im0, im1, flow, gin, g0, ws, n, ic, ih, iw, flow_channels);
   else {

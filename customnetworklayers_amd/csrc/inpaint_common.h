@@ -10,6 +10,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -41,6 +42,77 @@ inline int fail(int code, const char* fmt, ...) {
       return inpaint::fail(INPAINT_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
                            __FILE__, __LINE__);                                                \
   } while (0)
+
+// ---------------------------------------------------------------------------------------------
+// testing / tuning switches (INPAINT_* environment variables)
+//
+// Read once per process, on first use, and again only when somebody asks: *_reset_id() and inpaint_reload_env() do.
+// A variable changed in the middle of a run therefore switches no kernel until one of those calls.
+// ---------------------------------------------------------------------------------------------
+struct Knobs {
+  bool tv_tile_path = false;      // INPAINT_TV_PATH=tile: the LDS-tile kernels instead of the wave strips
+  bool tv_fuse = true;            // INPAINT_TV_FUSE=0: one forward iteration per launch
+  bool tv_fuse_adj = true;        // INPAINT_TV_FUSE_ADJ=0: one adjoint step per launch
+  int tv_fwd_rows = 0;            // INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strip height (0 = chosen per launch)
+  int tv_adj_rows = 0;
+  bool tgv_px_path = false;       // INPAINT_TGV_PATH=px: the per-pixel kernels
+  bool tgv_fuse = true;           // INPAINT_TGV_FUSE=0
+  bool tgv_fuse_adj = true;       // INPAINT_TGV_FUSE_ADJ=0
+  int tgv_fwd_rows = 0;           // INPAINT_TGV_FWD_ROWS / INPAINT_TGV_ADJ_ROWS
+  int tgv_adj_rows = 0;
+  int tgv_pair_waves = 0;         // INPAINT_TGV_PAIR_WAVES=1|2 (0 = by channel count)
+  int keep = -1;                  // INPAINT_KEEP=0|1|2 (INPAINT_KEEP_LAST=0 is INPAINT_KEEP=0); -1 = the id's own mode
+  double keep_gb = 32.0;          // INPAINT_KEEP_GB: budget of keep mode 2
+  bool quadfit_px_path = false;   // INPAINT_QUADFIT_PATH=px: one pixel per lane, no LDS windows
+  void load() {
+    *this = Knobs();
+    auto is = [](const char* name, const char* value) {
+      const char* e = getenv(name);
+      return e && strcmp(e, value) == 0;
+    };
+    auto rows = [](const char* name) {
+      const char* e = getenv(name);
+      const int v = e ? atoi(e) : 0;
+      return (v >= 1 && v <= 4096) ? v : 0;
+    };
+    tv_tile_path = is("INPAINT_TV_PATH", "tile");
+    tv_fuse = !is("INPAINT_TV_FUSE", "0");
+    tv_fuse_adj = !is("INPAINT_TV_FUSE_ADJ", "0");
+    tv_fwd_rows = rows("INPAINT_TV_FWD_ROWS");
+    tv_adj_rows = rows("INPAINT_TV_ADJ_ROWS");
+    tgv_px_path = is("INPAINT_TGV_PATH", "px");
+    tgv_fuse = !is("INPAINT_TGV_FUSE", "0");
+    tgv_fuse_adj = !is("INPAINT_TGV_FUSE_ADJ", "0");
+    tgv_fwd_rows = rows("INPAINT_TGV_FWD_ROWS");
+    tgv_adj_rows = rows("INPAINT_TGV_ADJ_ROWS");
+    tgv_pair_waves = is("INPAINT_TGV_PAIR_WAVES", "1") ? 1 : (is("INPAINT_TGV_PAIR_WAVES", "2") ? 2 : (getenv("INPAINT_TGV_PAIR_WAVES") ? 1 : 0));
+    if (is("INPAINT_KEEP_LAST", "0")) keep = 0;
+    if (const char* e = getenv("INPAINT_KEEP")) {
+      const int v = atoi(e);
+      if (v >= 0 && v <= 2) keep = v;
+    }
+    if (const char* e = getenv("INPAINT_KEEP_GB")) keep_gb = atof(e);
+    quadfit_px_path = is("INPAINT_QUADFIT_PATH", "px");
+  }
+};
+struct KnobsHolder {
+  Knobs k;
+  bool loaded = false;
+};
+inline KnobsHolder& knobs_holder() {
+  static KnobsHolder h;
+  return h;
+}
+inline const Knobs& knobs() {
+  KnobsHolder& h = knobs_holder();
+  if (!h.loaded) { h.k.load(); h.loaded = true; }
+  return h.k;
+}
+inline void reload_knobs() {
+  KnobsHolder& h = knobs_holder();
+  h.k.load();
+  h.loaded = true;
+}
 
 // ---------------------------------------------------------------------------------------------
 // schedule (reference: TVInpaintFista.cu:1499-1508,1523 and 1525-1532; the TGV driver repeats both)

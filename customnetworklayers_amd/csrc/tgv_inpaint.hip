@@ -720,6 +720,9 @@ struct Slot {
   int keep_mode = 2;
   int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tgvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
+  // shape and its whose every-row ring (keep mode 2) the device refused: later forwards of that shape go straight
+  // to keep mode 1 instead of freeing the arena and asking again on every call; cleared by reset_id
+  long long refused[5] = {0, 0, 0, 0, 0};
   int x05_mode = 0;     // how the last forward laid its rows out: 2 row = iteration, else row = iteration - first kept
   int x05_from = 0;     // first iteration whose x05 row the last forward kept
   bool x05_valid = false;
@@ -829,18 +832,10 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
 // The x05 rows the forward pass keeps.  INPAINT_KEEP=0|1|2 overrides the id's setting (INPAINT_KEEP_LAST=0 is the
 // older spelling of INPAINT_KEEP=0); keeping all rows needs its * state bytes, at most INPAINT_KEEP_GB (default 32).
 int resolve_keep_mode(const Slot& s, int n, int ic, int ih, int iw, int its) {
-  int mode = s.keep_mode;
-  if (const char* e = getenv("INPAINT_KEEP_LAST"))
-    if (strcmp(e, "0") == 0) mode = 0;
-  if (const char* e = getenv("INPAINT_KEEP")) {
-    const int v = atoi(e);
-    if (v >= 0 && v <= 2) mode = v;
-  }
+  int mode = knobs().keep >= 0 ? knobs().keep : s.keep_mode;
   if (mode == 2) {
-    double gb = 32.0;
-    if (const char* e = getenv("INPAINT_KEEP_GB")) gb = atof(e);
     const double bytes = 4.0 * 3 * n * ic * (double)ih * iw * its;
-    if (bytes > gb * 1073741824.0) mode = 1;
+    if (bytes > knobs().keep_gb * 1073741824.0) mode = 1;
   }
   return mode;
 }
@@ -855,6 +850,8 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
     return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
   if (n > 65535 || (ih + BY - 1) / BY > 65535)
     return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
+  if ((long long)ih * iw >= (1ll << 30))  // the strip kernels address a plane with 32-bit byte offsets
+    return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^30", (long long)ih * iw);
   if ((int)std::floor(std::sqrt((double)its)) > kMaxCheckpoints)
     return fail(INPAINT_ERR_ITS, "its=%d needs more than %d checkpoints", its, kMaxCheckpoints);
   return 0;
@@ -876,17 +873,13 @@ void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const flo
 // INPAINT_TGV_PATH=px forces the per-pixel kernels (used by the tests to keep both paths covered).
 // -------------------------------------------------------------------------------------------------
 bool use_strip(const Slot& s) {
-  const char* e = getenv("INPAINT_TGV_PATH");
-  if (e && strcmp(e, "px") == 0) return false;
+  if (knobs().tgv_px_path) return false;
   return s.ic >= 1 && s.ic <= 2;
 }
-int strip_rows(int n, int ih, int iw, int cols, const char* env_name, int lag) {
+int strip_rows(int n, int ih, int iw, int cols, int forced_rows, int lag) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap between
   // strips, but the launch should still keep every SIMD of the chip busy.
-  if (const char* e = getenv(env_name)) {
-    const int v = atoi(e);
-    if (v >= 1 && v <= 4096) return v;
-  }
+  if (forced_rows > 0) return forced_rows;
   const long long sx = (iw + cols - 1) / cols;
   return choose_strip_rows(sx * n, ih, 4, lag);
 }
@@ -895,10 +888,7 @@ int strip_rows(int n, int ih, int iw, int cols, const char* env_name, int lag) {
 // launch runs in ceil(workgroups / (4 * CUs)) rounds of (R + 3 pipeline rows + start-up) row steps each; the
 // strip height that minimises rounds x steps is taken (on 4 x 384 x 1248: 32 rows, 1008 workgroups, one round).
 int pair_split_rows(int n, int ih, int iw) {
-  if (const char* e = getenv("INPAINT_TGV_ADJ_ROWS")) {
-    const int v = atoi(e);
-    if (v >= 1 && v <= 4096) return v;
-  }
+  if (knobs().tgv_adj_rows > 0) return knobs().tgv_adj_rows;
   static int cus = 0;
   if (cus == 0) {
     int dev = 0;
@@ -926,7 +916,7 @@ template <int C>
 void launch_forward_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                           float* xout, const float* yin, float* yout, float* x05, float t) {
   auto kern = x05 ? tgvstrip::tgv_forward_strip<C, true> : tgvstrip::tgv_forward_strip<C, false>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, "INPAINT_TGV_FWD_ROWS", 6);
+  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, knobs().tgv_fwd_rows, 6);
   const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
@@ -955,7 +945,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c
   auto kern = tgvstrip::tgv_forward_strip2<C, false>;
   if (x05a && ring) kern = tgvstrip::tgv_forward_strip2<C, true, true>;
   else if (x05a) kern = tgvstrip::tgv_forward_strip2<C, true>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, "INPAINT_TGV_FWD_ROWS", 8);
+  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, knobs().tgv_fwd_rows, 8);
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
@@ -964,8 +954,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c
 }
 
 bool forward_pairs(const Slot& s) {
-  const char* e = getenv("INPAINT_TGV_FUSE");
-  if (e && strcmp(e, "0") == 0) return false;
+  if (!knobs().tgv_fuse) return false;
   return use_strip(s);
 }
 
@@ -987,7 +976,7 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, con
                           float* gxk_m1, float* gx_final, float t) {
   const int i = s.acc_cur, o = 1 - s.acc_cur;
   auto kern = gx_final ? tgvstrip::tgv_adjoint_strip<C, END, true, ADJ> : tgvstrip::tgv_adjoint_strip<C, END, false, ADJ>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, "INPAINT_TGV_ADJ_ROWS", 6);
+  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, knobs().tgv_adj_rows, 6);
   const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
@@ -1027,10 +1016,7 @@ void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b,
 // Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
 // (xc = slot j-2, or the checkpoint y when B is the segment's first iteration).
 // Whether the pair kernel runs its two steps in two wavefronts (the default with two channels).
-bool pair_split(int channels) {
-  const char* e = getenv("INPAINT_TGV_PAIR_WAVES");
-  return e ? strcmp(e, "2") == 0 : channels >= 2;
-}
+bool pair_split(int channels) { return knobs().tgv_pair_waves ? knobs().tgv_pair_waves == 2 : channels >= 2; }
 
 // TRUE_ADJ (the corrected gradient) exists for the two-wavefront kernel only; the caller checks pair_split().
 template <int C, bool BEND, bool TRUE_ADJ>
@@ -1043,7 +1029,7 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const bool split = pair_split(C);
   auto kern1 = gx_final ? tgvstrip::tgv_adjoint_strip2<C, BEND, true> : tgvstrip::tgv_adjoint_strip2<C, BEND, false>;
   const int R = split ? pair_split_rows(s.n, s.ih, s.iw)
-                      : strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, "INPAINT_TGV_ADJ_ROWS", 8);
+                      : strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, knobs().tgv_adj_rows, 8);
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
@@ -1072,8 +1058,7 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* c, const floa
 }
 
 bool adjoint_pairs(const Slot& s) {
-  const char* e = getenv("INPAINT_TGV_FUSE_ADJ");
-  if (e && strcmp(e, "0") == 0) return false;
+  if (!knobs().tgv_fuse_adj) return false;
   return forward_pairs(s);
 }
 
@@ -1091,11 +1076,14 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   s.forward_done = false;
   s.x05_valid = false;
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
+  const long long shape[5] = {n, ic, ih, iw, its};
+  if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
   rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
   if (rc && keep == 2) {  // no room for every x05 row: keep the last segment's instead and recompute the others
     (void)hipGetLastError();
     keep = 1;
     rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
+    if (!rc) std::copy(shape, shape + 5, s.refused);
   }
   if (rc) return rc;
   const size_t S3 = state_count(s), SB = S3 * sizeof(float);
@@ -1470,6 +1458,7 @@ int tgvinpaint_set_state(int id, const double* state6) {
 
 int tgvinpaint_reset_id(int id) {
   if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  reload_knobs();
   Slot& s = g_slots[id];
   if (s.arena.base) (void)hipStreamSynchronize(s.stream);
   int rc = s.arena.release();

@@ -491,6 +491,9 @@ struct Slot {
   int keep_mode = 2;
   int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
+  // shape and its whose every-row ring (keep mode 2) the device refused: later forwards of that shape go straight
+  // to keep mode 1 instead of freeing the arena and asking again on every call; cleared by reset_id
+  long long refused[5] = {0, 0, 0, 0, 0};
   int x05_mode = 0;     // how the last forward laid its rows out: 2 row = iteration, else row = iteration - first kept
   int x05_from = 0;     // first iteration whose x05 row the last forward kept
   bool x05_valid = false;
@@ -595,6 +598,8 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
     return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
   if (n > 65535 || (ih + TH - 1) / TH > 65535)
     return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
+  if ((long long)ih * iw >= (1ll << 30))  // the strip kernels address a plane with 32-bit byte offsets
+    return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^30", (long long)ih * iw);
   if ((int)std::floor(std::sqrt((double)its)) > kMaxCheckpoints)
     return fail(INPAINT_ERR_ITS, "its=%d needs more than %d checkpoints", its, kMaxCheckpoints);
   return 0;
@@ -604,36 +609,22 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
 // kernel selection: wave-strip kernels for 1..4 channels, the LDS-tile kernels otherwise.
 // INPAINT_TV_PATH=tile forces the tile kernels (used by the tests to keep both paths covered).
 // -------------------------------------------------------------------------------------------------
-bool force_tile_path() {
-  const char* e = getenv("INPAINT_TV_PATH");
-  return e && strcmp(e, "tile") == 0;
-}
+bool force_tile_path() { return knobs().tv_tile_path; }
 // The x05 rows the forward pass keeps.  INPAINT_KEEP=0|1|2 overrides the id's setting (INPAINT_KEEP_LAST=0 is the
 // older spelling of INPAINT_KEEP=0); keeping all rows needs its * field bytes, at most INPAINT_KEEP_GB (default 32).
 int resolve_keep_mode(const Slot& s, int n, int ic, int ih, int iw, int its) {
-  int mode = s.keep_mode;
-  if (const char* e = getenv("INPAINT_KEEP_LAST"))
-    if (strcmp(e, "0") == 0) mode = 0;
-  if (const char* e = getenv("INPAINT_KEEP")) {
-    const int v = atoi(e);
-    if (v >= 0 && v <= 2) mode = v;
-  }
+  int mode = knobs().keep >= 0 ? knobs().keep : s.keep_mode;
   if (mode == 2) {
-    double gb = 32.0;
-    if (const char* e = getenv("INPAINT_KEEP_GB")) gb = atof(e);
     const double bytes = 4.0 * n * ic * (double)ih * iw * its;
-    if (bytes > gb * 1073741824.0) mode = 1;
+    if (bytes > knobs().keep_gb * 1073741824.0) mode = 1;
   }
   return mode;
 }
-int strip_rows(int n, int ih, int iw, int cols, const char* env_name, int lag) {
+int strip_rows(int n, int ih, int iw, int cols, int forced_rows, int lag) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap
   // between strips, but the launch should still put about two wavefronts on each of the 1024 SIMDs
   // (measured on the 4 x 2 x 384 x 1248 workload: 16 rows beat 8 and 24).
-  if (const char* e = getenv(env_name)) {
-    const int v = atoi(e);
-    if (v >= 1 && v <= 4096) return v;
-  }
+  if (forced_rows > 0) return forced_rows;
   const long long sx = (iw + cols - 1) / cols;
   return choose_strip_rows(sx * n, ih, 4, lag);
 }
@@ -643,7 +634,7 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, co
                           const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
                           float t) {
   auto kern = x05 ? tvstrip::tv_forward_strip<C, true> : tvstrip::tv_forward_strip<C, false>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwdCols, "INPAINT_TV_FWD_ROWS", 6);
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwdCols, knobs().tv_fwd_rows, 6);
   const int sx = (s.iw + tvstrip::kFwdCols - 1) / tvstrip::kFwdCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
@@ -659,7 +650,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* d
   auto kern = tvstrip::tv_forward_strip2<C, false>;
   if (x05a && ring) kern = tvstrip::tv_forward_strip2<C, true, true>;
   else if (x05a) kern = tvstrip::tv_forward_strip2<C, true>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_FWD_ROWS", 8);
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_fwd_rows, 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
@@ -668,8 +659,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* d
 }
 
 bool forward_pairs(const Slot& s) {
-  const char* e = getenv("INPAINT_TV_FUSE");
-  if (e && strcmp(e, "0") == 0) return false;
+  if (!knobs().tv_fuse) return false;
   return !force_tile_path() && s.ic >= 1 && s.ic <= 4;
 }
 
@@ -711,7 +701,7 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, co
   const int i = s.acc_cur, o = 1 - s.acc_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, "INPAINT_TV_ADJ_ROWS", 6);
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, knobs().tv_adj_rows, 6);
   const int sx = (s.iw + tvstrip::kAdjCols - 1) / tvstrip::kAdjCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
@@ -754,7 +744,7 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
   const int i = s.acc_cur, o = 1 - s.acc_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip2<C, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2<C, BEND, false, TRUE_ADJ>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, "INPAINT_TV_ADJ_ROWS", 8);
+  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_adj_rows, 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
@@ -775,8 +765,7 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const flo
 }
 
 bool adjoint_pairs(const Slot& s) {
-  const char* e = getenv("INPAINT_TV_FUSE_ADJ");
-  if (e && strcmp(e, "0") == 0) return false;
+  if (!knobs().tv_fuse_adj) return false;
   // with 3 or 4 channels the pair kernel needs more than 256 registers (one wavefront per SIMD);
   // those take the one-step kernels
   return forward_pairs(s) && s.ic <= 2;
@@ -822,11 +811,14 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   s.forward_done = false;
   s.x05_valid = false;
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
+  const long long shape[5] = {n, ic, ih, iw, its};
+  if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
   rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
   if (rc && keep == 2) {  // no room for every x05 row: keep the last segment's instead and recompute the others
     (void)hipGetLastError();
     keep = 1;
     rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
+    if (!rc) std::copy(shape, shape + 5, s.refused);
   }
   if (rc) return rc;
   const size_t F = field_count(s), FB = F * sizeof(float);
@@ -1213,6 +1205,7 @@ int tvinpaint_set_state(int id, const double* state6) {
 
 int tvinpaint_reset_id(int id) {
   if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
+  reload_knobs();
   Slot& s = g_slots[id];
   if (s.arena.base) (void)hipStreamSynchronize(s.stream);
   int rc = s.arena.release();
@@ -1272,6 +1265,10 @@ int tvinpaint_guard_decide(int run, double av_gc, double av_running, double* mul
   if (av_out) *av_out = av;
   return action;
 }
+
+void inpaint_reload_env(void) { reload_knobs(); }
+
+int inpaint_keep_override(void) { return knobs().keep; }
 
 int tvinpaint_profile(int enable) {
   g_timer.enabled = enable != 0;

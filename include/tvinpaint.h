@@ -108,6 +108,13 @@ int tvinpaint_profile_read(double* total_ms, int* launches);
  * pairs per thread otherwise) and returns the four mismatch counts (host array).  All must be 0. */
 int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds);
 
+/* The INPAINT_* environment variables (testing and tuning switches: kernel selection, strip heights, keep-mode
+ * override and budget) are read once per process, on the first call that needs one, and again by every *_reset_id()
+ * and by this call; changing one in a running process has no effect until then. */
+void inpaint_reload_env(void);
+/* The keep mode INPAINT_KEEP / INPAINT_KEEP_LAST currently force on every id (-1: none), as last read. */
+int inpaint_keep_override(void);
+
 /* Diagnostic: the rate a plain device-to-device copy kernel reaches on the current GPU (bytes read + bytes written per
  * second, in GB/s, host pointer), to quote beside the published HBM peak.  Allocates and frees two buffers of `bytes`,
  * copies `repeats` times after a warm-up launch, timed with HIP events on `stream`; waits for the result. */

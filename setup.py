@@ -2,7 +2,8 @@
 
 `python setup.py build_ext --inplace` (or `install`) compiles the HIP library for gfx950 with hipcc
 into customnetworklayers_amd/libinpaint_hip.so; the Python modules bind it through its C ABI
-(include/*.h).  The reference builds one torch CUDAExtension per layer
+(include/*.h), with ctypes and, for the two inpainting layers, also as compiled PyTorch extensions
+(customnetworklayers_amd/cudaTV/tvInpaint_hip_ext.so, cudaTGV/tgvInpaint_hip_ext.so).  The reference builds one torch CUDAExtension per layer
 (cudaTV/setup.py:16-28, cudaTGV/setup.py:16-29, cudaQuadFit/setup.py:16-28, cudaMedian/setup.py:16-27 of the
 reference); the module names it produces -- tvInpaint_cuda_ext, tgvInpaint_cuda_ext, QuadFit_cuda_ext,
 median_cuda_ext -- are kept as importable top-level modules.
@@ -28,7 +29,9 @@ class BuildHip(Command):
         pass
 
     def run(self):
-        subprocess.check_call(["make", "-C", CSRC, "-j8"])
+        subprocess.check_call(["make", "-C", CSRC, "-j8", "all"])
+        # the compiled PyTorch bindings over the C ABI (host C++; the ctypes bindings need none of this)
+        subprocess.check_call(["make", "-C", CSRC, "-j8", "bindings"])
 
 
 class BuildPyWithHip(build_py):
@@ -43,7 +46,9 @@ setup(
     description="TV / TGV FISTA inpainting layers, quadratic fit and histogram median for MI355X (gfx950)",
     packages=["customnetworklayers_amd", "customnetworklayers_amd.cudaTV", "customnetworklayers_amd.cudaTGV",
               "customnetworklayers_amd.cudaQuadFit", "customnetworklayers_amd.cudaMedian"],
-    package_data={"customnetworklayers_amd": ["libinpaint_hip.so"]},
-    py_modules=["tvInpaint_cuda_ext", "tgvInpaint_cuda_ext", "QuadFit_cuda_ext", "median_cuda_ext"],
+    package_data={"customnetworklayers_amd": ["libinpaint_hip.so"], "customnetworklayers_amd.cudaTV": ["tvInpaint_hip_ext.so"],
+                  "customnetworklayers_amd.cudaTGV": ["tgvInpaint_hip_ext.so"]},
+    py_modules=["tvInpaint_cuda_ext", "tgvInpaint_cuda_ext", "QuadFit_cuda_ext", "median_cuda_ext", "TVInpainting",
+                "TGVInpainting", "QuadFitting", "median"],
     cmdclass={"build_ext": BuildHip, "build_py": BuildPyWithHip},
 )

@@ -87,6 +87,8 @@ def test_quadfit_warped_features_match_oracle(qf, flowaux_oracle, n, c, h, w):
 def test_quadfit_one_pixel_per_lane_kernels(qf, flowaux_oracle, n, c, h, w, monkeypatch):
     # INPAINT_QUADFIT_PATH=px: the kernels without LDS windows (a lane reads its taps from memory)
     monkeypatch.setenv("INPAINT_QUADFIT_PATH", "px")
+    from customnetworklayers_amd._lib import reload_env
+    reload_env()  # the switches are read once per process
     check_quadfit(qf, flowaux_oracle, random_quadfit(n, c, h, w, seed=31 + c), "px path random %dx%dx%dx%d" % (n, c, h, w))
     check_quadfit(qf, flowaux_oracle, workloads.quadfit_inputs(n, c, h, w, seed=32), "px path warped")
 
