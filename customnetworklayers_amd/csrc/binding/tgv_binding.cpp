@@ -6,8 +6,9 @@
 // writes (the reference allocates `channel`, lines 91 and 157), and the work is enqueued on PyTorch's current stream.
 #include <torch/extension.h>
 
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+// PyTorch on ROCm presents its HIP devices under the device type "cuda"; these are the guard and stream of that view
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <vector>
 
@@ -37,7 +38,7 @@ void check_shapes(const at::Tensor& d_x, const at::Tensor& d_y, const at::Tensor
     TORCH_CHECK(t->device() == d_b.device(), "all tensors must live on one device");
 }
 
-void* current_stream(const at::Tensor& t) { return c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
+void* current_stream(const at::Tensor& t) { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream(); }
 
 }  // namespace
 
@@ -52,7 +53,7 @@ std::vector<at::Tensor> tgvInpaint_forward(at::Tensor d_x, at::Tensor d_y, at::T
                                            int its, int id) {
   check_input(d_x, "d_x"); check_input(d_y, "d_y"); check_input(d_c, "d_c"); check_input(d_b, "d_b"); check_input(d_i, "d_i");
   check_shapes(d_x, d_y, d_c, d_b, d_i, "d_i");
-  const c10::hip::HIPGuard guard(d_b.device());
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(d_b.device());
   at::Tensor solution = at::empty_like(d_i);
   const int rc = tgvinpaint_forward(d_x.data_ptr<float>(), d_y.data_ptr<float>(), d_c.data_ptr<float>(), d_b.data_ptr<float>(),
                                     d_i.data_ptr<float>(), solution.data_ptr<float>(), (int)d_b.size(0), (int)d_b.size(1),
@@ -65,7 +66,7 @@ std::vector<at::Tensor> tgvInpaint_backward(at::Tensor d_iGf, at::Tensor d_x, at
                                             int its, int id) {
   check_input(d_x, "d_x"); check_input(d_y, "d_y"); check_input(d_c, "d_c"); check_input(d_b, "d_b"); check_input(d_iGf, "d_iGf");
   check_shapes(d_x, d_y, d_c, d_b, d_iGf, "d_iGf");
-  const c10::hip::HIPGuard guard(d_b.device());
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(d_b.device());
   at::Tensor d_oGx = at::empty_like(d_x), d_oGy = at::empty_like(d_y), d_oGc = at::empty_like(d_c);
   at::Tensor d_oGb = at::empty_like(d_b), d_oGi = at::empty_like(d_iGf);
   const int rc = tgvinpaint_backward(d_x.data_ptr<float>(), d_y.data_ptr<float>(), d_c.data_ptr<float>(), d_b.data_ptr<float>(),
