@@ -508,7 +508,8 @@ struct Slot {
   // per-segment fp32 accumulators, double-buffered: every adjoint step reads one set and writes the other
   float *acc_gc[2] = {nullptr, nullptr}, *acc_gx[2] = {nullptr, nullptr}, *acc_gy[2] = {nullptr, nullptr},
         *acc_gb[2] = {nullptr, nullptr};
-  int acc_cur = 0;
+  int acc_cur = 0;   // set of the shared accumulators (gc, gx, gy) the next adjoint launch reads
+  int accb_cur = 0;  // set of the per-channel accumulator (gb) the next adjoint step reads
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
   // strip path: one fp32 record per segment and tensor, added into the totals after the last segment
   float *seg_gc = nullptr, *seg_gx = nullptr, *seg_gy = nullptr, *seg_gb = nullptr;
@@ -606,8 +607,8 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
 }
 
 // -------------------------------------------------------------------------------------------------
-// kernel selection: wave-strip kernels for 1..4 channels, the LDS-tile kernels otherwise.
-// INPAINT_TV_PATH=tile forces the tile kernels (used by the tests to keep both paths covered).
+// kernel selection: the wave-strip kernels (more than 4 channels: in channel groups).
+// INPAINT_TV_PATH=tile forces the LDS-tile kernels written first (used by the tests as a second path).
 // -------------------------------------------------------------------------------------------------
 bool force_tile_path() { return knobs().tv_tile_path; }
 // The x05 rows the forward pass keeps.  INPAINT_KEEP=0|1|2 overrides the id's setting (INPAINT_KEEP_LAST=0 is the
@@ -629,6 +630,15 @@ int strip_rows(int n, int ih, int iw, int cols, int forced_rows, int lag) {
   return choose_strip_rows(sx * n, ih, 4, lag);
 }
 
+// Channel groups: the strip kernels are instantiated for 1..4 channels (the adjoint pair for 1..2).  More channels
+// run as consecutive launches over groups of up to kGroup channels, each launch getting the per-channel tensors
+// already moved to its first channel and the tensor's channel count as the plane stride.  Forward channels never
+// couple.  The adjoint couples them through gc, gwx, gwy only, and those are summed in channel order step by step:
+// one-step launches issued group after group reproduce that order exactly.
+constexpr int kGroup = 4;
+inline const float* at_channel(const Slot& s, const float* p, int ch0) { return p ? p + (size_t)ch0 * s.ih * s.iw : nullptr; }
+inline float* at_channel(const Slot& s, float* p, int ch0) { return p ? p + (size_t)ch0 * s.ih * s.iw : nullptr; }
+
 template <int C>
 void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                           const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
@@ -638,7 +648,7 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, co
   const int sx = (s.iw + tvstrip::kFwdCols - 1) / tvstrip::kFwdCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05, s.n, s.ih, s.iw, t, R, sx, sy, s.ic);
 }
 
 // Two forward iterations in one launch (strip path only): (xin, yin) = iterate k, (xout, yout) = iterate k+2;
@@ -655,12 +665,14 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* d
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB,
-                     (x05a && ring) ? tP : 0.f, R, sx, sy);
+                     (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic);
 }
+
+bool strip_path(const Slot& s) { return !force_tile_path() && s.ic >= 1; }
 
 bool forward_pairs(const Slot& s) {
   if (!knobs().tv_fuse) return false;
-  return !force_tile_path() && s.ic >= 1 && s.ic <= 4;
+  return strip_path(s);
 }
 
 // ring: xin / yin are the x05 rows of the two iterations before this pair and the iterate is rebuilt from them
@@ -668,24 +680,31 @@ bool forward_pairs(const Slot& s) {
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                          const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05a,
                          float* x05b, float tA, float tB, bool ring = false, float tP = 0.f) {
-  switch (s.ic) {
-    case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
-    case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
-    case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
-    default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP); break;
+  for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+    const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
+    float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *ga = at_channel(s, x05a, ch0), *gbb = at_channel(s, x05b, ch0);
+    switch (std::min(kGroup, s.ic - ch0)) {
+      case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
+      case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
+      case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
+      default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
+    }
   }
 }
 
 void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
                     float t) {
-  const bool strip = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
-  if (strip) {
-    switch (s.ic) {
-      case 1: launch_forward_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
-      case 2: launch_forward_strip<2>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
-      case 3: launch_forward_strip<3>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
-      default: launch_forward_strip<4>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05, t); break;
+  if (strip_path(s)) {
+    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+      const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
+      float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *gh = at_channel(s, x05, ch0);
+      switch (std::min(kGroup, s.ic - ch0)) {
+        case 1: launch_forward_strip<1>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+        case 2: launch_forward_strip<2>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+        case 3: launch_forward_strip<3>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+        default: launch_forward_strip<4>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+      }
     }
   } else {
     const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
@@ -694,20 +713,26 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const fl
   }
 }
 
+// One group of a one-step adjoint launch.  Shared accumulators (gc, gwx, gwy): set acc_cur in, the other out, flipped
+// by the caller after every launch; per-channel accumulators (gb): set accb_cur in, the other out, flipped once per
+// step.  last_group: this launch completes the step (a segment-start step then flushes the shared accumulators).
 template <int C, bool END, bool TRUE_ADJ>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                           const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
-                          float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
-  const int i = s.acc_cur, o = 1 - s.acc_cur;
+                          float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t, int ch0, bool last_group) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>;
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, knobs().tv_adj_rows, 6);
   const int sx = (s.iw + tvstrip::kAdjCols - 1) / tvstrip::kAdjCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i],
-                     s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final,
-                     s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, t, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, at_channel(s, b, ch0), at_channel(s, xa, ch0), at_channel(s, xb, ch0),
+                     at_channel(s, yck, ch0), s.acc_gc[i], s.acc_gc[o], at_channel(s, (const float*)s.acc_gb[ib], ch0),
+                     at_channel(s, s.acc_gb[ob], ch0), s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o],
+                     at_channel(s, g05_in, ch0), at_channel(s, g05_out, ch0), at_channel(s, gxk, ch0), at_channel(s, gxk_m1, ch0),
+                     at_channel(s, gx_final, ch0), s.seg_gc + sP, at_channel(s, s.seg_gb + sF, ch0), s.seg_gx + sP, s.seg_gy + sP,
+                     s.n, s.ih, s.iw, t, R, sx, sy, s.ic, last_group ? 1 : 0);
 }
 
 // One adjoint step: reads accumulator set acc_cur, writes the other one, then flips acc_cur.
@@ -716,22 +741,28 @@ template <bool END, bool TRUE_ADJ = false>
 bool launch_adjoint(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
                     float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
-  const bool strip = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
+  const bool strip = strip_path(s);
   if (strip) {
-    switch (s.ic) {
-      case 1: launch_adjoint_strip<1, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
-      case 2: launch_adjoint_strip<2, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
-      case 3: launch_adjoint_strip<3, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
-      default: launch_adjoint_strip<4, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t); break;
+    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+      const bool last = ch0 + kGroup >= s.ic;
+      switch (std::min(kGroup, s.ic - ch0)) {
+        case 1: launch_adjoint_strip<1, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+        case 2: launch_adjoint_strip<2, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+        case 3: launch_adjoint_strip<3, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+        default: launch_adjoint_strip<4, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+      }
+      s.acc_cur = 1 - s.acc_cur;
     }
+    s.accb_cur = 1 - s.accb_cur;
   } else {
     const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
     const int i = s.acc_cur, o = 1 - s.acc_cur;
     hipLaunchKernelGGL(tv_adjoint_iter<END>, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc[i],
                        s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in,
                        g05_out, gxk, gxk_m1, gx_final, s.ic, s.ih, s.iw, t);
+    s.acc_cur = 1 - s.acc_cur;
+    s.accb_cur = s.acc_cur;
   }
-  s.acc_cur = 1 - s.acc_cur;
   return strip;
 }
 
@@ -741,18 +772,20 @@ template <int C, bool BEND, bool TRUE_ADJ>
 void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                                const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                                float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
-  const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip2<C, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2<C, BEND, false, TRUE_ADJ>;
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_adj_rows, 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o],
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
                      s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
-                     s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy);
+                     s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
+// (one group only: a pair adds step A's and step B's terms of its channels back to back, which is the reference's
+// order of summation only when the launch holds every channel)
 template <bool BEND, bool TRUE_ADJ = false>
 void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c, const float* b,
                          const float* xa, const float* xb, const float* xc, const float* g05_in, float* g05_out,
@@ -762,12 +795,13 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const flo
   else
     launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
+  s.accb_cur = 1 - s.accb_cur;
 }
 
 bool adjoint_pairs(const Slot& s) {
   if (!knobs().tv_fuse_adj) return false;
-  // with 3 or 4 channels the pair kernel needs more than 256 registers (one wavefront per SIMD);
-  // those take the one-step kernels
+  // with 3 or 4 channels the pair kernel needs more than 256 registers (one wavefront per SIMD), and pairs over
+  // channel groups would sum the shared accumulators in another order; those take the one-step kernels
   return forward_pairs(s) && s.ic <= 2;
 }
 
@@ -952,18 +986,19 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
   const bool corr = s.grad_mode == 1;
-  if (corr && (force_tile_path() || s.ic > 4))
-    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (1..4 channels), got %d", s.ic);
+  if (corr && force_tile_path())
+    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TV_PATH=tile is set)");
   s.stream = stream;
   const size_t F = field_count(s), P = plane_count(s);
   const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
 
   hipLaunchKernelGGL(scrub_kernel, dim3(gF), dim3(256), 0, stream, gin, (long long)F);
   s.acc_cur = 0;
+  s.accb_cur = 0;
   // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
   // totals after the last segment, in the reference's order (TV.cu:1730 flushes after every segment: same bits,
   // but the totals are not read and rewritten ten times).
-  const bool seg_mode = !force_tile_path() && s.ic >= 1 && s.ic <= 4;
+  const bool seg_mode = strip_path(s);
   SegmentJobs sj;
   {
     float* segs[4] = {s.seg_gc, s.seg_gx, s.seg_gy, s.seg_gb};
@@ -1039,11 +1074,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
         if (corr)
           hipLaunchKernelGGL(tv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                             ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic,
                              (long long)ih * iw, (long long)P);
         else
           hipLaunchKernelGGL(tv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                             ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic,
                              (long long)ih * iw, (long long)P);
         pp_src = 1;
         j--;
@@ -1094,10 +1129,10 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       if (outer == nseg - 1 && j == len - 1) {
         if (corr)
           hipLaunchKernelGGL(tv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
-                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
         else
           hipLaunchKernelGGL(tv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
-                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = ring + (size_t)(j - 1) * F;
         if (timed_run == 0) g_timer.begin(stream);
@@ -1123,7 +1158,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     // iteration has already done it
     if (!flushed && seg_mode) {
       SegmentJobs st = sj;
-      float* accs[4] = {s.acc_gc[s.acc_cur], s.acc_gx[s.acc_cur], s.acc_gy[s.acc_cur], s.acc_gb[s.acc_cur]};
+      float* accs[4] = {s.acc_gc[s.acc_cur], s.acc_gx[s.acc_cur], s.acc_gy[s.acc_cur], s.acc_gb[s.accb_cur]};
       for (int k = 0; k < 4; k++) {
         st.acc[k] = accs[k];
         st.seg[k] = sj.seg[k] + (size_t)outer * sj.n[k];
@@ -1133,7 +1168,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[s.acc_cur], s.tot_gc, (long long)P);
     hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gx[s.acc_cur], s.tot_gx, (long long)P);
     hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gy[s.acc_cur], s.tot_gy, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[s.acc_cur], s.tot_gb, (long long)F);
+    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[s.accb_cur], s.tot_gb, (long long)F);
     }
     lastIt = k0;
   }

@@ -115,6 +115,12 @@ __device__ __forceinline__ void lds_barrier() {
 // -------------------------------------------------------------------------------------------------
 // Forward iteration, TV.cu:1194-1319 (and 1321-1455 when x05 is given).
 //
+// Channel groups: a launch serves C consecutive channels of a tensor with Ct channels per sample; the caller passes
+// the per-channel pointers already moved to the group's first channel.  (Forward channels never couple; the adjoint
+// couples them through the per-pixel accumulators gc, gwx, gwy only, summed in channel order, so groups launched in
+// channel order reproduce the sum of one launch over all channels.  flush_shared: only the last group of a
+// segment-start step stores the segment record of those three and zeroes them.)
+//
 // Per triangle (owner q) the two products
 //     E1 = (y_q - y_down) * (wy / m),   E2 = (y_q - y_right) * (wx / m),   m = max(1, |.|_q / delta)
 // are formed once; q subtracts both, the pixel below q subtracts -E1 and the pixel right of q
@@ -131,7 +137,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05,
-    int N, int H, int W, float t, int R, int strips_x, int strips_y) {
+    int N, int H, int W, float t, int R, int strips_x, int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kFwdCols, R, W, strips_x, strips_y, N)) return;
   const size_t HW = (size_t)H * W;
@@ -151,7 +157,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip(
   float *yo_p[C], *xo_p[C], *xh_p[C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t q = ((size_t)g.n * C + ch) * HW;
+    const size_t q = ((size_t)g.n * Ct + ch) * HW;
     y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
     yo_p[ch] = yout + q; xo_p[ch] = xout + q; xh_p[ch] = X05 ? x05 + q : nullptr;
   }
@@ -290,7 +296,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y) {
+    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
@@ -308,7 +314,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
   float *yo_p[C], *xo_p[C], *xa_p[C], *xb_p[C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t q = ((size_t)g.n * C + ch) * HW;
+    const size_t q = ((size_t)g.n * Ct + ch) * HW;
     y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
     yo_p[ch] = yout + q; xo_p[ch] = xout + q;
     xa_p[ch] = X05 ? x05a + q : nullptr; xb_p[ch] = X05 ? x05b + q : nullptr;
@@ -565,7 +571,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
     float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
-    float t, int R, int strips_x, int strips_y) {
+    float t, int R, int strips_x, int strips_y, int Ct, int flush_shared) {
   StripGeom g;
   if (!strip_geometry(g, kAdjCols, R, W, strips_x, strips_y, N)) return;
   const int Reff = min(R, H - g.hs);
@@ -585,7 +591,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
   float *g05o_p[C], *gxm_p[C], *gbo_p[C], *gxf_p[C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t q = ((size_t)g.n * C + ch) * HW;
+    const size_t q = ((size_t)g.n * Ct + ch) * HW;
     xa_p[ch] = x05a + q; xb_p[ch] = (END ? yck : x05b) + q;  // the checkpoint y travels in the y slot
     b_p[ch] = b + q; g_p[ch] = g05_in + q; gxi_p[ch] = gxk + q; gbi_p[ch] = gb_in + q;
     g05o_p[ch] = g05_out + q; gxm_p[ch] = gxk_m1 + q; gbo_p[ch] = gb + q;
@@ -733,7 +739,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
           stg(gxm_p[ch], roff, gxm);
           stg(g05o_p[ch], roff, g05v);
           if (END) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TV.cu:178-218)
-            seg_gb[((size_t)g.n * C + ch) * HW + (roff >> 2)] = gbv;
+            seg_gb[((size_t)g.n * Ct + ch) * HW + (roff >> 2)] = gbv;
             stg(gbo_p[ch], roff, 0.f);
           } else {
             stg(gbo_p[ch], roff, gbv);
@@ -745,7 +751,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
       dn4[ch] = n4;
     }
     if (!first.value && store_lane) {
-      if (END) {
+      if (END && flush_shared) {
         const size_t e = poff + (roff >> 2);
         seg_gc[e] = gcv;
         seg_gwx[e] = gwxv;
@@ -824,7 +830,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
     float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
-    float tA, float tB, int R, int strips_x, int strips_y) {
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
   const int Reff = min(R, H - g.hs);
@@ -843,7 +849,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
   float *g05o_p[C], *gxm_p[C], *gbo_p[C], *gxf_p[C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t q = ((size_t)g.n * C + ch) * HW;
+    const size_t q = ((size_t)g.n * Ct + ch) * HW;
     xa_p[ch] = x05a + q; xb_p[ch] = x05b + q; xc_p[ch] = x05c + q;  // x05c: x05[j-2], or the checkpoint y when BEND
     b_p[ch] = b + q; g_p[ch] = g05_in + q; gxi_p[ch] = gxk + q; gbi_p[ch] = gb_in + q;
     g05o_p[ch] = g05_out + q; gxm_p[ch] = gxk_m1 + q; gbo_p[ch] = gb + q;
@@ -1043,7 +1049,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
             stg(gxm_p[ch], roffB, gxm);
             stg(g05o_p[ch], roffB, g05v);
             if (BEND) {  // segment flush, fused (TV.cu:178-218)
-              seg_gb[((size_t)g.n * C + ch) * HW + (roffB >> 2)] = gbv;
+              seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
               stg(gbo_p[ch], roffB, 0.f);
             } else {
               stg(gbo_p[ch], roffB, gbv);

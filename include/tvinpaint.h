@@ -72,8 +72,8 @@ int tvinpaint_guard_stats(int id, double* stats25);
  * 1724-1727), iteration 0 is back-propagated too (the reference stops before it and returns g_x[1] as the gradient
  * wrt the start, 1696-1729, 1816), and the multipliers 0.1 / 0.1 / 1.0 and the global 0.1 (63-69) are 1.  The
  * clamp of the adjoint iterates (797-799), the upstream scrub and the output guard stay.  With them inactive the
- * result is the gradient of the forward pass (tests compare it with automatic differentiation).  Strip kernels
- * only (1..4 channels); same speed as the default. */
+ * result is the gradient of the forward pass (tests compare it with automatic differentiation).  Any channel
+ * count; same speed as the default. */
 int tvinpaint_gradient_mode(int id, int mode);
 
 /* Which intermediate iterates (the x05 rows of TVInpaintFista.cu:1678-1687) the next forwards on `id` keep for

@@ -84,10 +84,27 @@ def test_forward_backward_match_oracle(ext, tv_oracle, n, c, h, w, its):
     compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 5, 20, 64, 6),      # 4 + 1
+    (2, 6, 37, 101, 9),     # 4 + 2, ragged, odd its
+    (1, 7, 19, 126, 20),    # 4 + 3, several segments
+    (2, 8, 45, 130, 12),    # 4 + 4
+    (1, 9, 11, 62, 8),      # three groups
+])
+def test_more_than_four_channels_run_in_channel_groups(ext, tv_oracle, n, c, h, w, its):
+    # the strip kernels hold up to four channels; more run as launches over groups of channels, whose shared
+    # accumulators (confidence and edge-weight gradients) are summed group after group in the reference's order
+    d = tv_inputs(n, c, h, w, seed=300 + c, conf_density=0.3)
+    got, ref = run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2)
+    compare("%d channels in groups" % c, got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
-def test_tile_kernels_when_forced_or_needed(ext, tv_oracle, n, c, h, w, its, monkeypatch):
-    # up to 4 channels normally take the wave-strip kernels; force the LDS-tile kernels
-    # (5 channels always takes them)
+def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
+    # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first
     d = tv_inputs(n, c, h, w, seed=77 + c, conf_density=0.3)
     ref = run_oracle(tv_oracle, d, its, 2)
     compare("default path c=%d" % c, run_gpu(ext, d, its, 2), ref)
@@ -309,7 +326,7 @@ CORRECTED = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale
 
 @pytest.mark.parametrize("n,c,h,w,its", [
     (1, 2, 64, 128, 20), (2, 3, 37, 101, 9), (1, 1, 16, 64, 2), (1, 4, 19, 126, 6), (1, 2, 1, 70, 4),
-    (1, 1, 33, 1, 4), (3, 2, 130, 200, 50), (1, 2, 21, 64, 3),
+    (1, 1, 33, 1, 4), (3, 2, 130, 200, 50), (1, 2, 21, 64, 3), (1, 6, 23, 70, 10),
 ])
 def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # gradient_mode 1: y as the forward pass made it, no checkpoint stand-in at segment starts, iteration 0
@@ -376,6 +393,7 @@ def test_corrected_gradient_needs_the_strip_kernels(ext, monkeypatch):
     d = tv_inputs(1, 5, 12, 20, seed=1, conf_density=0.3)
     dev = torch.device("cuda:0")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    monkeypatch.setenv("INPAINT_TV_PATH", "tile")  # the LDS-tile kernels have no corrected form
     try:
         ext.reset_id(2)
         ext.gradient_mode(2, 1)
