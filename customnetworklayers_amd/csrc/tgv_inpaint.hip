@@ -741,7 +741,8 @@ struct Slot {
   // per-segment fp32 accumulators, double-buffered: a strip-kernel step reads one set and writes the other
   float *acc_gc[2] = {nullptr, nullptr}, *acc_gx[2] = {nullptr, nullptr}, *acc_gy[2] = {nullptr, nullptr},
         *acc_gb[2] = {nullptr, nullptr};
-  int acc_cur = 0;
+  int acc_cur = 0;   // set of the shared accumulators (gc, gx, gy) the next adjoint launch reads
+  int accb_cur = 0;  // set of the per-channel accumulator (gb) the next adjoint step reads
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
   // strip path: one fp32 record per segment and tensor, added into the totals after the last segment
   float *seg_gc = nullptr, *seg_gx = nullptr, *seg_gy = nullptr, *seg_gb = nullptr;
@@ -872,10 +873,16 @@ void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const flo
 // kernel selection: wave-strip kernels for 1..2 flow channels, the per-pixel kernels otherwise.
 // INPAINT_TGV_PATH=px forces the per-pixel kernels (used by the tests to keep both paths covered).
 // -------------------------------------------------------------------------------------------------
-bool use_strip(const Slot& s) {
-  if (knobs().tgv_px_path) return false;
-  return s.ic >= 1 && s.ic <= 2;
-}
+bool use_strip(const Slot& s) { return !knobs().tgv_px_path && s.ic >= 1; }
+
+// Channel groups: the strip kernels are instantiated for one and two flow channels.  More channels run as consecutive
+// launches over groups of two, each getting the per-channel tensors already moved to its first channel and the
+// tensor's channel count as the plane stride.  Forward channels never couple; the adjoint couples them through the
+// five shared accumulators (gc and the two channels of gwx, gwy) only, summed in channel order step by step, which
+// one-step launches issued group after group reproduce exactly.
+constexpr int kGroup = 2;
+inline const float* at_channel(const Slot& s, const float* p, int ch0) { return p ? p + (size_t)ch0 * s.ih * s.iw : nullptr; }
+inline float* at_channel(const Slot& s, float* p, int ch0) { return p ? p + (size_t)ch0 * s.ih * s.iw : nullptr; }
 int strip_rows(int n, int ih, int iw, int cols, int forced_rows, int lag) {
   // Rows per wavefront: taller strips amortise the start-up latency and the one-row overlap between
   // strips, but the launch should still keep every SIMD of the chip busy.
@@ -921,14 +928,18 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* c, con
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);  // a multiple of 8: one share per XCD
   hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xout, yin, yout, x05, s.n, s.ih, s.iw, t,
-                     R, sx, sy);
+                     R, sx, sy, s.ic);
 }
 
 void launch_forward(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                     const float* yin, float* yout, float* x05, float t) {
   if (use_strip(s)) {
-    if (s.ic == 1) launch_forward_strip<1>(s, stream, c, b, xin, xout, yin, yout, x05, t);
-    else launch_forward_strip<2>(s, stream, c, b, xin, xout, yin, yout, x05, t);
+    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+      const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
+      float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *gh = at_channel(s, x05, ch0);
+      if (s.ic - ch0 == 1) launch_forward_strip<1>(s, stream, c, gb, gxi, gxo, gyi, gyo, gh, t);
+      else launch_forward_strip<2>(s, stream, c, gb, gxi, gxo, gyi, gyo, gh, t);
+    }
     return;
   }
   const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
@@ -950,7 +961,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b,
-                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy);
+                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic);
 }
 
 bool forward_pairs(const Slot& s) {
@@ -964,25 +975,33 @@ bool forward_pairs(const Slot& s) {
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                          const float* yin, float* yout, float* x05a, float* x05b, float tA, float tB,
                          const float* xin_aux = nullptr, bool store_x_aux = true, bool ring = false, float tP = 0.f) {
-  if (s.ic == 1)
-    launch_forward_pair_strip<1>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP);
-  else
-    launch_forward_pair_strip<2>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP);
+  for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+    const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gxa = at_channel(s, xin_aux, ch0), *gyi = at_channel(s, yin, ch0);
+    float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *ga = at_channel(s, x05a, ch0), *gbb = at_channel(s, x05b, ch0);
+    if (s.ic - ch0 == 1)
+      launch_forward_pair_strip<1>(s, stream, c, gb, gxi, gxa, gxo, gyi, gyo, ga, gbb, store_x_aux, tA, tB, ring, tP);
+    else
+      launch_forward_pair_strip<2>(s, stream, c, gb, gxi, gxa, gxo, gyi, gyo, ga, gbb, store_x_aux, tA, tB, ring, tP);
+  }
 }
 
+// One group of a one-step adjoint launch.  Shared accumulators: set acc_cur in, the other out, flipped by the caller
+// after every launch; the per-channel accumulator gb: set accb_cur in, the other out, flipped once per step.
 template <int C, bool END, int ADJ>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
                           const float* xb, const float* yck, const float* g05_in, float* g05_out, const float* gxk,
-                          float* gxk_m1, float* gx_final, float t) {
-  const int i = s.acc_cur, o = 1 - s.acc_cur;
+                          float* gxk_m1, float* gx_final, float t, int ch0) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
   auto kern = gx_final ? tgvstrip::tgv_adjoint_strip<C, END, true, ADJ> : tgvstrip::tgv_adjoint_strip<C, END, false, ADJ>;
   const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, knobs().tgv_adj_rows, 6);
   const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, xb, yck, s.acc_gc[i], s.acc_gc[o],
-                     s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1,
-                     gx_final, s.n, s.ih, s.iw, t, R, sx, sy);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, at_channel(s, b, ch0), at_channel(s, xa, ch0),
+                     at_channel(s, xb, ch0), at_channel(s, yck, ch0), s.acc_gc[i], s.acc_gc[o],
+                     at_channel(s, (const float*)s.acc_gb[ib], ch0), at_channel(s, s.acc_gb[ob], ch0), s.acc_gx[i], s.acc_gx[o],
+                     s.acc_gy[i], s.acc_gy[o], at_channel(s, g05_in, ch0), at_channel(s, g05_out, ch0), at_channel(s, gxk, ch0),
+                     at_channel(s, gxk_m1, ch0), at_channel(s, gx_final, ch0), s.n, s.ih, s.iw, t, R, sx, sy, s.ic);
 }
 
 // One adjoint step.  Strip path: y is rebuilt inside the kernel from xa = x05[k], xb = x05[k-1] (END:
@@ -995,9 +1014,12 @@ void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b,
                     const float* yck, const float* g05_in, float* g05_out, float* gxk, float* gxk_m1, float* gx_final,
                     float t) {
   if (use_strip(s)) {
-    if (s.ic == 1) launch_adjoint_strip<1, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
-    else launch_adjoint_strip<2, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t);
-    s.acc_cur = 1 - s.acc_cur;
+    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+      if (s.ic - ch0 == 1) launch_adjoint_strip<1, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0);
+      else launch_adjoint_strip<2, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0);
+      s.acc_cur = 1 - s.acc_cur;
+    }
+    s.accb_cur = 1 - s.accb_cur;
     return;
   }
   const float* y = yck;
@@ -1007,10 +1029,10 @@ void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b,
                        (long long)s.ih * s.iw, P, t);
     y = s.yk;
   }
-  const int a = s.acc_cur;
+  const int a = s.acc_cur;  // (the per-pixel kernels update their accumulators in place: both indices stay put)
   const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
   hipLaunchKernelGGL(tgv_adjoint_px<END>, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, s.acc_gc[a],
-                     s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
+                     s.acc_gb[s.accb_cur], s.acc_gx[a], s.acc_gy[a], g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
 }
 
 // Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
@@ -1023,7 +1045,7 @@ template <int C, bool BEND, bool TRUE_ADJ>
 void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
                                const float* xb, const float* xc, const float* g05_in, float* g05_out, const float* gxk,
                                float* gxk_m1, float* gx_final, float tA, float tB) {
-  const int i = s.acc_cur, o = 1 - s.acc_cur;
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
   // two channels: the two steps run in two wavefronts of a workgroup (one strip per 128-thread workgroup);
   // one channel: both steps fit one wavefront's registers (four strips per 256-thread workgroup)
   const bool split = pair_split(C);
@@ -1034,9 +1056,9 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const long long waves = (long long)sx * sy * s.n;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
 #define TGV_PAIR_ARGS                                                                                                      \
-  s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], \
+  s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob], s.acc_gx[i], s.acc_gx[o], \
       s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + 2 * sP, s.seg_gy + 2 * sP, s.n, s.ih,  \
-      s.iw, tA, tB, R, sx, sy
+      s.iw, tA, tB, R, sx, sy, s.ic
   if (split) {
     const dim3 grid((unsigned)((waves + 7) / 8 * 8)), block(128);
     if (gx_final) hipLaunchKernelGGL((tgvstrip::tgv_adjoint_strip2w<C, BEND, true, TRUE_ADJ>), grid, block, 0, stream, TGV_PAIR_ARGS);
@@ -1055,11 +1077,14 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* c, const floa
   if (s.ic == 1) launch_adjoint_pair_strip<1, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   else launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
+  s.accb_cur = 1 - s.accb_cur;
 }
 
 bool adjoint_pairs(const Slot& s) {
   if (!knobs().tgv_fuse_adj) return false;
-  return forward_pairs(s);
+  // one group only: a pair adds step A's and step B's terms of its channels back to back, which is the reference's
+  // order of summation only when the launch holds every channel
+  return forward_pairs(s) && s.ic <= kGroup;
 }
 
 }  // namespace
@@ -1162,7 +1187,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
   const bool corr = s.grad_mode == 1;
   if (corr && !use_strip(s))
-    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (1 or 2 channels), got %d", s.ic);
+    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TGV_PATH=px is set)");
   s.stream = stream;
   const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
   const int gS = grid_stride((long long)S3), gF = grid_stride((long long)F), gP = grid_stride((long long)P),
@@ -1215,6 +1240,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     int k = 0;
     for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.yk, s.gx_final}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
     s.acc_cur = 0;
+    s.accb_cur = 0;
     z.ptr[k] = s.acc_gb[0]; z.bytes[k++] = (long long)F * 4;
     z.ptr[k] = s.acc_gc[0]; z.bytes[k++] = (long long)P * 4;
     z.ptr[k] = s.acc_gx[0]; z.bytes[k++] = (long long)P * 8;
@@ -1281,11 +1307,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       if (outer == nseg - 1 && j >= 0) {
         if (corr)
           hipLaunchKernelGGL(tgv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                             ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic,
                              (long long)ih * iw, (long long)P);
         else
           hipLaunchKernelGGL(tgv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
-                             ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic,
+                             ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic,
                              (long long)ih * iw, (long long)P);
         pp_src = 1;
         j--;
@@ -1335,10 +1361,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       if (outer == nseg - 1 && j == len - 1) {
         if (corr)
           hipLaunchKernelGGL(tgv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
-                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
         else
           hipLaunchKernelGGL(tgv_adjoint_first<false>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b, xa,
-                             s.acc_gc[s.acc_cur], s.acc_gb[s.acc_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
+                             s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic, (long long)ih * iw, (long long)P);
       } else if (j > 0) {
         const float* xb = ring + (size_t)(j - 1) * S3;
         if (timed_run == 0) g_timer.begin(stream);
@@ -1364,7 +1390,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     if (!flushed && seg_mode) {
       SegmentJobs st = sj;
       const int a = s.acc_cur;
-      float* accs[4] = {s.acc_gc[a], s.acc_gx[a], s.acc_gy[a], s.acc_gb[a]};
+      float* accs[4] = {s.acc_gc[a], s.acc_gx[a], s.acc_gy[a], s.acc_gb[s.accb_cur]};
       for (int k = 0; k < 4; k++) {
         st.acc[k] = accs[k];
         st.seg[k] = sj.seg[k] + (size_t)outer * sj.n[k];
@@ -1375,7 +1401,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[a], s.tot_gc, (long long)P);
       hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
       hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
-      hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[a], s.tot_gb, (long long)F);
+      hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[s.accb_cur], s.tot_gb, (long long)F);
     }
     lastIt = k0;
   }
@@ -1389,7 +1415,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
     const int last = pairs ? pp_src : 0;
     hipLaunchKernelGGL((tgv_adjoint_px<false, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, s.ckpt_y,
-                       s.acc_gc[a], s.acc_gb[a], s.acc_gx[a], s.acc_gy[a], s.g05[last], s.gx_final, s.gxk[last],
+                       s.acc_gc[a], s.acc_gb[s.accb_cur], s.acc_gx[a], s.acc_gy[a], s.g05[last], s.gx_final, s.gxk[last],
                        s.gxk[1 - last], s.ckpt_y, s.ic, s.ih, s.iw, 0.f);
     hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
     hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));

@@ -74,10 +74,10 @@ __global__ __launch_bounds__(256) void tgv_forward_strip(
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
     const float* __restrict__ xin, float* __restrict__ xout, const float* __restrict__ yin,
     float* __restrict__ yout, float* __restrict__ x05, int N, int H, int W, float t, int R, int strips_x,
-    int strips_y) {
+    int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kCols, R, W, strips_x, strips_y, N)) return;
-  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
   const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip(
   float *yo_p[3][C], *xo_p[3][C], *xh_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    b_p[ch] = b + ((size_t)g.n * C + ch) * HW;
+    b_p[ch] = b + ((size_t)g.n * Ct + ch) * HW;
 #pragma unroll
     for (int v = 0; v < 3; v++) {
       const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
@@ -257,11 +257,11 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
     const float* __restrict__ xin, const float* __restrict__ xin_aux, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int store_x_aux, int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y) {
+    int store_x_aux, int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
-  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
   const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
   float *yo_p[3][C], *xo_p[3][C], *xa_p[3][C], *xb_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    b_p[ch] = b + ((size_t)g.n * C + ch) * HW;
+    b_p[ch] = b + ((size_t)g.n * Ct + ch) * HW;
 #pragma unroll
     for (int v = 0; v < 3; v++) {
       const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
@@ -557,11 +557,11 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
     const float* __restrict__ gwx_in, float* __restrict__ gwx, const float* __restrict__ gwy_in,
     float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
     const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, int N, int H, int W,
-    float t, int R, int strips_x, int strips_y) {
+    float t, int R, int strips_x, int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kCols, R, W, strips_x, strips_y, N)) return;
   const int Reff = min(R, H - g.hs);
-  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
   const bool store_lane = g.lane > 0 && g.lane < 63 && g.col_ok;
@@ -581,7 +581,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
   float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t qb = ((size_t)g.n * C + ch) * HW;
+    const size_t qb = ((size_t)g.n * Ct + ch) * HW;
     b_p[ch] = b + qb; gbi_p[ch] = gb_in + qb; gbo_p[ch] = gb + qb;
 #pragma unroll
     for (int v = 0; v < 3; v++) {
@@ -929,12 +929,12 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
     float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
     const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
-    float tA, float tB, int R, int strips_x, int strips_y) {
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
   StripGeom g;
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
   const int Reff = min(R, H - g.hs);
   const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
-  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
   const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
@@ -952,7 +952,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
   float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t qb = ((size_t)g.n * C + ch) * HW;
+    const size_t qb = ((size_t)g.n * Ct + ch) * HW;
     b_p[ch] = b + qb; gbi_p[ch] = gb_in + qb; gbo_p[ch] = gb + qb;
     xc_p[ch] = x05c + (size_t)g.n * 3 * CHW + (size_t)ch * HW;  // u of x05[j-2] (BEND: u of the checkpoint y)
 #pragma unroll
@@ -1282,7 +1282,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
             stg(g05o_p[1][ch], roffB, o.d1);
             stg(g05o_p[2][ch], roffB, o.d2);
             if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
-              seg_gb[((size_t)g.n * C + ch) * HW + (roffB >> 2)] = gbv;
+              seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
               stg(gbo_p[ch], roffB, 0.f);
             } else {
               stg(gbo_p[ch], roffB, gbv);
@@ -1393,7 +1393,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
     const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
-    float tA, float tB, int R, int strips_x, int strips_y) {
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
   constexpr int kHand = 7 * C + 5;  // floats step A hands to step B per row and lane
   __shared__ float hand[2][kHand][64];
   StripGeom g;
@@ -1401,7 +1401,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
   const int role = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront 0: step A, wavefront 1: step B
   const int Reff = min(R, H - g.hs);
   const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
-  const size_t HW = (size_t)H * W, CHW = HW * C;
+  const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
   const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
@@ -1420,7 +1420,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
   float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t qb = ((size_t)g.n * C + ch) * HW;
+    const size_t qb = ((size_t)g.n * Ct + ch) * HW;
     b_p[ch] = b + qb; gbi_p[ch] = gb_in + qb; gbo_p[ch] = gb + qb;
     xc_p[ch] = x05c + (size_t)g.n * 3 * CHW + (size_t)ch * HW;  // u of x05[j-2] (BEND: u of the checkpoint y)
 #pragma unroll
@@ -1891,7 +1891,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
               stg(g05o_p[1][ch], roffB, o.d1);
               stg(g05o_p[2][ch], roffB, o.d2);
               if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
-                seg_gb[((size_t)g.n * C + ch) * HW + (roffB >> 2)] = gbv;
+                seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
                 stg(gbo_p[ch], roffB, 0.f);
               } else {
                 stg(gbo_p[ch], roffB, gbv);

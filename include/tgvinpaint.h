@@ -53,8 +53,8 @@ int tgvinpaint_reset_id(int id);
  * its siblings (355), iteration 0 is back-propagated too (2851-2933, 3047), and the multipliers (87-93) are 1.  The
  * clamp of the adjoint iterates (562-583), the upstream check and the output guard stay.  With them inactive the
  * result is the gradient of the forward pass (tests compare it with the float64 oracle that automatic differentiation
- * pins).  Strip kernels only (1 or 2 channels); two adjoint
- * steps per launch with two channels (5% slower than the default), one with one channel. */
+ * pins).  Any channel count; two adjoint steps per launch with two channels (5% slower than the default), one
+ * otherwise. */
 int tgvinpaint_gradient_mode(int id, int mode);
 
 /* Which intermediate iterates (the x05 rows of TGVInpaintFista.cu:2775-2814) the next forwards on `id` keep for

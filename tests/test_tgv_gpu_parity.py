@@ -100,10 +100,26 @@ def test_forward_backward_match_oracle(ext, tgv_oracle, n, c, h, w, its):
     compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 3, 20, 64, 6),      # 2 + 1
+    (2, 4, 37, 101, 9),     # 2 + 2, ragged, odd its
+    (1, 5, 19, 126, 20),    # three groups, several segments
+    (1, 3, 45, 130, 12),
+])
+def test_more_than_two_channels_run_in_channel_groups(ext, tgv_oracle, n, c, h, w, its):
+    # the strip kernels hold up to two flow channels; more run as launches over groups of channels, whose shared
+    # accumulators (confidence and weight gradients) are summed group after group in the reference's order
+    d = varying_inputs(n, c, h, w, seed=300 + c)
+    got, ref = run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2)
+    compare("%d channels in groups" % c, got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 33, 64, 9), (1, 3, 20, 64, 6)])
-def test_per_pixel_kernels_when_forced_or_needed(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
-    # up to 2 flow channels normally take the wave-strip kernels; force the per-pixel kernels
-    # (3 channels always takes them)
+def test_per_pixel_kernels_when_forced(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
+    # every channel count normally takes the wave-strip kernels; force the per-pixel kernels written first
     d = varying_inputs(n, c, h, w, seed=77 + c)
     ref = run_oracle(tgv_oracle, d, its, 2)
     compare("default path c=%d" % c, run_gpu(ext, d, its, 2), ref)
@@ -383,7 +399,7 @@ CORRECTED = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale
 
 @pytest.mark.parametrize("n,c,h,w,its", [
     (1, 2, 64, 128, 20), (2, 1, 37, 101, 9), (1, 1, 16, 64, 2), (1, 2, 1, 70, 4), (1, 1, 33, 1, 4),
-    (2, 2, 90, 200, 30), (1, 2, 21, 63, 3),
+    (2, 2, 90, 200, 30), (1, 2, 21, 63, 3), (1, 3, 23, 70, 10),
 ])
 def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tgv_oracle, n, c, h, w, its):
     # gradient_mode 1: y (all three variables) as the forward pass made it, no checkpoint stand-in at segment starts,
@@ -446,10 +462,11 @@ def test_corrected_gradient_is_the_gradient_of_the_forward_pass(ext, tgv_oracle)
     assert rel_err(plain[3], true[3]) > 0.5  # the reference's gradient is a different vector
 
 
-def test_corrected_gradient_needs_the_strip_kernels(ext):
+def test_corrected_gradient_needs_the_strip_kernels(ext, monkeypatch):
     d = varying_inputs(1, 3, 12, 20, seed=1)
     dev = torch.device("cuda:0")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    monkeypatch.setenv("INPAINT_TGV_PATH", "px")  # the per-pixel kernels have no corrected form
     try:
         ext.reset_id(2)
         ext.gradient_mode(2, 1)
