@@ -1362,7 +1362,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
 // The same two adjoint steps per launch, split over the two wavefronts of a 128-thread workgroup:
 // wavefront 0 runs step A (local iteration j) one row ahead and hands each row's results -- g05[j],
 // the partial g_x[j] and the seven accumulators -- to wavefront 1 through LDS (7C+5 floats per lane,
-// two slots, one LDS-only barrier per row); wavefront 1 runs step B (j-1) on them and stores.  Each
+// four slots, one LDS-only barrier per two rows); wavefront 1 runs step B (j-1) on them and stores.  Each
 // wavefront holds one step's registers, so two workgroup pairs fit a SIMD where tgv_adjoint_strip2
 // at two channels leaves room for one wavefront.  Arithmetic and memory traffic are those of
 // tgv_adjoint_strip2 (wavefront 1 re-reads the weights, b and u of x05[j-1] from the cache).
@@ -1395,7 +1395,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
   constexpr int kHand = 7 * C + 5;  // floats step A hands to step B per row and lane
-  __shared__ float hand[2][kHand][64];
+  __shared__ float hand[4][kHand][64];  // four slots: A runs up to two rows ahead of the barrier B waits at
   StripGeom g;
   if (!strip_geometry_block(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
   const int role = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront 0: step A, wavefront 1: step B
@@ -1709,7 +1709,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       const int h = g.hs - 2 + k;
       const bool in_img = g.col_ok && h >= 0 && h < H;
       const bool dmaskA = h >= 0 && h < H - 1;
-      float (*slot)[64] = hand[k & 1];
+      float (*slot)[64] = hand[k & 3];
       float gcv = late.gc_i;
       Acc accA{late.gwx0_i, late.gwx1_i, late.gwy0_i, late.gwy1_i};
 #pragma unroll
@@ -1742,6 +1742,12 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       slot[7 * C + 4][g.lane] = accA.gwy1;
     };
 
+    // A publishes two rows per barrier: the barrier after an odd row k makes rows k-1 and k visible to step B, which
+    // works on them while A fills the other two slots (one barrier per row made each wavefront wait for the other's
+    // slowest row)
+    auto publish = [&](int k) {
+      if (k & 1) lds_barrier();
+    };
     Adj2ARow<C> b0, b1, b2;
     Adj2Late<C> late;
     load_row(0, b0);
@@ -1752,7 +1758,6 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     absorb(1, b1);
     step(0, b0, b1, late, kNo);
     load_row(3, b0);
-    lds_barrier();
     absorb(2, b2);
     step(1, b1, b2, late, kYes);
     load_row(4, b1);
@@ -1762,27 +1767,26 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     step(2, b2, b0, late, kYes);
     load_row(5, b2);
     load_late(3, late);
-    lds_barrier();
     for (int k = 3; k <= klast; k += 3) {  // cur / next rotate through (b0,b1) (b1,b2) (b2,b0)
       absorb(k + 1, b1);
       step(k, b0, b1, late, kYes);
       load_row(k + 3, b0);
       load_late(k + 1, late);
-      lds_barrier();
+      publish(k);
       if (k + 1 > klast) break;
       absorb(k + 2, b2);
       step(k + 1, b1, b2, late, kYes);
       load_row(k + 4, b1);
       load_late(k + 2, late);
-      lds_barrier();
+      publish(k + 1);
       if (k + 2 > klast) break;
       absorb(k + 3, b0);
       step(k + 2, b2, b0, late, kYes);
       load_row(k + 5, b2);
       load_late(k + 3, late);
-      lds_barrier();
+      publish(k + 2);
     }
-    lds_barrier();  // the interval in which step B works on the last row
+    if (!(klast & 1)) lds_barrier();  // an even last row has not been published yet
   } else {
     // ---------------------------------- step B ----------------------------------
     auto load_row = [&](int k, Adj2BRow<C>& in) {
@@ -1853,7 +1857,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
       const bool dmaskB = h - 1 >= 0 && h - 1 < H - 1;
       const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
-      float (*slot)[64] = hand[k & 1];
+      float (*slot)[64] = hand[k & 3];
       float nG[3][C], ngxm[3][C], ngb[C];
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
@@ -1931,38 +1935,40 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       }
     };
 
+    // B waits before every even row for the barrier that published it and the row after it
+    auto await = [&](int k) {
+      if (!(k & 1)) lds_barrier();
+    };
     Adj2BRow<C> b0, b1, b2;
     load_row(0, b0);
     load_row(1, b1);
     load_row(2, b2);
-    lds_barrier();  // the interval in which step A works on the first row
+    lds_barrier();  // rows 0 and 1
     absorb(0, b0);
     step(0, b0, kNo, kNo);
     load_row(3, b0);
-    lds_barrier();
     absorb(1, b1);
     step(1, b1, kNo, kNo);
     load_row(4, b1);
-    lds_barrier();
+    lds_barrier();  // rows 2 and 3 (or the last row)
     absorb(2, b2);
     step(2, b2, kYes, kNo);
     load_row(5, b2);
-    lds_barrier();
     for (int k = 3; k <= klast; k += 3) {
+      await(k);
       absorb(k, b0);
       step(k, b0, kYes, kYes);
       load_row(k + 3, b0);
-      lds_barrier();
       if (k + 1 > klast) break;
+      await(k + 1);
       absorb(k + 1, b1);
       step(k + 1, b1, kYes, kYes);
       load_row(k + 4, b1);
-      lds_barrier();
       if (k + 2 > klast) break;
+      await(k + 2);
       absorb(k + 2, b2);
       step(k + 2, b2, kYes, kYes);
       load_row(k + 5, b2);
-      lds_barrier();
     }
   }
 }
