@@ -64,12 +64,13 @@ def test_tgv_full_length_sample_matches_oracle(ext):
     o = TGVOracle()
     o.set_quirks()
     cfg = CONFIGS[2]
-    d = tgv_inputs(1, cfg["c"], 192, 416, seed=3, **cfg["gen"])  # a ninth of a sample, all 100 iterations
+    d = tgv_inputs(1, cfg["c"], cfg["h"], cfg["w"], seed=3, **cfg["gen"])  # one whole sample, all 100 iterations
+    print("case 1x%dx%dx%d its=%d" % (cfg["c"], cfg["h"], cfg["w"], cfg["its"]), flush=True)
     got = gpu_layer(ext, d, cfg["its"], 3)
     o.reset_id(3)
     sol = o.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], cfg["its"], 3)
     grads = o.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], cfg["its"], 3)
     rel = lambda a, r: float(np.abs(a - r).max() / max(np.abs(r).max(), 1e-30))
     errs = [rel(a, r) for a, r in zip(got, [sol] + list(grads))]
-    print("\n[tgv 1x2x192x416 its=100] out %.2e grads %s" % (errs[0], ["%.2e" % e for e in errs[1:]]), flush=True)
+    print("\n[tgv 1x2x384x1248 its=100] out %.2e grads %s" % (errs[0], ["%.2e" % e for e in errs[1:]]), flush=True)
     assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3
