@@ -1395,7 +1395,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
   constexpr int kHand = 7 * C + 5;  // floats step A hands to step B per row and lane
-  __shared__ float hand[4][kHand][64];  // four slots: A runs up to two rows ahead of the barrier B waits at
+#ifndef TGV_ROWS_PER_BARRIER
+#define TGV_ROWS_PER_BARRIER 2
+#endif
+  constexpr int kP = TGV_ROWS_PER_BARRIER;  // rows step A publishes per barrier
+  __shared__ float hand[2 * kP][kHand][64];  // A fills kP slots while B works on the kP before them
   StripGeom g;
   if (!strip_geometry_block(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
   const int role = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront 0: step A, wavefront 1: step B
@@ -1709,7 +1713,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       const int h = g.hs - 2 + k;
       const bool in_img = g.col_ok && h >= 0 && h < H;
       const bool dmaskA = h >= 0 && h < H - 1;
-      float (*slot)[64] = hand[k & 3];
+      float (*slot)[64] = hand[k % (2 * kP)];
       float gcv = late.gc_i;
       Acc accA{late.gwx0_i, late.gwx1_i, late.gwy0_i, late.gwy1_i};
 #pragma unroll
@@ -1742,11 +1746,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       slot[7 * C + 4][g.lane] = accA.gwy1;
     };
 
-    // A publishes two rows per barrier: the barrier after an odd row k makes rows k-1 and k visible to step B, which
-    // works on them while A fills the other two slots (one barrier per row made each wavefront wait for the other's
-    // slowest row)
+    // A publishes kP rows per barrier: the barrier after row k with k % kP == kP - 1 makes rows k-kP+1 .. k visible to
+    // step B, which works on them while A fills the other kP slots (one barrier per row made each wavefront wait for
+    // the other's slowest row)
     auto publish = [&](int k) {
-      if (k & 1) lds_barrier();
+      if (k % kP == kP - 1) lds_barrier();
     };
     Adj2ARow<C> b0, b1, b2;
     Adj2Late<C> late;
@@ -1758,15 +1762,17 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     absorb(1, b1);
     step(0, b0, b1, late, kNo);
     load_row(3, b0);
+    publish(0);
     absorb(2, b2);
     step(1, b1, b2, late, kYes);
     load_row(4, b1);
     load_late(2, late);
-    lds_barrier();
+    publish(1);
     absorb(3, b0);
     step(2, b2, b0, late, kYes);
     load_row(5, b2);
     load_late(3, late);
+    publish(2);
     for (int k = 3; k <= klast; k += 3) {  // cur / next rotate through (b0,b1) (b1,b2) (b2,b0)
       absorb(k + 1, b1);
       step(k, b0, b1, late, kYes);
@@ -1786,7 +1792,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       load_late(k + 3, late);
       publish(k + 2);
     }
-    if (!(klast & 1)) lds_barrier();  // an even last row has not been published yet
+    if (klast % kP != kP - 1) lds_barrier();  // the last rows have not been published yet
   } else {
     // ---------------------------------- step B ----------------------------------
     auto load_row = [&](int k, Adj2BRow<C>& in) {
@@ -1857,7 +1863,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
       const bool dmaskB = h - 1 >= 0 && h - 1 < H - 1;
       const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
-      float (*slot)[64] = hand[k & 3];
+      float (*slot)[64] = hand[k % (2 * kP)];
       float nG[3][C], ngxm[3][C], ngb[C];
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
@@ -1935,22 +1941,23 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       }
     };
 
-    // B waits before every even row for the barrier that published it and the row after it
+    // B waits before every row k with k % kP == 0 for the barrier that published rows k .. k+kP-1
     auto await = [&](int k) {
-      if (!(k & 1)) lds_barrier();
+      if (k % kP == 0) lds_barrier();
     };
     Adj2BRow<C> b0, b1, b2;
     load_row(0, b0);
     load_row(1, b1);
     load_row(2, b2);
-    lds_barrier();  // rows 0 and 1
+    await(0);
     absorb(0, b0);
     step(0, b0, kNo, kNo);
     load_row(3, b0);
+    await(1);
     absorb(1, b1);
     step(1, b1, kNo, kNo);
     load_row(4, b1);
-    lds_barrier();  // rows 2 and 3 (or the last row)
+    await(2);
     absorb(2, b2);
     step(2, b2, kYes, kNo);
     load_row(5, b2);
