@@ -28,7 +28,8 @@ COUNTERS = {
             files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="2207eb7"),
     2: dict(traffic=(2 * 174492 + 148961) * 1024, step=(2 * 13776080 + 14750333) * 1024, lds=688464 * 64 * 8, rocprof_ms=0.12699,
             files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="2207eb7"),
-    5: dict(traffic=(2 * 408180 + 340500) * 1024, files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
+    5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
+            files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="HEADREV"),
     6: dict(traffic=(2 * 131080 + 247100) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
 }
 MEASURED_TRAFFIC_BYTES = {k: v["traffic"] for k, v in COUNTERS.items()}
@@ -144,8 +145,10 @@ def bench_flowaux(args, cfg, d):
         # floats per pixel: forward reads both feature maps and the flow, writes 3; backward reads both maps,
         # flow and upstream, writes g0, zero-fills g1 and read-modify-writes it
         # per-source pass of the backward (the dominant kernel): both maps, flow, upstream in; g0 and 5 coefficients out
-        bpp = dict(forward=4 * (2 * c + 5), backward=4 * (5 * c + 5), kernel=4 * (3 * c + 10))
-        kernel = "quadfit_tiles<1,2> (backward, per-source pass)"
+        # per-source pass of the backward: both maps, flow, upstream in; g0 and 5 coefficients out (the inverse map not counted)
+        # gather pass (the dominant kernel): first map, 5 coefficients, list length and up to 4 list entries in; g1 out
+        bpp = dict(forward=4 * (2 * c + 5), backward=4 * (5 * c + 5), kernel=4 * (2 * c + 10), sources=4 * (3 * c + 10))
+        kernel = "quadfit_gather_tiles<2> (backward, gather pass)"
         shape = "features %dx%dx%d" % (c, h, w)
     else:
         from customnetworklayers_amd.cudaMedian import median_cuda_ext as ext
@@ -161,7 +164,6 @@ def bench_flowaux(args, cfg, d):
         fwd(), bwd()
     torch.cuda.synchronize()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    lib.flowaux_profile(1)  # HIP events around the dominant kernel, on the stream it is launched on
     t0 = time.perf_counter()
     for e in ev:  # events on the stream the kernels are launched on (torch's current stream)
         e[0].record(); fwd(); e[1].record(); bwd(); e[2].record()
@@ -169,10 +171,20 @@ def bench_flowaux(args, cfg, d):
     elapsed = time.perf_counter() - t0
     f_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     b_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
-    tot_ms, launches = ctypes.c_double(0), ctypes.c_int(0)
-    lib.flowaux_profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
-    lib.flowaux_profile(0)
-    k_ms = tot_ms.value / max(launches.value, 1)
+
+    def kernel_ms(which):
+        """HIP events around one kernel of the backward pass, on the stream it is launched on; steps outside the timed region."""
+        lib.flowaux_profile(which)
+        for _ in range(args.steps):
+            bwd()
+        torch.cuda.synchronize()
+        tot_ms, launches = ctypes.c_double(0), ctypes.c_int(0)
+        lib.flowaux_profile_read(ctypes.byref(tot_ms), ctypes.byref(launches))
+        lib.flowaux_profile(0)
+        return tot_ms.value / max(launches.value, 1), launches.value
+
+    k_ms, launches_timed = kernel_ms(2 if cfg["kind"] == "quadfit" else 1)
+    src_ms = kernel_ms(1)[0] if cfg["kind"] == "quadfit" else None
     value = px / (elapsed / args.steps) / 1e6
     achieved = bpp["kernel"] * px / (k_ms * 1e-3) / 1e9 if k_ms > 0 else 0.0
     out = {
@@ -187,8 +199,14 @@ def bench_flowaux(args, cfg, d):
                       "backward_GBps": round(bpp["backward"] * px / (b_ms * 1e-3) / 1e9, 1)},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
-                     "bytes_per_launch": bpp["kernel"] * px, "avg_launch_ms": round(k_ms, 5), "launches_timed": launches.value},
+                     "bytes_per_launch": bpp["kernel"] * px, "avg_launch_ms": round(k_ms, 5), "launches_timed": launches_timed,
+                     "counters_from": COUNTERS[args.config]["files"] + " @ " + COUNTERS[args.config]["commit"]},
     }
+    if src_ms is not None:  # the second kernel of the backward pass
+        cnt = COUNTERS[args.config]
+        out["roofline"]["per_source_pass"] = {
+            "kernel": "quadfit_sources_resident<32,true>", "avg_launch_ms": round(src_ms, 5), "bytes_per_launch": bpp["sources"] * px,
+            "achieved": round(bpp["sources"] * px / (src_ms * 1e-3) / 1e9, 1), "traffic": cnt["sources_traffic"]}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = flowaux_cpu_baseline(cfg, d)
     print(json.dumps(out))

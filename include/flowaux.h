@@ -64,8 +64,9 @@ int medimax_backward(const float* vol, const float* gin, float* gvol, int n, int
                      void* stream);
 
 /* Measurement hooks, as tvinpaint_profile / tvinpaint_profile_read: with profiling on, every backward
- * call brackets its dominant kernel (the per-source pass of the quadratic fit, the whole-histogram kernel of
- * the median) with a HIP event pair on the caller's stream; _read waits for them and returns their total. */
+ * call brackets one kernel with a HIP event pair on the caller's stream; _read waits for them and returns their
+ * total.  enable = 1: the per-source pass of the quadratic fit, the whole-histogram kernel of the median;
+ * enable = 2: the gather pass of the quadratic fit (the median as for 1); 0 switches the events off. */
 int flowaux_profile(int enable);
 int flowaux_profile_read(double* total_ms, int* launches);
 

@@ -65,7 +65,9 @@ def check_quadfit(qf, o, d, name):
 @pytest.mark.parametrize("n,c,h,w,fc", [
     (1, 4, 9, 11, 2),       # tiny
     (2, 5, 33, 70, 3),      # odd sizes, three flow channels, two samples
-    (1, 32, 64, 128, 2),    # many channels
+    (1, 32, 64, 128, 2),    # many channels: the backward pass keeps every channel's taps in registers, all 32 in use
+    (1, 31, 37, 140, 2),    # one channel short of that
+    (1, 33, 40, 130, 2),    # one channel too many for it: the second map is read twice
     (3, 7, 17, 300, 2),     # several blocks per row
     (1, 1, 1, 1, 2),        # a single pixel
     (1, 3, 1, 200, 2),      # a single row
@@ -76,7 +78,7 @@ def test_quadfit_random_inputs_match_oracle(qf, flowaux_oracle, n, c, h, w, fc):
     check_quadfit(qf, flowaux_oracle, d, "random %dx%dx%dx%d fc=%d" % (n, c, h, w, fc))
 
 
-@pytest.mark.parametrize("n,c,h,w", [(2, 8, 96, 160), (1, 16, 50, 333)])
+@pytest.mark.parametrize("n,c,h,w", [(2, 8, 96, 160), (1, 16, 50, 333), (1, 32, 70, 200)])
 def test_quadfit_warped_features_match_oracle(qf, flowaux_oracle, n, c, h, w):
     d = workloads.quadfit_inputs(n, c, h, w, seed=3)
     out = check_quadfit(qf, flowaux_oracle, d, "warped %dx%dx%dx%d" % (n, c, h, w))
@@ -93,10 +95,21 @@ def test_quadfit_one_pixel_per_lane_kernels(qf, flowaux_oracle, n, c, h, w, monk
     check_quadfit(qf, flowaux_oracle, workloads.quadfit_inputs(n, c, h, w, seed=32), "px path warped")
 
 
-def test_quadfit_flow_that_scatters_the_tile(qf, flowaux_oracle):
-    # a flow that varies by tens of pixels inside one 64 x 8 tile: most taps fall outside the LDS window
-    d = random_quadfit(1, 4, 64, 256, seed=33, amp=40.0)
-    check_quadfit(qf, flowaux_oracle, d, "scattered")
+@pytest.mark.parametrize("c", [4, 32, 40])
+def test_quadfit_flow_that_scatters_the_tile(qf, flowaux_oracle, c):
+    # a flow that varies by tens of pixels inside one tile: most taps fall outside the LDS window
+    d = random_quadfit(1, c, 64, 256, seed=33, amp=40.0)
+    check_quadfit(qf, flowaux_oracle, d, "scattered, %d channels" % c)
+
+
+@pytest.mark.parametrize("n,c,h,w", [(2, 6, 40, 90), (1, 32, 33, 150)])
+def test_quadfit_backward_that_reads_the_second_map_twice(qf, flowaux_oracle, n, c, h, w, monkeypatch):
+    # INPAINT_QUADFIT_PATH=reread: the backward kernel of more than 32 channels, forced for fewer
+    monkeypatch.setenv("INPAINT_QUADFIT_PATH", "reread")
+    from customnetworklayers_amd._lib import reload_env
+    reload_env()
+    check_quadfit(qf, flowaux_oracle, random_quadfit(n, c, h, w, seed=41 + c), "reread random %dx%dx%dx%d" % (n, c, h, w))
+    check_quadfit(qf, flowaux_oracle, workloads.quadfit_inputs(n, c, h, w, seed=42), "reread warped")
 
 
 def test_quadfit_non_finite_displacements_count_as_outside(qf, flowaux_oracle):
