@@ -29,7 +29,7 @@ COUNTERS = {
     2: dict(traffic=(2 * 174492 + 148961) * 1024, step=(2 * 13776080 + 14750333) * 1024, lds=688464 * 64 * 8, rocprof_ms=0.12699,
             files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="2207eb7"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
-            files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="HEADREV"),
+            files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
     6: dict(traffic=(2 * 131080 + 247100) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
 }
 MEASURED_TRAFFIC_BYTES = {k: v["traffic"] for k, v in COUNTERS.items()}
