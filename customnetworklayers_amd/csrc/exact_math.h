@@ -52,4 +52,20 @@ __device__ __forceinline__ float exact_sqrt(float x) {
   return out;
 }
 
+// Values of lanes outside the image read as +0: inside(v) is v where `ok` held and +0 elsewhere, bit for bit what
+// `ok ? v : 0.f` gives.  The loaded bits are ANDed with an all-ones / all-zeros word whose origin the empty asm hides
+// from the optimizer; written as a conditional, a group of such values is compiled into a branch that zeroes all of
+// them and then copies all of them.
+struct LaneMask {
+  unsigned keep;
+  __device__ __forceinline__ explicit LaneMask(bool ok) : keep(ok ? 0xffffffffu : 0u) { asm("" : "+v"(keep)); }
+  __device__ __forceinline__ float operator()(float v) const { return __uint_as_float(__float_as_uint(v) & keep); }
+};
+// The same values from the plain conditional, for the kernels in which the AND form costs registers they do not have.
+struct LaneSelect {
+  bool ok;
+  __device__ __forceinline__ explicit LaneSelect(bool ok_) : ok(ok_) {}
+  __device__ __forceinline__ float operator()(float v) const { return ok ? v : 0.f; }
+};
+
 }  // namespace inpaint

@@ -126,15 +126,16 @@ __global__ __launch_bounds__(256) void tgv_forward_strip(
   auto absorb = [&](int k, FwdRow<C>& o) {
     const int h = g.hs - 1 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
+    const inpaint::LaneMask inside(ok);
     o.rc1 = rcp_refined(1.f + o.c);
     o.wxs = (ok && rmask) ? o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-    o.bxs = ok ? o.bxs : 0.f;
-    o.bys = ok ? o.bys : 0.f;
+    o.bxs = inside(o.bxs);
+    o.bys = inside(o.bys);
 #pragma unroll
     for (int ch = 0; ch < C; ch++)
 #pragma unroll
-      for (int v = 0; v < 3; v++) o.y[v][ch] = ok ? o.y[v][ch] : 0.f;
+      for (int v = 0; v < 3; v++) o.y[v][ch] = inside(o.y[v][ch]);
   };
 
   float upFa[C], upG1y[C], upG2y[C];  // terms handed down to the row below
@@ -321,6 +322,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
   auto absorb = [&](int k, Fwd2Row<C>& o) {
     const int h = g.hs - 2 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
+    const inpaint::LaneMask inside(ok);
     if (RING) {  // o.y holds x05[j-1], o.x holds x05[j-2]
       const float rc1 = rcp_refined(1.f + o.c);
 #pragma unroll
@@ -339,12 +341,12 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     }
     o.wxs = (ok && rmask) ? o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-    o.bxs = ok ? o.bxs : 0.f;
-    o.bys = ok ? o.bys : 0.f;
+    o.bxs = inside(o.bxs);
+    o.bys = inside(o.bys);
 #pragma unroll
     for (int ch = 0; ch < C; ch++)
 #pragma unroll
-      for (int v = 0; v < 3; v++) o.y[v][ch] = ok ? o.y[v][ch] : 0.f;
+      for (int v = 0; v < 3; v++) o.y[v][ch] = inside(o.y[v][ch]);
   };
 
   struct Tri {  // the six products of one triangle (TGV.cu:1669-1684)
@@ -630,34 +632,35 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
   auto absorb = [&](int k, AdjRow<C>& o) {
     const int h = g.hs - 1 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
-    o.c = ok ? o.c : 0.f;
+    const inpaint::LaneMask inside(ok);
+    o.c = inside(o.c);
     o.rc1 = rcp_refined(1.f + o.c);
     o.opc_d = 1. + (double)o.c;
     o.wxs = (ok && rmask) ? o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-    o.bxs = ok ? o.bxs : 0.f;
-    o.bys = ok ? o.bys : 0.f;
+    o.bxs = inside(o.bxs);
+    o.bys = inside(o.bys);
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.y[0][ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+      const float xa = inside(o.xa[ch]), xb = inside(o.y[0][ch]), bv = inside(o.bb[ch]);
       if (ADJ) {
         const float xn = tvstrip::prox_huber1(xa, o.c, o.rc1, bv);
         const float xo = ADJ == 2 ? xb : tvstrip::prox_huber1(xb, o.c, o.rc1, bv);
         o.y[0][ch] = xn + t * (xn - xo);  // TGV.cu:1773
 #pragma unroll
         for (int v = 1; v < 3; v++) {
-          const float xv = ok ? o.y[v][ch] : 0.f, xp = ok ? o.yp[v - 1][ch] : 0.f;
+          const float xv = inside(o.y[v][ch]), xp = inside(o.yp[v - 1][ch]);
           o.y[v][ch] = xv + t * (xv - xp);  // TGV.cu:1686-1690
         }
       } else {
         o.y[0][ch] = END ? xb : tvstrip::rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
-        o.y[1][ch] = ok ? o.y[1][ch] : 0.f;
-        o.y[2][ch] = ok ? o.y[2][ch] : 0.f;
+        o.y[1][ch] = inside(o.y[1][ch]);
+        o.y[2][ch] = inside(o.y[2][ch]);
       }
       o.xa[ch] = xa;
       o.bb[ch] = bv;
 #pragma unroll
-      for (int v = 0; v < 3; v++) o.g[v][ch] = ok ? o.g[v][ch] : 0.f;
+      for (int v = 0; v < 3; v++) o.g[v][ch] = inside(o.g[v][ch]);
     }
   };
 
@@ -1010,16 +1013,17 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
   auto absorb = [&](int k, Adj2Row<C>& o) {
     const int h = g.hs - 2 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
-    o.c = ok ? o.c : 0.f;
+    const inpaint::LaneMask inside(ok);
+    o.c = inside(o.c);
     const float rc1 = rcp_refined(1.f + o.c);
     const double opc_d = 1. + (double)o.c;
     o.wxs = (ok && rmask) ? o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-    o.bxs = ok ? o.bxs : 0.f;
-    o.bys = ok ? o.bys : 0.f;
+    o.bxs = inside(o.bxs);
+    o.bys = inside(o.bys);
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      const float xa = ok ? o.xa0[ch] : 0.f, xb = ok ? o.xb0[ch] : 0.f, xc = ok ? o.yB[0][ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+      const float xa = inside(o.xa0[ch]), xb = inside(o.xb0[ch]), xc = inside(o.yB[0][ch]), bv = inside(o.bb[ch]);
       o.yA[0][ch] = tvstrip::rebuild_y_fast(bv, xa, xb, o.c, rc1, opc_d, tA);
       o.yB[0][ch] = BEND ? xc : tvstrip::rebuild_y_fast(bv, xb, xc, o.c, rc1, opc_d, tB);
       o.xa0[ch] = xa;
@@ -1027,11 +1031,11 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
       o.bb[ch] = bv;
 #pragma unroll
       for (int v = 1; v < 3; v++) {
-        o.yA[v][ch] = ok ? o.yA[v][ch] : 0.f;
-        o.yB[v][ch] = ok ? o.yB[v][ch] : 0.f;
+        o.yA[v][ch] = inside(o.yA[v][ch]);
+        o.yB[v][ch] = inside(o.yB[v][ch]);
       }
 #pragma unroll
-      for (int v = 0; v < 3; v++) o.g[v][ch] = ok ? o.g[v][ch] : 0.f;
+      for (int v = 0; v < 3; v++) o.g[v][ch] = inside(o.g[v][ch]);
     }
   };
 
@@ -1676,16 +1680,17 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     auto absorb = [&](int k, Adj2ARow<C>& o) {
       const int h = g.hs - 2 + k;
       const bool ok = g.col_ok && h >= 0 && h < H;
-      o.c = ok ? o.c : 0.f;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
       const float rc1 = rcp_refined(1.f + o.c);
       const double opc_d = 1. + (double)o.c;
       o.wxs = (ok && rmask) ? o.wxs : 0.f;
       o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-      o.bxs = ok ? o.bxs : 0.f;
-      o.bys = ok ? o.bys : 0.f;
+      o.bxs = inside(o.bxs);
+      o.bys = inside(o.bys);
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
-        const float xa = ok ? o.xa0[ch] : 0.f, xb = ok ? o.xb0[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+        const float xa = inside(o.xa0[ch]), xb = inside(o.xb0[ch]), bv = inside(o.bb[ch]);
         if (TRUE_ADJ) {
           const float pa = tvstrip::prox_huber1(xa, o.c, rc1, bv), pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
           o.yA[0][ch] = pa + tA * (pa - pb);  // TGV.cu:1773
@@ -1696,11 +1701,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
         o.bb[ch] = bv;
 #pragma unroll
         for (int v = 1; v < 3; v++) {
-          const float xv = ok ? o.yA[v][ch] : 0.f;
-          o.yA[v][ch] = TRUE_ADJ ? xv + tA * (xv - (ok ? o.pv[v - 1][ch] : 0.f)) : xv;  // TGV.cu:1686-1690
+          const float xv = inside(o.yA[v][ch]);
+          o.yA[v][ch] = TRUE_ADJ ? xv + tA * (xv - inside(o.pv[v - 1][ch])) : xv;  // TGV.cu:1686-1690
         }
 #pragma unroll
-        for (int v = 0; v < 3; v++) o.g[v][ch] = ok ? o.g[v][ch] : 0.f;
+        for (int v = 0; v < 3; v++) o.g[v][ch] = inside(o.g[v][ch]);
       }
     };
     float dnA[C][6];
@@ -1819,16 +1824,17 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     auto absorb = [&](int k, Adj2BRow<C>& o) {
       const int h = g.hs - 2 + k;
       const bool ok = g.col_ok && h >= 0 && h < H;
-      o.c = ok ? o.c : 0.f;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
       const float rc1 = rcp_refined(1.f + o.c);
       const double opc_d = 1. + (double)o.c;
       o.wxs = (ok && rmask) ? o.wxs : 0.f;
       o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-      o.bxs = ok ? o.bxs : 0.f;
-      o.bys = ok ? o.bys : 0.f;
+      o.bxs = inside(o.bxs);
+      o.bys = inside(o.bys);
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
-        const float xb = ok ? o.xb0[ch] : 0.f, xc = ok ? o.yB[0][ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+        const float xb = inside(o.xb0[ch]), xc = inside(o.yB[0][ch]), bv = inside(o.bb[ch]);
         if (TRUE_ADJ) {
           const float pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
           const float pc = BEND ? xc : tvstrip::prox_huber1(xc, o.c, rc1, bv);
@@ -1840,8 +1846,8 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
         o.bb[ch] = bv;
 #pragma unroll
         for (int v = 1; v < 3; v++) {
-          const float xv = ok ? o.yB[v][ch] : 0.f;
-          o.yB[v][ch] = TRUE_ADJ ? xv + tB * (xv - (ok ? o.pv[v - 1][ch] : 0.f)) : xv;
+          const float xv = inside(o.yB[v][ch]);
+          o.yB[v][ch] = TRUE_ADJ ? xv + tB * (xv - inside(o.pv[v - 1][ch])) : xv;
         }
       }
     };

@@ -599,8 +599,8 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
     return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
   if (n > 65535 || (ih + TH - 1) / TH > 65535)
     return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
-  if ((long long)ih * iw >= (1ll << 30))  // the strip kernels address a plane with 32-bit byte offsets
-    return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^30", (long long)ih * iw);
+  if ((long long)ih * iw >= (1ll << 29))  // the strip kernels address two planes of a tensor with one 32-bit byte offset
+    return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^29", (long long)ih * iw);
   if ((int)std::floor(std::sqrt((double)its)) > kMaxCheckpoints)
     return fail(INPAINT_ERR_ITS, "its=%d needs more than %d checkpoints", its, kMaxCheckpoints);
   return 0;

@@ -626,14 +626,15 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
   auto absorb = [&](int k, AdjRow<C>& o) {
     const int h = g.hs - 1 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
-    o.c = ok ? o.c : 0.f;
+    const inpaint::LaneMask inside(ok);
+    o.c = inside(o.c);
     o.rc1 = rcp_refined(1.f + o.c);
     o.opc_d = 1. + (double)o.c;
     o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.y[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+      const float xa = inside(o.xa[ch]), xb = inside(o.y[ch]), bv = inside(o.bb[ch]);
       if (TRUE_ADJ) {
         const float xn = prox_huber1(xa, o.c, o.rc1, bv);
         const float xo = END ? xb : prox_huber1(xb, o.c, o.rc1, bv);
@@ -641,7 +642,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
       } else {
         o.y[ch] = END ? xb : rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, t);
       }
-      o.g[ch] = ok ? o.g[ch] : 0.f;
+      o.g[ch] = inside(o.g[ch]);
       o.xa[ch] = xa;
       o.bb[ch] = bv;
     }
@@ -845,16 +846,17 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
   const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
   const float *const gci_p = gc_in + poff, *const gwxi_p = gwx_in + poff, *const gwyi_p = gwy_in + poff;
   float *const gco_p = gc + poff, *const gwxo_p = gwx + poff, *const gwyo_p = gwy + poff;
-  const float *xa_p[C], *xb_p[C], *xc_p[C], *b_p[C], *g_p[C], *gxi_p[C], *gbi_p[C];
-  float *g05o_p[C], *gxm_p[C], *gbo_p[C], *gxf_p[C];
+  // One base pointer per tensor (the sample's first channel); channel ch sits chs[ch] bytes further (a 32-bit
+  // offset: the host refuses planes of 2^29 pixels and more).  A pointer pair per tensor AND channel does not fit the
+  // scalar registers: the compiler parks the surplus in lanes of a vector register and re-reads it at every row.
+  const size_t q0 = (size_t)g.n * Ct * HW;
+  const float *const xa_p = x05a + q0, *const xb_p = x05b + q0, *const xc_p = x05c + q0;  // x05c: x05[j-2], or the checkpoint y when BEND
+  const float *const b_p = b + q0, *const g_p = g05_in + q0, *const gxi_p = gxk + q0, *const gbi_p = gb_in + q0;
+  float *const g05o_p = g05_out + q0, *const gxm_p = gxk_m1 + q0, *const gbo_p = gb + q0;
+  float *const gxf_p = FINAL ? gx_final + q0 : nullptr;
+  unsigned chs[C];
 #pragma unroll
-  for (int ch = 0; ch < C; ch++) {
-    const size_t q = ((size_t)g.n * Ct + ch) * HW;
-    xa_p[ch] = x05a + q; xb_p[ch] = x05b + q; xc_p[ch] = x05c + q;  // x05c: x05[j-2], or the checkpoint y when BEND
-    b_p[ch] = b + q; g_p[ch] = g05_in + q; gxi_p[ch] = gxk + q; gbi_p[ch] = gb_in + q;
-    g05o_p[ch] = g05_out + q; gxm_p[ch] = gxk_m1 + q; gbo_p[ch] = gb + q;
-    gxf_p[ch] = FINAL ? gx_final + q : nullptr;
-  }
+  for (int ch = 0; ch < C; ch++) chs[ch] = (unsigned)ch * (4u * (unsigned)HW);
   const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
   const int o_lo = g.hs, o_hi = g.hs + Reff - 1;                       // output rows
 
@@ -871,13 +873,13 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     in.wys = ldg(wy_p, off_w);
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      in.xa[ch] = ldg(xa_p[ch], off);
-      in.xb[ch] = ldg(xb_p[ch], off);
-      in.yB[ch] = ldg(xc_p[ch], off);
-      in.bb[ch] = ldg(b_p[ch], off);
-      in.g[ch] = ldg(g_p[ch], off);
-      in.gx_i[ch] = ldg(gxi_p[ch], off_a);
-      in.gb_i[ch] = ldg(gbi_p[ch], off_o);
+      in.xa[ch] = ldg(xa_p, off + chs[ch]);
+      in.xb[ch] = ldg(xb_p, off + chs[ch]);
+      in.yB[ch] = ldg(xc_p, off + chs[ch]);
+      in.bb[ch] = ldg(b_p, off + chs[ch]);
+      in.g[ch] = ldg(g_p, off + chs[ch]);
+      in.gx_i[ch] = ldg(gxi_p, off_a + chs[ch]);
+      in.gb_i[ch] = ldg(gbi_p, off_o + chs[ch]);
     }
     in.gc_i = ldg(gci_p, off_o);
     in.gwx_i = ldg(gwxi_p, off_o);
@@ -886,14 +888,15 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
   auto absorb = [&](int k, Adj2Row<C>& o) {
     const int h = g.hs - 2 + k;
     const bool ok = g.col_ok && h >= 0 && h < H;
-    o.c = ok ? o.c : 0.f;
+    const std::conditional_t<BEND, inpaint::LaneSelect, inpaint::LaneMask> inside(ok);  // (the segment-end pair is short of registers)
+    o.c = inside(o.c);
     o.rc1 = rcp_refined(1.f + o.c);
     o.opc_d = 1. + (double)o.c;
     o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
     o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
-      const float xa = ok ? o.xa[ch] : 0.f, xb = ok ? o.xb[ch] : 0.f, xc = ok ? o.yB[ch] : 0.f, bv = ok ? o.bb[ch] : 0.f;
+      const float xa = inside(o.xa[ch]), xb = inside(o.xb[ch]), xc = inside(o.yB[ch]), bv = inside(o.bb[ch]);
       if (TRUE_ADJ) {
         const float pa = prox_huber1(xa, o.c, o.rc1, bv), pb = prox_huber1(xb, o.c, o.rc1, bv);
         const float pc = BEND ? xc : prox_huber1(xc, o.c, o.rc1, bv);
@@ -905,7 +908,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
         o.yA[ch] = rebuild_from(ra, rb, tA);
         o.yB[ch] = BEND ? xc : rebuild_from(rb, rebuild_pieces(bv, xc, o.c, o.rc1, o.opc_d), tB);
       }
-      o.g[ch] = ok ? o.g[ch] : 0.f;
+      o.g[ch] = inside(o.g[ch]);
       o.xa[ch] = xa;
       o.xb[ch] = xb;
       o.bb[ch] = bv;
@@ -1045,14 +1048,14 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
           gcB += gc_add;
           const float gbv = pgb[ch] + gb_add;
           if (store_lane) {
-            if (FINAL) stg(gxf_p[ch], roffB, df);
-            stg(gxm_p[ch], roffB, gxm);
-            stg(g05o_p[ch], roffB, g05v);
+            if (FINAL) stg(gxf_p, roffB + chs[ch], df);
+            stg(gxm_p, roffB + chs[ch], gxm);
+            stg(g05o_p, roffB + chs[ch], g05v);
             if (BEND) {  // segment flush, fused (TV.cu:178-218)
               seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
-              stg(gbo_p[ch], roffB, 0.f);
+              stg(gbo_p, roffB + chs[ch], 0.f);
             } else {
-              stg(gbo_p[ch], roffB, gbv);
+              stg(gbo_p, roffB + chs[ch], gbv);
             }
           }
         }

@@ -79,10 +79,10 @@ def test_planes_beyond_32_bit_offsets_are_refused():
     from customnetworklayers_amd._lib import last_error, lib
 
     p = ctypes.c_void_p(16)  # never dereferenced: the size check comes first
-    assert lib.tvinpaint_forward(p, p, p, p, p, p, 1, 1, 32768, 32768, 4, 0, None) == 2
-    assert "2^30" in last_error()
-    assert lib.tgvinpaint_forward(p, p, p, p, p, p, 1, 1, 32768, 32768, 4, 0, None) == 2
-    assert lib.tvinpaint_forward_noalloc(p, p, p, p, p, p, 1, 1, 32768, 32768, 4, None) == 2
+    assert lib.tvinpaint_forward(p, p, p, p, p, p, 1, 1, 16384, 32768, 4, 0, None) == 2
+    assert "2^29" in last_error()
+    assert lib.tgvinpaint_forward(p, p, p, p, p, p, 1, 1, 16384, 32768, 4, 0, None) == 2
+    assert lib.tvinpaint_forward_noalloc(p, p, p, p, p, p, 1, 1, 16384, 32768, 4, None) == 2
 
 
 def test_setup_py_builds_everything_from_a_clean_copy(tmp_path):
