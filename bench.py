@@ -24,10 +24,10 @@ HBM_PEAK_GBS = 8000.0
 #             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
 #   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
 COUNTERS = {
-    1: dict(traffic=(2 * 86991 + 67917) * 1024, step=(2 * 6743585 + 6203882) * 1024, lds=0, rocprof_ms=0.05829,
-            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="2207eb7"),
-    2: dict(traffic=(2 * 174492 + 148961) * 1024, step=(2 * 13776080 + 14750333) * 1024, lds=688464 * 64 * 8, rocprof_ms=0.12699,
-            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="2207eb7"),
+    1: dict(traffic=(2 * 87029 + 68278) * 1024, step=(2 * 6746728 + 6225147) * 1024, lds=0, rocprof_ms=0.05478,
+            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="60960d4"),
+    2: dict(traffic=(2 * 174356 + 149259) * 1024, step=(2 * 13756219 + 14751401) * 1024, lds=688464 * 64 * 8, rocprof_ms=0.12652,
+            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="60960d4"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
     6: dict(traffic=(2 * 131080 + 247100) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
