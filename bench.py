@@ -505,8 +505,8 @@ def main():
                     help="configs 1 and 2: time the opt-in corrected gradient instead of the reference's (not the headline)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus %d is not supported (samples shard trivially, "
-              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the samples of a batch are "
+              "independent: more GPUs would each take a share of them, with no communication)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
