@@ -1398,7 +1398,9 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
     float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
-  constexpr int kHand = 7 * C + 5;  // floats step A hands to step B per row and lane
+  // floats step A hands to step B per row and lane: its results (7C + 5) and the row's inputs that both steps need
+  // (c, four weights, b and the u of x05[j-1]: 2C + 5), which B would otherwise read from memory a second time
+  constexpr int kHand = 9 * C + 10;
 #ifndef TGV_ROWS_PER_BARRIER
 #define TGV_ROWS_PER_BARRIER 2
 #endif
@@ -1698,6 +1700,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
           o.yA[0][ch] = tvstrip::rebuild_y_fast(bv, xa, xb, o.c, rc1, opc_d, tA);
         }
         o.xa0[ch] = xa;
+        o.xb0[ch] = xb;
         o.bb[ch] = bv;
 #pragma unroll
         for (int v = 1; v < 3; v++) {
@@ -1749,6 +1752,17 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       slot[7 * C + 2][g.lane] = accA.gwx1;
       slot[7 * C + 3][g.lane] = accA.gwy0;
       slot[7 * C + 4][g.lane] = accA.gwy1;
+      // row k's inputs as A absorbed them (zero outside the image): B takes them from here
+      slot[7 * C + 5][g.lane] = cur.c;
+      slot[7 * C + 6][g.lane] = cur.wxs;
+      slot[7 * C + 7][g.lane] = cur.wys;
+      slot[7 * C + 8][g.lane] = cur.bxs;
+      slot[7 * C + 9][g.lane] = cur.bys;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        slot[7 * C + 10 + ch][g.lane] = cur.bb[ch];
+        slot[8 * C + 10 + ch][g.lane] = cur.xb0[ch];
+      }
     };
 
     // A publishes kP rows per barrier: the barrier after row k with k % kP == kP - 1 makes rows k-kP+1 .. k visible to
@@ -1800,17 +1814,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     if (klast % kP != kP - 1) lds_barrier();  // the last rows have not been published yet
   } else {
     // ---------------------------------- step B ----------------------------------
-    auto load_row = [&](int k, Adj2BRow<C>& in) {
+    auto load_row = [&](int k, Adj2BRow<C>& in) {  // (c, the weights, b and x05[j-1]'s u come from step A, see absorb)
       unsigned off, off_w;
       row_offsets(k, off, off_w);
-      in.c = ldg(cf_p, off);
-      in.wxs = ldg(wx_p, off_w);
-      in.wys = ldg(wy_p, off_w);
-      in.bxs = ldg(bx_p, off_w);
-      in.bys = ldg(by_p, off_w);
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
-        in.xb0[ch] = ldg(xb_p[0][ch], off);
         in.yB[1][ch] = ldg(xb_p[1][ch], off);
         in.yB[2][ch] = ldg(xb_p[2][ch], off);
         in.yB[0][ch] = ldg(xc_p[ch], off);
@@ -1818,23 +1826,23 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
           in.pv[0][ch] = ldg(pv_p[1][0][ch], off);
           in.pv[1][ch] = ldg(pv_p[1][1][ch], off);
         }
-        in.bb[ch] = ldg(b_p[ch], off);
       }
     };
-    auto absorb = [&](int k, Adj2BRow<C>& o) {
+    auto absorb = [&](int k, Adj2BRow<C>& o) {  // after await(k): row k's slot is visible
       const int h = g.hs - 2 + k;
       const bool ok = g.col_ok && h >= 0 && h < H;
       const inpaint::LaneMask inside(ok);
-      o.c = inside(o.c);
+      const float (*slot)[64] = hand[k % (2 * kP)];
+      o.c = slot[7 * C + 5][g.lane];  // already zero outside the image
+      o.wxs = slot[7 * C + 6][g.lane];
+      o.wys = slot[7 * C + 7][g.lane];
+      o.bxs = slot[7 * C + 8][g.lane];
+      o.bys = slot[7 * C + 9][g.lane];
       const float rc1 = rcp_refined(1.f + o.c);
       const double opc_d = 1. + (double)o.c;
-      o.wxs = (ok && rmask) ? o.wxs : 0.f;
-      o.wys = (ok && h < H - 1) ? o.wys : 0.f;
-      o.bxs = inside(o.bxs);
-      o.bys = inside(o.bys);
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
-        const float xb = inside(o.xb0[ch]), xc = inside(o.yB[0][ch]), bv = inside(o.bb[ch]);
+        const float xb = slot[8 * C + 10 + ch][g.lane], xc = inside(o.yB[0][ch]), bv = slot[7 * C + 10 + ch][g.lane];
         if (TRUE_ADJ) {
           const float pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
           const float pc = BEND ? xc : tvstrip::prox_huber1(xc, o.c, rc1, bv);
