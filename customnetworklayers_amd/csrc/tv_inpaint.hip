@@ -784,6 +784,43 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
+// Rows per strip of the two-wavefront pair kernel.  Its workgroups (one strip each) are resident four per CU, so a
+// launch runs in ceil(workgroups / (4 * CUs)) rounds of (R + pipeline rows + start-up) row steps each; the strip
+// height that minimises rounds x steps is taken.
+int pair_split_rows(int n, int ih, int iw) {
+  if (knobs().tv_adj_rows > 0) return knobs().tv_adj_rows;
+  const long long cap = 4ll * compute_unit_count();
+  const long long sx = (iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols;
+  int best = 16;
+  long long best_cost = -1;
+  for (int R = 8; R <= 64; R++) {
+    const long long wg = sx * ((ih + R - 1) / R) * n;
+    const long long cost = ((wg + cap - 1) / cap) * (R + 7);
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = R;
+    }
+  }
+  return best;
+}
+
+// 3 and 4 channels: the two steps of a pair in two wavefronts of a workgroup (one strip per 128-thread workgroup)
+template <int C, bool BEND, bool TRUE_ADJ>
+void launch_adjoint_pair_split(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                               const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
+                               float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
+  auto kern = gx_final ? tvstrip::tv_adjoint_strip2w<C, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2w<C, BEND, false, TRUE_ADJ>;
+  const int R = pair_split_rows(s.n, s.ih, s.iw);
+  const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
+  const long long strips = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(128);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
+                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+                     s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
+}
+
 // (one group only: a pair adds step A's and step B's terms of its channels back to back, which is the reference's
 // order of summation only when the launch holds every channel)
 template <bool BEND, bool TRUE_ADJ = false>
@@ -792,17 +829,22 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const flo
                          const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   if (s.ic == 1)
     launch_adjoint_pair_strip<1, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
-  else
+  else if (s.ic == 2)
     launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 3)
+    launch_adjoint_pair_split<3, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else
+    launch_adjoint_pair_split<4, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
   s.accb_cur = 1 - s.accb_cur;
 }
 
 bool adjoint_pairs(const Slot& s) {
   if (!knobs().tv_fuse_adj) return false;
-  // with 3 or 4 channels the pair kernel needs more than 256 registers (one wavefront per SIMD), and pairs over
-  // channel groups would sum the shared accumulators in another order; those take the one-step kernels
-  return forward_pairs(s) && s.ic <= 2;
+  // one channel group only (up to 4 channels): pairs over channel groups would sum the shared accumulators in
+  // another order; more channels take the one-step kernel, group after group.  With 3 or 4 channels the two steps
+  // need more than one wavefront's registers and run in two wavefronts.
+  return forward_pairs(s) && s.ic <= kGroup;
 }
 
 // -------------------------------------------------------------------------------------------------

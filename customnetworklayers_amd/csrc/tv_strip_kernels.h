@@ -1119,4 +1119,402 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
   }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Two adjoint steps per launch in TWO wavefronts of a 128-thread workgroup (one strip per workgroup),
+// for the channel counts whose two steps do not fit one wavefront's registers (3 and 4).  Same
+// arithmetic, same rows and lanes as tv_adjoint_strip2: wavefront 0 runs step A (iteration j) on row
+// k of the strip, wavefront 1 runs step B (iteration j-1) on row k-1.  What A computes for a row and
+// B continues -- g05[j] and the partial g_x[j] per channel, the per-channel gb and the three shared
+// accumulators with A's terms added (all channels of A first, then all channels of B: the reference's
+// order) -- travels through LDS together with the row's inputs both steps need (c, 1/(1+c), the
+// scaled weights, b and x05[j-1]), 5C + 7 floats per lane and row.  A publishes kP rows per barrier
+// into 2 kP slots; B works on the kP rows before them.  Both wavefronts pass the same number of
+// barriers, ceil((klast + 1) / kP).
+// -------------------------------------------------------------------------------------------------
+template <int C>
+struct Adj2wRow {
+  float c, rc1, wxs, wys;
+  float xa[C], xb[C], yA[C], bb[C], g[C], gx_i[C], gb_i[C], gc_i, gwx_i, gwy_i;
+  double opc_d;
+};
+
+template <int C, bool BEND, bool FINAL, bool TRUE_ADJ = false>
+__global__ __launch_bounds__(128) void tv_adjoint_strip2w(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
+    const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
+    const float* __restrict__ x05c, const float* __restrict__ gc_in, float* __restrict__ gc,
+    const float* __restrict__ gb_in, float* __restrict__ gb, const float* __restrict__ gwx_in,
+    float* __restrict__ gwx, const float* __restrict__ gwy_in, float* __restrict__ gwy,
+    const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
+    float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
+  constexpr int kP = 2;                 // rows step A publishes per barrier
+  constexpr int kHand = 5 * C + 7;      // floats per lane and row
+  __shared__ float hand[2 * kP][kHand][64];
+  StripGeom g;
+  if (!strip_geometry_block(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
+  const int role = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront 0: step A, wavefront 1: step B
+  const int Reff = min(R, H - g.hs);
+  const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
+  const size_t HW = (size_t)H * W;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
+  const bool wx_ok = g.col_ok && g.w < W - 1;
+  const double optA = 1. + (double)tA, optB = 1. + (double)tB;
+  const size_t poff = (size_t)g.n * HW;
+  const size_t q0 = (size_t)g.n * Ct * HW;  // one base pointer per tensor, channel ch chs[ch] bytes further
+  unsigned chs[C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) chs[ch] = (unsigned)ch * (4u * (unsigned)HW);
+  const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
+  const int o_lo = g.hs, o_hi = g.hs + Reff - 1;                       // output rows
+
+  constexpr float kGX = TRUE_ADJ ? 1.f : kLocalGXMult, kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
+  struct Tri {  // everything one triangle contributes (see tv_adjoint_strip)
+    float O1, O2, O3, O4, n3, n4, l1, l3, l4, ux, uy;
+  };
+  auto triangle = [&](float yk, float yd, float gk, float gd, float wxv, float wyv, auto end_form) {
+    Tri r;
+    const float yrt = from_right_lane(yk);
+    const float grt = from_right_lane(gk);
+    const float d1 = yk - yd, d2 = yk - yrt;
+    const float a1 = d1 * d1 * wyv;
+    const float a2 = d2 * d2 * wxv;
+    const float hub = exact_sqrt(a2 + a1);
+    const bool act = hub > kDelta;
+    float nom = inpaint::exact_div(kDelta, hub);
+    float denom = inpaint::exact_div(nom, 2.f * hub * hub);
+    nom = act ? nom : 1.f;
+    denom = act ? denom : 0.f;
+    const float gpd = gk - gd, gpr = gk - grt;
+    r.O1 = gpd * (wyv * nom);
+    r.O2 = gpr * (wxv * nom);
+    const float P1 = gpd * wyv * d1;
+    const float P2 = gpr * wxv * d2;
+    const float dd = denom * 2.0f;
+    const float tp = dd * (d1 * wyv + d2 * wxv);  // minus the reference's factor, exactly; O3, O4 carry the sign
+    const float tu = dd * d1 * wyv;
+    const float tl = dd * d2 * wxv;
+    r.O3 = -(P1 * tp);
+    r.O4 = -(P2 * tp);
+    r.n3 = P1 * tu;
+    r.n4 = P2 * tu;
+    r.l1 = from_left_lane(r.O2);
+    r.l3 = from_left_lane(P2 * tl);
+    r.l4 = from_left_lane(P1 * tl);
+    if (!end_form.value) {  // TV.cu:749-769
+      r.ux = kGX * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
+      r.uy = kGX * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
+    } else {  // TV.cu:1019-1037
+      const float ux_a = kGX * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
+      const float uy_a = kGX * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
+      r.ux = act ? ux_a : kGX * d2 * gpr;
+      r.uy = act ? uy_a : kGX * d1 * gpd;
+    }
+    return r;
+  };
+  // pixel update: J^T assembly, momentum adjoint, prox adjoint (TV.cu:668-743, 796-828)
+  auto update = [&](float gk, const Tri& t, float a1_, float a3_, float a4_, float gxv, double opt, float tmom,
+                    float conf, float rc1, float rc2, double opc_d, float bv, float xh, float& df, float& gxm,
+                    float& g05v, float& gc_add, float& gb_add) {
+    float tt = gk;
+    tt -= -a1_;
+    tt -= a3_;
+    tt -= a4_;
+    tt -= -t.l1;
+    tt -= t.l3;
+    tt -= t.l4;
+    tt -= t.O1;
+    tt -= t.O2;
+    tt -= t.O3;
+    tt -= t.O4;
+    df = (float)((double)gxv + opt * (double)tt);
+    df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
+    gxm = -tmom * tt;
+    const float diff = bv - xh;
+    const float sign = (diff < 0) ? -1.f : 1.f;
+    const bool quad = (opc_d >= (double)(sign * diff));
+    const float opc = 1.f + conf;
+    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
+    const float g05_q = div_by(df, opc, rc1);
+    const float gb_q = div_by(df * conf, opc, rc1) * 1.0f;
+    const bool mid = !quad && (conf >= sign * diff);
+    g05v = quad ? g05_q : (mid ? 0.f : df);
+    gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kGC);
+    gb_add = quad ? gb_q : (mid ? df * 1.0f : 0.f);
+  };
+  const std::true_type kYes{};
+  const std::false_type kNo{};
+
+  if (role == 0) {
+    // ---------------------------------- step A ----------------------------------
+    const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
+    const float *const gci_p = gc_in + poff, *const gwxi_p = gwx_in + poff, *const gwyi_p = gwy_in + poff;
+    const float *const xa_p = x05a + q0, *const xb_p = x05b + q0, *const b_p = b + q0, *const g_p = g05_in + q0;
+    const float *const gxi_p = gxk + q0, *const gbi_p = gb_in + q0;
+    auto load_row = [&](int k, Adj2wRow<C>& in) {
+      const int kk = min(k, klast + 1);
+      const int h = g.hs - 2 + kk;
+      const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+      // what a row does not need is read from a row the strip needs anyway (no extra cache lines)
+      const unsigned off_w = (unsigned)min(max(h, 0), h_hi) * W4 + wc;
+      const unsigned off_a = (unsigned)min(max(h, h_lo), h_hi) * W4 + wc;
+      const unsigned off_o = (unsigned)min(max(h, o_lo), o_hi) * W4 + wc;
+      in.c = ldg(cf_p, off);
+      in.wxs = ldg(wx_p, off_w);
+      in.wys = ldg(wy_p, off_w);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.xa[ch] = ldg(xa_p, off + chs[ch]);
+        in.xb[ch] = ldg(xb_p, off + chs[ch]);
+        in.bb[ch] = ldg(b_p, off + chs[ch]);
+        in.g[ch] = ldg(g_p, off + chs[ch]);
+        in.gx_i[ch] = ldg(gxi_p, off_a + chs[ch]);
+        in.gb_i[ch] = ldg(gbi_p, off_o + chs[ch]);
+      }
+      in.gc_i = ldg(gci_p, off_o);
+      in.gwx_i = ldg(gwxi_p, off_o);
+      in.gwy_i = ldg(gwyi_p, off_o);
+    };
+    auto absorb = [&](int k, Adj2wRow<C>& o) {
+      const int h = g.hs - 2 + k;
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
+      o.rc1 = rcp_refined(1.f + o.c);
+      o.opc_d = 1. + (double)o.c;
+      o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
+      o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xa = inside(o.xa[ch]), xb = inside(o.xb[ch]), bv = inside(o.bb[ch]);
+        if (TRUE_ADJ) {
+          const float pa = prox_huber1(xa, o.c, o.rc1, bv), pb = prox_huber1(xb, o.c, o.rc1, bv);
+          o.yA[ch] = pa + tA * (pa - pb);
+        } else {
+          o.yA[ch] = rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, tA);
+        }
+        o.g[ch] = inside(o.g[ch]);
+        o.xa[ch] = xa;
+        o.xb[ch] = xb;
+        o.bb[ch] = bv;
+      }
+    };
+    float dA1[C], dA3[C], dA4[C];  // terms handed down to the row below
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) dA1[ch] = dA3[ch] = dA4[ch] = 0.f;
+
+    auto step = [&](int k, const Adj2wRow<C>& cur, const Adj2wRow<C>& nxt, auto do_a) {
+      const int h = g.hs - 2 + k;
+      const bool in_img = g.col_ok && h >= 0 && h < H;
+      float (*slot)[64] = hand[k % (2 * kP)];
+      float gcv = cur.gc_i, gwxv = cur.gwx_i, gwyv = cur.gwy_i;
+      const float rc2A = rcp_refined((1.f + cur.c) * (1.f + cur.c));
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const Tri t = triangle(cur.yA[ch], nxt.yA[ch], cur.g[ch], nxt.g[ch], cur.wxs, cur.wys, kNo);
+        const float a1_ = dA1[ch], a3_ = dA3[ch], a4_ = dA4[ch];
+        dA1[ch] = t.O1; dA3[ch] = t.n3; dA4[ch] = t.n4;
+        float nG = 0.f, ngxm = 0.f, ngb = cur.gb_i[ch];
+        if (do_a.value) {
+          if (g.w < W - 1) gwxv = gwxv - t.ux;
+          if (h < H - 1) gwyv = gwyv - t.uy;
+          float df, gxm, g05v, gc_add, gb_add;
+          update(cur.g[ch], t, a1_, a3_, a4_, cur.gx_i[ch], optA, tA, cur.c, cur.rc1, rc2A, cur.opc_d, cur.bb[ch],
+                 cur.xa[ch], df, gxm, g05v, gc_add, gb_add);
+          gcv += gc_add;
+          ngb += gb_add;
+          nG = in_img ? g05v : 0.f;  // B reads zero padding outside the image
+          ngxm = gxm;
+        }
+        slot[ch][g.lane] = nG;
+        slot[C + ch][g.lane] = ngxm;
+        slot[2 * C + ch][g.lane] = ngb;
+        slot[3 * C + ch][g.lane] = cur.bb[ch];
+        slot[4 * C + ch][g.lane] = cur.xb[ch];
+      }
+      slot[5 * C + 0][g.lane] = gcv;
+      slot[5 * C + 1][g.lane] = gwxv;
+      slot[5 * C + 2][g.lane] = gwyv;
+      slot[5 * C + 3][g.lane] = cur.c;
+      slot[5 * C + 4][g.lane] = cur.rc1;
+      slot[5 * C + 5][g.lane] = cur.wxs;
+      slot[5 * C + 6][g.lane] = cur.wys;
+    };
+    // the barrier after row k with k % kP == kP - 1 makes rows k-kP+1 .. k visible to step B
+    auto publish = [&](int k) {
+      if (k % kP == kP - 1) lds_barrier();
+    };
+    Adj2wRow<C> b0, b1, b2;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    absorb(0, b0);
+    absorb(1, b1);
+    step(0, b0, b1, kNo);
+    load_row(3, b0);
+    publish(0);
+    for (int k = 1; k <= klast; k += 3) {  // cur / next rotate through (b1,b2) (b2,b0) (b0,b1)
+      absorb(k + 1, b2);
+      step(k, b1, b2, kYes);
+      load_row(k + 3, b1);
+      publish(k);
+      if (k + 1 > klast) break;
+      absorb(k + 2, b0);
+      step(k + 1, b2, b0, kYes);
+      load_row(k + 4, b2);
+      publish(k + 1);
+      if (k + 2 > klast) break;
+      absorb(k + 3, b1);
+      step(k + 2, b0, b1, kYes);
+      load_row(k + 5, b0);
+      publish(k + 2);
+    }
+    if (klast % kP != kP - 1) lds_barrier();  // the last rows have not been published yet
+  } else {
+    // ---------------------------------- step B ----------------------------------
+    const float* const xc_p = x05c + q0;  // x05[j-2], or the checkpoint y when BEND
+    float *const gco_p = gc + poff, *const gwxo_p = gwx + poff, *const gwyo_p = gwy + poff;
+    float *const g05o_p = g05_out + q0, *const gxm_p = gxk_m1 + q0, *const gbo_p = gb + q0;
+    float *const gxf_p = FINAL ? gx_final + q0 : nullptr;
+    struct RowB {
+      float xc[C];
+    };
+    auto load_row = [&](int k, RowB& in) {
+      const int kk = min(k, klast + 1);
+      const int h = g.hs - 2 + kk;
+      const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) in.xc[ch] = ldg(xc_p, off + chs[ch]);
+    };
+    const std::integral_constant<bool, BEND && !TRUE_ADJ> kBEnd{};  // the corrected gradient has one arithmetic form
+    float dB1[C], dB3[C], dB4[C];
+    // row k-1 as step B sees it
+    float pG[C], pgxm[C], pyB[C], pxb[C], pbb[C], pgb[C], pgc = 0.f, pgwx = 0.f, pgwy = 0.f;
+    float pc = 0.f, prc1 = 1.f, pwxs = 0.f, pwys = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      dB1[ch] = dB3[ch] = dB4[ch] = 0.f;
+      pG[ch] = pgxm[ch] = pyB[ch] = pxb[ch] = pbb[ch] = pgb[ch] = 0.f;
+    }
+
+    auto step = [&](int k, const RowB& in, auto tri_b, auto do_b) {
+      const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const inpaint::LaneMask inside(ok);
+      const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+      const float (*slot)[64] = hand[k % (2 * kP)];
+      float nG[C], ngxm[C], ngb[C], bbv[C], xbv[C], yB[C];
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        nG[ch] = slot[ch][g.lane];
+        ngxm[ch] = slot[C + ch][g.lane];
+        ngb[ch] = slot[2 * C + ch][g.lane];
+        bbv[ch] = slot[3 * C + ch][g.lane];
+        xbv[ch] = slot[4 * C + ch][g.lane];
+      }
+      const float gcv = slot[5 * C + 0][g.lane], gwxv = slot[5 * C + 1][g.lane], gwyv = slot[5 * C + 2][g.lane];
+      const float cc = slot[5 * C + 3][g.lane], rc1 = slot[5 * C + 4][g.lane];
+      const float wxs = slot[5 * C + 5][g.lane], wys = slot[5 * C + 6][g.lane];
+      const double opc_d = 1. + (double)cc;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {  // y of iteration j-1 on row k (the row below B's)
+        const float xc = inside(in.xc[ch]);
+        if (TRUE_ADJ) {
+          const float pb = prox_huber1(xbv[ch], cc, rc1, bbv[ch]);
+          const float pcv = BEND ? xc : prox_huber1(xc, cc, rc1, bbv[ch]);
+          yB[ch] = pb + tB * (pb - pcv);
+        } else {
+          yB[ch] = BEND ? xc : rebuild_y_fast(bbv[ch], xbv[ch], xc, cc, rc1, opc_d, tB);
+        }
+      }
+      if (tri_b.value) {
+        float gcB = pgc, gwxB = pgwx, gwyB = pgwy;
+        const float rc2B = rcp_refined((1.f + pc) * (1.f + pc));
+        const double popc_d = 1. + (double)pc;
+#pragma unroll
+        for (int ch = 0; ch < C; ch++) {
+          const Tri t = triangle(pyB[ch], yB[ch], pG[ch], nG[ch], pwxs, pwys, kBEnd);
+          const float a1_ = dB1[ch], a3_ = dB3[ch], a4_ = dB4[ch];
+          dB1[ch] = t.O1; dB3[ch] = t.n3; dB4[ch] = t.n4;
+          if (do_b.value) {
+            if (g.w < W - 1) gwxB = gwxB - t.ux;
+            if (h - 1 < H - 1) gwyB = gwyB - t.uy;
+            float df, gxm, g05v, gc_add, gb_add;
+            update(pG[ch], t, a1_, a3_, a4_, pgxm[ch], optB, tB, pc, prc1, rc2B, popc_d, pbb[ch], pxb[ch], df, gxm, g05v,
+                   gc_add, gb_add);
+            gcB += gc_add;
+            const float gbv = pgb[ch] + gb_add;
+            if (store_lane) {
+              if (FINAL) stg(gxf_p, roffB + chs[ch], df);
+              stg(gxm_p, roffB + chs[ch], gxm);
+              stg(g05o_p, roffB + chs[ch], g05v);
+              if (BEND) {  // segment flush, fused (TV.cu:178-218)
+                seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
+                stg(gbo_p, roffB + chs[ch], 0.f);
+              } else {
+                stg(gbo_p, roffB + chs[ch], gbv);
+              }
+            }
+          }
+        }
+        if (do_b.value && store_lane) {
+          if (BEND) {
+            const size_t e = poff + (roffB >> 2);
+            seg_gc[e] = gcB;
+            seg_gwx[e] = gwxB;
+            seg_gwy[e] = gwyB;
+            stg(gco_p, roffB, 0.f);
+            stg(gwxo_p, roffB, 0.f);
+            stg(gwyo_p, roffB, 0.f);
+          } else {
+            stg(gco_p, roffB, gcB);
+            stg(gwxo_p, roffB, gwxB);
+            stg(gwyo_p, roffB, gwyB);
+          }
+        }
+      }
+      pgc = gcv; pgwx = gwxv; pgwy = gwyv;
+      pc = cc; prc1 = rc1; pwxs = wxs; pwys = wys;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        pG[ch] = nG[ch]; pgxm[ch] = ngxm[ch]; pgb[ch] = ngb[ch];
+        pyB[ch] = yB[ch]; pxb[ch] = xbv[ch]; pbb[ch] = bbv[ch];
+      }
+    };
+    // B waits before every row k with k % kP == 0 for the barrier that published rows k .. k+kP-1
+    auto await = [&](int k) {
+      if (k % kP == 0) lds_barrier();
+    };
+    RowB b0, b1, b2;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    await(0);
+    step(0, b0, kNo, kNo);
+    load_row(3, b0);
+    await(1);
+    step(1, b1, kNo, kNo);
+    load_row(4, b1);
+    await(2);
+    step(2, b2, kYes, kNo);
+    load_row(5, b2);
+    for (int k = 3; k <= klast; k += 3) {
+      await(k);
+      step(k, b0, kYes, kYes);
+      load_row(k + 3, b0);
+      if (k + 1 > klast) break;
+      await(k + 1);
+      step(k + 1, b1, kYes, kYes);
+      load_row(k + 4, b1);
+      if (k + 2 > klast) break;
+      await(k + 2);
+      step(k + 2, b2, kYes, kYes);
+      load_row(k + 5, b2);
+    }
+  }
+}
+
 }  // namespace tvstrip

@@ -102,6 +102,27 @@ def test_more_than_four_channels_run_in_channel_groups(ext, tv_oracle, n, c, h, 
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 3, 23, 75, 17),     # odd its: first step, single step and pairs
+    (2, 4, 45, 130, 26),    # several strips wide, several segments
+    (1, 4, 3, 200, 6),      # fewer rows than the pair kernel's row lag
+    (1, 3, 2, 59, 4),
+    (1, 3, 70, 61, 8),      # one column more than a strip
+    (2, 4, 130, 200, 50),   # several strips high
+    (1, 4, 100, 60, 5),
+    (1, 3, 33, 1, 4),       # a single column
+])
+def test_three_and_four_channels_pair_in_two_wavefronts(ext, tv_oracle, n, c, h, w, its):
+    # with 3 or 4 channels the two adjoint steps of a launch run in two wavefronts of a workgroup and hand their
+    # row results over through LDS; every gradient is bit-equal to the oracle's
+    d = tv_inputs(n, c, h, w, seed=500 + c + h + its, conf_density=0.3)
+    got, ref = run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2)
+    compare("%d channels, two wavefronts" % c, got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
 def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first
