@@ -84,10 +84,13 @@ __global__ __launch_bounds__(256) void selftest_rsqrt_kernel(unsigned long long*
   if (bad3) atomicAdd(&counts[3], (unsigned long long)bad3);
 }
 
-// plain streaming copy, 16 bytes per lane and trip
-__global__ __launch_bounds__(256) void copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, long long n16) {
+// plain streaming copy, 16 bytes per lane.  One element per thread when the grid covers the buffer, with
+// non-temporal loads and stores: the fastest of the shapes measured on this GPU for 1 GiB (6.6 TB/s read + written;
+// the same loop on 8192 persistent workgroups reaches 4.6-4.9, a grid of half that many elements per thread 6.2).
+typedef float copy_v4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void copy_kernel(const copy_v4* __restrict__ src, copy_v4* __restrict__ dst, long long n16) {
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (long long)gridDim.x * blockDim.x)
-    dst[i] = src[i];
+    __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 int run_selftest(void (*kernel)(unsigned long long*, unsigned int), unsigned long long* host4, unsigned int rounds) {
@@ -125,7 +128,7 @@ extern "C" int inpaint_copy_bandwidth(long long bytes, int repeats, double* gbps
   if (bytes < 16 || repeats < 1 || !gbps_host) return inpaint::fail(INPAINT_ERR_ARG, "bad arguments");
   hipStream_t stream = (hipStream_t)stream_;
   const long long n16 = bytes / 16;
-  float4 *src = nullptr, *dst = nullptr;
+  copy_v4 *src = nullptr, *dst = nullptr;
   INPAINT_HIP(hipMalloc((void**)&src, (size_t)n16 * 16));
   if (hipMalloc((void**)&dst, (size_t)n16 * 16) != hipSuccess) {
     (void)hipFree(src);
@@ -135,7 +138,7 @@ extern "C" int inpaint_copy_bandwidth(long long bytes, int repeats, double* gbps
   hipEvent_t e0, e1;
   INPAINT_HIP(hipEventCreate(&e0));
   INPAINT_HIP(hipEventCreate(&e1));
-  const int grid = (int)std::min<long long>((n16 + 255) / 256, 256LL * 32);
+  const int grid = (int)std::min<long long>((n16 + 255) / 256, (1LL << 31) - 1);  // one element per thread
   hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, stream, src, dst, n16);
   INPAINT_HIP(hipEventRecord(e0, stream));
   for (int r = 0; r < repeats; r++) hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, stream, src, dst, n16);
