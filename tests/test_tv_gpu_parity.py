@@ -123,6 +123,22 @@ def test_three_and_four_channels_pair_in_two_wavefronts(ext, tv_oracle, n, c, h,
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("c", [2, 3, 4])
+@pytest.mark.parametrize("rows", ["3", "8", "13", "64"])
+def test_pair_kernels_at_forced_strip_heights(ext, tv_oracle, c, rows, monkeypatch):
+    # INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strips shorter and taller than the image, ragged last strips
+    d = tv_inputs(2, c, 50, 140, seed=610 + c, conf_density=0.3)
+    ref = run_oracle(tv_oracle, d, 12, 2)
+    monkeypatch.setenv("INPAINT_TV_FWD_ROWS", rows)
+    monkeypatch.setenv("INPAINT_TV_ADJ_ROWS", rows)
+    from customnetworklayers_amd._lib import reload_env
+    reload_env()
+    got = run_gpu(ext, d, 12, 2)
+    compare("strip height %s, %d channels" % (rows, c), got, ref)
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
 def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first
