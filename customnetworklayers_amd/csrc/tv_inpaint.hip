@@ -599,8 +599,9 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
     return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
   if (n > 65535 || (ih + TH - 1) / TH > 65535)
     return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
-  if ((long long)ih * iw >= (1ll << 29))  // the strip kernels address two planes of a tensor with one 32-bit byte offset
-    return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^29", (long long)ih * iw);
+  // the strip kernels address up to four planes of a tensor with one 32-bit byte offset from a common base pointer
+  if ((long long)ih * iw * std::min(std::max(ic, 2), 4) >= (1ll << 30))
+    return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^29 (2^28 with more than 3 channels)", (long long)ih * iw);
   if ((int)std::floor(std::sqrt((double)its)) > kMaxCheckpoints)
     return fail(INPAINT_ERR_ITS, "its=%d needs more than %d checkpoints", its, kMaxCheckpoints);
   return 0;
@@ -821,8 +822,45 @@ void launch_adjoint_pair_split(const Slot& s, hipStream_t stream, const float* d
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
-// (one group only: a pair adds step A's and step B's terms of its channels back to back, which is the reference's
-// order of summation only when the launch holds every channel)
+// 5 to 8 channels: two channel groups, step A and step B of each in a wavefront of its own (one strip per 256-thread
+// workgroup, two workgroups resident per CU)
+int pair_quad_rows(int n, int ih, int iw) {
+  if (knobs().tv_adj_rows > 0) return knobs().tv_adj_rows;
+  const long long cap = 2ll * compute_unit_count();
+  const long long sx = (iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols;
+  int best = 16;
+  long long best_cost = -1;
+  for (int R = 8; R <= 96; R++) {
+    const long long wg = sx * ((ih + R - 1) / R) * n;
+    const long long cost = ((wg + cap - 1) / cap) * (R + 12);  // 3 rows of start-up and two intervals of three rows behind
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = R;
+    }
+  }
+  return best;
+}
+
+template <int CM, int C1, bool BEND, bool TRUE_ADJ>
+void launch_adjoint_pair_quad(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                              const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
+                              float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
+  auto kern = gx_final ? tvstrip::tv_adjoint_strip4w<CM, C1, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip4w<CM, C1, BEND, false, TRUE_ADJ>;
+  const int R = pair_quad_rows(s.n, s.ih, s.iw);
+  const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
+  const long long strips = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(256);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
+                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+                     s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
+}
+
+constexpr int kPairChannels = 8;  // the most channels a pair launch holds (two groups of four)
+
+// (a pair adds step A's and step B's terms of its channels in the reference's order of summation only when the
+// launch holds every channel)
 template <bool BEND, bool TRUE_ADJ = false>
 void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c, const float* b,
                          const float* xa, const float* xb, const float* xc, const float* g05_in, float* g05_out,
@@ -833,18 +871,26 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const flo
     launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   else if (s.ic == 3)
     launch_adjoint_pair_split<3, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
-  else
+  else if (s.ic == 4)
     launch_adjoint_pair_split<4, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 5)
+    launch_adjoint_pair_quad<3, 2, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 6)
+    launch_adjoint_pair_quad<3, 3, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 7)
+    launch_adjoint_pair_quad<4, 3, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else
+    launch_adjoint_pair_quad<4, 4, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
   s.accb_cur = 1 - s.accb_cur;
 }
 
 bool adjoint_pairs(const Slot& s) {
   if (!knobs().tv_fuse_adj) return false;
-  // one channel group only (up to 4 channels): pairs over channel groups would sum the shared accumulators in
-  // another order; more channels take the one-step kernel, group after group.  With 3 or 4 channels the two steps
-  // need more than one wavefront's registers and run in two wavefronts.
-  return forward_pairs(s) && s.ic <= kGroup;
+  // the launch must hold every channel (pairs over launches of channel groups would sum the shared accumulators in
+  // another order): one wavefront for 1 or 2 channels, two for 3 or 4, four (two channel groups) for 5 to 8; more
+  // channels take the one-step kernel, group after group
+  return forward_pairs(s) && s.ic <= kPairChannels;
 }
 
 // -------------------------------------------------------------------------------------------------

@@ -1517,4 +1517,460 @@ __global__ __launch_bounds__(128) void tv_adjoint_strip2w(
   }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Two adjoint steps per launch for 5..8 channels: FOUR wavefronts per strip (256-thread workgroup).
+// The channels are split into two groups (the first CM, the second C1 <= CM of them); wavefronts 0 and
+// 1 run step A on group 0 and group 1, wavefronts 2 and 3 step B on group 0 and group 1, each as the
+// matching half of tv_adjoint_strip2w.  The reference adds the terms of the three shared accumulators in
+// the order A(ch 0 .. C-1), B(ch 0 .. C-1); here
+//   A0 adds its terms to the accumulators read from memory and hands them on (LDS),
+//   A1 adds its terms to what A0 handed on,
+//   B0 does not touch the accumulators: it hands its terms on, one by one (gc term, ux, uy per channel),
+//   B1 takes the accumulators after A1, adds B0's terms in channel order, then its own, and stores.
+// Time runs in intervals of three rows with one LDS-only barrier between them: in interval t A0 works
+// on rows 3t .. 3t+2, A1 and B0 on the three rows before, B1 on the three before those; every record
+// is written in one interval and read in the next, so two sets of three row slots per record type
+// suffice.  Every wavefront passes the same number of barriers (blocks + 2).
+// -------------------------------------------------------------------------------------------------
+template <int CM, int C1, bool BEND, bool FINAL, bool TRUE_ADJ = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tv_adjoint_strip4w(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
+    const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
+    const float* __restrict__ x05c, const float* __restrict__ gc_in, float* __restrict__ gc,
+    const float* __restrict__ gb_in, float* __restrict__ gb, const float* __restrict__ gwx_in,
+    float* __restrict__ gwx, const float* __restrict__ gwy_in, float* __restrict__ gwy,
+    const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
+    float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
+  static_assert(C1 >= 1 && C1 <= CM, "the second group is the smaller one");
+  constexpr int kSlots = 6;                     // two sets of three rows
+  __shared__ float handA[2][kSlots][3 * CM + 3][64];  // per group: g05[j], partial g_x[j], gb per channel; the accumulators
+  __shared__ float handT[kSlots][3 * CM][64];         // B0's terms: gc term, ux, uy per channel
+  StripGeom g;
+  if (!strip_geometry_block(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int Reff = min(R, H - g.hs);
+  const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
+  const int nblocks = (klast + 3) / 3;
+  const size_t HW = (size_t)H * W;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
+  const bool wx_ok = g.col_ok && g.w < W - 1;
+  const double optA = 1. + (double)tA, optB = 1. + (double)tB;
+  const size_t poff = (size_t)g.n * HW;
+  const unsigned plane4 = 4u * (unsigned)HW;  // bytes from one channel to the next
+  const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
+  const int o_lo = g.hs, o_hi = g.hs + Reff - 1;                       // output rows
+
+  constexpr float kGX = TRUE_ADJ ? 1.f : kLocalGXMult, kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
+  struct Tri {  // everything one triangle contributes (see tv_adjoint_strip)
+    float O1, O2, O3, O4, n3, n4, l1, l3, l4, ux, uy;
+  };
+  auto triangle = [&](float yk, float yd, float gk, float gd, float wxv, float wyv, auto end_form) {
+    Tri r;
+    const float yrt = from_right_lane(yk);
+    const float grt = from_right_lane(gk);
+    const float d1 = yk - yd, d2 = yk - yrt;
+    const float a1 = d1 * d1 * wyv;
+    const float a2 = d2 * d2 * wxv;
+    const float hub = exact_sqrt(a2 + a1);
+    const bool act = hub > kDelta;
+    float nom = inpaint::exact_div(kDelta, hub);
+    float denom = inpaint::exact_div(nom, 2.f * hub * hub);
+    nom = act ? nom : 1.f;
+    denom = act ? denom : 0.f;
+    const float gpd = gk - gd, gpr = gk - grt;
+    r.O1 = gpd * (wyv * nom);
+    r.O2 = gpr * (wxv * nom);
+    const float P1 = gpd * wyv * d1;
+    const float P2 = gpr * wxv * d2;
+    const float dd = denom * 2.0f;
+    const float tp = dd * (d1 * wyv + d2 * wxv);  // minus the reference's factor, exactly; O3, O4 carry the sign
+    const float tu = dd * d1 * wyv;
+    const float tl = dd * d2 * wxv;
+    r.O3 = -(P1 * tp);
+    r.O4 = -(P2 * tp);
+    r.n3 = P1 * tu;
+    r.n4 = P2 * tu;
+    r.l1 = from_left_lane(r.O2);
+    r.l3 = from_left_lane(P2 * tl);
+    r.l4 = from_left_lane(P1 * tl);
+    if (!end_form.value) {  // TV.cu:749-769
+      r.ux = kGX * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
+      r.uy = kGX * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
+    } else {  // TV.cu:1019-1037
+      const float ux_a = kGX * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
+      const float uy_a = kGX * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
+      r.ux = act ? ux_a : kGX * d2 * gpr;
+      r.uy = act ? uy_a : kGX * d1 * gpd;
+    }
+    return r;
+  };
+  // pixel update: J^T assembly, momentum adjoint, prox adjoint (TV.cu:668-743, 796-828)
+  auto update = [&](float gk, const Tri& t, float a1_, float a3_, float a4_, float gxv, double opt, float tmom,
+                    float conf, float rc1, float rc2, double opc_d, float bv, float xh, float& df, float& gxm,
+                    float& g05v, float& gc_add, float& gb_add) {
+    float tt = gk;
+    tt -= -a1_;
+    tt -= a3_;
+    tt -= a4_;
+    tt -= -t.l1;
+    tt -= t.l3;
+    tt -= t.l4;
+    tt -= t.O1;
+    tt -= t.O2;
+    tt -= t.O3;
+    tt -= t.O4;
+    df = (float)((double)gxv + opt * (double)tt);
+    df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
+    gxm = -tmom * tt;
+    const float diff = bv - xh;
+    const float sign = (diff < 0) ? -1.f : 1.f;
+    const bool quad = (opc_d >= (double)(sign * diff));
+    const float opc = 1.f + conf;
+    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
+    const float g05_q = div_by(df, opc, rc1);
+    const float gb_q = div_by(df * conf, opc, rc1) * 1.0f;
+    const bool mid = !quad && (conf >= sign * diff);
+    g05v = quad ? g05_q : (mid ? 0.f : df);
+    gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kGC);
+    gb_add = quad ? gb_q : (mid ? df * 1.0f : 0.f);
+  };
+  const std::true_type kYes{};
+  const std::false_type kNo{};
+
+  // ------------------------------------------ step A on one group ------------------------------------------
+  auto role_a = [&](auto channels, auto group) {
+    constexpr int C = decltype(channels)::value, G = decltype(group)::value;
+    const size_t q0 = ((size_t)g.n * Ct + (G ? CM : 0)) * HW;  // the group's first channel; channel ch plane4 * ch bytes further
+    const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
+    const float *const gci_p = gc_in + poff, *const gwxi_p = gwx_in + poff, *const gwyi_p = gwy_in + poff;
+    const float *const xa_p = x05a + q0, *const xb_p = x05b + q0, *const b_p = b + q0, *const g_p = g05_in + q0;
+    const float *const gxi_p = gxk + q0, *const gbi_p = gb_in + q0;
+    struct Row {
+      float c, rc1, wxs, wys;
+      float xa[C], xb[C], yA[C], bb[C], g[C], gx_i[C], gb_i[C], gc_i, gwx_i, gwy_i;
+      double opc_d;
+    };
+    auto load_row = [&](int k, Row& in) {
+      const int kk = min(k, klast + 1);
+      const int h = g.hs - 2 + kk;
+      const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+      const unsigned off_w = (unsigned)min(max(h, 0), h_hi) * W4 + wc;
+      const unsigned off_a = (unsigned)min(max(h, h_lo), h_hi) * W4 + wc;
+      const unsigned off_o = (unsigned)min(max(h, o_lo), o_hi) * W4 + wc;
+      in.c = ldg(cf_p, off);
+      in.wxs = ldg(wx_p, off_w);
+      in.wys = ldg(wy_p, off_w);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.xa[ch] = ldg(xa_p, off + plane4 * ch);
+        in.xb[ch] = ldg(xb_p, off + plane4 * ch);
+        in.bb[ch] = ldg(b_p, off + plane4 * ch);
+        in.g[ch] = ldg(g_p, off + plane4 * ch);
+        in.gx_i[ch] = ldg(gxi_p, off_a + plane4 * ch);
+        in.gb_i[ch] = ldg(gbi_p, off_o + plane4 * ch);
+      }
+      if (G == 0) {  // the second group continues the first group's sums
+        in.gc_i = ldg(gci_p, off_o);
+        in.gwx_i = ldg(gwxi_p, off_o);
+        in.gwy_i = ldg(gwyi_p, off_o);
+      } else {
+        in.gc_i = in.gwx_i = in.gwy_i = 0.f;
+      }
+    };
+    auto absorb = [&](int k, Row& o) {
+      const int h = g.hs - 2 + k;
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
+      o.rc1 = rcp_refined(1.f + o.c);
+      o.opc_d = 1. + (double)o.c;
+      o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
+      o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xa = inside(o.xa[ch]), xb = inside(o.xb[ch]), bv = inside(o.bb[ch]);
+        if (TRUE_ADJ) {
+          const float pa = prox_huber1(xa, o.c, o.rc1, bv), pb = prox_huber1(xb, o.c, o.rc1, bv);
+          o.yA[ch] = pa + tA * (pa - pb);
+        } else {
+          o.yA[ch] = rebuild_y_fast(bv, xa, xb, o.c, o.rc1, o.opc_d, tA);
+        }
+        o.g[ch] = inside(o.g[ch]);
+        o.xa[ch] = xa;
+        o.bb[ch] = bv;
+      }
+    };
+    float dA1[C], dA3[C], dA4[C];  // terms handed down to the row below
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) dA1[ch] = dA3[ch] = dA4[ch] = 0.f;
+
+    auto step = [&](int k, const Row& cur, const Row& nxt, auto do_a) {
+      const int h = g.hs - 2 + k;
+      const bool in_img = g.col_ok && h >= 0 && h < H;
+      float (*slot)[64] = handA[G][k % kSlots];
+      float gcv, gwxv, gwyv;
+      if (G == 0) {
+        gcv = cur.gc_i; gwxv = cur.gwx_i; gwyv = cur.gwy_i;
+      } else {  // what the first group made of the row's accumulators, one interval ago
+        const float (*prev)[64] = handA[0][k % kSlots];
+        gcv = prev[3 * CM + 0][g.lane]; gwxv = prev[3 * CM + 1][g.lane]; gwyv = prev[3 * CM + 2][g.lane];
+      }
+      const float rc2A = rcp_refined((1.f + cur.c) * (1.f + cur.c));
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const Tri t = triangle(cur.yA[ch], nxt.yA[ch], cur.g[ch], nxt.g[ch], cur.wxs, cur.wys, kNo);
+        const float a1_ = dA1[ch], a3_ = dA3[ch], a4_ = dA4[ch];
+        dA1[ch] = t.O1; dA3[ch] = t.n3; dA4[ch] = t.n4;
+        float nG = 0.f, ngxm = 0.f, ngb = cur.gb_i[ch];
+        if (do_a.value) {
+          if (g.w < W - 1) gwxv = gwxv - t.ux;
+          if (h < H - 1) gwyv = gwyv - t.uy;
+          float df, gxm, g05v, gc_add, gb_add;
+          update(cur.g[ch], t, a1_, a3_, a4_, cur.gx_i[ch], optA, tA, cur.c, cur.rc1, rc2A, cur.opc_d, cur.bb[ch],
+                 cur.xa[ch], df, gxm, g05v, gc_add, gb_add);
+          gcv += gc_add;
+          ngb += gb_add;
+          nG = in_img ? g05v : 0.f;  // B reads zero padding outside the image
+          ngxm = gxm;
+        }
+        slot[ch][g.lane] = nG;
+        slot[CM + ch][g.lane] = ngxm;
+        slot[2 * CM + ch][g.lane] = ngb;
+      }
+      slot[3 * CM + 0][g.lane] = gcv;
+      slot[3 * CM + 1][g.lane] = gwxv;
+      slot[3 * CM + 2][g.lane] = gwyv;
+    };
+    Row b0, b1, b2;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    for (int t = 0; t < G; t++) lds_barrier();  // group 1 works one interval behind group 0
+    absorb(0, b0);
+    absorb(1, b1);
+    step(0, b0, b1, kNo);
+    load_row(3, b0);
+    absorb(2, b2);
+    step(1, b1, b2, kYes);
+    load_row(4, b1);
+    absorb(3, b0);
+    step(2, b2, b0, kYes);
+    load_row(5, b2);
+    lds_barrier();
+    for (int blk = 1; blk < nblocks; blk++) {  // b0 holds row k (absorbed), b1 and b2 rows k+1, k+2 (loaded)
+      const int k = 3 * blk;
+      absorb(k + 1, b1);
+      step(k, b0, b1, kYes);
+      load_row(k + 3, b0);
+      if (k + 1 <= klast) {
+        absorb(k + 2, b2);
+        step(k + 1, b1, b2, kYes);
+        load_row(k + 4, b1);
+      }
+      if (k + 2 <= klast) {
+        absorb(k + 3, b0);
+        step(k + 2, b2, b0, kYes);
+        load_row(k + 5, b2);
+      }
+      lds_barrier();
+    }
+    for (int t = G; t < 2; t++) lds_barrier();  // the intervals in which only the wavefronts behind still work
+  };
+
+  // ------------------------------------------ step B on one group ------------------------------------------
+  auto role_b = [&](auto channels, auto group) {
+    constexpr int C = decltype(channels)::value, G = decltype(group)::value;
+    const size_t q0 = ((size_t)g.n * Ct + (G ? CM : 0)) * HW;
+    const int ch0 = G ? CM : 0;
+    const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
+    const float *const xb_p = x05b + q0, *const xc_p = x05c + q0, *const b_p = b + q0;  // x05c: x05[j-2], or the checkpoint y when BEND
+    float *const gco_p = gc + poff, *const gwxo_p = gwx + poff, *const gwyo_p = gwy + poff;
+    float *const g05o_p = g05_out + q0, *const gxm_p = gxk_m1 + q0, *const gbo_p = gb + q0;
+    float *const gxf_p = FINAL ? gx_final + q0 : nullptr;
+    struct Row {
+      float c, rc1, wxs, wys;
+      float xb[C], yB[C], bb[C];  // yB is loaded as x05[j-2] (or the checkpoint y) and rebuilt in place
+    };
+    auto load_row = [&](int k, Row& in) {
+      const int kk = min(k, klast + 1);
+      const int h = g.hs - 2 + kk;
+      const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+      const unsigned off_w = (unsigned)min(max(h, 0), h_hi) * W4 + wc;
+      in.c = ldg(cf_p, off);
+      in.wxs = ldg(wx_p, off_w);
+      in.wys = ldg(wy_p, off_w);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.xb[ch] = ldg(xb_p, off + plane4 * ch);
+        in.yB[ch] = ldg(xc_p, off + plane4 * ch);
+        in.bb[ch] = ldg(b_p, off + plane4 * ch);
+      }
+    };
+    auto absorb = [&](int k, Row& o) {
+      const int h = g.hs - 2 + k;
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
+      o.rc1 = rcp_refined(1.f + o.c);
+      const double opc_d = 1. + (double)o.c;
+      o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
+      o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xb = inside(o.xb[ch]), xc = inside(o.yB[ch]), bv = inside(o.bb[ch]);
+        if (TRUE_ADJ) {
+          const float pb = prox_huber1(xb, o.c, o.rc1, bv);
+          const float pcv = BEND ? xc : prox_huber1(xc, o.c, o.rc1, bv);
+          o.yB[ch] = pb + tB * (pb - pcv);
+        } else {
+          o.yB[ch] = BEND ? xc : rebuild_y_fast(bv, xb, xc, o.c, o.rc1, opc_d, tB);
+        }
+        o.xb[ch] = xb;
+        o.bb[ch] = bv;
+      }
+    };
+    const std::integral_constant<bool, BEND && !TRUE_ADJ> kBEnd{};  // the corrected gradient has one arithmetic form
+    float dB1[C], dB3[C], dB4[C];
+    // row k-1 as step B sees it
+    float pG[C], pgxm[C], pyB[C], pxb[C], pbb[C], pgb[C], pgc = 0.f, pgwx = 0.f, pgwy = 0.f;
+    float pc = 0.f, prc1 = 1.f, pwxs = 0.f, pwys = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      dB1[ch] = dB3[ch] = dB4[ch] = 0.f;
+      pG[ch] = pgxm[ch] = pyB[ch] = pxb[ch] = pbb[ch] = pgb[ch] = 0.f;
+    }
+
+    auto step = [&](int k, const Row& cur, auto tri_b, auto do_b) {
+      const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
+      const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+      const float (*slot)[64] = handA[G][k % kSlots];
+      float (*terms)[64] = handT[k % kSlots];
+      float nG[C], ngxm[C], ngb[C];
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        nG[ch] = slot[ch][g.lane];
+        ngxm[ch] = slot[CM + ch][g.lane];
+        ngb[ch] = slot[2 * CM + ch][g.lane];
+      }
+      float gcv = 0.f, gwxv = 0.f, gwyv = 0.f;
+      if (G == 1) {  // the row's accumulators with every A term added
+        gcv = slot[3 * CM + 0][g.lane]; gwxv = slot[3 * CM + 1][g.lane]; gwyv = slot[3 * CM + 2][g.lane];
+      }
+      if (tri_b.value) {
+        float gcB = pgc, gwxB = pgwx, gwyB = pgwy;
+        if (G == 1 && do_b.value) {  // the first group's B terms, in channel order, before this group's
+#pragma unroll
+          for (int ch = 0; ch < CM; ch++) {
+            if (g.w < W - 1) gwxB = gwxB - terms[CM + ch][g.lane];
+            if (h - 1 < H - 1) gwyB = gwyB - terms[2 * CM + ch][g.lane];
+            gcB += terms[ch][g.lane];
+          }
+        }
+        const float rc2B = rcp_refined((1.f + pc) * (1.f + pc));
+        const double popc_d = 1. + (double)pc;
+#pragma unroll
+        for (int ch = 0; ch < C; ch++) {
+          const Tri t = triangle(pyB[ch], cur.yB[ch], pG[ch], nG[ch], pwxs, pwys, kBEnd);
+          const float a1_ = dB1[ch], a3_ = dB3[ch], a4_ = dB4[ch];
+          dB1[ch] = t.O1; dB3[ch] = t.n3; dB4[ch] = t.n4;
+          if (do_b.value) {
+            float df, gxm, g05v, gc_add, gb_add;
+            update(pG[ch], t, a1_, a3_, a4_, pgxm[ch], optB, tB, pc, prc1, rc2B, popc_d, pbb[ch], pxb[ch], df, gxm, g05v,
+                   gc_add, gb_add);
+            if (G == 0) {
+              terms[ch][g.lane] = gc_add;
+              terms[CM + ch][g.lane] = t.ux;
+              terms[2 * CM + ch][g.lane] = t.uy;
+            } else {
+              if (g.w < W - 1) gwxB = gwxB - t.ux;
+              if (h - 1 < H - 1) gwyB = gwyB - t.uy;
+              gcB += gc_add;
+            }
+            const float gbv = pgb[ch] + gb_add;
+            if (store_lane) {
+              if (FINAL) stg(gxf_p, roffB + plane4 * ch, df);
+              stg(gxm_p, roffB + plane4 * ch, gxm);
+              stg(g05o_p, roffB + plane4 * ch, g05v);
+              if (BEND) {  // segment flush, fused (TV.cu:178-218)
+                seg_gb[((size_t)g.n * Ct + ch0 + ch) * HW + (roffB >> 2)] = gbv;
+                stg(gbo_p, roffB + plane4 * ch, 0.f);
+              } else {
+                stg(gbo_p, roffB + plane4 * ch, gbv);
+              }
+            }
+          }
+        }
+        if (G == 1 && do_b.value && store_lane) {
+          if (BEND) {
+            const size_t e = poff + (roffB >> 2);
+            seg_gc[e] = gcB;
+            seg_gwx[e] = gwxB;
+            seg_gwy[e] = gwyB;
+            stg(gco_p, roffB, 0.f);
+            stg(gwxo_p, roffB, 0.f);
+            stg(gwyo_p, roffB, 0.f);
+          } else {
+            stg(gco_p, roffB, gcB);
+            stg(gwxo_p, roffB, gwxB);
+            stg(gwyo_p, roffB, gwyB);
+          }
+        }
+      }
+      pgc = gcv; pgwx = gwxv; pgwy = gwyv;
+      pc = cur.c; prc1 = cur.rc1; pwxs = cur.wxs; pwys = cur.wys;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        pG[ch] = nG[ch]; pgxm[ch] = ngxm[ch]; pgb[ch] = ngb[ch];
+        pyB[ch] = cur.yB[ch]; pxb[ch] = cur.xb[ch]; pbb[ch] = cur.bb[ch];
+      }
+    };
+    Row b0, b1, b2;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    for (int t = 0; t < 1 + G; t++) lds_barrier();  // one interval behind the group's step A
+    absorb(0, b0);
+    step(0, b0, kNo, kNo);
+    load_row(3, b0);
+    absorb(1, b1);
+    step(1, b1, kNo, kNo);
+    load_row(4, b1);
+    absorb(2, b2);
+    step(2, b2, kYes, kNo);
+    load_row(5, b2);
+    lds_barrier();
+    for (int blk = 1; blk < nblocks; blk++) {  // b0, b1, b2 hold rows k, k+1, k+2 (loaded)
+      const int k = 3 * blk;
+      absorb(k, b0);
+      step(k, b0, kYes, kYes);
+      load_row(k + 3, b0);
+      if (k + 1 <= klast) {
+        absorb(k + 1, b1);
+        step(k + 1, b1, kYes, kYes);
+        load_row(k + 4, b1);
+      }
+      if (k + 2 <= klast) {
+        absorb(k + 2, b2);
+        step(k + 2, b2, kYes, kYes);
+        load_row(k + 5, b2);
+      }
+      lds_barrier();
+    }
+    for (int t = 1 + G; t < 2; t++) lds_barrier();
+  };
+
+  const std::integral_constant<int, CM> kFirst{};
+  const std::integral_constant<int, C1> kSecond{};
+  const std::integral_constant<int, 0> kG0{};
+  const std::integral_constant<int, 1> kG1{};
+  if (wave == 0) role_a(kFirst, kG0);
+  else if (wave == 1) role_a(kSecond, kG1);
+  else if (wave == 2) role_b(kFirst, kG0);
+  else role_b(kSecond, kG1);
+}
+
 }  // namespace tvstrip

@@ -123,7 +123,31 @@ def test_three_and_four_channels_pair_in_two_wavefronts(ext, tv_oracle, n, c, h,
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("c", [2, 3, 4])
+@pytest.mark.parametrize("n,c,h,w,its", [
+    (1, 5, 23, 75, 17),     # groups of 3 + 2; odd its: first step, single step and pairs
+    (2, 6, 45, 130, 26),    # 3 + 3; several strips wide, several segments
+    (1, 7, 3, 200, 6),      # 4 + 3; fewer rows than one interval of the pipeline
+    (1, 8, 2, 59, 4),       # 4 + 4
+    (1, 5, 70, 61, 8),      # one column more than a strip
+    (2, 8, 130, 200, 50),   # several strips high
+    (1, 7, 100, 60, 5),
+    (1, 6, 33, 1, 4),       # a single column
+    (1, 8, 4, 64, 6),       # rows: exactly one block of three after the start-up rows
+    (1, 5, 5, 64, 6),
+    (1, 6, 6, 64, 6),
+])
+def test_five_to_eight_channels_pair_in_four_wavefronts(ext, tv_oracle, n, c, h, w, its):
+    # two channel groups, step A and step B of each in a wavefront of its own; the shared accumulators travel
+    # A(group 0) -> A(group 1) -> B(group 1), which also adds B(group 0)'s terms first: the reference's order
+    d = tv_inputs(n, c, h, w, seed=700 + c + h + its, conf_density=0.3)
+    got, ref = run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2)
+    compare("%d channels, four wavefronts" % c, got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("c", [2, 3, 4, 5, 8])
 @pytest.mark.parametrize("rows", ["3", "8", "13", "64"])
 def test_pair_kernels_at_forced_strip_heights(ext, tv_oracle, c, rows, monkeypatch):
     # INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strips shorter and taller than the image, ragged last strips
@@ -310,7 +334,7 @@ def test_module_surface_and_autograd(ext, tv_oracle):
     compare("module", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
 
 
-@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 40, 130, 20), (1, 1, 30, 70, 9), (1, 3, 20, 64, 6)])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 40, 130, 20), (1, 1, 30, 70, 9), (1, 3, 20, 64, 6), (1, 7, 25, 64, 12)])
 def test_kept_iterates_or_recomputed_segments_give_the_same_bits(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # keep mode 2 (default) stores every x05 row in the forward and recomputes nothing; mode 1 keeps the last
     # segment's rows, which serve one backward; mode 0 recomputes every segment as the reference does.  A second
@@ -363,7 +387,7 @@ CORRECTED = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale
 
 @pytest.mark.parametrize("n,c,h,w,its", [
     (1, 2, 64, 128, 20), (2, 3, 37, 101, 9), (1, 1, 16, 64, 2), (1, 4, 19, 126, 6), (1, 2, 1, 70, 4),
-    (1, 1, 33, 1, 4), (3, 2, 130, 200, 50), (1, 2, 21, 64, 3), (1, 6, 23, 70, 10),
+    (1, 1, 33, 1, 4), (3, 2, 130, 200, 50), (1, 2, 21, 64, 3), (1, 6, 23, 70, 10), (2, 8, 40, 126, 16), (1, 5, 9, 64, 7),
 ])
 def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # gradient_mode 1: y as the forward pass made it, no checkpoint stand-in at segment starts, iteration 0
