@@ -1070,11 +1070,52 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
 #undef TGV_PAIR_ARGS
 }
 
+// Rows per strip of the four-wavefront pair kernel (three and four channels).  Its 256-thread workgroups (one strip
+// each) are resident two per CU; a strip of R rows takes R + 3 pipeline rows, two intervals of two rows behind and the
+// start-up.
+int pair_quad_rows(int n, int ih, int iw) {
+  if (knobs().tgv_adj_rows > 0) return knobs().tgv_adj_rows;
+  const long long cap = 2ll * compute_unit_count();
+  const long long sx = (iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2;
+  int best = 16;
+  long long best_cost = -1;
+  for (int R = 8; R <= 96; R++) {
+    const long long wg = sx * ((ih + R - 1) / R) * n;
+    const long long cost = ((wg + cap - 1) / cap) * (R + 11);
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = R;
+    }
+  }
+  return best;
+}
+
+// 3 and 4 channels: two channel groups, step A and step B of each in a wavefront of its own
+template <int CM, int C1, bool BEND, bool TRUE_ADJ>
+void launch_adjoint_pair_quad(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
+                              const float* xb, const float* xc, const float* g05_in, float* g05_out, const float* gxk,
+                              float* gxk_m1, float* gx_final, float tA, float tB) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  auto kern = gx_final ? tgvstrip::tgv_adjoint_strip4w<CM, C1, BEND, true, TRUE_ADJ> : tgvstrip::tgv_adjoint_strip4w<CM, C1, BEND, false, TRUE_ADJ>;
+  const int R = pair_quad_rows(s.n, s.ih, s.iw);
+  const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
+  const long long strips = (long long)sx * sy * s.n;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
+  const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(256);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib],
+                     s.acc_gb[ob], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final,
+                     s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + 2 * sP, s.seg_gy + 2 * sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
+}
+
+constexpr int kPairChannels = 4;  // the most channels a pair launch holds (two groups of two)
+
 template <bool BEND, bool TRUE_ADJ = false>
 void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa, const float* xb,
                          const float* xc, const float* g05_in, float* g05_out, const float* gxk, float* gxk_m1,
                          float* gx_final, float tA, float tB) {
   if (s.ic == 1) launch_adjoint_pair_strip<1, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 3) launch_adjoint_pair_quad<2, 1, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 4) launch_adjoint_pair_quad<2, 2, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   else launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   s.acc_cur = 1 - s.acc_cur;
   s.accb_cur = 1 - s.accb_cur;
@@ -1082,9 +1123,10 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* c, const floa
 
 bool adjoint_pairs(const Slot& s) {
   if (!knobs().tgv_fuse_adj) return false;
-  // one group only: a pair adds step A's and step B's terms of its channels back to back, which is the reference's
-  // order of summation only when the launch holds every channel
-  return forward_pairs(s) && s.ic <= kGroup;
+  // a pair adds step A's and step B's terms of its channels back to back, which is the reference's order of summation
+  // only when the launch holds every channel: one or two wavefronts for 1 or 2 channels, four (two channel groups) for
+  // 3 or 4; more channels take the one-step kernel, group after group
+  return forward_pairs(s) && s.ic <= kPairChannels;
 }
 
 }  // namespace

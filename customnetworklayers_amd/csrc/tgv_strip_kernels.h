@@ -1,4 +1,4 @@
-// Wave-strip kernels of the TGV layer (the default path for up to 2 flow channels).
+// Wave-strip kernels of the TGV layer (the default path; adjoint pairs hold up to 4 flow channels, more run in groups).
 //
 // Same execution scheme as the TV layer's strip kernels: one wavefront owns 62 adjacent columns (one
 // pixel per lane, lanes 0 and 63 are aprons) by R rows of one sample and walks them top to bottom
@@ -1992,6 +1992,706 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       load_row(k + 5, b2);
     }
   }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Two adjoint steps per launch for three and four flow channels: FOUR wavefronts per strip (256-thread
+// workgroup).  The channels are split into two groups (the first CM, the second C1 <= CM of them);
+// wavefronts 0 and 1 run step A on group 0 and group 1, wavefronts 2 and 3 step B on group 0 and
+// group 1, each as the matching half of tgv_adjoint_strip2w.  The reference adds the terms of the five
+// shared accumulators (gc, two channels of gwx, two of gwy) in the order A(ch 0 .. C-1), B(ch 0 .. C-1);
+// here
+//   A0 adds its terms to the accumulators read from memory and hands them on (LDS),
+//   A1 adds its terms to what A0 handed on,
+//   B0 does not touch the accumulators: it hands its terms on, one by one -- the gc term and, per weight
+//      accumulator, the float that is added and the double that is subtracted after it (zero where the
+//      Huber term is inactive: x - 0.0 is x),
+//   B1 takes the accumulators after A1, applies B0's terms in channel order, then its own, and stores.
+// Time runs in intervals of two rows with one LDS-only barrier between them: in interval t A0 works on
+// rows 2t, 2t+1, A1 and B0 on the two rows before, B1 on the two before those; every record is written
+// in one interval and read in the next, so two sets of two row slots per record type suffice.  Every
+// wavefront passes the same number of barriers (intervals + 2).  Step B reads c, the weights, b and the
+// u of x05[j-1] from memory itself (the records of two groups plus B0's terms fill the 64 KB of LDS a
+// workgroup may hold).
+// -------------------------------------------------------------------------------------------------
+template <int CM, int C1, bool BEND, bool FINAL, bool TRUE_ADJ = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tgv_adjoint_strip4w(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
+    const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
+    const float* __restrict__ x05a, const float* __restrict__ x05b, const float* __restrict__ x05c,
+    const float* __restrict__ gc_in, float* __restrict__ gc, const float* __restrict__ gb_in, float* __restrict__ gb,
+    const float* __restrict__ gwx_in, float* __restrict__ gwx, const float* __restrict__ gwy_in,
+    float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
+    const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
+  static_assert(C1 >= 1 && C1 <= CM, "the second group is the smaller one");
+  constexpr int kP = 2;                // rows per interval
+  constexpr int kSlots = 2 * kP;       // two sets of kP row slots
+  constexpr int kRec = 7 * CM + 5;     // step A's results per row and lane: g05[j] (3), partial g_x[j] (3), gb per channel; the accumulators
+  __shared__ float handA[2][kSlots][kRec][64];
+  __shared__ float termF[kSlots][5 * CM][64];   // B0's terms: per channel the gc term and the four floats that are added
+  __shared__ double termD[kSlots][4 * CM][64];  // ... and the four doubles that are subtracted after them
+  StripGeom g;
+  if (!strip_geometry_block(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int Reff = min(R, H - g.hs);
+  const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
+  const size_t HW = (size_t)H * W, CHW = HW * Ct;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
+  const bool rmask = g.col_ok && g.w < W - 1;
+  const double optA = 1. + (double)tA, optB = 1. + (double)tB;
+  const float gxm = TRUE_ADJ ? 1.f : kLocalGXMult;
+  constexpr float kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
+  const size_t poff = (size_t)g.n * HW;
+  const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
+  const int o_lo = g.hs, o_hi = g.hs + Reff - 1;                       // output rows
+
+  const auto row_offsets = [&](int k, unsigned& off, unsigned& off_w) {
+    const int kk = min(k, klast + 1);
+    const int h = g.hs - 2 + kk;
+    off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+    off_w = (unsigned)min(max(h, 0), h_hi) * W4 + wc;
+  };
+
+  // Huber weight, activity and weight derivative of one term, in the main or the segment-start form
+  auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
+    if (end_form.value) {  // TGV.cu:1132-1138
+      const float hub = exact_sqrt(A);
+      Wt = exact_div(1.0f, fmaxf(1.f, exact_div(hub, delta)));
+      act = hub > delta;
+      hub2 = hub * hub;
+      dW = exact_div(Wt, hub2);
+    } else {  // TGV.cu:313-319
+      const float hub = rsq_exact(A);
+      Wt = fminf(1.f, hub * delta);
+      act = Wt < 1.0f;
+      hub2 = hub * hub;
+      dW = Wt * hub2;
+    }
+  };
+
+  struct Acc {  // the weight-gradient accumulators of one pixel
+    float gwx0, gwx1, gwy0, gwy1;
+  };
+  // what one channel's triangle does to them: x = (float)((double)(x + add) - sub), sub = 0 where the term is inactive
+  struct AccTerms {
+    float add_wx0, add_wy0, add_wx1, add_wy1;
+    double sub_wx0, sub_wy0, sub_wx1, sub_wy1;
+  };
+  auto apply_terms = [](Acc& acc, const AccTerms& t) {
+    acc.gwx0 = (float)((double)(acc.gwx0 + t.add_wx0) - t.sub_wx0);
+    acc.gwy0 = (float)((double)(acc.gwy0 + t.add_wy0) - t.sub_wy0);
+    acc.gwx1 = (float)((double)(acc.gwx1 + t.add_wx1) - t.sub_wx1);
+    acc.gwy1 = (float)((double)(acc.gwy1 + t.add_wy1) - t.sub_wy1);
+  };
+  struct T3 {
+    float t0, t1, t2;
+  };
+  // One pixel of one step: the triangle owned by the pixel (all shares), the terms handed down
+  // (dn[6], read then replaced) and, when upd, the pixel's weight-gradient terms and J^T g.
+  auto pixel = [&](float yk, float y1c, float y2c, float yd, float y1d, float y2d, float gk, float g1k, float g2k,
+                   float gd, float g1d, float g2d, float wxv, float wyv, float bX, float bY, bool dmask, float* dn,
+                   AccTerms& at, auto end_form, auto upd) {
+    const float yr = from_right_lane(yk), y1r = from_right_lane(y1c), y2r = from_right_lane(y2c);
+    const float gr = from_right_lane(gk), g1r = from_right_lane(g1k), g2r = from_right_lane(g2k);
+    // ---- coupling term ----
+    const float aij_1 = rmask ? ((yr - yk) - y1c) : 0.f;
+    const float aij_2 = dmask ? ((yd - yk) - y2c) : 0.f;
+    float Wt, dW, hub2;
+    bool act;
+    huber(aij_2 * aij_2 * wyv + aij_1 * aij_1 * wxv, kD0, Wt, act, dW, hub2, end_form);
+    const float dy1 = gk - gr + g1k;
+    const float dy2 = gk - gd + g2k;
+    const float a1 = aij_1 * wxv, a2 = aij_2 * wyv;
+    const float deriv = dy1 * a1 + dy2 * a2;
+    const float Da = Wt * dy2 * wyv, Db = Wt * dy1 * wxv;
+    const float Ea = act ? deriv * (a2 * dW) : 0.f;
+    const float Eb = act ? deriv * (a1 * dW) : 0.f;
+    const float E0 = act ? deriv * ((a1 + a2) * dW) : 0.f;
+    // ---- smoothness term of v1 ----
+    const float u11 = rmask ? (y1r - y1c) : 0.f;
+    const float u12 = dmask ? (y1d - y1c) : 0.f;
+    float W1, dW1, h1sq;
+    bool act1;
+    huber((u11 * u11 + u12 * u12) * bX, kD1, W1, act1, dW1, h1sq, end_form);
+    const float dg1x = g1k - g1r, dg1y = g1k - g1d;
+    const float H1x = rmask ? bX * W1 * dg1x : 0.f;
+    const float H1y = dmask ? bX * W1 * dg1y : 0.f;
+    const float S1 = dg1x * u11 + dg1y * u12;
+    const float dv1 = dg1x * u11 * bX + dg1y * u12 * bX;
+    const float R1 = act1 ? bX * dW1 * (u11 + u12) * dv1 : 0.f;
+    const float N1y = act1 ? bX * (dW1 * bX * u12) * S1 : 0.f;
+    const float N1x = act1 ? bX * (dW1 * bX * u11) * S1 : 0.f;
+    // ---- smoothness term of v2 ----
+    const float u21 = rmask ? (y2r - y2c) : 0.f;
+    const float u22 = dmask ? (y2d - y2c) : 0.f;
+    float W2, dW2, h2sq;
+    bool act2;
+    huber((u21 * u21 + u22 * u22) * bY, kD2, W2, act2, dW2, h2sq, end_form);
+    const float dg2x = g2k - g2r, dg2y = g2k - g2d;
+    const float H2x = rmask ? bY * W2 * dg2x : 0.f;
+    const float H2y = dmask ? bY * W2 * dg2y : 0.f;
+    const float S2 = dg2x * u21 + dg2y * u22;
+    const float dv2 = dg2x * u21 * bY + dg2y * u22 * bY;
+    const float R2 = act2 ? bY * dW2 * (u21 + u22) * dv2 : 0.f;
+    const float dW2_below = (end_form.value || TRUE_ADJ) ? dW2 : exact_div(W2, h2sq);  // TGV.cu:355
+    const float N2y = act2 ? bY * (dW2_below * bY * u22) * S2 : 0.f;
+    const float N2x = act2 ? bY * (dW2 * bY * u21) * S2 : 0.f;
+
+    const float lDb = from_left_lane(Db), lEb = from_left_lane(Eb);
+    const float lH1 = from_left_lane(H1x), lN1 = from_left_lane(N1x);
+    const float lH2 = from_left_lane(H2x), lN2 = from_left_lane(N2x);
+    const float aDa = dn[0], aEa = dn[1], aH1 = dn[2], aN1 = dn[3], aH2 = dn[4], aN2 = dn[5];
+    dn[0] = Da; dn[1] = Ea; dn[2] = H1y; dn[3] = N1y; dn[4] = H2y; dn[5] = N2y;
+    T3 r{0.f, 0.f, 0.f};
+    if (upd.value) {
+      if (end_form.value) {
+        at.add_wx0 = gxm * dy1 * aij_1 * Wt;
+        at.add_wy0 = gxm * dy2 * aij_2 * Wt;
+      } else {
+        at.add_wx0 = gxm * dy1 * (aij_1 * Wt);
+        at.add_wy0 = gxm * dy2 * (aij_2 * Wt);
+      }
+      {
+        const double sy = (double)(gxm * (aij_2 * dW * aij_2)) * 0.5 * (double)deriv;
+        const double sx = (double)(gxm * (aij_1 * dW * aij_1)) * 0.5 * (double)deriv;
+        at.sub_wy0 = act ? sy : 0.0;
+        at.sub_wx0 = act ? sx : 0.0;
+      }
+      at.add_wx1 = gxm * S1 * W1;
+      {
+        const double s1 = (double)(gxm * (u12 * dW1 * u12 + u11 * dW1 * u11)) * 0.5 * (double)dv1;
+        at.sub_wx1 = act1 ? s1 : 0.0;
+      }
+      at.add_wy1 = gxm * S2 * W2;
+      {
+        const double s2 = (double)(gxm * (u22 * dW2 * u22 + u21 * dW2 * u21)) * 0.5 * (double)dv2;
+        at.sub_wy1 = act2 ? s2 : 0.0;
+      }
+      float t0 = gk, t1 = g1k, t2 = g2k;
+      t0 -= -aDa;
+      t0 += -aEa;
+      t1 -= -aH1;
+      t1 += -aN1;
+      t2 -= -aH2;
+      t2 += -aN2;
+      t0 -= -lDb;
+      t0 += -lEb;
+      t1 -= -lH1;
+      t1 += -lN1;
+      t2 -= -lH2;
+      t2 += -lN2;
+      if (end_form.value) {
+        t0 -= dy2 * wyv * Wt;
+        t0 -= dy1 * wxv * Wt;
+        t1 -= Wt * (g1k - gr + gk) * wxv;
+        t2 -= Wt * (g2k - gd + gk) * wyv;
+      } else {
+        t0 -= Wt * (dy2 * wyv + dy1 * wxv);
+        t1 -= Db;
+        t2 -= Da;
+      }
+      t0 += E0;
+      t2 += Ea;
+      t1 += Eb;
+      if (end_form.value) {
+        t1 -= H1y;
+        t1 -= H1x;
+      } else {
+        t1 -= H1x;
+        t1 -= H1y;
+      }
+      t1 += R1;
+      t2 -= H2x;
+      t2 -= H2y;
+      t2 += R2;
+      r.t0 = t0; r.t1 = t1; r.t2 = t2;
+    }
+    return r;
+  };
+  // momentum adjoint of the three variables and prox adjoint of u (TGV.cu:560-612)
+  struct Tail {
+    float df, d1, d2, gxm0, gxm1, gxm2, g05v, gc_add, gb_add;
+  };
+  auto tail = [&](const T3& t, float gx0, float gx1, float gx2, double opt, float tm, float conf, float bv, float xh) {
+    Tail o;
+    o.gxm1 = -tm * t.t1;
+    float d1 = (float)((double)gx1 + opt * (double)t.t1);
+    o.d1 = fmaxf(-kClipLocalGrad, fminf(d1, kClipLocalGrad));
+    o.gxm2 = -tm * t.t2;
+    float d2 = (float)((double)gx2 + opt * (double)t.t2);
+    o.d2 = fmaxf(-kClipLocalGrad, fminf(d2, kClipLocalGrad));
+    float df = (float)((double)gx0 + opt * (double)t.t0);
+    df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
+    o.df = df;
+    o.gxm0 = -tm * t.t0;
+    const float rc1 = rcp_refined(1.f + conf);
+    const float rc2 = rcp_refined((1.f + conf) * (1.f + conf));
+    const double opc_d = 1. + (double)conf;
+    const float diff = bv - xh;
+    const float sign = (diff < 0) ? -1.f : 1.f;
+    const bool quad = (opc_d >= (double)(sign * diff));
+    const float opc = 1.f + conf;
+    const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
+    const float g05_q = div_by(df, opc, rc1);
+    const float gb_q = div_by(df * conf, opc, rc1) * 1.0f;
+    const bool mid = !quad && (conf >= sign * diff);
+    o.g05v = quad ? g05_q : (mid ? 0.f : df);
+    o.gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kGC);
+    o.gb_add = quad ? gb_q : (mid ? df * 1.0f : 0.f);
+    return o;
+  };
+
+  const std::true_type kYes{};
+  const std::false_type kNo{};
+
+  // ------------------------------------------ step A on one group ------------------------------------------
+  auto role_a = [&](auto channels, auto group) {
+    constexpr int C = decltype(channels)::value, G = decltype(group)::value;
+    constexpr int chb = G ? CM : 0;  // the group's first channel
+    const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
+                       *const cf_p = cf + poff;
+    const float *const gci_p = gc_in + poff, *const gwx0i_p = gwx_in + 2 * poff, *const gwx1i_p = gwx_in + 2 * poff + HW,
+                       *const gwy0i_p = gwy_in + 2 * poff, *const gwy1i_p = gwy_in + 2 * poff + HW;
+    const float *xa_p[3][C], *xb0_p[C], *pv_p[2][C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const size_t qb = ((size_t)g.n * Ct + chb + ch) * HW;
+      b_p[ch] = b + qb; gbi_p[ch] = gb_in + qb;
+      xb0_p[ch] = x05b + (size_t)g.n * 3 * CHW + (size_t)(chb + ch) * HW;
+#pragma unroll
+      for (int v = 0; v < 3; v++) {
+        const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)(chb + ch) * HW;
+        xa_p[v][ch] = x05a + q;
+        if (v > 0) pv_p[v - 1][ch] = x05b + q;  // corrected gradient: the aux rows before A's, for the momentum of aux y
+        g_p[v][ch] = g05_in + q; gxi_p[v][ch] = gxk + q;
+      }
+    }
+    auto load_row = [&](int k, Adj2ARow<C>& in) {
+      unsigned off, off_w;
+      row_offsets(k, off, off_w);
+      in.c = ldg(cf_p, off);
+      in.wxs = ldg(wx_p, off_w);
+      in.wys = ldg(wy_p, off_w);
+      in.bxs = ldg(bx_p, off_w);
+      in.bys = ldg(by_p, off_w);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.xa0[ch] = ldg(xa_p[0][ch], off);
+        in.yA[1][ch] = ldg(xa_p[1][ch], off);
+        in.yA[2][ch] = ldg(xa_p[2][ch], off);
+        in.xb0[ch] = ldg(xb0_p[ch], off);
+        if (TRUE_ADJ) {
+          in.pv[0][ch] = ldg(pv_p[0][ch], off);
+          in.pv[1][ch] = ldg(pv_p[1][ch], off);
+        }
+        in.bb[ch] = ldg(b_p[ch], off);
+#pragma unroll
+        for (int v = 0; v < 3; v++) in.g[v][ch] = ldg(g_p[v][ch], off);
+      }
+    };
+    auto load_late = [&](int k, Adj2Late<C>& in) {  // what A's update of row k and the accumulators of that pixel need
+      const int h = g.hs - 2 + min(k, klast);
+      const unsigned off_a = (unsigned)min(max(h, h_lo), h_hi) * W4 + wc;
+      const unsigned off_o = (unsigned)min(max(h, o_lo), o_hi) * W4 + wc;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.gb_i[ch] = ldg(gbi_p[ch], off_o);
+#pragma unroll
+        for (int v = 0; v < 3; v++) in.gx_i[v][ch] = ldg(gxi_p[v][ch], off_a);
+      }
+      if (G == 0) {  // the second group continues the first group's sums
+        in.gc_i = ldg(gci_p, off_o);
+        in.gwx0_i = ldg(gwx0i_p, off_o);
+        in.gwx1_i = ldg(gwx1i_p, off_o);
+        in.gwy0_i = ldg(gwy0i_p, off_o);
+        in.gwy1_i = ldg(gwy1i_p, off_o);
+      } else {
+        in.gc_i = in.gwx0_i = in.gwx1_i = in.gwy0_i = in.gwy1_i = 0.f;
+      }
+    };
+    auto absorb = [&](int k, Adj2ARow<C>& o) {
+      const int h = g.hs - 2 + k;
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
+      const float rc1 = rcp_refined(1.f + o.c);
+      const double opc_d = 1. + (double)o.c;
+      o.wxs = (ok && rmask) ? o.wxs : 0.f;
+      o.wys = (ok && h < H - 1) ? o.wys : 0.f;
+      o.bxs = inside(o.bxs);
+      o.bys = inside(o.bys);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xa = inside(o.xa0[ch]), xb = inside(o.xb0[ch]), bv = inside(o.bb[ch]);
+        if (TRUE_ADJ) {
+          const float pa = tvstrip::prox_huber1(xa, o.c, rc1, bv), pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
+          o.yA[0][ch] = pa + tA * (pa - pb);  // TGV.cu:1773
+        } else {
+          o.yA[0][ch] = tvstrip::rebuild_y_fast(bv, xa, xb, o.c, rc1, opc_d, tA);
+        }
+        o.xa0[ch] = xa;
+        o.bb[ch] = bv;
+#pragma unroll
+        for (int v = 1; v < 3; v++) {
+          const float xv = inside(o.yA[v][ch]);
+          o.yA[v][ch] = TRUE_ADJ ? xv + tA * (xv - inside(o.pv[v - 1][ch])) : xv;  // TGV.cu:1686-1690
+        }
+#pragma unroll
+        for (int v = 0; v < 3; v++) o.g[v][ch] = inside(o.g[v][ch]);
+      }
+    };
+    float dnA[C][6];
+#pragma unroll
+    for (int ch = 0; ch < C; ch++)
+#pragma unroll
+      for (int i = 0; i < 6; i++) dnA[ch][i] = 0.f;
+
+    auto step = [&](int k, const Adj2ARow<C>& cur, const Adj2ARow<C>& nxt, const Adj2Late<C>& late, auto do_a) {
+      const int h = g.hs - 2 + k;
+      const bool in_img = g.col_ok && h >= 0 && h < H;
+      const bool dmaskA = h >= 0 && h < H - 1;
+      float (*slot)[64] = handA[G][k % kSlots];
+      float gcv;
+      Acc accA;
+      if (G == 0) {
+        gcv = late.gc_i;
+        accA = Acc{late.gwx0_i, late.gwx1_i, late.gwy0_i, late.gwy1_i};
+      } else {  // what the first group made of the row's accumulators, one interval ago
+        const float (*prev)[64] = handA[0][k % kSlots];
+        gcv = prev[7 * CM + 0][g.lane];
+        accA = Acc{prev[7 * CM + 1][g.lane], prev[7 * CM + 2][g.lane], prev[7 * CM + 3][g.lane], prev[7 * CM + 4][g.lane]};
+      }
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        AccTerms at;
+        const T3 t = pixel(cur.yA[0][ch], cur.yA[1][ch], cur.yA[2][ch], nxt.yA[0][ch], nxt.yA[1][ch], nxt.yA[2][ch],
+                           cur.g[0][ch], cur.g[1][ch], cur.g[2][ch], nxt.g[0][ch], nxt.g[1][ch], nxt.g[2][ch], cur.wxs,
+                           cur.wys, cur.bxs, cur.bys, dmaskA, dnA[ch], at, kNo, do_a);
+        float nG[3] = {0.f, 0.f, 0.f}, ngxm[3] = {0.f, 0.f, 0.f};
+        float ngb = late.gb_i[ch];
+        if (do_a.value) {
+          apply_terms(accA, at);
+          const Tail o = tail(t, late.gx_i[0][ch], late.gx_i[1][ch], late.gx_i[2][ch], optA, tA, cur.c, cur.bb[ch], cur.xa0[ch]);
+          gcv += o.gc_add;
+          ngb += o.gb_add;
+          nG[0] = in_img ? o.g05v : 0.f;  // B reads zero padding outside the image
+          nG[1] = in_img ? o.d1 : 0.f;
+          nG[2] = in_img ? o.d2 : 0.f;
+          ngxm[0] = o.gxm0; ngxm[1] = o.gxm1; ngxm[2] = o.gxm2;
+        }
+#pragma unroll
+        for (int v = 0; v < 3; v++) {
+          slot[v * CM + ch][g.lane] = nG[v];
+          slot[3 * CM + v * CM + ch][g.lane] = ngxm[v];
+        }
+        slot[6 * CM + ch][g.lane] = ngb;
+      }
+      slot[7 * CM + 0][g.lane] = gcv;
+      slot[7 * CM + 1][g.lane] = accA.gwx0;
+      slot[7 * CM + 2][g.lane] = accA.gwx1;
+      slot[7 * CM + 3][g.lane] = accA.gwy0;
+      slot[7 * CM + 4][g.lane] = accA.gwy1;
+    };
+    // the barrier after row k with k % kP == kP - 1 ends the interval of rows k-kP+1 .. k
+    auto publish = [&](int k) {
+      if (k % kP == kP - 1) lds_barrier();
+    };
+    Adj2ARow<C> b0, b1, b2;
+    Adj2Late<C> late;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    load_late(1, late);
+    for (int t = 0; t < G; t++) lds_barrier();  // group 1 works one interval behind group 0
+    absorb(0, b0);
+    absorb(1, b1);
+    step(0, b0, b1, late, kNo);
+    load_row(3, b0);
+    publish(0);
+    absorb(2, b2);
+    step(1, b1, b2, late, kYes);
+    load_row(4, b1);
+    load_late(2, late);
+    publish(1);
+    absorb(3, b0);
+    step(2, b2, b0, late, kYes);
+    load_row(5, b2);
+    load_late(3, late);
+    publish(2);
+    for (int k = 3; k <= klast; k += 3) {  // cur / next rotate through (b0,b1) (b1,b2) (b2,b0)
+      absorb(k + 1, b1);
+      step(k, b0, b1, late, kYes);
+      load_row(k + 3, b0);
+      load_late(k + 1, late);
+      publish(k);
+      if (k + 1 > klast) break;
+      absorb(k + 2, b2);
+      step(k + 1, b1, b2, late, kYes);
+      load_row(k + 4, b1);
+      load_late(k + 2, late);
+      publish(k + 1);
+      if (k + 2 > klast) break;
+      absorb(k + 3, b0);
+      step(k + 2, b2, b0, late, kYes);
+      load_row(k + 5, b2);
+      load_late(k + 3, late);
+      publish(k + 2);
+    }
+    if (klast % kP != kP - 1) lds_barrier();    // the last interval was a short one
+    for (int t = G; t < 2; t++) lds_barrier();  // the intervals in which only the wavefronts behind still work
+  };
+
+  // ------------------------------------------ step B on one group ------------------------------------------
+  auto role_b = [&](auto channels, auto group) {
+    constexpr int C = decltype(channels)::value, G = decltype(group)::value;
+    constexpr int chb = G ? CM : 0;
+    const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
+                       *const cf_p = cf + poff;
+    float *const gco_p = gc + poff, *const gwx0o_p = gwx + 2 * poff, *const gwx1o_p = gwx + 2 * poff + HW,
+                 *const gwy0o_p = gwy + 2 * poff, *const gwy1o_p = gwy + 2 * poff + HW;
+    const float *xb_p[3][C], *xc_p[C], *pv_p[2][C], *b_p[C];
+    float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      const size_t qb = ((size_t)g.n * Ct + chb + ch) * HW;
+      b_p[ch] = b + qb; gbo_p[ch] = gb + qb;
+      xc_p[ch] = x05c + (size_t)g.n * 3 * CHW + (size_t)(chb + ch) * HW;  // u of x05[j-2] (BEND: u of the checkpoint y)
+#pragma unroll
+      for (int v = 0; v < 3; v++) {
+        const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)(chb + ch) * HW;
+        xb_p[v][ch] = ((BEND && v > 0 && !TRUE_ADJ) ? x05c : x05b) + q;  // B's aux y: x05[j-1], or the checkpoint when BEND
+        if (v > 0) pv_p[v - 1][ch] = x05c + q;  // corrected gradient: the aux rows before B's
+        g05o_p[v][ch] = g05_out + q; gxm_p[v][ch] = gxk_m1 + q; gxf_p[v][ch] = FINAL ? gx_final + q : nullptr;
+      }
+    }
+    auto load_row = [&](int k, Adj2BRow<C>& in) {
+      unsigned off, off_w;
+      row_offsets(k, off, off_w);
+      in.c = ldg(cf_p, off);
+      in.wxs = ldg(wx_p, off_w);
+      in.wys = ldg(wy_p, off_w);
+      in.bxs = ldg(bx_p, off_w);
+      in.bys = ldg(by_p, off_w);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.xb0[ch] = ldg(x05b + (size_t)g.n * 3 * CHW + (size_t)(chb + ch) * HW, off);
+        in.bb[ch] = ldg(b_p[ch], off);
+        in.yB[1][ch] = ldg(xb_p[1][ch], off);
+        in.yB[2][ch] = ldg(xb_p[2][ch], off);
+        in.yB[0][ch] = ldg(xc_p[ch], off);
+        if (TRUE_ADJ) {
+          in.pv[0][ch] = ldg(pv_p[0][ch], off);
+          in.pv[1][ch] = ldg(pv_p[1][ch], off);
+        }
+      }
+    };
+    auto absorb = [&](int k, Adj2BRow<C>& o) {
+      const int h = g.hs - 2 + k;
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const inpaint::LaneMask inside(ok);
+      o.c = inside(o.c);
+      const float rc1 = rcp_refined(1.f + o.c);
+      const double opc_d = 1. + (double)o.c;
+      o.wxs = (ok && rmask) ? o.wxs : 0.f;
+      o.wys = (ok && h < H - 1) ? o.wys : 0.f;
+      o.bxs = inside(o.bxs);
+      o.bys = inside(o.bys);
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xb = inside(o.xb0[ch]), xc = inside(o.yB[0][ch]), bv = inside(o.bb[ch]);
+        if (TRUE_ADJ) {
+          const float pb = tvstrip::prox_huber1(xb, o.c, rc1, bv);
+          const float pc = BEND ? xc : tvstrip::prox_huber1(xc, o.c, rc1, bv);
+          o.yB[0][ch] = pb + tB * (pb - pc);
+        } else {
+          o.yB[0][ch] = BEND ? xc : tvstrip::rebuild_y_fast(bv, xb, xc, o.c, rc1, opc_d, tB);
+        }
+        o.xb0[ch] = xb;
+        o.bb[ch] = bv;
+#pragma unroll
+        for (int v = 1; v < 3; v++) {
+          const float xv = inside(o.yB[v][ch]);
+          o.yB[v][ch] = TRUE_ADJ ? xv + tB * (xv - inside(o.pv[v - 1][ch])) : xv;
+        }
+      }
+    };
+    const std::integral_constant<bool, BEND && !TRUE_ADJ> kBEnd{};  // the corrected gradient has one arithmetic form
+    float dnB[C][6];
+    // row k-1 as step B sees it
+    float pG[3][C], pgxm[3][C], pyB[3][C], pxb0[C], pbb[C], pgb[C], pgc = 0.f;
+    Acc pacc{0.f, 0.f, 0.f, 0.f};
+    float pc = 0.f, pwxs = 0.f, pwys = 0.f, pbxs = 0.f, pbys = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      pxb0[ch] = pbb[ch] = pgb[ch] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 6; i++) dnB[ch][i] = 0.f;
+#pragma unroll
+      for (int v = 0; v < 3; v++) pG[v][ch] = pgxm[v][ch] = pyB[v][ch] = 0.f;
+    }
+
+    auto step = [&](int k, const Adj2BRow<C>& cur, auto tri_b, auto do_b) {
+      const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
+      const bool dmaskB = h - 1 >= 0 && h - 1 < H - 1;
+      const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+      const float (*slot)[64] = handA[G][k % kSlots];
+      float (*tf)[64] = termF[k % kSlots];
+      double (*td)[64] = termD[k % kSlots];
+      float nG[3][C], ngxm[3][C], ngb[C];
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+#pragma unroll
+        for (int v = 0; v < 3; v++) {
+          nG[v][ch] = slot[v * CM + ch][g.lane];
+          ngxm[v][ch] = slot[3 * CM + v * CM + ch][g.lane];
+        }
+        ngb[ch] = slot[6 * CM + ch][g.lane];
+      }
+      float gcv = 0.f;
+      Acc accA{0.f, 0.f, 0.f, 0.f};
+      if (G == 1) {  // the row's accumulators with every A term added
+        gcv = slot[7 * CM + 0][g.lane];
+        accA = Acc{slot[7 * CM + 1][g.lane], slot[7 * CM + 2][g.lane], slot[7 * CM + 3][g.lane], slot[7 * CM + 4][g.lane]};
+      }
+      if (tri_b.value) {
+        float gcB = pgc;
+        Acc accB = pacc;
+        if (G == 1 && do_b.value) {  // the first group's B terms, in channel order, before this group's
+#pragma unroll
+          for (int ch = 0; ch < CM; ch++) {
+            AccTerms at;
+            at.add_wx0 = tf[5 * ch + 1][g.lane]; at.add_wy0 = tf[5 * ch + 2][g.lane];
+            at.add_wx1 = tf[5 * ch + 3][g.lane]; at.add_wy1 = tf[5 * ch + 4][g.lane];
+            at.sub_wx0 = td[4 * ch + 0][g.lane]; at.sub_wy0 = td[4 * ch + 1][g.lane];
+            at.sub_wx1 = td[4 * ch + 2][g.lane]; at.sub_wy1 = td[4 * ch + 3][g.lane];
+            apply_terms(accB, at);
+            gcB += tf[5 * ch + 0][g.lane];
+          }
+        }
+#pragma unroll
+        for (int ch = 0; ch < C; ch++) {
+          AccTerms at;
+          const T3 t = pixel(pyB[0][ch], pyB[1][ch], pyB[2][ch], cur.yB[0][ch], cur.yB[1][ch], cur.yB[2][ch], pG[0][ch],
+                             pG[1][ch], pG[2][ch], nG[0][ch], nG[1][ch], nG[2][ch], pwxs, pwys, pbxs, pbys, dmaskB,
+                             dnB[ch], at, kBEnd, do_b);
+          if (do_b.value) {
+            const Tail o = tail(t, pgxm[0][ch], pgxm[1][ch], pgxm[2][ch], optB, tB, pc, pbb[ch], pxb0[ch]);
+            if (G == 0) {
+              tf[5 * ch + 0][g.lane] = o.gc_add;
+              tf[5 * ch + 1][g.lane] = at.add_wx0; tf[5 * ch + 2][g.lane] = at.add_wy0;
+              tf[5 * ch + 3][g.lane] = at.add_wx1; tf[5 * ch + 4][g.lane] = at.add_wy1;
+              td[4 * ch + 0][g.lane] = at.sub_wx0; td[4 * ch + 1][g.lane] = at.sub_wy0;
+              td[4 * ch + 2][g.lane] = at.sub_wx1; td[4 * ch + 3][g.lane] = at.sub_wy1;
+            } else {
+              apply_terms(accB, at);
+              gcB += o.gc_add;
+            }
+            const float gbv = pgb[ch] + o.gb_add;
+            if (store_lane) {
+              if (FINAL) {
+                stg(gxf_p[0][ch], roffB, o.df);
+                stg(gxf_p[1][ch], roffB, o.d1);
+                stg(gxf_p[2][ch], roffB, o.d2);
+              }
+              stg(gxm_p[0][ch], roffB, o.gxm0);
+              stg(gxm_p[1][ch], roffB, o.gxm1);
+              stg(gxm_p[2][ch], roffB, o.gxm2);
+              stg(g05o_p[0][ch], roffB, o.g05v);
+              stg(g05o_p[1][ch], roffB, o.d1);
+              stg(g05o_p[2][ch], roffB, o.d2);
+              if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
+                seg_gb[((size_t)g.n * Ct + chb + ch) * HW + (roffB >> 2)] = gbv;
+                stg(gbo_p[ch], roffB, 0.f);
+              } else {
+                stg(gbo_p[ch], roffB, gbv);
+              }
+            }
+          }
+        }
+        if (G == 1 && do_b.value && store_lane) {
+          if (BEND) {
+            const size_t e1 = poff + (roffB >> 2), e2 = 2 * poff + (roffB >> 2);
+            seg_gc[e1] = gcB;
+            seg_gwx[e2] = accB.gwx0;
+            seg_gwx[e2 + HW] = accB.gwx1;
+            seg_gwy[e2] = accB.gwy0;
+            seg_gwy[e2 + HW] = accB.gwy1;
+            stg(gco_p, roffB, 0.f);
+            stg(gwx0o_p, roffB, 0.f);
+            stg(gwx1o_p, roffB, 0.f);
+            stg(gwy0o_p, roffB, 0.f);
+            stg(gwy1o_p, roffB, 0.f);
+          } else {
+            stg(gco_p, roffB, gcB);
+            stg(gwx0o_p, roffB, accB.gwx0);
+            stg(gwx1o_p, roffB, accB.gwx1);
+            stg(gwy0o_p, roffB, accB.gwy0);
+            stg(gwy1o_p, roffB, accB.gwy1);
+          }
+        }
+      }
+      pgc = gcv; pacc = accA;
+      pc = cur.c; pwxs = cur.wxs; pwys = cur.wys; pbxs = cur.bxs; pbys = cur.bys;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        pgb[ch] = ngb[ch]; pxb0[ch] = cur.xb0[ch]; pbb[ch] = cur.bb[ch];
+#pragma unroll
+        for (int v = 0; v < 3; v++) { pG[v][ch] = nG[v][ch]; pgxm[v][ch] = ngxm[v][ch]; pyB[v][ch] = cur.yB[v][ch]; }
+      }
+    };
+
+    // B waits before every row k with k % kP == 0 for the barrier that ended the interval in which rows k .. k+kP-1 were handed over
+    auto await = [&](int k) {
+      if (k % kP == 0) lds_barrier();
+    };
+    Adj2BRow<C> b0, b1, b2;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    for (int t = 0; t < G; t++) lds_barrier();  // group 1 works one interval behind group 0
+    await(0);
+    absorb(0, b0);
+    step(0, b0, kNo, kNo);
+    load_row(3, b0);
+    await(1);
+    absorb(1, b1);
+    step(1, b1, kNo, kNo);
+    load_row(4, b1);
+    await(2);
+    absorb(2, b2);
+    step(2, b2, kYes, kNo);
+    load_row(5, b2);
+    for (int k = 3; k <= klast; k += 3) {
+      await(k);
+      absorb(k, b0);
+      step(k, b0, kYes, kYes);
+      load_row(k + 3, b0);
+      if (k + 1 > klast) break;
+      await(k + 1);
+      absorb(k + 1, b1);
+      step(k + 1, b1, kYes, kYes);
+      load_row(k + 4, b1);
+      if (k + 2 > klast) break;
+      await(k + 2);
+      absorb(k + 2, b2);
+      step(k + 2, b2, kYes, kYes);
+      load_row(k + 5, b2);
+    }
+    for (int t = G; t < 2; t++) lds_barrier();
+  };
+
+  const std::integral_constant<int, CM> kFirst{};
+  const std::integral_constant<int, C1> kSecond{};
+  const std::integral_constant<int, 0> kG0{};
+  const std::integral_constant<int, 1> kG1{};
+  if (wave == 0) role_a(kFirst, kG0);
+  else if (wave == 1) role_a(kSecond, kG1);
+  else if (wave == 2) role_b(kFirst, kG0);
+  else role_b(kSecond, kG1);
 }
 
 

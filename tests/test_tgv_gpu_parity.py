@@ -191,7 +191,25 @@ def test_adjoint_pair_strip_heights(ext, tgv_oracle, rows, monkeypatch):
     compare("strip height %s" % rows, run_gpu(ext, d, 12, 2), ref)
 
 
-@pytest.mark.parametrize("c", [1, 2])
+@pytest.mark.parametrize("rows", ["", "1", "2", "3", "5", "8", "13", "64"])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 3, 50, 140, 12), (1, 4, 37, 121, 9), (1, 4, 3, 200, 6), (2, 3, 1, 70, 4),
+                                         (1, 4, 33, 1, 4)])
+def test_three_and_four_channels_pair_in_four_wavefronts(ext, tgv_oracle, n, c, h, w, its, rows, monkeypatch):
+    # three and four channels: the pair runs in four wavefronts of a workgroup (two channel groups; the five shared
+    # accumulators travel A0 -> A1 -> B1, which applies B0's terms first); strips shorter and taller than the image,
+    # strips of one interval and of several, ragged last strips, images narrower than the aprons
+    d = varying_inputs(n, c, h, w, seed=131 + c + h)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    if rows:
+        monkeypatch.setenv("INPAINT_TGV_ADJ_ROWS", rows)
+    got = run_gpu(ext, d, its, 2)
+    compare("four-wavefront pair c=%d %dx%d rows=%s" % (c, h, w, rows or "chosen"), got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("c", [1, 2, 3, 4])
 @pytest.mark.parametrize("its", [2, 3, 4, 5, 6, 8, 16, 17, 26])
 def test_every_pairing_of_the_reverse_sweep(ext, tgv_oracle, c, its):
     # segment lengths 2, 4, 6 ... and their mixes: first step + pairs, first + single + pairs,
@@ -346,7 +364,7 @@ def test_module_surface_and_autograd(ext, tgv_oracle):
     compare("module", (sol.detach().permute(2, 0, 1).unsqueeze(0).cpu().numpy(), got_grads, None), ref)
 
 
-@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 40, 130, 20), (1, 1, 30, 70, 9), (1, 3, 20, 64, 6)])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 40, 130, 20), (1, 1, 30, 70, 9), (1, 3, 20, 64, 6), (1, 4, 45, 70, 20)])
 def test_kept_iterates_or_recomputed_segments_give_the_same_bits(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
     # keep mode 2 (default) stores every x05 row in the forward and recomputes nothing; mode 1 keeps the last
     # segment's rows, which serve one backward; mode 0 recomputes every segment as the reference does.  A second
@@ -399,7 +417,7 @@ CORRECTED = dict(end_uses_ckpt_y=0, skip_iter0_adjoint=0, getyk_rebuild=0, scale
 
 @pytest.mark.parametrize("n,c,h,w,its", [
     (1, 2, 64, 128, 20), (2, 1, 37, 101, 9), (1, 1, 16, 64, 2), (1, 2, 1, 70, 4), (1, 1, 33, 1, 4),
-    (2, 2, 90, 200, 30), (1, 2, 21, 63, 3), (1, 3, 23, 70, 10),
+    (2, 2, 90, 200, 30), (1, 2, 21, 63, 3), (1, 3, 23, 70, 10), (2, 4, 41, 130, 20),
 ])
 def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tgv_oracle, n, c, h, w, its):
     # gradient_mode 1: y (all three variables) as the forward pass made it, no checkpoint stand-in at segment starts,
