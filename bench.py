@@ -477,6 +477,36 @@ def bench_layer(config, steps, warmup, corrected=False, keep=None, detail=True):
     return out, cfg
 
 
+def bench_channels(kind, c, steps, warmup):
+    """One TV or TGV layer at the headline's image size with c channels (the reference accepts any channel count)."""
+    import torch
+
+    from customnetworklayers_amd import workloads
+
+    ext = layer_of(kind)[0]
+    n, h, w, its = 4, 384, 1248, 100
+    make = workloads.tv_inputs if kind == "tv" else workloads.tgv_inputs
+    d = make(n, c, h, w, seed=0, conf_density=0.2)
+    t = {k: torch.from_numpy(v).to("cuda:0") for k, v in d.items()}
+
+    def step():
+        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 0)
+        return ext.backward(t["grad"], t["dx"], t["dy"], t["dc"], t["db"], its, 0)
+
+    ext.reset_id(0)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    ext.reset_id(0)
+    return {"value": round(n * h * w * its / sec / 1e6, 2), "unit": "Mpixel-iter/s", "ms_per_step": round(sec * 1e3, 4), "steps": steps,
+            "warmup": warmup, "workload": "%s inpainting fwd+bwd, N=%d, flow %dx%dx%d fp32, %d FISTA iterations" % (kind.upper(), n, c, h, w, its)}
+
+
 def copy_ceiling():
     """What a plain copy kernel over 1 GiB reaches on this GPU (read + written bytes per second)."""
     import torch
@@ -536,6 +566,12 @@ def main():
         other["config3_hierarchy"] = dict({k: o[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup")}, workload=o["config"]["workload"])
         o, _ = bench_layer(4, 3, 1, detail=False)
         other["config4_stress"] = dict(leg(o), workload=o["config"]["workload"], slot_bytes=o["config"]["slot_bytes"])
+        # more channels than the two of the configurations: time per step against (C/2) x the two-channel time
+        two = {"tv": out["ms_per_step"], "tgv": other["config2_tgv"]["ms_per_step"]}
+        for kind, c in (("tv", 4), ("tv", 8), ("tgv", 4)):
+            o = bench_channels(kind, c, 3, 1)
+            o["x_of_two_channel_time_per_channel_pair"] = round(o["ms_per_step"] / (two[kind] * c / 2), 3)
+            other["%s_%d_channels" % (kind, c)] = o
         out["other_configs"] = other
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
