@@ -36,6 +36,7 @@ def _load():
     lib.tvinpaint_profile.argtypes = [_int]
     lib.tvinpaint_profile_read.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_int)]
     lib.inpaint_selftest_math.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_uint]
+    lib.inpaint_selftest_division_pairs.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_ulonglong)]
     lib.inpaint_reload_env.restype = None
     lib.inpaint_copy_bandwidth.argtypes = [ctypes.c_longlong, _int, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     lib.tvinpaint_last_error.restype = ctypes.c_char_p

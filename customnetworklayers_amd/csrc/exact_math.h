@@ -1,43 +1,55 @@
-// Correctly rounded fp32 division and square root for operands in the layer's working range,
+// Correctly rounded fp32 division, reciprocal and square root for operands in the layer's working range,
 // cheaper than the compiler's general IEEE expansions.
 //
-// The compiler expands a / b into div_scale, rcp, four fused refinement steps, div_fmas and
-// div_fixup; the scale / fixup instructions only matter for operands near the ends of the exponent
-// range, denormals, zeros and infinities in the denominator.  The sequences below are the same
-// Newton-Raphson core (reciprocal refined once, quotient corrected twice with exact fma residuals)
-// without that range handling, so they return the same bits whenever the operands are ordinary:
+// The compiler expands a / b into div_scale, rcp, four fused refinement steps, div_fmas and div_fixup (one
+// refinement of the reciprocal, two corrections of the quotient); the scale / fixup instructions only matter for
+// operands near the ends of the exponent range, denormals, zeros and infinities in the denominator.  The sequences
+// below drop that range handling AND the second correction of the quotient:
+//   r = rcp(d) refined once        is the correctly rounded 1 / d for every float d in [2^-40, 2^40],
+//   q = n r corrected once         (q + fma(-d, q, n) r) is the correctly rounded n / d for ALL 2^46 pairs of mantissas
+//                                  (n, d in [1, 2)), hence for every pair of ordinary operands: the three operations are
+//                                  exact up to a common power of two as long as nothing underflows.
+// Both facts hold for this GPU's v_rcp_f32 and are checked exhaustively on the device against the compiler's `/`
+// (inpaint_selftest_rsqrt for the reciprocal, inpaint_selftest_division_pairs for the quotient: 7.0e13 pairs, about
+// 40 s).  They return the compiler's bits whenever the operands are ordinary:
 //   denominators here are >= 0.02 (1 + c, max(1, .), a triangle norm above delta) and finite,
 //   numerators are zero or of ordinary magnitude.
 // The reciprocal is a separate step so that several numerators can share one denominator.
+// x / c for the two Huber thresholds c = 0.1f, 0.2f needs no reciprocal instruction at all: with R = RN(1 / c)
+// (10.0f and 5.0f; |c R - 1| = 2^-26) one correction of x R is within 2^-26 ulp of x / c, and a quotient by a
+// 24-bit c is never closer than 2^-25 ulp to a rounding boundary (checked exhaustively as well).
 // exact_sqrt is v_sqrt_f32 (1 ulp) plus the one-ulp-up / one-ulp-down residual test; inputs below
 // 2^-96 would need the compiler's pre-scaling to stay exact and callers do not need them exact
 // (a triangle norm that small is far below the Huber threshold).
 //
-// inpaint_selftest_math() (C ABI) compares all three against the compiler's `/` and sqrtf on the
-// GPU: exhaustively where the domain is one float, on structured + random pairs otherwise.
+// inpaint_selftest_math() (C ABI) compares them against the compiler's `/` and sqrtf on the GPU:
+// exhaustively where the domain is one float, on structured + random pairs over a wide range of exponents otherwise.
 #pragma once
 
 #include <hip/hip_runtime.h>
 
 namespace inpaint {
 
-// reciprocal of d, refined: |r - 1/d| is far below half an ulp except in rare last-bit cases
+// reciprocal of d, refined once: the correctly rounded 1 / d
 __device__ __forceinline__ float rcp_refined(float d) {
   float r = __builtin_amdgcn_rcpf(d);
   const float e = __builtin_fmaf(-d, r, 1.0f);
   return __builtin_fmaf(e, r, r);
 }
+__device__ __forceinline__ float exact_rcp(float d) { return rcp_refined(d); }
 
 // n / d given r = rcp_refined(d)
 __device__ __forceinline__ float div_by(float n, float d, float r) {
-  float q = n * r;
-  float e = __builtin_fmaf(-d, q, n);
-  q = __builtin_fmaf(e, r, q);
-  e = __builtin_fmaf(-d, q, n);
+  const float q = n * r;
+  const float e = __builtin_fmaf(-d, q, n);
   return __builtin_fmaf(e, r, q);
 }
 
 __device__ __forceinline__ float exact_div(float n, float d) { return div_by(n, d, rcp_refined(d)); }
+
+// x / 0.1f and x / 0.2f (the Huber thresholds)
+__device__ __forceinline__ float div_by_tenth(float x) { return div_by(x, 0.1f, 10.0f); }
+__device__ __forceinline__ float div_by_fifth(float x) { return div_by(x, 0.2f, 5.0f); }
 
 __device__ __forceinline__ float exact_sqrt(float x) {
   const float s = __builtin_amdgcn_sqrtf(x);

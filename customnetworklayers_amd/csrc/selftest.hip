@@ -18,7 +18,7 @@ __device__ inline unsigned int mix(unsigned int x) {  // integer hash, good enou
 }
 
 // counts[0]: sqrt over every float in [2^-96, FLT_MAX] plus 0 and +inf
-// counts[1]: x / 0.1f over 0 and every float in [2^-96, 2^96]
+// counts[1]: div_by_tenth(x) against x / 0.1f over 0 and every float in [2^-96, 2^96]
 // counts[2]: n / d on hashed pairs, d in [2^-6, 2^40), |n| in [2^-60, 2^60) or 0, plus structured
 //            denominators (all-ones and single-bit mantissas)
 // counts[3]: shared-reciprocal form, two numerators per denominator in [1, 2^24)
@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* count
   for (unsigned long long i = tid; i <= 0x7f800000ULL; i += stride) {
     const float x = __uint_as_float((unsigned int)i);
     if (x == 0.f || x >= 1.2621774e-29f) bad0 += !same_bits(exact_sqrt(x), sqrtf(x));
-    if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) bad1 += !same_bits(exact_div(x, 0.1f), x / 0.1f);
+    if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) bad1 += !same_bits(div_by_tenth(x), x / 0.1f);
   }
   for (unsigned int k = 0; k < pair_rounds; k++) {
     const unsigned int h1 = mix(tid * 2654435761U + k * 40503U + 17U), h2 = mix(h1 ^ 0x9e3779b9U);
@@ -57,8 +57,9 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* count
 }
 
 // counts[0]: rsq_exact(x) against 1.0f / sqrtf(x) over 0 and every float in [2^-96, 2^96]
-// counts[1]: x / 0.2f over the same set (the TGV layer's Huber threshold)
-// counts[2]: 1 / m over every float m in [1, 2^40): the segment-start kernel's Huber weight
+// counts[1]: div_by_fifth(x) against x / 0.2f over the same set (the TGV layer's Huber threshold)
+// counts[2]: exact_rcp(m) against 1 / m over every float m in [2^-40, 2^40): the reciprocal that every division starts
+//            from, and the segment-start kernel's Huber weight
 // counts[3]: w / h2 on hashed pairs, w in (2^-20, 1], h2 in [2^-14, 2^6): its weight derivative
 __global__ __launch_bounds__(256) void selftest_rsqrt_kernel(unsigned long long* counts, unsigned int pair_rounds) {
   const unsigned int tid = blockIdx.x * blockDim.x + threadIdx.x;
@@ -68,9 +69,9 @@ __global__ __launch_bounds__(256) void selftest_rsqrt_kernel(unsigned long long*
     const float x = __uint_as_float((unsigned int)i);
     if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) {
       bad0 += !same_bits(tgvstrip::rsq_exact(x), 1.0f / sqrtf(x));
-      bad1 += !same_bits(exact_div(x, 0.2f), x / 0.2f);
+      bad1 += !same_bits(div_by_fifth(x), x / 0.2f);
     }
-    if (x >= 1.0f && x < 1.0995116e12f) bad2 += !same_bits(exact_div(1.0f, x), 1.0f / x);
+    if (x >= 9.094947e-13f && x < 1.0995116e12f) bad2 += !same_bits(exact_rcp(x), 1.0f / x);
   }
   for (unsigned int k = 0; k < pair_rounds; k++) {
     const unsigned int h1 = mix(tid * 2654435761U + k * 40503U + 29U), h2 = mix(h1 ^ 0x9e3779b9U);
@@ -93,6 +94,27 @@ __global__ __launch_bounds__(256) void copy_kernel(const copy_v4* __restrict__ s
     __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// Every quotient of ordinary operands is, up to a power of two, n / d with n, d in [1, 2): all 2^23 x 2^23 pairs of
+// mantissas, the library's division (reciprocal refined once, quotient corrected once) against the compiler's IEEE
+// expansion.  One thread per denominator; blockIdx.y selects a sixteenth of the numerators.
+// counts[0]: mismatches of div_by; counts[1]: mismatches of the uncorrected n * r (a check of the check: about a
+// quarter of all pairs).
+__global__ __launch_bounds__(256) void selftest_pairs_kernel(unsigned long long* counts, unsigned first_mantissa) {
+  const unsigned dm = first_mantissa + blockIdx.x * blockDim.x + threadIdx.x;
+  const float d = __uint_as_float(0x3f800000u | dm);
+  const float r = rcp_refined(d);
+  unsigned bad0 = 0, bad1 = 0;
+  const unsigned n0 = blockIdx.y * (0x800000u / 16), n1 = n0 + 0x800000u / 16;
+  for (unsigned nm = n0; nm < n1; nm++) {
+    const float n = __uint_as_float(0x3f800000u | nm);
+    const float ref = n / d;
+    bad0 += !same_bits(div_by(n, d, r), ref);
+    bad1 += !same_bits(n * r, ref);
+  }
+  if (bad0) atomicAdd(&counts[0], (unsigned long long)bad0);
+  if (bad1) atomicAdd(&counts[1], (unsigned long long)bad1);
+}
+
 int run_selftest(void (*kernel)(unsigned long long*, unsigned int), unsigned long long* host4, unsigned int rounds) {
   unsigned long long* dev = nullptr;
   INPAINT_HIP(hipMalloc((void**)&dev, 4 * sizeof(unsigned long long)));
@@ -108,6 +130,24 @@ int run_selftest(void (*kernel)(unsigned long long*, unsigned int), unsigned lon
 
 extern "C" int inpaint_selftest_rsqrt(unsigned long long* mismatches4_host, unsigned int pair_rounds) {
   return run_selftest(selftest_rsqrt_kernel, mismatches4_host, pair_rounds);
+}
+
+// Slices first_slice .. first_slice + slices - 1 of the 64 slices of 2^17 denominator mantissas each (all 2^23
+// numerator mantissas per denominator: 1.1e12 pairs and about 0.6 s per slice on an MI355X).
+extern "C" int inpaint_selftest_division_pairs(unsigned int first_slice, unsigned int slices, unsigned long long* mismatches2_host) {
+  if (first_slice >= 64 || slices < 1 || first_slice + slices > 64 || !mismatches2_host)
+    return inpaint::fail(INPAINT_ERR_ARG, "slices %u .. %u of 64", first_slice, first_slice + slices);
+  unsigned long long* dev = nullptr;
+  INPAINT_HIP(hipMalloc((void**)&dev, 2 * sizeof(unsigned long long)));
+  INPAINT_HIP(hipMemset(dev, 0, 2 * sizeof(unsigned long long)));
+  for (unsigned int s = first_slice; s < first_slice + slices; s++) {
+    hipLaunchKernelGGL(selftest_pairs_kernel, dim3((1u << 17) / 256, 16), dim3(256), 0, 0, dev, s << 17);
+    INPAINT_HIP(hipGetLastError());
+    INPAINT_HIP(hipDeviceSynchronize());  // one launch at a time: each runs for about half a second
+  }
+  INPAINT_HIP(hipMemcpy(mismatches2_host, dev, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+  INPAINT_HIP(hipFree(dev));
+  return 0;
 }
 
 extern "C" int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds) {

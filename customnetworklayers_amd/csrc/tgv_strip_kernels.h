@@ -25,6 +25,8 @@ namespace tgvstrip {
 
 using inpaint::div_by;
 using inpaint::exact_div;
+using inpaint::exact_rcp;
+using inpaint::div_by_fifth;
 using inpaint::exact_sqrt;
 using inpaint::rcp_refined;
 using tvstrip::from_left_lane;
@@ -39,6 +41,7 @@ using tvstrip::StripGeom;
 constexpr int kCols = 62;  // output columns per wavefront (lanes 0 and 63 are aprons)
 constexpr int kCols2 = 60;  // two fused forward iterations (lanes 0, 1, 62, 63 are aprons)
 constexpr float kD0 = 0.2f, kD1 = 0.2f, kD2 = 0.2f;  // TGV.cu:58-60
+static_assert(kD0 == 0.2f && kD1 == 0.2f && kD2 == 0.2f, "the segment-start form divides by the threshold with div_by_fifth");
 constexpr float kClipLocalGrad = 2000.0f;            // TGV.cu:78
 constexpr float kLocalGCMult = 0.1f;                 // TGV.cu:87
 constexpr float kLocalGXMult = 0.1f;                 // TGV.cu:89
@@ -46,7 +49,7 @@ constexpr float kLocalGXMult = 0.1f;                 // TGV.cu:89
 // 1.0f / sqrtf(x) with both operations correctly rounded; +inf at 0.  Inputs below 2^-96 may be
 // one ulp off, which no caller can see: their Huber weight is 1 either way.
 __device__ __forceinline__ float rsq_exact(float x) {
-  const float r = exact_div(1.0f, exact_sqrt(x));
+  const float r = exact_rcp(exact_sqrt(x));
   return (x == 0.0f) ? __builtin_inff() : r;
 }
 
@@ -673,7 +676,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2) {
     if (END) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
-      Wt = exact_div(1.0f, fmaxf(1.f, exact_div(hub, delta)));
+      Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
       act = hub > delta;
       hub2 = hub * hub;
       dW = exact_div(Wt, hub2);
@@ -1043,7 +1046,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
     if (end_form.value) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
-      Wt = exact_div(1.0f, fmaxf(1.f, exact_div(hub, delta)));
+      Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
       act = hub > delta;
       hub2 = hub * hub;
       dW = exact_div(Wt, hub2);
@@ -1460,7 +1463,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
     if (end_form.value) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
-      Wt = exact_div(1.0f, fmaxf(1.f, exact_div(hub, delta)));
+      Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
       act = hub > delta;
       hub2 = hub * hub;
       dW = exact_div(Wt, hub2);
@@ -2060,7 +2063,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
     if (end_form.value) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
-      Wt = exact_div(1.0f, fmaxf(1.f, exact_div(hub, delta)));
+      Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
       act = hub > delta;
       hub2 = hub * hub;
       dW = exact_div(Wt, hub2);

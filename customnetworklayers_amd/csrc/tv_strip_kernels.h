@@ -35,6 +35,7 @@ constexpr int kFwdCols = 63;      // output columns per wavefront, forward (lane
 constexpr int kAdjCols = 62;      // adjoint (lanes 0 and 63 are aprons)
 constexpr int kFwd2Cols = 60;     // two fused forward iterations (lanes 0, 1, 62, 63 are aprons)
 constexpr float kDelta = 0.1f;    // TV.cu:44
+static_assert(kDelta == 0.1f, "the forward pass divides by the threshold with div_by_tenth");
 constexpr float kL = 0.125f;      // TV.cu:1478
 constexpr float kClipLocalGrad = 10000.0f;  // TV.cu:52
 constexpr float kLocalGCMult = 0.1f;        // TV.cu:63
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip(
       const float d1 = yc - nxt.y[ch];
       const float d2 = yc - cur.yr[ch];
       const float hub = exact_sqrt(d1 * d1 * cur.wys + d2 * d2 * cur.wxs);
-      const float m = fmaxf(1.f, inpaint::exact_div(hub, kDelta));
+      const float m = fmaxf(1.f, inpaint::div_by_tenth(hub));
       const float rm = rcp_refined(m);
       const float e1 = d1 * div_by(cur.wys, m, rm);
       const float e2 = d2 * div_by(cur.wxs, m, rm);
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     const float d1 = yc - yd;
     const float d2 = yc - from_right_lane(yc);
     const float hub = exact_sqrt(d1 * d1 * wys + d2 * d2 * wxs);
-    const float m = fmaxf(1.f, inpaint::exact_div(hub, kDelta));
+    const float m = fmaxf(1.f, inpaint::div_by_tenth(hub));
     const float rm = rcp_refined(m);
     e1 = d1 * div_by(wys, m, rm);
     e2 = d2 * div_by(wxs, m, rm);

@@ -85,7 +85,7 @@ int tgvinpaint_guard_decide(int run, double av_gc, double av_running, double* mu
 int tgvinpaint_profile(int enable);
 int tgvinpaint_profile_read(double* total_ms, int* launches);
 
-/* Diagnostic, like inpaint_selftest_math: the TGV strip kernels' 1/sqrt(x), x/0.2f, 1/m and w/h^2
+/* Diagnostic, like inpaint_selftest_math: the TGV strip kernels' 1/sqrt(x), x/0.2f, the reciprocal 1/m over [2^-40, 2^40) and w/h^2
  * against the compiler's IEEE expansions on the GPU (host array of four mismatch counts, all 0). */
 int inpaint_selftest_rsqrt(unsigned long long* mismatches4_host, unsigned int pair_rounds);
 

@@ -103,10 +103,18 @@ int tvinpaint_guard_decide(int run, double av_gc, double av_running, double* mul
 int tvinpaint_profile(int enable);
 int tvinpaint_profile_read(double* total_ms, int* launches);
 
-/* Diagnostic: compares the library's cheap correctly-rounded division / square root with the
+/* Diagnostic (no counterpart in the reference): compares the library's cheap correctly-rounded division / square root with the
  * compiler's IEEE expansions on the GPU (exhaustively over single floats, on `pair_rounds` hashed
  * pairs per thread otherwise) and returns the four mismatch counts (host array).  All must be 0. */
 int inpaint_selftest_math(unsigned long long* mismatches4_host, unsigned int pair_rounds);
+
+/* Diagnostic: the library's division (reciprocal refined once, quotient corrected once) against the compiler's IEEE
+ * expansion on ALL pairs of mantissas, n / d with n, d in [1, 2) -- every quotient of ordinary operands is one of
+ * these up to a power of two.  The 2^23 denominator mantissas come in 64 slices of 2^17 (each with all 2^23
+ * numerators: 1.1e12 pairs, about 0.6 s on an MI355X); the call checks slices first_slice .. first_slice + slices - 1
+ * and returns two counts (host array): mismatches of the division, which must be 0, and mismatches of the
+ * uncorrected product n * (1 / d), about a quarter of the pairs (shows that the comparison sees a wrong last bit). */
+int inpaint_selftest_division_pairs(unsigned int first_slice, unsigned int slices, unsigned long long* mismatches2_host);
 
 /* The INPAINT_* environment variables (testing and tuning switches: kernel selection, strip heights, keep-mode
  * override and budget) are read once per process, on the first call that needs one, and again by every *_reset_id()
