@@ -654,19 +654,31 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, co
 
 // Two forward iterations in one launch (strip path only): (xin, yin) = iterate k, (xout, yout) = iterate k+2;
 // x05a / x05b receive the pre-prox values of iterations k and k+1 when given.
+// groups: the launch covers that many consecutive channel groups of C channels (one wavefront per strip and group)
 template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                                const float* b, const float* xin, float* xout, const float* yin, float* yout,
-                               float* x05a, float* x05b, float tA, float tB, bool ring, float tP) {
+                               float* x05a, float* x05b, float tA, float tB, bool ring, float tP, int groups = 1) {
   auto kern = tvstrip::tv_forward_strip2<C, false>;
   if (x05a && ring) kern = tvstrip::tv_forward_strip2<C, true, true>;
   else if (x05a) kern = tvstrip::tv_forward_strip2<C, true>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_fwd_rows, 8);
+  const int R = strip_rows(s.n * groups, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_fwd_rows, 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
-  const long long waves = (long long)sx * sy * s.n;
+  const long long waves = (long long)sx * sy * s.n * groups;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB,
-                     (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic);
+                     (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic, groups);
+}
+
+// A launch that cannot give every SIMD of the chip a wavefront lasts as long as one wavefront needs for its strip, and
+// that time is proportional to the channels the wavefront carries: such launches run one channel per wavefront.
+bool forward_split_channels(const Slot& s) {
+  if (s.ic < 2 || s.ic > kGroup) return false;
+  if (knobs().tv_fwd_split >= 0) return knobs().tv_fwd_split == 1;
+  const long long sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols;
+  // (measured, two channels, 50 iterations: 2 x 112 x 256 0.187 -> 0.162 ms per forward pass, 2 x 224 x 512 0.221 -> 0.197 ms,
+  // 2 x 448 x 1024 no difference)
+  return sx * ((s.ih + 1) / 2) * s.n <= 8ll * compute_unit_count();  // strips of two rows: at most two wavefronts per SIMD
 }
 
 bool strip_path(const Slot& s) { return !force_tile_path() && s.ic >= 1; }
@@ -681,6 +693,10 @@ bool forward_pairs(const Slot& s) {
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                          const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05a,
                          float* x05b, float tA, float tB, bool ring = false, float tP = 0.f) {
+  if (forward_split_channels(s)) {
+    launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP, s.ic);
+    return;
+  }
   for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
     const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
     float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *ga = at_channel(s, x05a, ch0), *gbb = at_channel(s, x05b, ch0);

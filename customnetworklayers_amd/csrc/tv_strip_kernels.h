@@ -297,9 +297,13 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct) {
+    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct, int groups) {
+  // groups > 1: the launch covers `groups` consecutive channel groups of C channels each, every strip once per group
+  // (forward channels never couple): small images then spread over more wavefronts, each with a shorter row step
   StripGeom g;
-  if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
+  if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N * groups, 2)) return;
+  const int ch_first = (g.n % groups) * C;
+  g.n /= groups;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
   const size_t HW = (size_t)H * W;
   const unsigned W4 = 4u * (unsigned)W;
@@ -315,7 +319,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
   float *yo_p[C], *xo_p[C], *xa_p[C], *xb_p[C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    const size_t q = ((size_t)g.n * Ct + ch) * HW;
+    const size_t q = ((size_t)g.n * Ct + ch_first + ch) * HW;
     y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
     yo_p[ch] = yout + q; xo_p[ch] = xout + q;
     xa_p[ch] = X05 ? x05a + q : nullptr; xb_p[ch] = X05 ? x05b + q : nullptr;

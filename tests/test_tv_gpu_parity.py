@@ -163,6 +163,26 @@ def test_pair_kernels_at_forced_strip_heights(ext, tv_oracle, c, rows, monkeypat
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("keep", ["0", "2"])
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 50, 140, 12), (1, 3, 37, 121, 9), (2, 4, 20, 64, 20), (1, 2, 3, 200, 6)])
+def test_forward_pairs_with_one_channel_per_wavefront(ext, tv_oracle, n, c, h, w, its, split, keep, monkeypatch):
+    # launches too small to fill the chip run the forward pairs with one channel per wavefront (all channel groups in one
+    # launch); INPAINT_TV_FWD_SPLIT forces either layout, with the iterates kept (keep mode 2: the pairs rebuild their input
+    # from the x05 rows) and recomputed (keep mode 0)
+    d = tv_inputs(n, c, h, w, seed=640 + c + h, conf_density=0.3)
+    ref = run_oracle(tv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TV_FWD_SPLIT", split)
+    monkeypatch.setenv("INPAINT_KEEP", keep)
+    from customnetworklayers_amd._lib import reload_env
+    reload_env()
+    got = run_gpu(ext, d, its, 2)
+    compare("forward split %s, keep %s, %d channels" % (split, keep, c), got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
 def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first
