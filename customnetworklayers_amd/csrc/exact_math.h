@@ -18,9 +18,9 @@
 // x / c for the two Huber thresholds c = 0.1f, 0.2f needs no reciprocal instruction at all: with R = RN(1 / c)
 // (10.0f and 5.0f; |c R - 1| = 2^-26) one correction of x R is within 2^-26 ulp of x / c, and a quotient by a
 // 24-bit c is never closer than 2^-25 ulp to a rounding boundary (checked exhaustively as well).
-// exact_sqrt is v_sqrt_f32 (1 ulp) plus the one-ulp-up / one-ulp-down residual test; inputs below
-// 2^-96 would need the compiler's pre-scaling to stay exact and callers do not need them exact
-// (a triangle norm that small is far below the Huber threshold).
+// exact_sqrt is v_rsq_f32 (1 ulp) turned into the root and corrected once; inputs below 2^-96 would need the
+// compiler's pre-scaling to stay exact and callers do not need them exact (a triangle norm that small is far below the
+// Huber threshold).
 //
 // inpaint_selftest_math() (C ABI) compares them against the compiler's `/` and sqrtf on the GPU:
 // exhaustively where the domain is one float, on structured + random pairs over a wide range of exponents otherwise.
@@ -51,17 +51,15 @@ __device__ __forceinline__ float exact_div(float n, float d) { return div_by(n, 
 __device__ __forceinline__ float div_by_tenth(float x) { return div_by(x, 0.1f, 10.0f); }
 __device__ __forceinline__ float div_by_fifth(float x) { return div_by(x, 0.2f, 5.0f); }
 
+// sqrt(x), correctly rounded, for x = 0 and every finite x >= 2^-96: v_rsq_f32 (1 ulp) gives the root x * y and half its
+// reciprocal y / 2, and one Newton correction with the exact fma residual lands on the correctly rounded value for every
+// such x (checked exhaustively).  The clamp keeps y finite at x = 0, where the root and the residual are 0.  +inf is not
+// in the domain (the product inf * 0 is NaN); smaller positive x may be one ulp off, denormals more.
 __device__ __forceinline__ float exact_sqrt(float x) {
-  const float s = __builtin_amdgcn_sqrtf(x);
-  const float s_dn = __int_as_float(__float_as_int(s) - 1);
-  const float s_up = __int_as_float(__float_as_int(s) + 1);
-  const float r_dn = __builtin_fmaf(-s_dn, s, x);
-  const float r_up = __builtin_fmaf(-s_up, s, x);
-  // x = 0 and x = +inf need no case of their own: their residuals are 0 or NaN, both tests fail and s itself
-  // (0 or +inf) is returned
-  float out = (r_dn <= 0.0f) ? s_dn : s;
-  out = (r_up > 0.0f) ? s_up : out;
-  return out;
+  const float y = __builtin_amdgcn_rsqf(fmaxf(x, 1.17549435e-38f));
+  const float s = x * y;
+  const float e = __builtin_fmaf(-s, s, x);
+  return __builtin_fmaf(e, 0.5f * y, s);
 }
 
 // Values of lanes outside the image read as +0: inside(v) is v where `ok` held and +0 elsewhere, bit for bit what

@@ -17,7 +17,7 @@ __device__ inline unsigned int mix(unsigned int x) {  // integer hash, good enou
   return x;
 }
 
-// counts[0]: sqrt over every float in [2^-96, FLT_MAX] plus 0 and +inf
+// counts[0]: sqrt over 0 and every finite float in [2^-96, FLT_MAX]
 // counts[1]: div_by_tenth(x) against x / 0.1f over 0 and every float in [2^-96, 2^96]
 // counts[2]: n / d on hashed pairs, d in [2^-6, 2^40), |n| in [2^-60, 2^60) or 0, plus structured
 //            denominators (all-ones and single-bit mantissas)
@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* count
   const unsigned int tid = blockIdx.x * blockDim.x + threadIdx.x;
   const unsigned int stride = gridDim.x * blockDim.x;
   unsigned int bad0 = 0, bad1 = 0, bad2 = 0, bad3 = 0;
-  for (unsigned long long i = tid; i <= 0x7f800000ULL; i += stride) {
+  for (unsigned long long i = tid; i < 0x7f800000ULL; i += stride) {
     const float x = __uint_as_float((unsigned int)i);
     if (x == 0.f || x >= 1.2621774e-29f) bad0 += !same_bits(exact_sqrt(x), sqrtf(x));
     if (x == 0.f || (x >= 1.2621774e-29f && x <= 7.9228163e28f)) bad1 += !same_bits(div_by_tenth(x), x / 0.1f);
