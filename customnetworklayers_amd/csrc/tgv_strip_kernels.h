@@ -409,7 +409,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
   };
 
   float upA[3][C], upB[3][C];  // terms handed down to the next row (Fa, G1y, G2y), per iteration
-  float pyB[3][C], pxB[3][C], pbb[C], pc = 0.f, pwxs = 0.f, pwys = 0.f, pbxs = 0.f, pbys = 0.f;
+  float pyB[3][C], pxB[3][C], pbb[C], pc = 0.f, prc1 = 1.f, pwxs = 0.f, pwys = 0.f, pbxs = 0.f, pbys = 0.f;
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
     pbb[ch] = 0.f;
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
     const bool storeA = store_lane && k >= 2 && k <= Reff + 1;
     const float rc1A = rcp_refined(1.f + cur.c);
-    const float rc1B = rcp_refined(1.f + pc);
+    const float rc1B = prc1;  // iteration A formed it for this row one step ago
     float nyB[3][C], nxB[3][C];
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
         }
       }
     }
-    pc = cur.c; pwxs = cur.wxs; pwys = cur.wys; pbxs = cur.bxs; pbys = cur.bys;
+    pc = cur.c; prc1 = rc1A; pwxs = cur.wxs; pwys = cur.wys; pbxs = cur.bxs; pbys = cur.bys;
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       pbb[ch] = cur.bb[ch];

@@ -396,7 +396,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
   };
 
   float upA[C], upB[C];        // triangle terms handed down to the next row, per iteration
-  float pyB[C], pxB[C], pbb[C], pc = 0.f, pwxs = 0.f, pwys = 0.f;  // row k-1 as iteration B sees it
+  float pyB[C], pxB[C], pbb[C], pc = 0.f, prc1 = 1.f, pwxs = 0.f, pwys = 0.f;  // row k-1 as iteration B sees it
 #pragma unroll
   for (int ch = 0; ch < C; ch++) upA[ch] = upB[ch] = pyB[ch] = pxB[ch] = pbb[ch] = 0.f;
 
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
     const bool storeA = store_lane && k >= 2 && k <= Reff + 1;  // A's pre-prox value, output rows only
     const float rc1A = rcp_refined(1.f + cur.c);
-    const float rc1B = rcp_refined(1.f + pc);
+    const float rc1B = prc1;  // iteration A formed it for this row one step ago
     float nyB[C], nxB[C];
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
@@ -447,7 +447,7 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
         }
       }
     }
-    pc = cur.c; pwxs = cur.wxs; pwys = cur.wys;
+    pc = cur.c; prc1 = rc1A; pwxs = cur.wxs; pwys = cur.wys;
 #pragma unroll
     for (int ch = 0; ch < C; ch++) { pyB[ch] = nyB[ch]; pxB[ch] = nxB[ch]; pbb[ch] = cur.bb[ch]; }
   };
@@ -1000,7 +1000,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
   float dA1[C], dA3[C], dA4[C], dB1[C], dB3[C], dB4[C];  // terms handed down, per step
   // row k-1 as step B sees it
   float pG[C], pgxm[C], pyB[C], pxb[C], pbb[C], pgb[C], pgc = 0.f, pgwx = 0.f, pgwy = 0.f;
-  float pc = 0.f, prc1 = 1.f, pwxs = 0.f, pwys = 0.f;
+  float pc = 0.f, prc1 = 1.f, prc2 = 1.f, pwxs = 0.f, pwys = 0.f;
   double popc_d = 1.;
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
@@ -1038,7 +1038,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
     }
     if (tri_b.value) {
       float gcB = pgc, gwxB = pgwx, gwyB = pgwy;
-      const float rc2B = rcp_refined((1.f + pc) * (1.f + pc));
+      const float rc2B = prc2;  // step A formed it for this row one step ago
 #pragma unroll
       for (int ch = 0; ch < C; ch++) {
         const Tri t = triangle(pyB[ch], cur.yB[ch], pG[ch], nG[ch], pwxs, pwys, kBEnd);
@@ -1082,7 +1082,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
       }
     }
     pgc = gcv; pgwx = gwxv; pgwy = gwyv;
-    pc = cur.c; prc1 = cur.rc1; popc_d = cur.opc_d; pwxs = cur.wxs; pwys = cur.wys;
+    pc = cur.c; prc1 = cur.rc1; prc2 = rc2A; popc_d = cur.opc_d; pwxs = cur.wxs; pwys = cur.wys;
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       pG[ch] = nG[ch]; pgxm[ch] = ngxm[ch]; pgb[ch] = ngb[ch];
