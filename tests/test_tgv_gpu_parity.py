@@ -209,6 +209,38 @@ def test_three_and_four_channels_pair_in_four_wavefronts(ext, tgv_oracle, n, c, 
         assert np.array_equal(a, b)
 
 
+REGIMES = {
+    # name: (scale of the flow, confidence values, edge-weight values, beta values)
+    "large flows": (1e4, (0.0, 0.3, 1.0), (1e-3, 1.0), (2.0,)),
+    "tiny flows": (1e-6, (0.0, 0.3, 1.0), (1e-3, 1.0), (2.0,)),
+    "confidence from 1e-8 to 1e3": (8.0, (0.0, 1e-8, 1e-3, 1.0, 1e3), (0.2, 1.0), (2.0,)),
+    "weights from 0 to 1 and beta from 1e-3 to 40": (8.0, (0.0, 0.5), (0.0, 1e-12, 1e-3, 1.0), (1e-3, 0.5, 2.0, 40.0)),
+    "flat image, no data": (0.0, (0.0,), (1.0,), (2.0,)),
+}
+
+
+@pytest.mark.parametrize("c", [1, 2, 3])
+@pytest.mark.parametrize("regime", sorted(REGIMES))
+def test_unusual_magnitudes_stay_bit_equal(ext, tgv_oracle, regime, c):
+    # as for the TV layer: magnitudes far from the benchmark's must leave every output bit-equal to the oracle
+    scale, confs, weights, betas = REGIMES[regime]
+    n, h, w, its = 2, 37, 131, 12
+    d = varying_inputs(n, c, h, w, seed=900 + c)
+    rng = np.random.default_rng(23 + c)
+    d["db"] = (d["db"] * np.float32(scale / 8.0)).astype(np.float32)
+    d["di"][:, :c] = d["db"]
+    d["di"][:, c:] *= np.float32(scale / 8.0)
+    d["dc"] = rng.choice(np.array(confs, np.float32), size=d["dc"].shape).astype(np.float32)
+    for k in ("dx", "dy"):
+        d[k][:, 0] = rng.choice(np.array(weights, np.float32), size=d[k][:, 0].shape)
+        d[k][:, 1] = rng.choice(np.array(betas, np.float32), size=d[k][:, 1].shape)
+    got, ref = run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2)
+    compare("%s, %d channels" % (regime, c), got, ref)
+    assert np.array_equal(got[0], ref[0], equal_nan=True)
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b, equal_nan=True)
+
+
 @pytest.mark.parametrize("c", [1, 2, 3, 4])
 @pytest.mark.parametrize("its", [2, 3, 4, 5, 6, 8, 16, 17, 26])
 def test_every_pairing_of_the_reverse_sweep(ext, tgv_oracle, c, its):

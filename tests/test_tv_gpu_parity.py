@@ -183,6 +183,38 @@ def test_forward_pairs_with_one_channel_per_wavefront(ext, tv_oracle, n, c, h, w
         assert np.array_equal(a, b)
 
 
+REGIMES = {
+    # name: (scale of the flow, confidence values, edge-weight values)
+    "large flows": (1e4, (0.0, 0.3, 1.0), (1e-3, 1.0)),
+    "tiny flows": (1e-6, (0.0, 0.3, 1.0), (1e-3, 1.0)),
+    "confidence from 1e-8 to 1e3": (8.0, (0.0, 1e-8, 1e-3, 1.0, 1e3), (0.2, 1.0)),
+    "weights from 0 to 50": (8.0, (0.0, 0.5), (0.0, 1e-12, 1e-3, 1.0, 50.0)),
+    "flat image, no data": (0.0, (0.0,), (1.0,)),
+}
+
+
+@pytest.mark.parametrize("c", [1, 2, 3])
+@pytest.mark.parametrize("regime", sorted(REGIMES))
+def test_unusual_magnitudes_stay_bit_equal(ext, tv_oracle, regime, c):
+    # the short division / reciprocal / square root sequences return the compiler's bits for ordinary operands; inputs far
+    # from the benchmark's magnitudes (flows of 1e4 and 1e-6 pixels, confidences and weights over many decades, zero weights,
+    # an image without any gradient) must therefore leave every output bit-equal to the oracle
+    scale, confs, weights = REGIMES[regime]
+    n, h, w, its = 2, 37, 131, 12
+    d = tv_inputs(n, c, h, w, seed=900 + c, conf_density=0.5)
+    rng = np.random.default_rng(17 + c)
+    d["db"] = (d["db"] * np.float32(scale / 8.0)).astype(np.float32)
+    d["di"] = d["db"].copy()
+    d["dc"] = rng.choice(np.array(confs, np.float32), size=d["dc"].shape).astype(np.float32)
+    d["dx"] = rng.choice(np.array(weights, np.float32), size=d["dx"].shape).astype(np.float32)
+    d["dy"] = rng.choice(np.array(weights, np.float32), size=d["dy"].shape).astype(np.float32)
+    got, ref = run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2)
+    compare("%s, %d channels" % (regime, c), got, ref)
+    assert np.array_equal(got[0], ref[0], equal_nan=True)
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b, equal_nan=True)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
 def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first
