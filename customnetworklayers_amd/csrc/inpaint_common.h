@@ -56,6 +56,7 @@ struct Knobs {
   int tv_fwd_rows = 0;            // INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strip height (0 = chosen per launch)
   int tv_adj_rows = 0;
   int tv_fwd_split = -1;          // INPAINT_TV_FWD_SPLIT=0|1: forward pairs with one channel per wavefront (-1 = by the size of the launch)
+  int tv_adj_split = -1;          // INPAINT_TV_ADJ_SPLIT=0|1: the same for the adjoint pairs of two channels
   bool tgv_px_path = false;       // INPAINT_TGV_PATH=px: the per-pixel kernels
   bool tgv_fuse = true;           // INPAINT_TGV_FUSE=0
   bool tgv_fuse_adj = true;       // INPAINT_TGV_FUSE_ADJ=0
@@ -83,6 +84,7 @@ struct Knobs {
     tv_fwd_rows = rows("INPAINT_TV_FWD_ROWS");
     tv_adj_rows = rows("INPAINT_TV_ADJ_ROWS");
     tv_fwd_split = is("INPAINT_TV_FWD_SPLIT", "1") ? 1 : (is("INPAINT_TV_FWD_SPLIT", "0") ? 0 : -1);
+    tv_adj_split = is("INPAINT_TV_ADJ_SPLIT", "1") ? 1 : (is("INPAINT_TV_ADJ_SPLIT", "0") ? 0 : -1);
     tgv_px_path = is("INPAINT_TGV_PATH", "px");
     tgv_fuse = !is("INPAINT_TGV_FUSE", "0");
     tgv_fuse_adj = !is("INPAINT_TGV_FUSE_ADJ", "0");

@@ -873,6 +873,30 @@ void launch_adjoint_pair_quad(const Slot& s, hipStream_t stream, const float* dx
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
+// Two channels, one per wavefront (one strip per 128-thread workgroup), for launches that cannot fill the chip
+bool adjoint_split_channels(const Slot& s) {
+  if (s.ic != 2) return false;
+  if (knobs().tv_adj_split >= 0) return knobs().tv_adj_split == 1;
+  const long long sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols;
+  return sx * ((s.ih + 1) / 2) * s.n <= 8ll * compute_unit_count();  // as forward_split_channels
+}
+
+template <bool BEND, bool TRUE_ADJ>
+void launch_adjoint_pair_channels(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
+                                  const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
+                                  float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
+  const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
+  auto kern = gx_final ? tvstrip::tv_adjoint_strip2c<BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2c<BEND, false, TRUE_ADJ>;
+  const int R = strip_rows(2 * s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_adj_rows, 9);
+  const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
+  const long long strips = (long long)sx * sy * s.n;
+  const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(128);
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
+                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+                     s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
+}
+
 constexpr int kPairChannels = 8;  // the most channels a pair launch holds (two groups of four)
 
 // (a pair adds step A's and step B's terms of its channels in the reference's order of summation only when the
@@ -883,6 +907,8 @@ void launch_adjoint_pair(Slot& s, hipStream_t stream, const float* dx, const flo
                          const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   if (s.ic == 1)
     launch_adjoint_pair_strip<1, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
+  else if (s.ic == 2 && adjoint_split_channels(s))
+    launch_adjoint_pair_channels<BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   else if (s.ic == 2)
     launch_adjoint_pair_strip<2, BEND, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, xc, g05_in, g05_out, gxk, gxk_m1, gx_final, tA, tB);
   else if (s.ic == 3)

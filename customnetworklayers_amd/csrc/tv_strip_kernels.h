@@ -1125,6 +1125,355 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
 }
 
 // -------------------------------------------------------------------------------------------------
+// The same two adjoint steps per launch for TWO channels with ONE CHANNEL PER WAVEFRONT (128-thread workgroup, one strip
+// per workgroup), for launches that cannot fill the chip: such a launch lasts as long as one wavefront needs for its
+// strip, and a wavefront with one channel needs half the time per row.  Both wavefronts run tv_adjoint_strip2's row loop
+// on their own channel.  The channels meet in the three shared accumulators only, which the reference sums in the order
+// A(ch 0), A(ch 1), B(ch 0), B(ch 1): wavefront 0 does not touch them but hands its terms (gc term, ux, uy of step A and
+// of step B, six floats per row and lane) through LDS to wavefront 1, which works one row step behind, reads the
+// accumulators, applies channel 0's terms before its own and stores.  One LDS-only barrier per row step; both wavefronts
+// pass klast + 2 of them.
+// -------------------------------------------------------------------------------------------------
+template <bool BEND, bool FINAL, bool TRUE_ADJ = false>
+__global__ __launch_bounds__(128) void tv_adjoint_strip2c(
+    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
+    const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
+    const float* __restrict__ x05c, const float* __restrict__ gc_in, float* __restrict__ gc,
+    const float* __restrict__ gb_in, float* __restrict__ gb, const float* __restrict__ gwx_in,
+    float* __restrict__ gwx, const float* __restrict__ gwy_in, float* __restrict__ gwy,
+    const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
+    float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
+    float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
+    float tA, float tB, int R, int strips_x, int strips_y, int Ct) {
+  constexpr int C = 1;  // channels per wavefront
+  __shared__ float terms[2][6][64];  // wavefront 0's terms of a row step: gc term, ux, uy of step A and of step B
+  StripGeom g;
+  if (!strip_geometry_block(g, kFwd2Cols, R, W, strips_x, strips_y, N, 2)) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int Reff = min(R, H - g.hs);
+  const int klast = Reff + 2;  // strip row k is image row hs - 2 + k
+  const size_t HW = (size_t)H * W;
+  const unsigned W4 = 4u * (unsigned)W;
+  const unsigned wc = g.col_ok ? 4u * g.w : 0u;
+  const bool store_lane = g.lane > 1 && g.lane < 62 && g.col_ok;
+  const bool wx_ok = g.col_ok && g.w < W - 1;
+  const double optA = 1. + (double)tA, optB = 1. + (double)tB;
+  const size_t poff = (size_t)g.n * HW;
+  const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
+  const float *const gci_p = gc_in + poff, *const gwxi_p = gwx_in + poff, *const gwyi_p = gwy_in + poff;
+  float *const gco_p = gc + poff, *const gwxo_p = gwx + poff, *const gwyo_p = gwy + poff;
+  // One base pointer per tensor (the sample's first channel); channel ch sits chs[ch] bytes further (a 32-bit
+  // offset: the host refuses planes of 2^29 pixels and more).  A pointer pair per tensor AND channel does not fit the
+  // scalar registers: the compiler parks the surplus in lanes of a vector register and re-reads it at every row.
+  const size_t q0 = ((size_t)g.n * Ct + wave) * HW;  // this wavefront's channel
+  const float *const xa_p = x05a + q0, *const xb_p = x05b + q0, *const xc_p = x05c + q0;  // x05c: x05[j-2], or the checkpoint y when BEND
+  const float *const b_p = b + q0, *const g_p = g05_in + q0, *const gxi_p = gxk + q0, *const gbi_p = gb_in + q0;
+  float *const g05o_p = g05_out + q0, *const gxm_p = gxk_m1 + q0, *const gbo_p = gb + q0;
+  float *const gxf_p = FINAL ? gx_final + q0 : nullptr;
+  unsigned chs[C];
+#pragma unroll
+  for (int ch = 0; ch < C; ch++) chs[ch] = (unsigned)ch * (4u * (unsigned)HW);
+  const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
+  const int o_lo = g.hs, o_hi = g.hs + Reff - 1;                       // output rows
+
+  auto run = [&](auto role) {
+    constexpr int ROLE = decltype(role)::value;  // 0: channel 0, hands its accumulator terms on; 1: channel 1, owns the accumulators
+    auto load_row = [&](int k, Adj2Row<C>& in) {
+      const int kk = min(k, klast + 1);
+      const int h = g.hs - 2 + kk;
+      const unsigned off = (unsigned)(h < 0 ? 0 : (h >= H ? H - 1 : h)) * W4 + wc;
+      // what a row does not need is read from a row the strip needs anyway (no extra cache lines)
+      const unsigned off_w = (unsigned)min(max(h, 0), h_hi) * W4 + wc;
+      const unsigned off_a = (unsigned)min(max(h, h_lo), h_hi) * W4 + wc;
+      const unsigned off_o = (unsigned)min(max(h, o_lo), o_hi) * W4 + wc;
+      in.c = ldg(cf_p, off);
+      in.wxs = ldg(wx_p, off_w);
+      in.wys = ldg(wy_p, off_w);
+  #pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        in.xa[ch] = ldg(xa_p, off + chs[ch]);
+        in.xb[ch] = ldg(xb_p, off + chs[ch]);
+        in.yB[ch] = ldg(xc_p, off + chs[ch]);
+        in.bb[ch] = ldg(b_p, off + chs[ch]);
+        in.g[ch] = ldg(g_p, off + chs[ch]);
+        in.gx_i[ch] = ldg(gxi_p, off_a + chs[ch]);
+        in.gb_i[ch] = ldg(gbi_p, off_o + chs[ch]);
+      }
+      in.gc_i = ldg(gci_p, off_o);
+      in.gwx_i = ldg(gwxi_p, off_o);
+      in.gwy_i = ldg(gwyi_p, off_o);
+    };
+    auto absorb = [&](int k, Adj2Row<C>& o) {
+      const int h = g.hs - 2 + k;
+      const bool ok = g.col_ok && h >= 0 && h < H;
+      const std::conditional_t<BEND, inpaint::LaneSelect, inpaint::LaneMask> inside(ok);  // (the segment-end pair is short of registers)
+      o.c = inside(o.c);
+      o.rc1 = rcp_refined(1.f + o.c);
+      o.opc_d = 1. + (double)o.c;
+      o.wxs = (ok && wx_ok) ? kL * o.wxs : 0.f;
+      o.wys = (ok && h < H - 1) ? kL * o.wys : 0.f;
+  #pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float xa = inside(o.xa[ch]), xb = inside(o.xb[ch]), xc = inside(o.yB[ch]), bv = inside(o.bb[ch]);
+        if (TRUE_ADJ) {
+          const float pa = prox_huber1(xa, o.c, o.rc1, bv), pb = prox_huber1(xb, o.c, o.rc1, bv);
+          const float pc = BEND ? xc : prox_huber1(xc, o.c, o.rc1, bv);
+          o.yA[ch] = pa + tA * (pa - pb);
+          o.yB[ch] = pb + tB * (pb - pc);
+        } else {
+          // rebuild_y_fast(bv, xa, xb, ..., tA) and rebuild_y_fast(bv, xb, xc, ..., tB) with the pieces of xb formed once
+          const RebuildPieces ra = rebuild_pieces(bv, xa, o.c, o.rc1, o.opc_d), rb = rebuild_pieces(bv, xb, o.c, o.rc1, o.opc_d);
+          o.yA[ch] = rebuild_from(ra, rb, tA);
+          o.yB[ch] = BEND ? xc : rebuild_from(rb, rebuild_pieces(bv, xc, o.c, o.rc1, o.opc_d), tB);
+        }
+        o.g[ch] = inside(o.g[ch]);
+        o.xa[ch] = xa;
+        o.xb[ch] = xb;
+        o.bb[ch] = bv;
+      }
+    };
+
+    constexpr float kGX = TRUE_ADJ ? 1.f : kLocalGXMult, kGC = TRUE_ADJ ? 1.f : kLocalGCMult;
+    struct Tri {  // everything one triangle contributes (see tv_adjoint_strip)
+      float O1, O2, O3, O4, n3, n4, l1, l3, l4, ux, uy;
+    };
+    auto triangle = [&](float yk, float yd, float gk, float gd, float wxv, float wyv, auto end_form) {
+      Tri r;
+      const float yrt = from_right_lane(yk);
+      const float grt = from_right_lane(gk);
+      const float d1 = yk - yd, d2 = yk - yrt;
+      const float a1 = d1 * d1 * wyv;
+      const float a2 = d2 * d2 * wxv;
+      const float hub = exact_sqrt(a2 + a1);
+      const bool act = hub > kDelta;
+      float nom = inpaint::exact_div(kDelta, hub);
+      float denom = inpaint::exact_div(nom, 2.f * hub * hub);
+      nom = act ? nom : 1.f;
+      denom = act ? denom : 0.f;
+      const float gpd = gk - gd, gpr = gk - grt;
+      r.O1 = gpd * (wyv * nom);
+      r.O2 = gpr * (wxv * nom);
+      const float P1 = gpd * wyv * d1;
+      const float P2 = gpr * wxv * d2;
+      const float dd = denom * 2.0f;
+      // the reference's factor dd * ((yd - yk) * wyv + (yrt - yk) * wxv) is minus this one, exactly: a - b = -(b - a),
+      // (-a) * w = -(a * w) and (-a) + (-b) = -(a + b) in IEEE arithmetic; O3, O4 carry the sign
+      const float tp = dd * (d1 * wyv + d2 * wxv);
+      const float tu = dd * d1 * wyv;
+      const float tl = dd * d2 * wxv;
+      r.O3 = -(P1 * tp);
+      r.O4 = -(P2 * tp);
+      r.n3 = P1 * tu;
+      r.n4 = P2 * tu;
+      r.l1 = from_left_lane(r.O2);
+      r.l3 = from_left_lane(P2 * tl);
+      r.l4 = from_left_lane(P1 * tl);
+      if (!end_form.value) {  // TV.cu:749-769
+        r.ux = kGX * d2 * (gpr * (nom - a2 * denom) - gpd * d2 * d1 * denom * wyv);
+        r.uy = kGX * d1 * (gpd * (nom - a1 * denom) - gpr * d1 * d2 * denom * wxv);
+      } else {  // TV.cu:1019-1037
+        const float ux_a = kGX * (gpr * d2 * (nom - a2 * denom) - gpd * d2 * d2 * d1 * denom * wyv);
+        const float uy_a = kGX * (gpd * d1 * (nom - a1 * denom) - gpr * d1 * d1 * d2 * denom * wxv);
+        r.ux = act ? ux_a : kGX * d2 * gpr;
+        r.uy = act ? uy_a : kGX * d1 * gpd;
+      }
+      return r;
+    };
+    // pixel update: J^T assembly, momentum adjoint, prox adjoint (TV.cu:668-743, 796-828)
+    auto update = [&](float gk, const Tri& t, float a1_, float a3_, float a4_, float gxv, double opt, float tmom,
+                      float conf, float rc1, float rc2, double opc_d, float bv, float xh, float& df, float& gxm,
+                      float& g05v, float& gc_add, float& gb_add) {
+      float tt = gk;
+      tt -= -a1_;
+      tt -= a3_;
+      tt -= a4_;
+      tt -= -t.l1;
+      tt -= t.l3;
+      tt -= t.l4;
+      tt -= t.O1;
+      tt -= t.O2;
+      tt -= t.O3;
+      tt -= t.O4;
+      df = (float)((double)gxv + opt * (double)tt);
+      df = fmaxf(-kClipLocalGrad, fminf(df, kClipLocalGrad));
+      gxm = -tmom * tt;
+      const float diff = bv - xh;
+      const float sign = (diff < 0) ? -1.f : 1.f;
+      const bool quad = (opc_d >= (double)(sign * diff));
+      const float opc = 1.f + conf;
+      const float gc_q = df * (div_by(bv, opc, rc1) - div_by(conf * bv + xh, opc * opc, rc2)) * kGC;
+      const float g05_q = div_by(df, opc, rc1);
+      const float gb_q = div_by(df * conf, opc, rc1) * 1.0f;
+      const bool mid = !quad && (conf >= sign * diff);
+      g05v = quad ? g05_q : (mid ? 0.f : df);
+      gc_add = quad ? gc_q : (mid ? 0.f : sign * df * kGC);
+      gb_add = quad ? gb_q : (mid ? df * 1.0f : 0.f);
+    };
+
+    float dA1[C], dA3[C], dA4[C], dB1[C], dB3[C], dB4[C];  // terms handed down, per step
+    // row k-1 as step B sees it
+    float pG[C], pgxm[C], pyB[C], pxb[C], pbb[C], pgb[C], pgc = 0.f, pgwx = 0.f, pgwy = 0.f;
+    float pc = 0.f, prc1 = 1.f, prc2 = 1.f, pwxs = 0.f, pwys = 0.f;
+    double popc_d = 1.;
+  #pragma unroll
+    for (int ch = 0; ch < C; ch++) {
+      dA1[ch] = dA3[ch] = dA4[ch] = dB1[ch] = dB3[ch] = dB4[ch] = 0.f;
+      pG[ch] = pgxm[ch] = pyB[ch] = pxb[ch] = pbb[ch] = pgb[ch] = 0.f;
+    }
+    const std::true_type kYes{};
+    const std::false_type kNo{};
+    const std::integral_constant<bool, BEND && !TRUE_ADJ> kBEnd{};  // the corrected gradient has one arithmetic form
+
+    auto step = [&](int k, const Adj2Row<C>& cur, const Adj2Row<C>& nxt, auto do_a, auto tri_b, auto do_b) {
+      const int h = g.hs - 2 + k;  // A's row; B's row is h - 1
+      const bool in_img = g.col_ok && h >= 0 && h < H;
+      const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+      float nG[C], ngxm[C], ngb[C];
+      float (*slot)[64] = terms[k & 1];
+      float gcv = cur.gc_i, gwxv = cur.gwx_i, gwyv = cur.gwy_i;
+      if (ROLE == 1 && do_a.value) {  // channel 0's terms of this row first
+        if (g.w < W - 1) gwxv = gwxv - slot[1][g.lane];
+        if (h < H - 1) gwyv = gwyv - slot[2][g.lane];
+        gcv += slot[0][g.lane];
+      }
+      const float rc2A = rcp_refined((1.f + cur.c) * (1.f + cur.c));
+  #pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const Tri t = triangle(cur.yA[ch], nxt.yA[ch], cur.g[ch], nxt.g[ch], cur.wxs, cur.wys, kNo);
+        const float a1_ = dA1[ch], a3_ = dA3[ch], a4_ = dA4[ch];
+        dA1[ch] = t.O1; dA3[ch] = t.n3; dA4[ch] = t.n4;
+        nG[ch] = 0.f; ngxm[ch] = 0.f; ngb[ch] = cur.gb_i[ch];
+        if (do_a.value) {
+          float df, gxm, g05v, gc_add, gb_add;
+          update(cur.g[ch], t, a1_, a3_, a4_, cur.gx_i[ch], optA, tA, cur.c, cur.rc1, rc2A, cur.opc_d, cur.bb[ch],
+                 cur.xa[ch], df, gxm, g05v, gc_add, gb_add);
+          if (ROLE == 1) {
+            if (g.w < W - 1) gwxv = gwxv - t.ux;
+            if (h < H - 1) gwyv = gwyv - t.uy;
+            gcv += gc_add;
+          } else {
+            slot[0][g.lane] = gc_add;
+            slot[1][g.lane] = t.ux;
+            slot[2][g.lane] = t.uy;
+          }
+          ngb[ch] += gb_add;
+          nG[ch] = in_img ? g05v : 0.f;  // B reads zero padding outside the image
+          ngxm[ch] = gxm;
+        }
+      }
+      if (tri_b.value) {
+        float gcB = pgc, gwxB = pgwx, gwyB = pgwy;
+        if (ROLE == 1 && do_b.value) {  // channel 0's terms of B's row first
+          if (g.w < W - 1) gwxB = gwxB - slot[4][g.lane];
+          if (h - 1 < H - 1) gwyB = gwyB - slot[5][g.lane];
+          gcB += slot[3][g.lane];
+        }
+        const float rc2B = prc2;  // step A formed it for this row one step ago
+  #pragma unroll
+        for (int ch = 0; ch < C; ch++) {
+          const Tri t = triangle(pyB[ch], cur.yB[ch], pG[ch], nG[ch], pwxs, pwys, kBEnd);
+          const float a1_ = dB1[ch], a3_ = dB3[ch], a4_ = dB4[ch];
+          dB1[ch] = t.O1; dB3[ch] = t.n3; dB4[ch] = t.n4;
+          if (do_b.value) {
+            float df, gxm, g05v, gc_add, gb_add;
+            update(pG[ch], t, a1_, a3_, a4_, pgxm[ch], optB, tB, pc, prc1, rc2B, popc_d, pbb[ch], pxb[ch], df, gxm, g05v,
+                   gc_add, gb_add);
+            if (ROLE == 1) {
+              if (g.w < W - 1) gwxB = gwxB - t.ux;
+              if (h - 1 < H - 1) gwyB = gwyB - t.uy;
+              gcB += gc_add;
+            } else {
+              slot[3][g.lane] = gc_add;
+              slot[4][g.lane] = t.ux;
+              slot[5][g.lane] = t.uy;
+            }
+            const float gbv = pgb[ch] + gb_add;
+            if (store_lane) {
+              if (FINAL) stg(gxf_p, roffB + chs[ch], df);
+              stg(gxm_p, roffB + chs[ch], gxm);
+              stg(g05o_p, roffB + chs[ch], g05v);
+              if (BEND) {  // segment flush, fused (TV.cu:178-218)
+                seg_gb[((size_t)g.n * Ct + wave + ch) * HW + (roffB >> 2)] = gbv;
+                stg(gbo_p, roffB + chs[ch], 0.f);
+              } else {
+                stg(gbo_p, roffB + chs[ch], gbv);
+              }
+            }
+          }
+        }
+        if (ROLE == 1 && do_b.value && store_lane) {
+          if (BEND) {
+            const size_t e = poff + (roffB >> 2);
+            seg_gc[e] = gcB;
+            seg_gwx[e] = gwxB;
+            seg_gwy[e] = gwyB;
+            stg(gco_p, roffB, 0.f);
+            stg(gwxo_p, roffB, 0.f);
+            stg(gwyo_p, roffB, 0.f);
+          } else {
+            stg(gco_p, roffB, gcB);
+            stg(gwxo_p, roffB, gwxB);
+            stg(gwyo_p, roffB, gwyB);
+          }
+        }
+      }
+      pgc = gcv; pgwx = gwxv; pgwy = gwyv;
+      pc = cur.c; prc1 = cur.rc1; prc2 = rc2A; popc_d = cur.opc_d; pwxs = cur.wxs; pwys = cur.wys;
+  #pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        pG[ch] = nG[ch]; pgxm[ch] = ngxm[ch]; pgb[ch] = ngb[ch];
+        pyB[ch] = cur.yB[ch]; pxb[ch] = cur.xb[ch]; pbb[ch] = cur.bb[ch];
+      }
+    };
+
+    Adj2Row<C> b0, b1, b2, b3;
+    load_row(0, b0);
+    load_row(1, b1);
+    load_row(2, b2);
+    load_row(3, b3);
+    if (ROLE == 1) lds_barrier();  // one row step behind wavefront 0
+    absorb(0, b0);
+    absorb(1, b1);
+    step(0, b0, b1, kNo, kNo, kNo);
+    lds_barrier();
+    load_row(4, b0);
+    absorb(2, b2);
+    step(1, b1, b2, kYes, kNo, kNo);
+    lds_barrier();
+    load_row(5, b1);
+    absorb(3, b3);
+    step(2, b2, b3, kYes, kYes, kNo);
+    lds_barrier();
+    load_row(6, b2);
+    for (int k = 3; k <= klast; k += 4) {  // cur / next rotate through (b3,b0) (b0,b1) (b1,b2) (b2,b3)
+      absorb(k + 1, b0);
+      step(k, b3, b0, kYes, kYes, kYes);
+      lds_barrier();
+      load_row(k + 4, b3);
+      if (k + 1 > klast) break;
+      absorb(k + 2, b1);
+      step(k + 1, b0, b1, kYes, kYes, kYes);
+      lds_barrier();
+      load_row(k + 5, b0);
+      if (k + 2 > klast) break;
+      absorb(k + 3, b2);
+      step(k + 2, b1, b2, kYes, kYes, kYes);
+      lds_barrier();
+      load_row(k + 6, b1);
+      if (k + 3 > klast) break;
+      absorb(k + 4, b3);
+      step(k + 3, b2, b3, kYes, kYes, kYes);
+      lds_barrier();
+      load_row(k + 7, b2);
+    }
+
+    if (ROLE == 0) lds_barrier();  // wavefront 1's last row step
+  };
+  if (wave == 0) run(std::integral_constant<int, 0>{});
+  else run(std::integral_constant<int, 1>{});
+}
+
+// -------------------------------------------------------------------------------------------------
 // Two adjoint steps per launch in TWO wavefronts of a 128-thread workgroup (one strip per workgroup),
 // for the channel counts whose two steps do not fit one wavefront's registers (3 and 4).  Same
 // arithmetic, same rows and lanes as tv_adjoint_strip2: wavefront 0 runs step A (iteration j) on row

@@ -147,14 +147,18 @@ def test_five_to_eight_channels_pair_in_four_wavefronts(ext, tv_oracle, n, c, h,
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("split", ["0", "1"])
 @pytest.mark.parametrize("c", [2, 3, 4, 5, 8])
-@pytest.mark.parametrize("rows", ["3", "8", "13", "64"])
-def test_pair_kernels_at_forced_strip_heights(ext, tv_oracle, c, rows, monkeypatch):
-    # INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strips shorter and taller than the image, ragged last strips
+@pytest.mark.parametrize("rows", ["1", "3", "8", "13", "64"])
+def test_pair_kernels_at_forced_strip_heights(ext, tv_oracle, c, rows, split, monkeypatch):
+    # INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strips shorter and taller than the image, ragged last strips; all channels
+    # per wavefront and one channel per wavefront (forward pairs up to four channels, adjoint pairs at two)
     d = tv_inputs(2, c, 50, 140, seed=610 + c, conf_density=0.3)
     ref = run_oracle(tv_oracle, d, 12, 2)
     monkeypatch.setenv("INPAINT_TV_FWD_ROWS", rows)
     monkeypatch.setenv("INPAINT_TV_ADJ_ROWS", rows)
+    monkeypatch.setenv("INPAINT_TV_FWD_SPLIT", split)
+    monkeypatch.setenv("INPAINT_TV_ADJ_SPLIT", split)
     from customnetworklayers_amd._lib import reload_env
     reload_env()
     got = run_gpu(ext, d, 12, 2)
@@ -165,14 +169,17 @@ def test_pair_kernels_at_forced_strip_heights(ext, tv_oracle, c, rows, monkeypat
 
 @pytest.mark.parametrize("keep", ["0", "2"])
 @pytest.mark.parametrize("split", ["0", "1"])
-@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 50, 140, 12), (1, 3, 37, 121, 9), (2, 4, 20, 64, 20), (1, 2, 3, 200, 6)])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 50, 140, 12), (1, 3, 37, 121, 9), (2, 4, 20, 64, 20), (1, 2, 3, 200, 6), (1, 2, 1, 70, 4),
+                                         (1, 2, 33, 1, 4), (2, 2, 45, 130, 17)])
 def test_forward_pairs_with_one_channel_per_wavefront(ext, tv_oracle, n, c, h, w, its, split, keep, monkeypatch):
     # launches too small to fill the chip run the forward pairs with one channel per wavefront (all channel groups in one
-    # launch); INPAINT_TV_FWD_SPLIT forces either layout, with the iterates kept (keep mode 2: the pairs rebuild their input
+    # launch) and, at two channels, the adjoint pairs likewise (channel 0's accumulator terms handed to channel 1's wavefront
+    # through LDS); INPAINT_TV_FWD_SPLIT / INPAINT_TV_ADJ_SPLIT force either layout, with the iterates kept (keep mode 2: the pairs rebuild their input
     # from the x05 rows) and recomputed (keep mode 0)
     d = tv_inputs(n, c, h, w, seed=640 + c + h, conf_density=0.3)
     ref = run_oracle(tv_oracle, d, its, 2)
     monkeypatch.setenv("INPAINT_TV_FWD_SPLIT", split)
+    monkeypatch.setenv("INPAINT_TV_ADJ_SPLIT", split)  # (two channels: the adjoint pairs likewise)
     monkeypatch.setenv("INPAINT_KEEP", keep)
     from customnetworklayers_amd._lib import reload_env
     reload_env()
@@ -455,17 +462,27 @@ def test_corrected_gradient_matches_the_oracle_with_the_same_quirks_off(ext, tv_
     dev = torch.device("cuda:0")
     t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
     try:
-        for keep in (2, 1, 0):
-            ext.reset_id(2)
-            ext.gradient_mode(2, 1)
-            ext.keep_iterates(2, keep)
-            (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
-            grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
-            got = (sol.cpu().numpy(), [g.cpu().numpy() for g in grads], None)
-            compare("corrected, keep %d" % keep, got, ref)
-            for a, b in zip(got[1], ref[1]):
-                assert np.array_equal(a, b)
+        # two channels: also with all channels in one wavefront and with one channel per wavefront forced (small launches
+        # pick the latter by themselves)
+        for split in ((None, "0", "1") if c == 2 else (None,)):
+            for name in ("INPAINT_TV_FWD_SPLIT", "INPAINT_TV_ADJ_SPLIT"):
+                if split is None:
+                    monkeypatch.delenv(name, raising=False)
+                else:
+                    monkeypatch.setenv(name, split)
+            for keep in (2, 1, 0):
+                ext.reset_id(2)  # (reads the switches again)
+                ext.gradient_mode(2, 1)
+                ext.keep_iterates(2, keep)
+                (sol,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 2)
+                grads = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 2)
+                got = (sol.cpu().numpy(), [g.cpu().numpy() for g in grads], None)
+                compare("corrected, keep %d, split %s" % (keep, split), got, ref)
+                for a, b in zip(got[1], ref[1]):
+                    assert np.array_equal(a, b)
     finally:
+        monkeypatch.delenv("INPAINT_TV_FWD_SPLIT", raising=False)
+        monkeypatch.delenv("INPAINT_TV_ADJ_SPLIT", raising=False)
         ext.reset_id(2)  # back to the reference's gradient
     compare("plain again", run_gpu(ext, d, its, 2), plain)
 
