@@ -30,7 +30,7 @@ COUNTERS = {
             files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="e333615"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
-    6: dict(traffic=(2 * 131080 + 247100) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="d1e1cc5"),
+    6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="9d70e42+"),
 }
 MEASURED_TRAFFIC_BYTES = {k: v["traffic"] for k, v in COUNTERS.items()}
 # Peak LDS rate: 128 B per clock and CU x 256 CUs x 2.4 GHz.
@@ -157,7 +157,7 @@ def bench_flowaux(args, cfg, d):
         bwd = lambda: ext.backward(t["grad"], t["vol"])  # noqa: E731
         # forward reads the histogram once (it may stop early) and writes 2; backward reads it, the upstream and writes it
         bpp = dict(forward=4 * (dd + 2), backward=4 * (2 * dd + 2), kernel=4 * (2 * dd + 2))
-        kernel = "median_rows_kernel<4,true> (backward)"
+        kernel = "median_stream_kernel<10,true> (backward)"
         shape = "histograms %dx%dx%d" % (h, w, dd)
     bpp["total"] = bpp["forward"] + bpp["backward"]  # "kernel": the dominant kernel alone
     for _ in range(args.warmup):

@@ -1126,71 +1126,111 @@ __global__ __launch_bounds__(256) void median_backward_kernel(const float* __res
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxRowBins = 255;
 
+// In: kBatch loads per lane are issued before the first of them is stored to LDS (a loop that stores each value right
+// after its load waits for memory once per element: 9 round trips per wavefront at 33 bins where one or two suffice).
 template <int VEC, bool OUT>
 __device__ __forceinline__ void stage_rows(const float* __restrict__ src, float* __restrict__ dst, float* tile, int total,
                                            int D, int Dp, int lane) {
   constexpr int kStep = 64 * VEC;
+  constexpr int kBatch = OUT ? 1 : 8;
+  if (VEC == 4 && Dp == D) {  // odd bin counts need no padding: the tile is a plain copy of the run, 16 bytes per lane and step
+    const int full = total & ~3;
+    if (OUT) {
+      for (int i = lane * 4; i < full; i += kStep) *reinterpret_cast<float4*>(dst + i) = *reinterpret_cast<const float4*>(tile + i);
+      for (int i = full + lane; i < total; i += 64) dst[i] = tile[i];
+    } else {
+      for (int i = lane * 4; i < full; i += kStep * 8) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = *reinterpret_cast<const float4*>(src + (i + u * kStep < full ? i + u * kStep : 0));
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+          if (i + u * kStep < full) *reinterpret_cast<float4*>(tile + i + u * kStep) = v[u];
+      }
+      for (int i = full + lane; i < total; i += 64) tile[i] = src[i];
+    }
+    return;
+  }
   const int qs = kStep / D, rs = kStep - qs * D;
   int i = lane * VEC;
   int px = i / D, b = i - px * D;
-  for (; i < total; i += kStep) {
-    if (VEC == 4 && i + 3 < total) {
-      float4 v;
-      if (!OUT) v = *reinterpret_cast<const float4*>(src + i);
-      float* e[4];
-      int pe = px, be = b;
+  for (; i < total; i += kStep * kBatch) {
+    float4 v4[kBatch];
+    float v1[kBatch];
+    if (!OUT) {  // unconditional loads (an index past the end re-reads the wavefront's first elements)
 #pragma unroll
-      for (int k = 0; k < 4; k++) {
-        e[k] = tile + pe * Dp + be;
-        if (++be >= D) { be = 0; pe++; }
-      }
-      if (OUT) {
-        v.x = *e[0]; v.y = *e[1]; v.z = *e[2]; v.w = *e[3];
-        *reinterpret_cast<float4*>(dst + i) = v;
-      } else {
-        *e[0] = v.x; *e[1] = v.y; *e[2] = v.z; *e[3] = v.w;
-      }
-    } else {
-      int pe = px, be = b;
-      for (int k = 0; k < VEC && i + k < total; k++) {
-        if (OUT) dst[i + k] = tile[pe * Dp + be];
-        else tile[pe * Dp + be] = src[i + k];
-        if (++be >= D) { be = 0; pe++; }
+      for (int u = 0; u < kBatch; u++) {
+        const int iu = i + u * kStep;
+        if (VEC == 4) v4[u] = *reinterpret_cast<const float4*>(src + (iu + 3 < total ? iu : 0));
+        else v1[u] = src[iu < total ? iu : 0];
       }
     }
-    b += rs;
-    px += qs;
-    if (b >= D) { b -= D; px++; }
+#pragma unroll
+    for (int u = 0; u < kBatch; u++) {
+      const int iu = i + u * kStep;
+      if (iu < total) {
+        if (VEC == 4 && iu + 3 < total) {
+          float* e[4];
+          int pe = px, be = b;
+#pragma unroll
+          for (int k = 0; k < 4; k++) {
+            e[k] = tile + pe * Dp + be;
+            if (++be >= D) { be = 0; pe++; }
+          }
+          if (OUT) {
+            float4 v;
+            v.x = *e[0]; v.y = *e[1]; v.z = *e[2]; v.w = *e[3];
+            *reinterpret_cast<float4*>(dst + iu) = v;
+          } else {
+            *e[0] = v4[u].x; *e[1] = v4[u].y; *e[2] = v4[u].z; *e[3] = v4[u].w;
+          }
+        } else {  // the run's last, partial vector (or VEC == 1)
+          int pe = px, be = b;
+          for (int k = 0; k < VEC && iu + k < total; k++) {
+            if (OUT) dst[iu + k] = tile[pe * Dp + be];
+            else tile[pe * Dp + be] = VEC == 4 ? src[iu + k] : v1[u];
+            if (++be >= D) { be = 0; pe++; }
+          }
+        }
+      }
+      b += rs;
+      px += qs;
+      if (b >= D) { b -= D; px++; }
+    }
   }
 }
 
 template <int VEC, bool BACKWARD>
 __global__ __launch_bounds__(64) void median_rows_kernel(const float* __restrict__ vol, const float* __restrict__ gin,
-                                                         float* __restrict__ res, long long P, long long HW, int D, int Dp) {
-  extern __shared__ float tile[];  // 64 rows of pitch Dp
+                                                         float* __restrict__ res, long long P, long long HW, int D, int Dp,
+                                                         long long first_tile) {
+  extern __shared__ __align__(16) float tile[];  // 64 rows of pitch Dp
   const int lane = threadIdx.x;
-  const long long p0 = (long long)blockIdx.x * 64;
+  const long long p0 = (first_tile + blockIdx.x) * 64;
   const int npx = (int)min((long long)64, P - p0);
   const int total = npx * D;
   stage_rows<VEC, false>(vol + p0 * D, nullptr, tile, total, D, Dp, lane);
   __syncthreads();
   float* row = tile + lane * Dp;
   // the walk of MM.cu:26-43 == MM.cu:59-75, without the early exit (the bins past the crossing are skipped by `found`)
+  // The crossing bin's interpolation (a double division) is formed once, after the walk: inside the loop it would run in
+  // every iteration in which ANY lane of the wavefront crosses.  The comparisons against 0.5 are the reference's
+  // (a float promoted to double compares as the float does).
   bool found = false;
   int cidx = 0;
   float score = 0.f, pmid = 1.f, alpha = 0.f;
   if (lane < npx) {
+#pragma unroll 4
     for (int c = 0; c < D; c++) {
       const float cScore = row[c];
-      const bool hit = !found && score < 0.5 && score + cScore >= 0.5;
-      if (hit) {
-        alpha = (1. - 2. * score - cScore) / (2. * cScore);  // MM.cu:34
-        pmid = cScore;
-        cidx = c;
-        found = true;
-      }
-      if (!found) score = score + cScore;
+      const float sum = score + cScore;
+      const bool hit = !found && score < 0.5f && sum >= 0.5f;
+      pmid = hit ? cScore : pmid;
+      cidx = hit ? c : cidx;
+      found = found || hit;
+      score = found ? score : sum;  // (the running sum stops in front of the crossing bin)
     }
+    if (found) alpha = (1. - 2. * score - pmid) / (2. * pmid);  // MM.cu:34
   }
   const long long p = p0 + lane;
   const long long n = p / HW, q = p - n * HW;
@@ -1207,29 +1247,132 @@ __global__ __launch_bounds__(64) void median_rows_kernel(const float* __restrict
     const float neg = -g0v / (2. * pmid);             // MM.cu:85
     const float pos = +g0v / (2. * pmid);             // MM.cu:88
     score = 0.f;
+#pragma unroll 4
     for (int c = 0; c < D; c++) {  // MM.cu:77-92; the crossing bin keeps the value of MM.cu:69
       const float cScore = row[c];
+      const float sum = score + cScore;
       float g = (found && c == cidx) ? cross : 0.f;
-      if (score + cScore < 0.5) g = neg;
-      else if (score >= 0.5) g = pos;
+      g = (sum < 0.5f) ? neg : ((score >= 0.5f) ? pos : g);
       row[c] = g;
-      score = score + cScore;
+      score = sum;
     }
   }
   __syncthreads();
   stage_rows<VEC, true>(nullptr, res + p0 * D, tile, total, D, Dp, lane);
 }
 
+// Workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight.
+__device__ __forceinline__ void lds_only_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// The same pass over FULL tiles of 64 pixels for odd bin counts up to 4 * NV - 1 (no padding: the tile in LDS is a plain
+// copy of the run), as a loop: a wavefront keeps the next tile's run in flight (NV 16-byte loads per lane, held in registers)
+// while it walks the current one.  With one tile per wavefront only a quarter of the resident wavefronts have loads in
+// flight at any time (the rest walk, store or are being launched), and the pass runs at half the rate memory allows.
+template <int NV, bool BACKWARD>
+__global__ __launch_bounds__(64) void median_stream_kernel(const float* __restrict__ vol, const float* __restrict__ gin,
+                                                           float* __restrict__ res, long long tiles, long long HW, int D) {
+  extern __shared__ __align__(16) float tile[];  // 64 rows of D floats
+  const int lane = threadIdx.x;
+  const int per = 16 * D;  // 16-byte elements of a tile
+  typedef float vec4 __attribute__((ext_vector_type(4)));  // (an array of HIP's float4 structs ends up in scratch memory)
+  vec4* tile4 = reinterpret_cast<vec4*>(tile);
+  vec4 v[NV];
+  float gn0 = 0.f, gn1 = 0.f;
+  // every load unconditional: an element past the run re-reads the lane's first one, and so does every element of the
+  // surplus fetch behind a wavefront's last tile (live = false)
+  auto fetch = [&](long long t, bool live) {
+    const vec4* src = reinterpret_cast<const vec4*>(vol) + t * per;
+    const int last = live ? per : 0;
+#pragma unroll
+    for (int u = 0; u < NV; u++) v[u] = __builtin_nontemporal_load(src + (lane + 64 * u < last ? lane + 64 * u : lane));  // read once
+    if (BACKWARD) {
+      const long long p = t * 64 + lane, n = p / HW, q = p - n * HW;
+      gn0 = gin[n * 2 * HW + q];
+      gn1 = gin[n * 2 * HW + HW + q];
+    }
+  };
+  long long t = blockIdx.x;
+  if (t >= tiles) return;
+  fetch(t, true);
+  const float* row = tile + lane * D;
+  for (; t < tiles; t += gridDim.x) {
+#pragma unroll
+    for (int u = 0; u < NV; u++)
+      if (lane + 64 * u < per) tile4[lane + 64 * u] = v[u];
+    const float g0v = gn0, g1v = gn1;
+    const long long tn = t + gridDim.x;
+    fetch(tn < tiles ? tn : t, tn < tiles);
+    lds_only_barrier();  // (a full barrier would also wait for the loads just issued)
+    bool found = false;
+    int cidx = 0;
+    float score = 0.f, pmid = 1.f, alpha = 0.f;
+#pragma unroll 4
+    for (int c = 0; c < D; c++) {  // the walk of median_rows_kernel
+      const float cScore = row[c];
+      const float sum = score + cScore;
+      const bool hit = !found && score < 0.5f && sum >= 0.5f;
+      pmid = hit ? cScore : pmid;
+      cidx = hit ? c : cidx;
+      found = found || hit;
+      score = found ? score : sum;
+    }
+    if (found) alpha = (1. - 2. * score - pmid) / (2. * pmid);  // MM.cu:34
+    if (!BACKWARD) {
+      const long long p = t * 64 + lane, n = p / HW, q = p - n * HW;
+      res[n * 2 * HW + q] = found ? (float)cidx - 0.f + alpha : 0.f;  // MM.cu:35
+      res[n * 2 * HW + HW + q] = found ? pmid : 0.f;
+    } else {
+      const float cross = g0v * alpha / (-pmid) + g1v;  // MM.cu:69
+      const float neg = -g0v / (2. * pmid);             // MM.cu:85
+      const float pos = +g0v / (2. * pmid);             // MM.cu:88
+      float* wrow = tile + lane * D;
+      score = 0.f;
+#pragma unroll 4
+      for (int c = 0; c < D; c++) {  // MM.cu:77-92; the crossing bin keeps the value of MM.cu:69
+        const float cScore = wrow[c];
+        const float sum = score + cScore;
+        float g = (found && c == cidx) ? cross : 0.f;
+        g = (sum < 0.5f) ? neg : ((score >= 0.5f) ? pos : g);
+        wrow[c] = g;
+        score = sum;
+      }
+      lds_only_barrier();
+      vec4* dst = reinterpret_cast<vec4*>(res) + t * per;
+#pragma unroll
+      for (int u = 0; u < NV; u++)
+        if (lane + 64 * u < per) dst[lane + 64 * u] = tile4[lane + 64 * u];
+    }
+    lds_only_barrier();  // the next tile overwrites the rows
+  }
+}
+
 template <bool BACKWARD>
 void launch_median_rows(const float* vol, const float* gin, float* res, long long P, long long HW, int D, bool aligned,
                         hipStream_t stream) {
   const int Dp = D | 1;
+  constexpr int kStreamNV = 10;
+  if (aligned && (D & 1) && D >= 5 && D < 4 * kStreamNV && P >= 64 && !inpaint::knobs().median_tile_per_wave) {
+    // full tiles in the streaming loop, the last partial tile (if any) below
+    const long long tiles = P / 64;
+    const long long waves = std::min<long long>(tiles, 16ll * inpaint::compute_unit_count());
+    hipLaunchKernelGGL((median_stream_kernel<kStreamNV, BACKWARD>), dim3((unsigned)waves), dim3(64), (size_t)64 * D * sizeof(float), stream,
+                       vol, gin, res, tiles, HW, D);
+    if (P % 64 == 0) return;
+    // (the kernel below takes its pixels from P and blockIdx: give it the last tile only)
+    hipLaunchKernelGGL((median_rows_kernel<4, BACKWARD>), dim3(1), dim3(64), (size_t)64 * Dp * sizeof(float), stream, vol, gin, res, P, HW, D,
+                       Dp, tiles);
+    return;
+  }
   const dim3 grid((unsigned)((P + 63) / 64)), block(64);
   const size_t lds = (size_t)64 * Dp * sizeof(float);
   if (aligned && D >= 4)
-    hipLaunchKernelGGL((median_rows_kernel<4, BACKWARD>), grid, block, lds, stream, vol, gin, res, P, HW, D, Dp);
+    hipLaunchKernelGGL((median_rows_kernel<4, BACKWARD>), grid, block, lds, stream, vol, gin, res, P, HW, D, Dp, 0ll);
   else
-    hipLaunchKernelGGL((median_rows_kernel<1, BACKWARD>), grid, block, lds, stream, vol, gin, res, P, HW, D, Dp);
+    hipLaunchKernelGGL((median_rows_kernel<1, BACKWARD>), grid, block, lds, stream, vol, gin, res, P, HW, D, Dp, 0ll);
 }
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }

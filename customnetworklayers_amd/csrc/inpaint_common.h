@@ -66,6 +66,7 @@ struct Knobs {
   int keep = -1;                  // INPAINT_KEEP=0|1|2 (INPAINT_KEEP_LAST=0 is INPAINT_KEEP=0); -1 = the id's own mode
   double keep_gb = 32.0;          // INPAINT_KEEP_GB: budget of keep mode 2
   bool quadfit_px_path = false;   // INPAINT_QUADFIT_PATH=px: one pixel per lane, no LDS windows
+  bool median_tile_per_wave = false;  // INPAINT_MEDIAN_PATH=tile: one tile of 64 pixels per wavefront for every bin count
   bool quadfit_reread = false;    // INPAINT_QUADFIT_PATH=reread: backward pass A reads the second map twice (any channel count)
   void load() {
     *this = Knobs();
@@ -99,6 +100,7 @@ struct Knobs {
     if (const char* e = getenv("INPAINT_KEEP_GB")) keep_gb = atof(e);
     quadfit_px_path = is("INPAINT_QUADFIT_PATH", "px");
     quadfit_reread = is("INPAINT_QUADFIT_PATH", "reread");
+    median_tile_per_wave = is("INPAINT_MEDIAN_PATH", "tile");
   }
 };
 struct KnobsHolder {

@@ -215,10 +215,30 @@ def check_median(med, o, vol, grad, name):
     (1, 6, 9, 300),      # beyond: the chunked kernels
     (2, 5, 7, 2),
     (1, 10, 13, 3),
+    (1, 37, 41, 39),     # the most bins the streaming kernel takes; full tiles and a partial one
+    (2, 30, 33, 5),      # the fewest
+    (3, 7, 11, 21),      # tiles of 64 pixels that straddle samples
+    (2, 50, 77, 33),
 ])
 def test_median_matches_oracle(med, flowaux_oracle, n, h, w, d):
     m = workloads.median_inputs(n, h, w, d, seed=n + h + w + d, empty_fraction=0.1)
     check_median(med, flowaux_oracle, m["vol"], m["grad"], "%dx%dx%dx%d" % (n, h, w, d))
+
+
+@pytest.mark.parametrize("n,h,w,d", [(2, 16, 20, 33), (1, 9, 31, 31), (3, 7, 11, 21)])
+def test_median_one_tile_per_wavefront_when_forced(med, flowaux_oracle, n, h, w, d, monkeypatch):
+    # odd bin counts up to 39 normally stream their full tiles through a loop that keeps the next tile's loads in flight;
+    # INPAINT_MEDIAN_PATH=tile keeps the one-tile-per-wavefront kernel (every other bin count's path) covered for them
+    from customnetworklayers_amd._lib import reload_env
+
+    m = workloads.median_inputs(n, h, w, d, seed=n + h + w + d, empty_fraction=0.1)
+    monkeypatch.setenv("INPAINT_MEDIAN_PATH", "tile")
+    reload_env()
+    try:
+        check_median(med, flowaux_oracle, m["vol"], m["grad"], "tile path %dx%dx%dx%d" % (n, h, w, d))
+    finally:
+        monkeypatch.delenv("INPAINT_MEDIAN_PATH")
+        reload_env()
 
 
 def test_median_buffers_without_16_byte_alignment(med, flowaux_oracle):
