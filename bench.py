@@ -30,7 +30,7 @@ COUNTERS = {
             files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="e333615"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
-    6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="9d70e42+"),
+    6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="26d8b66"),
 }
 MEASURED_TRAFFIC_BYTES = {k: v["traffic"] for k, v in COUNTERS.items()}
 # Peak LDS rate: 128 B per clock and CU x 256 CUs x 2.4 GHz.
