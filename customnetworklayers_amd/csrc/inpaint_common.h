@@ -529,14 +529,15 @@ static __global__ __launch_bounds__(256) void combine_segments_many(SegmentJobs 
     double t = 0.;
     int o = nseg - 1;
     for (; o >= 3; o -= 4) {  // four records in flight at a time; the additions keep their order
-      const float v0 = seg[(long long)o * n + i], v1 = seg[(long long)(o - 1) * n + i];
-      const float v2 = seg[(long long)(o - 2) * n + i], v3 = seg[(long long)(o - 3) * n + i];
+      // (the records are read once, long after they were written: non-temporal loads)
+      const float v0 = __builtin_nontemporal_load(seg + (long long)o * n + i), v1 = __builtin_nontemporal_load(seg + (long long)(o - 1) * n + i);
+      const float v2 = __builtin_nontemporal_load(seg + (long long)(o - 2) * n + i), v3 = __builtin_nontemporal_load(seg + (long long)(o - 3) * n + i);
       t = (double)v0 + t / 1.;
       t = (double)v1 + t / 1.;
       t = (double)v2 + t / 1.;
       t = (double)v3 + t / 1.;
     }
-    for (; o >= 0; o--) t = (double)seg[(long long)o * n + i] + t / 1.;
+    for (; o >= 0; o--) t = (double)__builtin_nontemporal_load(seg + (long long)o * n + i) + t / 1.;
     total[i] = t;
   }
 }
