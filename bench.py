@@ -24,10 +24,10 @@ HBM_PEAK_GBS = 8000.0
 #             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
 #   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
 COUNTERS = {
-    1: dict(traffic=(2 * 87068 + 68650) * 1024, step=(2 * 6748481 + 6242282) * 1024, lds=0, rocprof_ms=0.05247,
-            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="e333615"),
-    2: dict(traffic=(2 * 164299 + 148833) * 1024, step=(2 * 13219866 + 14762791) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.12038,
-            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="e333615"),
+    1: dict(traffic=(2 * 87069 + 68619) * 1024, step=(2 * 6745580 + 6265029) * 1024, lds=0, rocprof_ms=0.05232,
+            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="1f27574"),
+    2: dict(traffic=(2 * 164373 + 148800) * 1024, step=(2 * 13227465 + 14760773) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.12023,
+            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="1f27574"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
     6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="26d8b66"),
