@@ -548,6 +548,16 @@ static __global__ __launch_bounds__(256) void fill_zero_f32(float* __restrict__ 
     p[i] = 0.f;
 }
 
+// One source copied into two destinations (the starting point into both halves of checkpoint 0).
+static __global__ __launch_bounds__(256) void copy_twice_f32(const float* __restrict__ src, float* __restrict__ a, float* __restrict__ b,
+                                                             long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    const float v = src[i];
+    a[i] = v;
+    b[i] = v;
+  }
+}
+
 // Zero several buffers in one launch (blockIdx.y picks the buffer).
 struct ZeroList {
   void* ptr[24];
@@ -568,6 +578,28 @@ static __global__ __launch_bounds__(256) void scrub_kernel(float* __restrict__ g
        i += (long long)gridDim.x * blockDim.x) {
     const float v = g[i];
     if (!finite_value(v)) g[i] = 0.f;
+  }
+}
+
+// The start of a backward pass in one launch: the buffers of `z` zeroed (blockIdx.y < nz), the non-finite entries of the
+// caller's upstream gradient zeroed in place (blockIdx.y == nz, as scrub_kernel) and the guard's statistics of the
+// previous backward cleared (blockIdx.y == nz + 1, as guard_clear_kernel).  Launch with grid (blocks, nz + 2).
+static __global__ __launch_bounds__(256) void backward_prologue_many(ZeroList z, int nz, float* __restrict__ upstream,
+                                                                     long long upstream_n, GuardState* gs) {
+  const int job = blockIdx.y;
+  if (job < nz) {
+    uint32_t* p = static_cast<uint32_t*>(z.ptr[job]);
+    const long long n = z.bytes[job] / 4;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) p[i] = 0u;
+  } else if (job == nz) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < upstream_n; i += (long long)gridDim.x * blockDim.x) {
+      const float v = upstream[i];
+      if (!finite_value(v)) upstream[i] = 0.f;
+    }
+  } else if (blockIdx.x == 0 && threadIdx.x < 5) {
+    GuardStats zs;
+    zs.sum = 0; zs.tail_sum = 0; zs.max_bits = 0; zs.last_invalid1 = 0; zs.num_above = 0; zs.num_invalid = 0;
+    gs->stats[threadIdx.x] = zs;
   }
 }
 
@@ -603,10 +635,26 @@ struct FinalizeJobs {
   double chain_const[4];
   const double* chain_per_sample[4];
   long long per_sample[4];
+  // optional fifth job (grid.y == 5): a float tensor guarded as finalize_f32 does, with the guard's scale `f32_scale`
+  const float* f32_src = nullptr;
+  float* f32_out = nullptr;
+  long long f32_n = 0;
+  int f32_scale = 4;
 };
 static __global__ __launch_bounds__(256) void finalize_many(FinalizeJobs jobs, const GuardState* __restrict__ gs, GuardParams p,
                                                             float global_mult) {
   const int k = blockIdx.y;
+  if (k == 4) {  // (finalize_f32)
+    const double mult = gs->scale[jobs.f32_scale];
+    const float* __restrict__ src = jobs.f32_src;
+    float* __restrict__ out = jobs.f32_out;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < jobs.f32_n; i += (long long)gridDim.x * blockDim.x) {
+      float v = guard_limit(src[i], p);
+      if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
+      out[i] = 0.0f + v;
+    }
+    return;
+  }
   const double mult = gs->scale[k];
   const double* __restrict__ total = jobs.total[k];
   float* __restrict__ out = jobs.out[k];

@@ -1007,8 +1007,8 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
       hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, s.ckpt_x, (long long)F);
     }
   } else {
-    INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, FB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
-    INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, FB, hipMemcpyDeviceToDevice, stream));
+    hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
+                       (long long)F);  // checkpoint 0 = init
     // first iteration whose x05 row is kept, and the ring row of iteration k
     const int kl = s.iterations.empty() ? K : (keep == 2 ? 0 : (keep == 1 ? s.iterations.back() : K));
     auto ring_row = [&](int k) { return s.x05 + (size_t)(keep == 2 ? k : k - kl) * F; };
@@ -1122,7 +1122,6 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   const size_t F = field_count(s), P = plane_count(s);
   const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
 
-  hipLaunchKernelGGL(scrub_kernel, dim3(gF), dim3(256), 0, stream, gin, (long long)F);
   s.acc_cur = 0;
   s.accb_cur = 0;
   // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
@@ -1149,7 +1148,8 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 8; }
       z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
     }
-    hipLaunchKernelGGL(fill_zero_many, dim3(gF, k), dim3(256), 0, stream, z);
+    // one launch: these buffers zeroed, the upstream gradient scrubbed (TV.cu:1609-1623), the guard's statistics cleared
+    hipLaunchKernelGGL(backward_prologue_many, dim3(gF, k + 2), dim3(256), 0, stream, z, k, gin, (long long)F, s.guard);
   }
 
   // buffer roles of TV.cu:1638-1641: g05[0]/g05[1] and gxk[0]/gxk[1] ping-pong with the parity of
@@ -1312,7 +1312,6 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
                        s.gxk[last], s.gx_final, s.tot_gx, s.tot_gy, ic, ih, iw, (long long)P);
   }
   // output guard on the device (TV.cu:1760-1791), then scale and store (TV.cu:1795-1818)
-  hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
   const long long cnts[5] = {(long long)P, (long long)P, (long long)P, (long long)F, (long long)F};
   GuardJobs jobs;
@@ -1338,8 +1337,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     fin.chain_per_sample[k] = nullptr;
     fin.per_sample[k] = 1;
   }
-  hipLaunchKernelGGL(finalize_many, dim3(gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, corr ? 1.f : kGlobalGMult);
-  hipLaunchKernelGGL(finalize_f32, dim3(gF), dim3(256), 0, stream, s.gx_final, gi, (long long)F, s.guard, 4, kGuard);
+  fin.f32_src = s.gx_final;  // the gradient wrt the starting point, guarded as a float tensor (TV.cu:1784-1791,1816)
+  fin.f32_out = gi;
+  fin.f32_n = (long long)F;
+  fin.f32_scale = 4;
+  hipLaunchKernelGGL(finalize_many, dim3(gF, 5), dim3(256), 0, stream, fin, s.guard, kGuard, corr ? 1.f : kGlobalGMult);
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TV.cu:1829
   return 0;
