@@ -62,6 +62,7 @@ struct Knobs {
   bool tgv_fuse_adj = true;       // INPAINT_TGV_FUSE_ADJ=0
   int tgv_fwd_rows = 0;           // INPAINT_TGV_FWD_ROWS / INPAINT_TGV_ADJ_ROWS
   int tgv_adj_rows = 0;
+  int tgv_fwd_split = -1;         // INPAINT_TGV_FWD_SPLIT=0|1: forward pairs with one channel per wavefront (-1 = by the size of the launch)
   int tgv_pair_waves = 0;         // INPAINT_TGV_PAIR_WAVES=1|2 (0 = by channel count)
   int keep = -1;                  // INPAINT_KEEP=0|1|2 (INPAINT_KEEP_LAST=0 is INPAINT_KEEP=0); -1 = the id's own mode
   double keep_gb = 32.0;          // INPAINT_KEEP_GB: budget of keep mode 2
@@ -91,6 +92,7 @@ struct Knobs {
     tgv_fuse_adj = !is("INPAINT_TGV_FUSE_ADJ", "0");
     tgv_fwd_rows = rows("INPAINT_TGV_FWD_ROWS");
     tgv_adj_rows = rows("INPAINT_TGV_ADJ_ROWS");
+    tgv_fwd_split = is("INPAINT_TGV_FWD_SPLIT", "1") ? 1 : (is("INPAINT_TGV_FWD_SPLIT", "0") ? 0 : -1);
     tgv_pair_waves = is("INPAINT_TGV_PAIR_WAVES", "1") ? 1 : (is("INPAINT_TGV_PAIR_WAVES", "2") ? 2 : (getenv("INPAINT_TGV_PAIR_WAVES") ? 1 : 0));
     if (is("INPAINT_KEEP_LAST", "0")) keep = 0;
     if (const char* e = getenv("INPAINT_KEEP")) {

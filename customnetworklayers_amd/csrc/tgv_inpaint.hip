@@ -952,16 +952,27 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* c, const flo
 template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                                const float* xin_aux, float* xout, const float* yin, float* yout, float* x05a, float* x05b,
-                               bool store_x_aux, float tA, float tB, bool ring, float tP) {
+                               bool store_x_aux, float tA, float tB, bool ring, float tP, int groups = 1) {
   auto kern = tgvstrip::tgv_forward_strip2<C, false>;
   if (x05a && ring) kern = tgvstrip::tgv_forward_strip2<C, true, true>;
   else if (x05a) kern = tgvstrip::tgv_forward_strip2<C, true>;
-  const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols2, knobs().tgv_fwd_rows, 8);
+  const int R = strip_rows(s.n * groups, s.ih, s.iw, tgvstrip::kCols2, knobs().tgv_fwd_rows, 8);
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
-  const long long waves = (long long)sx * sy * s.n;
+  const long long waves = (long long)sx * sy * s.n * groups;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b,
-                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic);
+                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic, groups);
+}
+
+// One channel per wavefront, all channels in one launch (the C = 1 instantiation with the channel as a grid dimension;
+// forward channels never couple).  Unlike the TV layer this pays at every size: a wavefront with one channel needs 124
+// registers instead of 198, so four wavefronts share a SIMD instead of two, which hides more of the kernel's latency
+// than the repeated per-pixel work (c, the four weights, masks) costs: 4 x C x 384 x 1248, 100 iterations, forward pass:
+// C = 2 3.38 -> 3.33 ms, C = 4 6.93 -> 6.47 ms; 2 x 2 x 224 x 512, 50 iterations: 0.43 -> 0.32 ms.
+bool forward_split_channels(const Slot& s) {
+  if (s.ic < 2) return false;
+  if (knobs().tgv_fwd_split >= 0) return knobs().tgv_fwd_split == 1;
+  return true;
 }
 
 bool forward_pairs(const Slot& s) {
@@ -975,6 +986,10 @@ bool forward_pairs(const Slot& s) {
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                          const float* yin, float* yout, float* x05a, float* x05b, float tA, float tB,
                          const float* xin_aux = nullptr, bool store_x_aux = true, bool ring = false, float tP = 0.f) {
+  if (forward_split_channels(s)) {
+    launch_forward_pair_strip<1>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP, s.ic);
+    return;
+  }
   for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
     const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gxa = at_channel(s, xin_aux, ch0), *gyi = at_channel(s, yin, ch0);
     float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *ga = at_channel(s, x05a, ch0), *gbb = at_channel(s, x05b, ch0);

@@ -261,9 +261,14 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
     const float* __restrict__ xin, const float* __restrict__ xin_aux, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int store_x_aux, int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct) {
+    int store_x_aux, int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct,
+    int groups) {
+  // groups > 1: the launch covers `groups` consecutive channel groups of C channels each, every strip once per group
+  // (forward channels never couple)
   StripGeom g;
-  if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N, 2)) return;
+  if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N * groups, 2)) return;
+  const int ch_first = (g.n % groups) * C;
+  g.n /= groups;
   const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
   const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
@@ -279,10 +284,10 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
   float *yo_p[3][C], *xo_p[3][C], *xa_p[3][C], *xb_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
-    b_p[ch] = b + ((size_t)g.n * Ct + ch) * HW;
+    b_p[ch] = b + ((size_t)g.n * Ct + ch_first + ch) * HW;
 #pragma unroll
     for (int v = 0; v < 3; v++) {
-      const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)ch * HW;
+      const size_t q = (size_t)g.n * 3 * CHW + (size_t)v * CHW + (size_t)(ch_first + ch) * HW;
       // v1, v2 of an iterate equal the x05 rows of the iteration that made it (no prox on them): a recompute launch
       // reads them from the ring (xin_aux) instead of a second copy, and does not write that copy (store_x_aux == 0)
       y_p[v][ch] = yin + q; x_p[v][ch] = ((v > 0 && xin_aux) ? xin_aux : xin) + q;

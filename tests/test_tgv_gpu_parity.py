@@ -161,6 +161,24 @@ def test_fused_forward_strip_edges(ext, tgv_oracle, n, c, h, w, its):
     compare("%dx%dx%dx%d its=%d" % (n, c, h, w, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("keep", ["0", "2"])
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 50, 140, 12), (1, 3, 37, 121, 9), (2, 4, 20, 64, 20), (1, 2, 3, 200, 6), (1, 5, 19, 126, 10)])
+def test_forward_pairs_with_one_channel_per_wavefront(ext, tgv_oracle, n, c, h, w, its, split, keep, monkeypatch):
+    # the forward pairs run one channel per wavefront, all channels in one launch (the default from two channels on);
+    # INPAINT_TGV_FWD_SPLIT=0 keeps the launches over groups of two channels covered; with the iterates kept (the pairs
+    # rebuild their input from the x05 rows) and recomputed
+    d = varying_inputs(n, c, h, w, seed=640 + c + h)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    monkeypatch.setenv("INPAINT_TGV_FWD_SPLIT", split)
+    monkeypatch.setenv("INPAINT_KEEP", keep)
+    got = run_gpu(ext, d, its, 2)
+    compare("forward split %s, keep %s, %d channels" % (split, keep, c), got, ref)
+    assert np.array_equal(got[0], ref[0])
+    for a, b in zip(got[1], ref[1]):
+        assert np.array_equal(a, b)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 45, 130, 10)])
 def test_single_step_adjoint_strip_kernels(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
     # the reverse sweep may run two adjoint steps per launch; INPAINT_TGV_FUSE_ADJ=0 keeps the
@@ -183,11 +201,14 @@ def test_adjoint_pairs_in_one_or_two_wavefronts(ext, tgv_oracle, n, c, h, w, its
     compare("pair in %s wavefront(s) c=%d %dx%d" % (waves, c, h, w), run_gpu(ext, d, its, 2), ref)
 
 
+@pytest.mark.parametrize("split", ["0", "1"])
 @pytest.mark.parametrize("rows", ["8", "13", "64"])
-def test_adjoint_pair_strip_heights(ext, tgv_oracle, rows, monkeypatch):
+def test_adjoint_pair_strip_heights(ext, tgv_oracle, rows, split, monkeypatch):
     d = varying_inputs(2, 2, 50, 140, seed=97)
     ref = run_oracle(tgv_oracle, d, 12, 2)
     monkeypatch.setenv("INPAINT_TGV_ADJ_ROWS", rows)
+    monkeypatch.setenv("INPAINT_TGV_FWD_ROWS", rows)
+    monkeypatch.setenv("INPAINT_TGV_FWD_SPLIT", split)
     compare("strip height %s" % rows, run_gpu(ext, d, 12, 2), ref)
 
 
