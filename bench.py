@@ -24,10 +24,10 @@ HBM_PEAK_GBS = 8000.0
 #             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
 #   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
 COUNTERS = {
-    1: dict(traffic=(2 * 87069 + 68619) * 1024, step=(2 * 6745580 + 6265029) * 1024, lds=0, rocprof_ms=0.05232,
-            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="1f27574"),
-    2: dict(traffic=(2 * 164373 + 148800) * 1024, step=(2 * 13227465 + 14760773) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.12023,
-            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="1f27574"),
+    1: dict(traffic=(2 * 87073 + 68698) * 1024, step=(2 * 6738500 + 6268485) * 1024, lds=0, rocprof_ms=0.05199,
+            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="80cfba3"),
+    2: dict(traffic=(2 * 164402 + 148964) * 1024, step=(2 * 13839728 + 14761333) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.11997,
+            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="80cfba3"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
     6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="26d8b66"),
