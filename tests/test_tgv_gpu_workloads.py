@@ -74,3 +74,27 @@ def test_tgv_full_length_sample_matches_oracle(ext):
     errs = [rel(a, r) for a, r in zip(got, [sol] + list(grads))]
     print("\n[tgv 1x2x384x1248 its=100] out %.2e grads %s" % (errs[0], ["%.2e" % e for e in errs[1:]]), flush=True)
     assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3
+
+
+@pytest.mark.parametrize("c,parts", [(4, ((0, 2), (2, 4))), (3, ((0, 2), (2, 3)))])
+def test_tgv_wider_runs_contain_the_narrower_ones(ext, c, parts):
+    # 2 x C x 384 x 1248, 100 iterations with three and four channels (adjoint pairs in four wavefronts, two channel groups):
+    # the channels couple only through the gradients wrt confidence and weights, so the solution, g_b and g_init of any
+    # subset of channels must equal, bit for bit, a run on those channels alone (which takes the two- / one-wavefront kernels)
+    cfg = CONFIGS[2]
+    n = 2
+    d = tgv_inputs(n, c, cfg["h"], cfg["w"], seed=5, **cfg["gen"])
+    full = gpu_layer(ext, d, cfg["its"], 0)
+    assert all(np.isfinite(a).all() for a in full)
+    for lo, hi in parts:
+        sel = [v * c + ch for v in range(3) for ch in range(lo, hi)]  # u, v1, v2 of the chosen channels
+        sub = dict(d)
+        sub["db"] = d["db"][:, lo:hi]
+        sub["di"] = d["di"][:, sel]
+        sub["grad"] = d["grad"][:, sel]
+        part = gpu_layer(ext, sub, cfg["its"], 1)
+        np.testing.assert_array_equal(part[0], full[0][:, sel])
+        np.testing.assert_array_equal(part[4], full[4][:, lo:hi])  # g_b
+        np.testing.assert_array_equal(part[5], full[5][:, sel])    # g_init
+    ext.reset_id(0)
+    ext.reset_id(1)

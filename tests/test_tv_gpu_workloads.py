@@ -49,6 +49,25 @@ def test_headline_batch_equals_its_samples_run_alone(ext):
     np.testing.assert_array_equal(one_ch[5][0, 0], full[5][0, 0])  # g_init
 
 
+@pytest.mark.parametrize("c,parts", [(8, ((0, 4), (4, 8))), (5, ((0, 3), (3, 5))), (3, ((0, 2), (2, 3)))])
+def test_wider_runs_contain_the_narrower_ones(ext, c, parts):
+    # 2 x C x 384 x 1248, 100 iterations with 8, 5 and 3 channels (adjoint pairs in four / four / two wavefronts): the channels
+    # couple only through the gradients wrt confidence and weights, so the solution, g_b and g_init of any subset of
+    # channels must equal, bit for bit, a run on those channels alone (which takes another pair kernel)
+    cfg = CONFIGS[1]
+    d = tv_inputs(2, c, cfg["h"], cfg["w"], seed=5, **cfg["gen"])
+    full = gpu_layer(ext, d, cfg["its"], 0)
+    assert all(np.isfinite(a).all() for a in full)
+    for lo, hi in parts:
+        sub = {k: (v[:, lo:hi] if k in ("db", "di", "grad") else v) for k, v in d.items()}
+        part = gpu_layer(ext, sub, cfg["its"], 1)
+        np.testing.assert_array_equal(part[0], full[0][:, lo:hi])
+        np.testing.assert_array_equal(part[4], full[4][:, lo:hi])  # g_b
+        np.testing.assert_array_equal(part[5], full[5][:, lo:hi])  # g_init
+    ext.reset_id(0)
+    ext.reset_id(1)
+
+
 def test_stress_shape_matches_oracle(ext, tv_oracle):
     # 16 x 2 x 256 x 512, 200 iterations in the quoted workload; two samples here
     cfg = CONFIGS[4]
