@@ -31,6 +31,8 @@ def _load():
     lib.tvinpaint_schedule.argtypes = [_int, ctypes.POINTER(_int), ctypes.POINTER(_int)]
     lib.tvinpaint_step_sizes.argtypes = [_int, ctypes.POINTER(ctypes.c_float)]
     lib.tvinpaint_step_sizes.restype = None
+    lib.tvinpaint_selftest_guard.argtypes = [ctypes.c_void_p, ctypes.c_longlong, _int, _int, ctypes.c_double,
+                                             ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_guard_decide.argtypes = [_int, ctypes.c_double, ctypes.c_double,
                                            ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.tvinpaint_profile.argtypes = [_int]
@@ -51,6 +53,8 @@ def _load():
     lib.tgvinpaint_slot_bytes.argtypes = [_int]
     lib.tgvinpaint_slot_bytes.restype = ctypes.c_longlong
     lib.tgvinpaint_lipschitz.argtypes = [_int, ctypes.POINTER(ctypes.c_double), _int]
+    lib.tgvinpaint_selftest_guard.argtypes = [ctypes.c_void_p, ctypes.c_longlong, _int, _int, ctypes.c_double,
+                                              ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     lib.tgvinpaint_guard_decide.argtypes = [_int, ctypes.c_double, ctypes.c_double,
                                             ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.tgvinpaint_profile.argtypes = [_int]

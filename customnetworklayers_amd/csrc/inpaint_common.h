@@ -255,6 +255,7 @@ struct GuardState {  // lives in device memory, one per id
   double scale[5];   // multiplier chosen for the current backward (1, mult, or 0)
   double report[25]; // per tensor: mean |g|, max |g|, num_above, num_invalid, action
   GuardStats stats[5];
+  unsigned int tickets[5];  // blocks of pass 2 that have added their share of a tail sum (zero between launches)
   // pass 1 leaves per-block records here; they are combined in a fixed order (no atomics on one address, which
   // this GPU serialises at the memory side, and a mean that does not depend on the order of arrival)
   GuardStats partial[5][kGuardBlocks];
@@ -302,11 +303,12 @@ __device__ inline unsigned int wave_sum_u(unsigned int v) {
   return v;
 }
 
-// pass 1: sum, max, counts, position of the last non-finite entry (one set of atomics per block); with clamp_mean
+// pass 1: sum, max, counts, position of the last non-finite entry (one record per block); with clamp_mean
 // (TGV) an entry above max_tol enters the mean as max_tol, the TV layer's mean takes it as it is.
 // pass 2 (does nothing unless pass 1 saw a non-finite entry): sum of |g| behind the last one.
-// The five tensors of one backward in one launch each for pass 1, pass 2 and the final scaling (blockIdx.y picks
-// the tensor; blocks beyond a tensor's own grid find nothing to do).
+// pass 3: the decision.
+// The five tensors of one backward in one launch for pass 1, one for passes 2 and 3 and one for the final scaling
+// (blockIdx.y picks the tensor; blocks beyond a tensor's own grid find nothing to do).
 struct GuardJobs {
   const void* ptr[5];
   long long n[5];
@@ -397,11 +399,20 @@ __device__ __forceinline__ GuardStats guard_combine(const GuardStats* __restrict
   return r;
 }
 
+// Passes 2 and 3 of one tensor.  Pass 2 does nothing unless pass 1 saw a non-finite entry: then every block adds its
+// share of the sum of |g| behind the last one to stats->tail_sum and takes a ticket; the block with the last ticket has
+// every share in front of it and goes on to pass 3.  Without non-finite entries block 0 does.  Pass 3, one wavefront:
+// the partial records combined in a fixed order, then lane 0 turns the statistics into the tensor's multiplier and
+// updates its running mean.  Sequential running mean of the reference, av_{i+1} = (|g_i| + i av_i)/(i+1) with a
+// reset to 1000 * running mean at every non-finite entry, in closed form.
 template <class T>
-__device__ __forceinline__ void guard_tail_body(const T* __restrict__ g, long long n, const GuardStats* __restrict__ part,
-                                                GuardStats* __restrict__ st, double max_tol, bool clamp_mean) {
+__device__ __forceinline__ void guard_tail_decide_body(const T* __restrict__ g, long long n, GuardState* __restrict__ gs, int k,
+                                                       int run, const GuardParams& p, bool clamp_mean) {
+  const GuardStats* __restrict__ part = gs->partial[k];
+  GuardStats* __restrict__ st = &gs->stats[k];
   __shared__ unsigned long long s_last[4];
   __shared__ unsigned int s_invalid[4];
+  __shared__ int s_decide;
   {
     unsigned long long last = 0;
     unsigned int invalid = 0;
@@ -414,60 +425,59 @@ __device__ __forceinline__ void guard_tail_body(const T* __restrict__ g, long lo
     if ((threadIdx.x & 63) == 0) { s_last[threadIdx.x >> 6] = last; s_invalid[threadIdx.x >> 6] = invalid; }
     __syncthreads();
   }
-  if (s_invalid[0] + s_invalid[1] + s_invalid[2] + s_invalid[3] == 0) return;
-  unsigned long long last1 = s_last[0];
-  for (int k = 1; k < 4; k++) last1 = s_last[k] > last1 ? s_last[k] : last1;
-  const long long start = (long long)last1;
-  double s = 0;
-  for (long long i = start + (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    const double a = fabs((double)g[i]);
-    s += (clamp_mean && a > max_tol) ? max_tol : a;
-  }
-  s = wave_sum(s);
-  if ((threadIdx.x & 63) == 0 && s != 0) atomicAdd(&st->tail_sum, s);
-}
-
-static __global__ __launch_bounds__(256) void guard_tail_many(GuardJobs jobs, GuardState* __restrict__ gs, double max_tol,
-                                                              bool clamp_mean) {
-  const int k = blockIdx.y;
-  if (jobs.is_f32[k])
-    guard_tail_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], gs->partial[k], &gs->stats[k], max_tol, clamp_mean);
-  else
-    guard_tail_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], gs->partial[k], &gs->stats[k], max_tol, clamp_mean);
-}
-
-struct GuardCounts {
-  long long n[5];
-};
-
-// One wavefront per tensor (launch with 320 threads): combine the partial records, then lane 0 turns the
-// statistics into the tensor's multiplier and updates its running mean.  Sequential running mean of the reference,
-// av_{i+1} = (|g_i| + i av_i)/(i+1) with a reset to 1000*running mean at every non-finite entry, in closed form.
-static __global__ __launch_bounds__(320) void guard_decide_kernel(GuardState* gs, GuardCounts cnt, int run, GuardParams p) {
-  const int k = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (k >= 5 || blockIdx.x != 0) return;
-  GuardStats s = guard_combine(gs->partial[k], lane);
-  if (lane != 0) return;
-  s.tail_sum = gs->stats[k].tail_sum;  // pass 2 adds into it (cleared before pass 1)
-  gs->stats[k] = s;
-  const double n = (double)cnt.n[k];
-  double av_gc;
-  if (cnt.n[k] <= 0) {
-    av_gc = 0;
-  } else if (s.num_invalid == 0) {
-    av_gc = s.sum / n;
+  const bool any_invalid = s_invalid[0] + s_invalid[1] + s_invalid[2] + s_invalid[3] != 0;
+  if (!any_invalid) {
+    if (blockIdx.x != 0) return;
   } else {
-    av_gc = ((double)s.last_invalid1 * (gs->av[k] * 1000.) + s.tail_sum) / n;
+    unsigned long long last1 = s_last[0];
+    for (int w = 1; w < 4; w++) last1 = s_last[w] > last1 ? s_last[w] : last1;
+    double s = 0;
+    for (long long i = (long long)last1 + (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (long long)gridDim.x * blockDim.x) {
+      const double a = fabs((double)g[i]);
+      s += (clamp_mean && a > p.max_tolerance) ? p.max_tolerance : a;
+    }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0 && s != 0) atomicAdd(&st->tail_sum, s);
+    __threadfence();  // the share is visible to the device before the ticket is taken
+    __syncthreads();
+    if (threadIdx.x == 0) s_decide = atomicAdd(&gs->tickets[k], 1u) == gridDim.x - 1;
+    __syncthreads();
+    if (!s_decide) return;
+    __threadfence();
+  }
+  if (threadIdx.x >= 64) return;
+  const int lane = threadIdx.x;
+  GuardStats c = guard_combine(part, lane);
+  if (lane != 0) return;
+  // (cleared before pass 1; read where the other blocks' atomics have put it)
+  c.tail_sum = any_invalid ? atomicAdd(&st->tail_sum, 0.0) : 0.0;
+  if (any_invalid) gs->tickets[k] = 0;
+  *st = c;
+  double av_gc;
+  if (n <= 0) {
+    av_gc = 0;
+  } else if (c.num_invalid == 0) {
+    av_gc = c.sum / (double)n;
+  } else {
+    av_gc = ((double)c.last_invalid1 * (gs->av[k] * 1000.) + c.tail_sum) / (double)n;
   }
   double mult = 1.0;
-  int action = guard_decide_rule(run, av_gc, gs->av[k], mult, p);
+  const int action = guard_decide_rule(run, av_gc, gs->av[k], mult, p);
   gs->scale[k] = mult;
   gs->report[5 * k + 0] = av_gc;
-  gs->report[5 * k + 1] = __longlong_as_double((long long)s.max_bits);
-  gs->report[5 * k + 2] = s.num_above;
-  gs->report[5 * k + 3] = s.num_invalid;
+  gs->report[5 * k + 1] = __longlong_as_double((long long)c.max_bits);
+  gs->report[5 * k + 2] = c.num_above;
+  gs->report[5 * k + 3] = c.num_invalid;
   gs->report[5 * k + 4] = action;
+}
+
+// launch with grid (guard_grid(longest tensor), 5) and 256 threads
+static __global__ __launch_bounds__(256) void guard_tail_decide_many(GuardJobs jobs, GuardState* __restrict__ gs, int run,
+                                                                     GuardParams p, bool clamp_mean) {
+  const int k = blockIdx.y;
+  if (jobs.is_f32[k]) guard_tail_decide_body(static_cast<const float*>(jobs.ptr[k]), jobs.n[k], gs, k, run, p, clamp_mean);
+  else guard_tail_decide_body(static_cast<const double*>(jobs.ptr[k]), jobs.n[k], gs, k, run, p, clamp_mean);
 }
 
 static __global__ void guard_clear_kernel(GuardState* gs) {
@@ -476,6 +486,7 @@ static __global__ void guard_clear_kernel(GuardState* gs) {
     GuardStats z;
     z.sum = 0; z.tail_sum = 0; z.max_bits = 0; z.last_invalid1 = 0; z.num_above = 0; z.num_invalid = 0;
     gs->stats[k] = z;
+    gs->tickets[k] = 0;
   }
 }
 
@@ -602,6 +613,7 @@ static __global__ __launch_bounds__(256) void backward_prologue_many(ZeroList z,
     GuardStats zs;
     zs.sum = 0; zs.tail_sum = 0; zs.max_bits = 0; zs.last_invalid1 = 0; zs.num_above = 0; zs.num_invalid = 0;
     gs->stats[threadIdx.x] = zs;
+    gs->tickets[threadIdx.x] = 0;
   }
 }
 
@@ -671,6 +683,62 @@ static __global__ __launch_bounds__(256) void finalize_many(FinalizeJobs jobs, c
     const double chain = chain_per_sample ? chain_per_sample[i / per_sample] : chain_const;
     out[i] = (chain == 1.0) ? f : (float)(chain * (double)f);
   }
+}
+
+// Diagnostic: the device guard (the three kernels above, as a backward pass launches them) on one tensor handed over in
+// host memory.  `values`: n doubles, or n floats with is_f32 (then the tensor takes the slot of the gradient wrt the
+// starting point).  `out`: the n guarded values as floats (limit, kill / rescale; no global multiplier, no chain
+// factor).  result7: mean |g|, max |g|, entries above the tolerance, non-finite entries, action (0 plain / 1 rescaled
+// / 2 killed), the updated running mean, the multiplier.  Allocates and frees its own device memory.
+inline int guard_selftest(const void* values, long long n, bool is_f32, int run, double running_mean, const GuardParams& p,
+                          bool clamp_mean, float* out, double* result7) {
+  if (!values || !out || !result7 || n < 1) return fail(INPAINT_ERR_ARG, "guard selftest: null pointer or n < 1");
+  const int k = is_f32 ? 4 : 0;
+  const size_t bytes = (size_t)n * (is_f32 ? sizeof(float) : sizeof(double));
+  void* dv = nullptr;
+  float* dout = nullptr;
+  GuardState* gs = nullptr;
+  auto release = [&]() {
+    (void)hipFree(dv);
+    (void)hipFree(dout);
+    (void)hipFree(gs);
+  };
+  auto run_all = [&]() -> int {
+    INPAINT_HIP(hipMalloc(&dv, bytes));
+    INPAINT_HIP(hipMalloc((void**)&dout, (size_t)n * sizeof(float)));
+    INPAINT_HIP(hipMalloc((void**)&gs, sizeof(GuardState)));
+    INPAINT_HIP(hipMemcpy(dv, values, bytes, hipMemcpyHostToDevice));
+    INPAINT_HIP(hipMemset(gs, 0, sizeof(GuardState)));
+    INPAINT_HIP(hipMemcpy(&gs->av[k], &running_mean, sizeof(double), hipMemcpyHostToDevice));
+    GuardJobs jobs;
+    FinalizeJobs fin;
+    for (int j = 0; j < 5; j++) {
+      jobs.ptr[j] = nullptr; jobs.n[j] = 0; jobs.is_f32[j] = 0;
+      if (j < 4) {
+        fin.total[j] = nullptr; fin.out[j] = nullptr; fin.n[j] = 0;
+        fin.chain_const[j] = 1.0; fin.chain_per_sample[j] = nullptr; fin.per_sample[j] = 1;
+      }
+    }
+    jobs.ptr[k] = dv; jobs.n[k] = n; jobs.is_f32[k] = is_f32;
+    if (is_f32) {
+      fin.f32_src = static_cast<const float*>(dv); fin.f32_out = dout; fin.f32_n = n; fin.f32_scale = k;
+    } else {
+      fin.total[k] = static_cast<const double*>(dv); fin.out[k] = dout; fin.n[k] = n;
+    }
+    hipLaunchKernelGGL(guard_reduce_many, dim3(kGuardBlocks, 5), dim3(256), 0, 0, jobs, gs, p.max_tolerance, clamp_mean);
+    hipLaunchKernelGGL(guard_tail_decide_many, dim3(guard_grid(n), 5), dim3(256), 0, 0, jobs, gs, run, p, clamp_mean);
+    hipLaunchKernelGGL(finalize_many, dim3(grid_stride(n), 5), dim3(256), 0, 0, fin, gs, p, 1.f);
+    INPAINT_HIP(hipGetLastError());
+    INPAINT_HIP(hipDeviceSynchronize());
+    INPAINT_HIP(hipMemcpy(out, dout, (size_t)n * sizeof(float), hipMemcpyDeviceToHost));
+    INPAINT_HIP(hipMemcpy(result7, &gs->report[5 * k], 5 * sizeof(double), hipMemcpyDeviceToHost));
+    INPAINT_HIP(hipMemcpy(result7 + 5, &gs->av[k], sizeof(double), hipMemcpyDeviceToHost));
+    INPAINT_HIP(hipMemcpy(result7 + 6, &gs->scale[k], sizeof(double), hipMemcpyDeviceToHost));
+    return 0;
+  };
+  const int rc = run_all();
+  release();
+  return rc;
 }
 
 // Optional timing of a layer's dominant kernel with HIP events on the launch stream.  An event

@@ -1492,10 +1492,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     longest = std::max(longest, cnts[k]);
   }
   hipLaunchKernelGGL(guard_reduce_many, dim3(kGuardBlocks, 5), dim3(256), 0, stream, jobs, s.guard, kGuard.max_tolerance, true);
-  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, s.guard, kGuard.max_tolerance, true);
-  GuardCounts gcnt;
-  for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
-  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(320), 0, stream, s.guard, gcnt, s.run, kGuard);
+  hipLaunchKernelGGL(guard_tail_decide_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, s.guard, s.run, kGuard, true);
   const long long HW2 = 2LL * ih * iw;
   FinalizeJobs fin;
   float* outs[4] = {gc, gx, gy, gb};
@@ -1514,6 +1511,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TGV.cu:3061
   return 0;
+}
+
+int tgvinpaint_selftest_guard(const void* values, long long n, int is_f32, int run, double running_mean, float* out,
+                            double* result7) {
+  return guard_selftest(values, n, is_f32 != 0, run, running_mean, kGuard, true, out, result7);
 }
 
 int tgvinpaint_get_state(int id, double* state6) {

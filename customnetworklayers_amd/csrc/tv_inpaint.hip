@@ -877,8 +877,13 @@ void launch_adjoint_pair_quad(const Slot& s, hipStream_t stream, const float* dx
 bool adjoint_split_channels(const Slot& s) {
   if (s.ic != 2) return false;
   if (knobs().tv_adj_split >= 0) return knobs().tv_adj_split == 1;
+  // Split while strips of 16 rows, one wavefront for both channels, would leave the chip short of wavefronts: the
+  // unsplit kernel then has to take low strips, and walks 8 halo rows for each.  Measured, 50 iterations, backward pass
+  // unsplit -> split (16-row strips per CU in brackets): 1 x 384 x 1248 0.571 -> 0.523 ms (2.0), 2 x 384 x 1248
+  // 0.869 -> 0.855 (3.9), 2 x 448 x 1024 0.856 -> 0.850 (3.9), 4 x 300 x 900 0.959 -> 0.946 (4.5), 3 x 384 x 1248
+  // 1.191 -> 1.196 (5.9), 4 x 384 x 1248 slower (7.9).
   const long long sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols;
-  return sx * ((s.ih + 1) / 2) * s.n <= 8ll * compute_unit_count();  // as forward_split_channels
+  return sx * ((s.ih + 15) / 16) * s.n <= 5ll * compute_unit_count();
 }
 
 template <bool BEND, bool TRUE_ADJ>
@@ -1323,10 +1328,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     longest = std::max(longest, cnts[k]);
   }
   hipLaunchKernelGGL(guard_reduce_many, dim3(kGuardBlocks, 5), dim3(256), 0, stream, jobs, s.guard, kGuard.max_tolerance, false);
-  hipLaunchKernelGGL(guard_tail_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, s.guard, 0.0, false);
-  GuardCounts gcnt;
-  for (int k = 0; k < 5; k++) gcnt.n[k] = cnts[k];
-  hipLaunchKernelGGL(guard_decide_kernel, dim3(1), dim3(320), 0, stream, s.guard, gcnt, s.run, kGuard);
+  hipLaunchKernelGGL(guard_tail_decide_many, dim3(guard_grid(longest), 5), dim3(256), 0, stream, jobs, s.guard, s.run, kGuard, false);
   FinalizeJobs fin;
   float* outs[4] = {gc, gx, gy, gb};
   for (int k = 0; k < 4; k++) {
@@ -1345,6 +1347,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TV.cu:1829
   return 0;
+}
+
+int tvinpaint_selftest_guard(const void* values, long long n, int is_f32, int run, double running_mean, float* out,
+                            double* result7) {
+  return guard_selftest(values, n, is_f32 != 0, run, running_mean, kGuard, false, out, result7);
 }
 
 int tvinpaint_get_state(int id, double* state6) {

@@ -97,6 +97,17 @@ void tvinpaint_step_sizes(int its, float* out);
  * TVInpaintFista.cu:128-155).  Returns the action and writes the multiplier and the new running mean. */
 int tvinpaint_guard_decide(int run, double av_gc, double av_running, double* mult_out, double* av_out);
 
+/* Diagnostic (no counterpart in the reference as a separate call): the output guard as the backward pass runs it on
+ * the device (check_gradUpdate + update_correct_av_step_host, TVInpaintFista.cu:128-175, applied as
+ * TVInpaintFista.cu:1760-1818) on ONE tensor handed over in host memory, so that tensors with non-finite and
+ * out-of-tolerance entries can be checked.  values: n doubles, or n floats when is_f32 is set (the guard treats the
+ * gradient wrt the starting point as a float tensor).  out: the n guarded values as floats (non-finite and
+ * out-of-tolerance entries zeroed, then killed or rescaled; no further factor).  result7: mean |g| as the guard
+ * counts it, max |g|, entries above the tolerance, non-finite entries, action (0 plain / 1 rescaled / 2 killed), the
+ * updated running mean, the multiplier.  Allocates and frees its own device memory; synchronises the device. */
+int tvinpaint_selftest_guard(const void* values, long long n, int is_f32, int run, double running_mean, float* out,
+                             double* result7);
+
 /* Timing of the main adjoint kernel (the dominant one) with HIP events recorded on the launch
  * stream around every launch.  profile(1) starts collecting, profile_read waits for the recorded
  * events, returns their summed duration and count and clears the collection. */
