@@ -733,13 +733,15 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const fl
 // One group of a one-step adjoint launch.  Shared accumulators (gc, gwx, gwy): set acc_cur in, the other out, flipped
 // by the caller after every launch; per-channel accumulators (gb): set accb_cur in, the other out, flipped once per
 // step.  last_group: this launch completes the step (a segment-start step then flushes the shared accumulators).
-template <int C, bool END, bool TRUE_ADJ>
+template <int C, bool END, bool TRUE_ADJ, bool FIRST = false>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                           const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
-                          float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t, int ch0, bool last_group) {
+                          float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t, int ch0, bool last_group,
+                          const float* x05_last = nullptr) {
   const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
-  auto kern = gx_final ? tvstrip::tv_adjoint_strip<C, END, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ>;
+  auto kern = (gx_final && !FIRST) ? tvstrip::tv_adjoint_strip<C, END, !FIRST, TRUE_ADJ, FIRST>
+                                   : tvstrip::tv_adjoint_strip<C, END, false, TRUE_ADJ, FIRST>;
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kAdjCols, knobs().tv_adj_rows, 6);
   const int sx = (s.iw + tvstrip::kAdjCols - 1) / tvstrip::kAdjCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
@@ -749,7 +751,25 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* dx, co
                      at_channel(s, s.acc_gb[ob], ch0), s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o],
                      at_channel(s, g05_in, ch0), at_channel(s, g05_out, ch0), at_channel(s, gxk, ch0), at_channel(s, gxk_m1, ch0),
                      at_channel(s, gx_final, ch0), s.seg_gc + sP, at_channel(s, s.seg_gb + sF, ch0), s.seg_gx + sP, s.seg_gy + sP,
-                     s.n, s.ih, s.iw, t, R, sx, sy, s.ic, last_group ? 1 : 0);
+                     s.n, s.ih, s.iw, t, R, sx, sy, s.ic, last_group ? 1 : 0, at_channel(s, x05_last, ch0));
+}
+
+// The first two steps of the reverse sweep in one launch (strip path, at most kGroup channels, the second step not
+// a segment's first iteration): step j = len - 2 as launch_adjoint runs it, with the sweep's first step (the upstream
+// gradient `gin` through the prox at the last x05 row) done on the way in.  The accumulators start at zero in set
+// acc_cur; the launch writes the other set, then the sets flip as after any step.
+template <bool TRUE_ADJ>
+void launch_adjoint_first_two(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c, const float* b,
+                              const float* x05_last, const float* xa, const float* xb, const float* gin, float* g05_out,
+                              const float* gxk, float* gxk_m1, float t) {
+  switch (s.ic) {
+    case 1: launch_adjoint_strip<1, false, TRUE_ADJ, true>(s, stream, dx, dy, c, b, xa, xb, nullptr, gin, g05_out, gxk, gxk_m1, nullptr, t, 0, true, x05_last); break;
+    case 2: launch_adjoint_strip<2, false, TRUE_ADJ, true>(s, stream, dx, dy, c, b, xa, xb, nullptr, gin, g05_out, gxk, gxk_m1, nullptr, t, 0, true, x05_last); break;
+    case 3: launch_adjoint_strip<3, false, TRUE_ADJ, true>(s, stream, dx, dy, c, b, xa, xb, nullptr, gin, g05_out, gxk, gxk_m1, nullptr, t, 0, true, x05_last); break;
+    default: launch_adjoint_strip<4, false, TRUE_ADJ, true>(s, stream, dx, dy, c, b, xa, xb, nullptr, gin, g05_out, gxk, gxk_m1, nullptr, t, 0, true, x05_last); break;
+  }
+  s.acc_cur = 1 - s.acc_cur;
+  s.accb_cur = 1 - s.accb_cur;
 }
 
 // One adjoint step: reads accumulator set acc_cur, writes the other one, then flips acc_cur.
@@ -1206,7 +1226,14 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       // first step of the whole backward writes g05[1]; a segment's last launch leaves its result
       // where the next segment picks it up.
       int j = len - 1;
-      if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
+      if (outer == nseg - 1 && j >= 2 && s.ic <= kGroup && knobs().tv_fuse_first) {
+        // the sweep's first step rides on its second (a segment of at least four iterations: that one is an inner step)
+        const float *x_last = ring + (size_t)j * F, *xa = ring + (size_t)(j - 1) * F, *xb = ring + (size_t)(j - 2) * F;
+        if (corr) launch_adjoint_first_two<true>(s, stream, dx, dy, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);
+        else launch_adjoint_first_two<false>(s, stream, dx, dy, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);
+        pp_src = 0;
+        j -= 2;
+      } else if (outer == nseg - 1 && j >= 0) {  // (its < 2: no iterations, nothing to back-propagate)
         if (corr)
           hipLaunchKernelGGL(tv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
                              ring + (size_t)j * F, s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic,

@@ -563,6 +563,7 @@ __device__ __forceinline__ float prox_huber1(float yt, float c, float rc1, float
 template <int C>
 struct AdjRow {
   float c, rc1, wxs, wys, xa[C], y[C], bb[C], g[C];  // y is loaded as x05[k-1] (or the checkpoint y) and rebuilt in place
+  float xl[C];                                       // FIRST only: the last x05 row, which the first step linearises at
   float gc_i, gwx_i, gwy_i, gx_i[C], gb_i[C];        // accumulators and partial g_x the row's pixel update continues
   double opc_d;                                      // 1. + (double)c, the left side of the prox regime test
 };
@@ -570,7 +571,11 @@ struct AdjRow {
 // TRUE_ADJ selects the corrected gradient (not the reference's): y is the forward pass's own y (see prox_huber1;
 // with END the y slot carries the checkpointed x of the segment start, not the checkpointed y), the segment-start
 // step uses the main kernel's weight-gradient form, and the per-step multipliers are 1.
-template <int C, bool END, bool FINAL, bool TRUE_ADJ = false>
+// FIRST: this step is the second of the reverse sweep, and the launch performs the sweep's first step (TV.cu:222-287,
+// a pointwise map) on the way in: g05_in is the caller's upstream gradient and x05l the last x05 row; every row that is
+// loaded gets its incoming adjoint from them, and the strip's own rows add the first step's share to the accumulators
+// they have just read, channel by channel, before the step's own (the order of two launches).
+template <int C, bool END, bool FINAL, bool TRUE_ADJ = false, bool FIRST = false>
 __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
@@ -580,7 +585,8 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ g05_in, float* __restrict__ g05_out, const float* __restrict__ gxk,
     float* __restrict__ gxk_m1, float* __restrict__ gx_final, float* __restrict__ seg_gc,
     float* __restrict__ seg_gb, float* __restrict__ seg_gwx, float* __restrict__ seg_gwy, int N, int H, int W,
-    float t, int R, int strips_x, int strips_y, int Ct, int flush_shared) {
+    float t, int R, int strips_x, int strips_y, int Ct, int flush_shared, const float* __restrict__ x05l = nullptr) {
+  static_assert(!(FIRST && END), "the first step is fused into a segment's inner steps only");
   StripGeom g;
   if (!strip_geometry(g, kAdjCols, R, W, strips_x, strips_y, N)) return;
   const int Reff = min(R, H - g.hs);
@@ -596,7 +602,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
   const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const cf_p = cf + poff;
   const float *const gci_p = gc_in + poff, *const gwxi_p = gwx_in + poff, *const gwyi_p = gwy_in + poff;
   float *const gco_p = gc + poff, *const gwxo_p = gwx + poff, *const gwyo_p = gwy + poff;
-  const float *xa_p[C], *xb_p[C], *b_p[C], *g_p[C], *gxi_p[C], *gbi_p[C];
+  const float *xa_p[C], *xb_p[C], *b_p[C], *g_p[C], *gxi_p[C], *gbi_p[C], *xl_p[C];
   float *g05o_p[C], *gxm_p[C], *gbo_p[C], *gxf_p[C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
@@ -605,6 +611,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
     b_p[ch] = b + q; g_p[ch] = g05_in + q; gxi_p[ch] = gxk + q; gbi_p[ch] = gb_in + q;
     g05o_p[ch] = g05_out + q; gxm_p[ch] = gxk_m1 + q; gbo_p[ch] = gb + q;
     gxf_p[ch] = FINAL ? gx_final + q : nullptr;
+    xl_p[ch] = FIRST ? x05l + q : nullptr;
   }
 
   auto load_row = [&](int k, AdjRow<C>& in) {
@@ -625,6 +632,7 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
       in.y[ch] = ldg(xb_p[ch], off);
       in.bb[ch] = ldg(b_p[ch], off);
       in.g[ch] = ldg(g_p[ch], off);
+      if (FIRST) in.xl[ch] = ldg(xl_p[ch], off);
       in.gx_i[ch] = ldg(gxi_p[ch], off_p);
       in.gb_i[ch] = ldg(gbi_p[ch], off_p);
     }
@@ -654,6 +662,26 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
       o.g[ch] = inside(o.g[ch]);
       o.xa[ch] = xa;
       o.bb[ch] = bv;
+    }
+    if (FIRST) {
+      // the sweep's first step at this row (TV.cu:240-255): the upstream gradient through the prox at the last x05 row.
+      // The accumulators belong to the strip's own rows; what rows above and below make of them is never used.
+      const float opc = 1.f + o.c;
+      const float rc2 = rcp_refined(opc * opc);
+      float gcv = o.gc_i;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float df = o.g[ch], bv = o.bb[ch], xh = inside(o.xl[ch]);
+        const float diff = bv - xh;
+        const float sign = (diff < 0) ? -1.f : 1.f;
+        const bool quad = (o.opc_d >= (double)(sign * diff));
+        const float gc_q = df * (div_by(bv, opc, o.rc1) - div_by(o.c * bv + xh, opc * opc, rc2)) * kGC;
+        const float gb_q = div_by(df * o.c, opc, o.rc1) * 1.0f;
+        o.g[ch] = quad ? div_by(df, opc, o.rc1) : df;
+        gcv += quad ? gc_q : sign * df * kGC;
+        o.gb_i[ch] = quad ? o.gb_i[ch] + gb_q : 0.f;  // (TV.cu:254 writes zero outside the quadratic regime)
+      }
+      o.gc_i = gcv;
     }
   };
 

@@ -260,6 +260,23 @@ def test_every_pairing_of_the_reverse_sweep(ext, tv_oracle, its):
     compare("its=%d" % its, run_gpu(ext, d, its, 2), run_oracle(tv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("c", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("its", [4, 5, 9, 16, 50])
+def test_first_step_of_the_sweep_rides_on_the_second(ext, tv_oracle, c, its, monkeypatch):
+    # up to four channels, a last segment of at least four iterations: one launch does the sweep's first two steps
+    # (its = 4, 5: the last segment has two iterations, so the two steps stay apart; c = 5 always keeps them apart);
+    # INPAINT_TV_FUSE_FIRST=0 keeps the separate launches covered
+    d = tv_inputs(2, c, 37, 130, seed=500 + 10 * c + its, conf_density=0.4)
+    ref = run_oracle(tv_oracle, d, its, 2)
+    a = run_gpu(ext, d, its, 2)
+    compare("first two steps in one launch c=%d its=%d" % (c, its), a, ref)
+    monkeypatch.setenv("INPAINT_TV_FUSE_FIRST", "0")
+    b = run_gpu(ext, d, its, 2)
+    compare("first step in its own launch c=%d its=%d" % (c, its), b, ref)
+    for x, y in zip(a[1], b[1]):
+        np.testing.assert_array_equal(x, y)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [
     (1, 1, 9, 60, 8),       # exactly one fused strip wide (60 output columns)
     (1, 2, 11, 61, 8),      # one column more
