@@ -54,6 +54,7 @@ struct Knobs {
   bool tv_fuse = true;            // INPAINT_TV_FUSE=0: one forward iteration per launch
   bool tv_fuse_adj = true;        // INPAINT_TV_FUSE_ADJ=0: one adjoint step per launch
   bool tv_fuse_first = true;      // INPAINT_TV_FUSE_FIRST=0: the reverse sweep's first step in a launch of its own
+  bool tgv_fuse_first = true;     // INPAINT_TGV_FUSE_FIRST=0: the same for the TGV layer
   int tv_fwd_rows = 0;            // INPAINT_TV_FWD_ROWS / INPAINT_TV_ADJ_ROWS: strip height (0 = chosen per launch)
   int tv_adj_rows = 0;
   int tv_fwd_split = -1;          // INPAINT_TV_FWD_SPLIT=0|1: forward pairs with one channel per wavefront (-1 = by the size of the launch)
@@ -85,6 +86,7 @@ struct Knobs {
     tv_fuse = !is("INPAINT_TV_FUSE", "0");
     tv_fuse_adj = !is("INPAINT_TV_FUSE_ADJ", "0");
     tv_fuse_first = !is("INPAINT_TV_FUSE_FIRST", "0");
+    tgv_fuse_first = !is("INPAINT_TGV_FUSE_FIRST", "0");
     tv_fwd_rows = rows("INPAINT_TV_FWD_ROWS");
     tv_adj_rows = rows("INPAINT_TV_ADJ_ROWS");
     tv_fwd_split = is("INPAINT_TV_FWD_SPLIT", "1") ? 1 : (is("INPAINT_TV_FWD_SPLIT", "0") ? 0 : -1);

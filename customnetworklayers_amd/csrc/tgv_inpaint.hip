@@ -1002,12 +1002,13 @@ void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, cons
 
 // One group of a one-step adjoint launch.  Shared accumulators: set acc_cur in, the other out, flipped by the caller
 // after every launch; the per-channel accumulator gb: set accb_cur in, the other out, flipped once per step.
-template <int C, bool END, int ADJ>
+template <int C, bool END, int ADJ, bool FIRST = false>
 void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa,
                           const float* xb, const float* yck, const float* g05_in, float* g05_out, const float* gxk,
-                          float* gxk_m1, float* gx_final, float t, int ch0) {
+                          float* gxk_m1, float* gx_final, float t, int ch0, const float* x05_last = nullptr) {
   const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
-  auto kern = gx_final ? tgvstrip::tgv_adjoint_strip<C, END, true, ADJ> : tgvstrip::tgv_adjoint_strip<C, END, false, ADJ>;
+  auto kern = (gx_final && !FIRST) ? tgvstrip::tgv_adjoint_strip<C, END, !FIRST, ADJ, FIRST>
+                                   : tgvstrip::tgv_adjoint_strip<C, END, false, ADJ, FIRST>;
   const int R = strip_rows(s.n, s.ih, s.iw, tgvstrip::kCols, knobs().tgv_adj_rows, 6);
   const int sx = (s.iw + tgvstrip::kCols - 1) / tgvstrip::kCols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
@@ -1016,7 +1017,22 @@ void launch_adjoint_strip(const Slot& s, hipStream_t stream, const float* c, con
                      at_channel(s, xb, ch0), at_channel(s, yck, ch0), s.acc_gc[i], s.acc_gc[o],
                      at_channel(s, (const float*)s.acc_gb[ib], ch0), at_channel(s, s.acc_gb[ob], ch0), s.acc_gx[i], s.acc_gx[o],
                      s.acc_gy[i], s.acc_gy[o], at_channel(s, g05_in, ch0), at_channel(s, g05_out, ch0), at_channel(s, gxk, ch0),
-                     at_channel(s, gxk_m1, ch0), at_channel(s, gx_final, ch0), s.n, s.ih, s.iw, t, R, sx, sy, s.ic);
+                     at_channel(s, gxk_m1, ch0), at_channel(s, gx_final, ch0), s.n, s.ih, s.iw, t, R, sx, sy, s.ic,
+                     at_channel(s, x05_last, ch0));
+}
+
+// The first two steps of the reverse sweep in one launch (strip path, at most kGroup channels, the second step not a
+// segment's first iteration): step j = len - 2 as launch_adjoint runs it, with the sweep's first step (the upstream
+// gradient `gin` through the prox at the last x05 row) done on the way in.  The accumulators start at zero in set
+// acc_cur; the launch writes the other set, then the sets flip as after any step.
+template <int ADJ>
+void launch_adjoint_first_two(Slot& s, hipStream_t stream, const float* c, const float* b, const float* x05_last,
+                              const float* xa, const float* xb, const float* gin, float* g05_out, const float* gxk,
+                              float* gxk_m1, float t) {
+  if (s.ic == 1) launch_adjoint_strip<1, false, ADJ, true>(s, stream, c, b, xa, xb, nullptr, gin, g05_out, gxk, gxk_m1, nullptr, t, 0, x05_last);
+  else launch_adjoint_strip<2, false, ADJ, true>(s, stream, c, b, xa, xb, nullptr, gin, g05_out, gxk, gxk_m1, nullptr, t, 0, x05_last);
+  s.acc_cur = 1 - s.acc_cur;
+  s.accb_cur = 1 - s.accb_cur;
 }
 
 // One adjoint step.  Strip path: y is rebuilt inside the kernel from xa = x05[k], xb = x05[k-1] (END:
@@ -1189,8 +1205,8 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
     }
   } else {
     scale_weights(s, stream, dx, dy);
-    INPAINT_HIP(hipMemcpyAsync(s.ckpt_y, init, SB, hipMemcpyDeviceToDevice, stream));  // checkpoint 0 = init
-    INPAINT_HIP(hipMemcpyAsync(s.ckpt_x, init, SB, hipMemcpyDeviceToDevice, stream));
+    hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)S3)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
+                       (long long)S3);  // checkpoint 0 = init
     // first iteration whose x05 row is kept, and the ring row of iteration k
     const int kl = s.iterations.empty() ? K : (keep == 2 ? 0 : (keep == 1 ? s.iterations.back() : K));
     auto ring_row = [&](int k) { return s.x05 + (size_t)(keep == 2 ? k : k - kl) * S3; };
@@ -1361,7 +1377,14 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     if (pairs) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
       // `pp_src` = the g05 / g_x buffer the next launch reads; it flips once per launch
       int j = len - 1;
-      if (outer == nseg - 1 && j >= 0) {
+      if (outer == nseg - 1 && j >= 2 && s.ic <= kGroup && knobs().tgv_fuse_first) {
+        // the sweep's first step rides on its second (a segment of at least four iterations: that one is an inner step)
+        const float *x_last = ring + (size_t)j * S3, *xa = ring + (size_t)(j - 1) * S3, *xb = ring + (size_t)(j - 2) * S3;
+        if (corr) launch_adjoint_first_two<1>(s, stream, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);
+        else launch_adjoint_first_two<0>(s, stream, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);
+        pp_src = 0;
+        j -= 2;
+      } else if (outer == nseg - 1 && j >= 0) {
         if (corr)
           hipLaunchKernelGGL(tgv_adjoint_first<true>, dim3(grid1d((long long)P)), dim3(256), 0, stream, c, b,
                              ring + (size_t)j * S3, s.acc_gc[s.acc_cur], s.acc_gb[s.accb_cur], s.g05[1], gin, ic,

@@ -548,6 +548,7 @@ struct AdjRow {
   float c, rc1, wxs, wys, bxs, bys;
   float y[3][C];   // y[0]: loaded as x05[k-1] (or the checkpoint y) and rebuilt in place; y[1], y[2]: x05[k] aux (or checkpoint)
   float xa[C];     // x05[k] of u, for the prox regime
+  float xl[C];     // FIRST only: u of the last x05 row, which the sweep's first step linearises at
   float yp[2][C];  // corrected gradient only: aux of x05[k-1] (or of the checkpointed x), for the momentum of aux y
   float bb[C], g[3][C];
   float gx_i[3][C], gb_i[C], gc_i, gwx0_i, gwx1_i, gwy0_i, gwy1_i;
@@ -558,7 +559,12 @@ struct AdjRow {
 // with x+ = prox(x05[k]) and x- = prox(x05[k-1]) (ADJ == 1) or the checkpointed x of a segment start passed as
 // x05b (ADJ == 2); aux: x05[k] + t (x05[k] - x05[k-1]), momentum included (TGV.cu:1686-1690) --, the upper-triangle
 // v2 block multiplies by hub^2 like its siblings, and the per-step multipliers are 1.  END must be false then.
-template <int C, bool END, bool FINAL, int ADJ = 0>
+// FIRST: this step is the second of the reverse sweep, and the launch performs the sweep's first step (TGV.cu:151-218,
+// a pointwise map: the prox adjoint on u, the auxiliary variables pass through) on the way in: g05_in is the caller's
+// upstream gradient and x05l the last x05 row; every row that is loaded gets its incoming adjoint from them, and the
+// strip's own rows add the first step's share to the accumulators they have just read, channel by channel, before
+// the step's own (the order of two launches).
+template <int C, bool END, bool FINAL, int ADJ = 0, bool FIRST = false>
 __global__ __launch_bounds__(256) void tgv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
@@ -567,7 +573,8 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
     const float* __restrict__ gwx_in, float* __restrict__ gwx, const float* __restrict__ gwy_in,
     float* __restrict__ gwy, const float* __restrict__ g05_in, float* __restrict__ g05_out,
     const float* __restrict__ gxk, float* __restrict__ gxk_m1, float* __restrict__ gx_final, int N, int H, int W,
-    float t, int R, int strips_x, int strips_y, int Ct) {
+    float t, int R, int strips_x, int strips_y, int Ct, const float* __restrict__ x05l = nullptr) {
+  static_assert(!(FIRST && END), "the first step is fused into a segment's inner steps only");
   StripGeom g;
   if (!strip_geometry(g, kCols, R, W, strips_x, strips_y, N)) return;
   const int Reff = min(R, H - g.hs);
@@ -587,7 +594,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
                      *const gwy0i_p = gwy_in + 2 * poff, *const gwy1i_p = gwy_in + 2 * poff + HW;
   float *const gco_p = gc + poff, *const gwx0o_p = gwx + 2 * poff, *const gwx1o_p = gwx + 2 * poff + HW,
                *const gwy0o_p = gwy + 2 * poff, *const gwy1o_p = gwy + 2 * poff + HW;
-  const float *ys_p[3][C], *yp_p[2][C], *xa_p[C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
+  const float *ys_p[3][C], *yp_p[2][C], *xa_p[C], *xl_p[C], *b_p[C], *g_p[3][C], *gxi_p[3][C], *gbi_p[C];
   float *g05o_p[3][C], *gxm_p[3][C], *gbo_p[C], *gxf_p[3][C];
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
@@ -604,6 +611,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
       g05o_p[v][ch] = g05_out + q; gxm_p[v][ch] = gxk_m1 + q; gxf_p[v][ch] = FINAL ? gx_final + q : nullptr;
     }
     xa_p[ch] = x05a + (size_t)g.n * 3 * CHW + (size_t)ch * HW;
+    xl_p[ch] = FIRST ? x05l + (size_t)g.n * 3 * CHW + (size_t)ch * HW : nullptr;
   }
 
   auto load_row = [&](int k, AdjRow<C>& in) {
@@ -621,6 +629,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
 #pragma unroll
     for (int ch = 0; ch < C; ch++) {
       in.xa[ch] = ldg(xa_p[ch], off);
+      if (FIRST) in.xl[ch] = ldg(xl_p[ch], off);
       in.bb[ch] = ldg(b_p[ch], off);
       in.gb_i[ch] = ldg(gbi_p[ch], off_p);
 #pragma unroll
@@ -669,6 +678,26 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
       o.bb[ch] = bv;
 #pragma unroll
       for (int v = 0; v < 3; v++) o.g[v][ch] = inside(o.g[v][ch]);
+    }
+    if (FIRST) {
+      // the sweep's first step at this row (TGV.cu:166-182): the upstream gradient of u through the prox at the last
+      // x05 row.  The accumulators belong to the strip's own rows; what rows above and below make of them is never used.
+      const float opc = 1.f + o.c;
+      const float rc2 = rcp_refined(opc * opc);
+      float gcv = o.gc_i;
+#pragma unroll
+      for (int ch = 0; ch < C; ch++) {
+        const float df = o.g[0][ch], bv = o.bb[ch], xh = inside(o.xl[ch]);
+        const float diff = bv - xh;
+        const float sign = (diff < 0) ? -1.f : 1.f;
+        const bool quad = (o.opc_d >= (double)(sign * diff));
+        const float gc_q = df * (div_by(bv, opc, o.rc1) - div_by(o.c * bv + xh, opc * opc, rc2)) * kGC;
+        const float gb_q = div_by(df * o.c, opc, o.rc1) * 1.0f;
+        o.g[0][ch] = quad ? div_by(df, opc, o.rc1) : df;
+        gcv += quad ? gc_q : sign * df * kGC;
+        o.gb_i[ch] = quad ? o.gb_i[ch] + gb_q : 0.f;  // (TGV.cu:181 writes zero outside the quadratic regime)
+      }
+      o.gc_i = gcv;
     }
   };
 

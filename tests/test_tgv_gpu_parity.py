@@ -271,6 +271,23 @@ def test_every_pairing_of_the_reverse_sweep(ext, tgv_oracle, c, its):
     compare("c=%d its=%d" % (c, its), run_gpu(ext, d, its, 2), run_oracle(tgv_oracle, d, its, 2))
 
 
+@pytest.mark.parametrize("c", [1, 2, 3])
+@pytest.mark.parametrize("its", [4, 5, 9, 16, 50])
+def test_first_step_of_the_sweep_rides_on_the_second(ext, tgv_oracle, c, its, monkeypatch):
+    # one or two channels, a last segment of at least four iterations: one launch does the sweep's first two steps
+    # (its = 4, 5: the last segment has two iterations, so the two steps stay apart; c = 3 always keeps them apart);
+    # INPAINT_TGV_FUSE_FIRST=0 keeps the separate launches covered
+    d = varying_inputs(2, c, 37, 130, seed=600 + 10 * c + its)
+    ref = run_oracle(tgv_oracle, d, its, 2)
+    a = run_gpu(ext, d, its, 2)
+    compare("first two steps in one launch c=%d its=%d" % (c, its), a, ref)
+    monkeypatch.setenv("INPAINT_TGV_FUSE_FIRST", "0")
+    b = run_gpu(ext, d, its, 2)
+    compare("first step in its own launch c=%d its=%d" % (c, its), b, ref)
+    for x, y in zip(a[1], b[1]):
+        np.testing.assert_array_equal(x, y)
+
+
 def test_varying_beta_and_per_sample_lipschitz(ext, tgv_oracle):
     # sample 0: beta up to 9 (bound above 32, data dependent); sample 1: small beta (bound 32)
     d = varying_inputs(2, 2, 40, 56, seed=11)
