@@ -24,10 +24,10 @@ HBM_PEAK_GBS = 8000.0
 #             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
 #   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
 COUNTERS = {
-    1: dict(traffic=(2 * 87073 + 68698) * 1024, step=(2 * 6738500 + 6268485) * 1024, lds=0, rocprof_ms=0.05199,
-            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="80cfba3"),
-    2: dict(traffic=(2 * 164402 + 148964) * 1024, step=(2 * 13839728 + 14761333) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.11997,
-            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="80cfba3"),
+    1: dict(traffic=(2 * 87065 + 68623) * 1024, step=(2 * 6708660 + 6228365) * 1024, lds=0, rocprof_ms=0.05195,
+            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="c0e18f6"),
+    2: dict(traffic=(2 * 164318 + 148791) * 1024, step=(2 * 13770067 + 14681835) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.12007,
+            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="c0e18f6"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
     6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="26d8b66"),
@@ -561,7 +561,7 @@ def main():
                                             slot_bytes=o["config"]["slot_bytes"])
         o, _ = bench_layer(2, 4, 2, detail=False)
         other["config2_tgv"] = dict(leg(o), workload=o["config"]["workload"], slot_bytes=o["config"]["slot_bytes"])
-        hargs = argparse.Namespace(steps=5, warmup=2, no_cpu_baseline=True)
+        hargs = argparse.Namespace(steps=30, warmup=5, no_cpu_baseline=True)  # (2 ms steps: a short leg would time the empty queue at its start)
         o = bench_hierarchy(hargs, CONFIGS[3])
         other["config3_hierarchy"] = dict({k: o[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup")}, workload=o["config"]["workload"])
         o, _ = bench_layer(4, 3, 1, detail=False)
