@@ -1308,12 +1308,19 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       sj.n[k] = ns[k];
     }
   }
-  {
+  // The sweep's first step rides on its second when the last segment has at least four iterations (that second step
+  // is then an inner step) and one launch holds every channel.  That launch starts from zero accumulators without
+  // reading them, and every launch after it reads only what its predecessor wrote in full: nothing to clear.
+  const bool corr_pairs_ok = !corr || pair_split(s.ic);
+  const int nseg_all = (int)s.iterations.size();
+  const bool first_two = seg_mode && adjoint_pairs(s) && corr_pairs_ok && s.ic <= kGroup && knobs().tgv_fuse_first &&
+                         nseg_all > 0 && 2 * ((its - s.iterations[nseg_all - 1]) / 2) >= 4;
+  s.acc_cur = 0;
+  s.accb_cur = 0;
+  if (!first_two) {
     ZeroList z;
     int k = 0;
     for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.yk, s.gx_final}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
-    s.acc_cur = 0;
-    s.accb_cur = 0;
     z.ptr[k] = s.acc_gb[0]; z.bytes[k++] = (long long)F * 4;
     z.ptr[k] = s.acc_gc[0]; z.bytes[k++] = (long long)P * 4;
     z.ptr[k] = s.acc_gx[0]; z.bytes[k++] = (long long)P * 8;
@@ -1377,8 +1384,8 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     if (pairs) {  // reverse sweep (TGV.cu:2851-2933), two steps per launch
       // `pp_src` = the g05 / g_x buffer the next launch reads; it flips once per launch
       int j = len - 1;
-      if (outer == nseg - 1 && j >= 2 && s.ic <= kGroup && knobs().tgv_fuse_first) {
-        // the sweep's first step rides on its second (a segment of at least four iterations: that one is an inner step)
+      if (outer == nseg - 1 && first_two) {
+        // the sweep's first step rides on its second
         const float *x_last = ring + (size_t)j * S3, *xa = ring + (size_t)(j - 1) * S3, *xb = ring + (size_t)(j - 2) * S3;
         if (corr) launch_adjoint_first_two<1>(s, stream, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);
         else launch_adjoint_first_two<0>(s, stream, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);

@@ -562,8 +562,10 @@ struct AdjRow {
 // FIRST: this step is the second of the reverse sweep, and the launch performs the sweep's first step (TGV.cu:151-218,
 // a pointwise map: the prox adjoint on u, the auxiliary variables pass through) on the way in: g05_in is the caller's
 // upstream gradient and x05l the last x05 row; every row that is loaded gets its incoming adjoint from them, and the
-// strip's own rows add the first step's share to the accumulators they have just read, channel by channel, before
-// the step's own (the order of two launches).
+// strip's own rows add the first step's share to the accumulators, channel by channel, before the step's own (the
+// order of two launches).  The accumulators and the partial g_x start at zero here, so the launch does not read them
+// (gc_in, gb_in, gwx_in, gwy_in, gxk are not used) and the caller need not clear anything: every later launch reads
+// only what the launch before it wrote in full.
 template <int C, bool END, bool FINAL, int ADJ = 0, bool FIRST = false>
 __global__ __launch_bounds__(256) void tgv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
@@ -631,20 +633,20 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
       in.xa[ch] = ldg(xa_p[ch], off);
       if (FIRST) in.xl[ch] = ldg(xl_p[ch], off);
       in.bb[ch] = ldg(b_p[ch], off);
-      in.gb_i[ch] = ldg(gbi_p[ch], off_p);
+      in.gb_i[ch] = FIRST ? 0.f : ldg(gbi_p[ch], off_p);  // (FIRST: nothing accumulated yet, no partial g_x: zeros)
 #pragma unroll
       for (int v = 0; v < 3; v++) {
         in.y[v][ch] = ldg(ys_p[v][ch], off);
         if (ADJ && v > 0) in.yp[v - 1][ch] = ldg(yp_p[v - 1][ch], off);
         in.g[v][ch] = ldg(g_p[v][ch], off);
-        in.gx_i[v][ch] = ldg(gxi_p[v][ch], off_p);
+        in.gx_i[v][ch] = FIRST ? 0.f : ldg(gxi_p[v][ch], off_p);
       }
     }
-    in.gc_i = ldg(gci_p, off_p);
-    in.gwx0_i = ldg(gwx0i_p, off_p);
-    in.gwx1_i = ldg(gwx1i_p, off_p);
-    in.gwy0_i = ldg(gwy0i_p, off_p);
-    in.gwy1_i = ldg(gwy1i_p, off_p);
+    in.gc_i = FIRST ? 0.f : ldg(gci_p, off_p);
+    in.gwx0_i = FIRST ? 0.f : ldg(gwx0i_p, off_p);
+    in.gwx1_i = FIRST ? 0.f : ldg(gwx1i_p, off_p);
+    in.gwy0_i = FIRST ? 0.f : ldg(gwy0i_p, off_p);
+    in.gwy1_i = FIRST ? 0.f : ldg(gwy1i_p, off_p);
   };
   auto absorb = [&](int k, AdjRow<C>& o) {
     const int h = g.hs - 1 + k;

@@ -1164,11 +1164,19 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       sj.n[k] = k < 3 ? (long long)P : (long long)F;
     }
   }
+  // The sweep's first step rides on its second when the last segment has at least four iterations (that second step
+  // is then an inner step) and one launch holds every channel.  That launch starts from zero accumulators without
+  // reading them, and every launch after it reads only what its predecessor wrote in full: nothing to clear.
+  const int nseg = (int)s.iterations.size();
+  const bool first_two = seg_mode && adjoint_pairs(s) && s.ic <= kGroup && knobs().tv_fuse_first && nseg > 0 &&
+                         2 * ((its - s.iterations[nseg - 1]) / 2) >= 4;
   {
     ZeroList z;
     int k = 0;
-    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.gx_final, s.acc_gb[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)F * 4; }
-    for (float* p : {s.acc_gc[0], s.acc_gx[0], s.acc_gy[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 4; }
+    if (!first_two) {
+      for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.gx_final, s.acc_gb[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)F * 4; }
+      for (float* p : {s.acc_gc[0], s.acc_gx[0], s.acc_gy[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 4; }
+    }
     if (!seg_mode) {  // (the strip path writes every total when it adds up the segment records)
       for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 8; }
       z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
@@ -1183,7 +1191,6 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   // step (TV.cu:800 calls its store a debugging aid), so only that step stores it, into gx_final.
   int lastIt = its;
   int pp_src = 1;  // g05 / g_x buffer the next adjoint launch reads (pair path)
-  const int nseg = (int)s.iterations.size();
   for (int outer = nseg - 1; outer >= 0; outer--) {
     const int k0 = s.iterations[outer];
     const int len = 2 * ((lastIt - k0) / 2);
@@ -1226,8 +1233,8 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       // first step of the whole backward writes g05[1]; a segment's last launch leaves its result
       // where the next segment picks it up.
       int j = len - 1;
-      if (outer == nseg - 1 && j >= 2 && s.ic <= kGroup && knobs().tv_fuse_first) {
-        // the sweep's first step rides on its second (a segment of at least four iterations: that one is an inner step)
+      if (outer == nseg - 1 && first_two) {
+        // the sweep's first step rides on its second
         const float *x_last = ring + (size_t)j * F, *xa = ring + (size_t)(j - 1) * F, *xb = ring + (size_t)(j - 2) * F;
         if (corr) launch_adjoint_first_two<true>(s, stream, dx, dy, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);
         else launch_adjoint_first_two<false>(s, stream, dx, dy, c, b, x_last, xa, xb, gin, s.g05[0], s.gxk[1], s.gxk[0], s.steps[k0 + j - 1]);

@@ -573,8 +573,10 @@ struct AdjRow {
 // step uses the main kernel's weight-gradient form, and the per-step multipliers are 1.
 // FIRST: this step is the second of the reverse sweep, and the launch performs the sweep's first step (TV.cu:222-287,
 // a pointwise map) on the way in: g05_in is the caller's upstream gradient and x05l the last x05 row; every row that is
-// loaded gets its incoming adjoint from them, and the strip's own rows add the first step's share to the accumulators
-// they have just read, channel by channel, before the step's own (the order of two launches).
+// loaded gets its incoming adjoint from them, and the strip's own rows add the first step's share to the accumulators,
+// channel by channel, before the step's own (the order of two launches).  The accumulators and the partial g_x start at
+// zero here, so the launch does not read them (gc_in, gb_in, gwx_in, gwy_in, gxk are not used) and the caller need
+// not clear anything: every later launch reads only what the launch before it wrote in full.
 template <int C, bool END, bool FINAL, bool TRUE_ADJ = false, bool FIRST = false>
 __global__ __launch_bounds__(256) void tv_adjoint_strip(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
@@ -633,12 +635,13 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
       in.bb[ch] = ldg(b_p[ch], off);
       in.g[ch] = ldg(g_p[ch], off);
       if (FIRST) in.xl[ch] = ldg(xl_p[ch], off);
-      in.gx_i[ch] = ldg(gxi_p[ch], off_p);
-      in.gb_i[ch] = ldg(gbi_p[ch], off_p);
+      // (FIRST: nothing has been accumulated yet and there is no partial g_x: zeros, which nobody has to store first)
+      in.gx_i[ch] = FIRST ? 0.f : ldg(gxi_p[ch], off_p);
+      in.gb_i[ch] = FIRST ? 0.f : ldg(gbi_p[ch], off_p);
     }
-    in.gc_i = ldg(gci_p, off_p);
-    in.gwx_i = ldg(gwxi_p, off_p);
-    in.gwy_i = ldg(gwyi_p, off_p);
+    in.gc_i = FIRST ? 0.f : ldg(gci_p, off_p);
+    in.gwx_i = FIRST ? 0.f : ldg(gwxi_p, off_p);
+    in.gwy_i = FIRST ? 0.f : ldg(gwyi_p, off_p);
   };
   auto absorb = [&](int k, AdjRow<C>& o) {
     const int h = g.hs - 1 + k;
