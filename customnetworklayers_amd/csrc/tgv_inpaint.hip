@@ -746,6 +746,8 @@ struct Slot {
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
   // strip path: one fp32 record per segment and tensor, added into the totals after the last segment
   float *seg_gc = nullptr, *seg_gx = nullptr, *seg_gy = nullptr, *seg_gb = nullptr;
+  float* zeros = nullptr;  // a field of zeros (as large as the largest accumulator), never written after the slot is made: the accumulators a segment's first pair starts from
+  bool acc_fresh = false;  // the next pair launch starts a segment: its accumulators are zero, read from `zeros` (the pair that ended the segment before wrote none)
   int seg_cur = 0;  // segment the backward pass is in
   GuardState* guard = nullptr;
   double pending_av[5] = {0, 0, 0, 0, 0};
@@ -795,6 +797,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   need += Arena::padded(P, 8) + Arena::padded(2 * P, 8) * 2;
   need += Arena::padded(P * nck, 4) + Arena::padded(2 * P * nck, 4) * 2 + Arena::padded(F * nck, 4);
   need += Arena::padded((size_t)n, 8) + Arena::padded((size_t)n, 4) + Arena::padded(2, 4);
+  need += Arena::padded(std::max(F, 2 * P), 4);  // the field of zeros
   need += Arena::padded(1, sizeof(GuardState));
   rc = s.arena.reserve(need);
   if (rc) return rc;
@@ -820,8 +823,10 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   s.tot_gb = a.take<double>(F);
   s.seg_gc = a.take<float>(P * nck); s.seg_gx = a.take<float>(2 * P * nck); s.seg_gy = a.take<float>(2 * P * nck);
   s.seg_gb = a.take<float>(F * nck);
+  s.zeros = a.take<float>(std::max(F, 2 * P));
   s.guard = a.take<GuardState>(1);
   if (!s.guard) return fail(INPAINT_ERR_HIP, "arena layout overflow");
+  hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)std::max(F, 2 * P))), dim3(256), 0, stream, s.zeros, (long long)std::max(F, 2 * P));
   GuardState init;
   memset(&init, 0, sizeof(init));
   for (int k = 0; k < 5; k++) { init.av[k] = s.pending_av[k]; init.scale[k] = 1.0; }
@@ -1086,9 +1091,10 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const int sx = (s.iw + tgvstrip::kCols2 - 1) / tgvstrip::kCols2, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
+  const bool zf = s.acc_fresh;  // first pair of a segment: zero accumulators, read from the field of zeros
 #define TGV_PAIR_ARGS                                                                                                      \
-  s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob], s.acc_gx[i], s.acc_gx[o], \
-      s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + 2 * sP, s.seg_gy + 2 * sP, s.n, s.ih,  \
+  s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, zf ? s.zeros : s.acc_gc[i], s.acc_gc[o], zf ? s.zeros : s.acc_gb[ib], s.acc_gb[ob], zf ? s.zeros : s.acc_gx[i], s.acc_gx[o], \
+      zf ? s.zeros : s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + 2 * sP, s.seg_gy + 2 * sP, s.n, s.ih,  \
       s.iw, tA, tB, R, sx, sy, s.ic
   if (split) {
     const dim3 grid((unsigned)((waves + 7) / 8 * 8)), block(128);
@@ -1133,8 +1139,9 @@ void launch_adjoint_pair_quad(const Slot& s, hipStream_t stream, const float* c,
   const long long strips = (long long)sx * sy * s.n;
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(256);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib],
-                     s.acc_gb[ob], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final,
+  const bool zf = s.acc_fresh;  // first pair of a segment: zero accumulators, read from the field of zeros
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, xb, xc, zf ? s.zeros : s.acc_gc[i], s.acc_gc[o], zf ? s.zeros : s.acc_gb[ib],
+                     s.acc_gb[ob], zf ? s.zeros : s.acc_gx[i], s.acc_gx[o], zf ? s.zeros : s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final,
                      s.seg_gc + sP, s.seg_gb + sF, s.seg_gx + 2 * sP, s.seg_gy + 2 * sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
@@ -1423,6 +1430,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
         const float* xa = ring + (size_t)j * S3;
         const float* xb = ring + (size_t)(j - 1) * S3;
         float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
+        // A pair that ends a segment stores the segment's sums as a record; it does not write the zeros the next segment
+        // starts from (only the sweep's very last launch clears the accumulators): a segment's first pair reads zeros
+        // from the slot's field of zeros instead, which stays in the cache.
+        s.acc_fresh = outer < nseg - 1 && j == len - 1;
         if (j - 1 > 0) {
           const float* xc = ring + (size_t)(j - 2) * S3;
           if (timed_run == 0) g_timer.begin(stream);
@@ -1440,6 +1451,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
         }
         pp_src = 1 - pp_src;
       }
+      s.acc_fresh = false;
     } else
     for (int j = len - 1; j >= 0; j--) {  // reverse sweep (TGV.cu:2851-2933)
       const float t = s.steps[k0 + j];

@@ -938,12 +938,17 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
 }
 
 // -------------------------------------------------------------------------------------------------
+// Accumulators at a segment end, in all pair kernels below: a BEND launch stores the segment's sums as a record; the
+// zeros the reference leaves in the accumulators (TGVH.cu:178-216) are written by the very last launch of the sweep only
+// (FINAL).  After any other BEND launch the accumulator set it would have written holds stale values, and the caller
+// hands the next launch a field of zeros as gc_in / gb_in / gwx_in / gwy_in instead.
+// -------------------------------------------------------------------------------------------------
 // Two adjoint steps per launch (A = local iteration j, B = j-1): the arithmetic of
 // tgv_adjoint_strip applied twice, B one row behind A in the same wavefront (the scheme of
 // tvstrip::tv_adjoint_strip2).  A's g05[j] and partial g_x[j] stay in registers; the seven
 // accumulators are read and written once for both steps.  BEND: B is the segment's first iteration
 // (checkpoint y, segment-start arithmetic) and the segment flush is fused: the fp32 segment sums go into the
-// segment's record (added into the fp64 totals after the last segment) and the accumulators are left at zero.  FINAL: B's completed g_x is stored.
+// segment's record (added into the fp64 totals after the last segment).  FINAL: B's completed g_x is stored and the accumulators are left at zero.
 // To fit two wavefronts per SIMD the row buffers hold only what a row's neighbours need; the fields
 // that only the pixel's own update reads (partial g_x, accumulators) are loaded one step ahead into a
 // single set of registers.
@@ -1324,9 +1329,9 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
             stg(g05o_p[0][ch], roffB, o.g05v);
             stg(g05o_p[1][ch], roffB, o.d1);
             stg(g05o_p[2][ch], roffB, o.d2);
-            if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
+            if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record; zero at the sweep's end (TGVH.cu:178-216)
               seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
-              stg(gbo_p[ch], roffB, 0.f);
+              if (FINAL) stg(gbo_p[ch], roffB, 0.f);
             } else {
               stg(gbo_p[ch], roffB, gbv);
             }
@@ -1341,11 +1346,11 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
           seg_gwx[e2 + HW] = accB.gwx1;
           seg_gwy[e2] = accB.gwy0;
           seg_gwy[e2 + HW] = accB.gwy1;
-          stg(gco_p, roffB, 0.f);
-          stg(gwx0o_p, roffB, 0.f);
-          stg(gwx1o_p, roffB, 0.f);
-          stg(gwy0o_p, roffB, 0.f);
-          stg(gwy1o_p, roffB, 0.f);
+          if (FINAL) stg(gco_p, roffB, 0.f);
+          if (FINAL) stg(gwx0o_p, roffB, 0.f);
+          if (FINAL) stg(gwx1o_p, roffB, 0.f);
+          if (FINAL) stg(gwy0o_p, roffB, 0.f);
+          if (FINAL) stg(gwy1o_p, roffB, 0.f);
         } else {
           stg(gco_p, roffB, gcB);
           stg(gwx0o_p, roffB, accB.gwx0);
@@ -1953,9 +1958,9 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
               stg(g05o_p[0][ch], roffB, o.g05v);
               stg(g05o_p[1][ch], roffB, o.d1);
               stg(g05o_p[2][ch], roffB, o.d2);
-              if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
+              if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record; zero at the sweep's end (TGVH.cu:178-216)
                 seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)] = gbv;
-                stg(gbo_p[ch], roffB, 0.f);
+                if (FINAL) stg(gbo_p[ch], roffB, 0.f);
               } else {
                 stg(gbo_p[ch], roffB, gbv);
               }
@@ -1970,11 +1975,11 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
             seg_gwx[e2 + HW] = accB.gwx1;
             seg_gwy[e2] = accB.gwy0;
             seg_gwy[e2 + HW] = accB.gwy1;
-            stg(gco_p, roffB, 0.f);
-            stg(gwx0o_p, roffB, 0.f);
-            stg(gwx1o_p, roffB, 0.f);
-            stg(gwy0o_p, roffB, 0.f);
-            stg(gwy1o_p, roffB, 0.f);
+            if (FINAL) stg(gco_p, roffB, 0.f);
+            if (FINAL) stg(gwx0o_p, roffB, 0.f);
+            if (FINAL) stg(gwx1o_p, roffB, 0.f);
+            if (FINAL) stg(gwy0o_p, roffB, 0.f);
+            if (FINAL) stg(gwy1o_p, roffB, 0.f);
           } else {
             stg(gco_p, roffB, gcB);
             stg(gwx0o_p, roffB, accB.gwx0);
@@ -2642,9 +2647,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
               stg(g05o_p[0][ch], roffB, o.g05v);
               stg(g05o_p[1][ch], roffB, o.d1);
               stg(g05o_p[2][ch], roffB, o.d2);
-              if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record, then zero (TGVH.cu:178-216)
+              if (BEND) {  // segment flush, fused: fp32 segment sum into the segment's record; zero at the sweep's end (TGVH.cu:178-216)
                 seg_gb[((size_t)g.n * Ct + chb + ch) * HW + (roffB >> 2)] = gbv;
-                stg(gbo_p[ch], roffB, 0.f);
+                if (FINAL) stg(gbo_p[ch], roffB, 0.f);
               } else {
                 stg(gbo_p[ch], roffB, gbv);
               }
@@ -2659,11 +2664,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             seg_gwx[e2 + HW] = accB.gwx1;
             seg_gwy[e2] = accB.gwy0;
             seg_gwy[e2 + HW] = accB.gwy1;
-            stg(gco_p, roffB, 0.f);
-            stg(gwx0o_p, roffB, 0.f);
-            stg(gwx1o_p, roffB, 0.f);
-            stg(gwy0o_p, roffB, 0.f);
-            stg(gwy1o_p, roffB, 0.f);
+            if (FINAL) stg(gco_p, roffB, 0.f);
+            if (FINAL) stg(gwx0o_p, roffB, 0.f);
+            if (FINAL) stg(gwx1o_p, roffB, 0.f);
+            if (FINAL) stg(gwy0o_p, roffB, 0.f);
+            if (FINAL) stg(gwy1o_p, roffB, 0.f);
           } else {
             stg(gco_p, roffB, gcB);
             stg(gwx0o_p, roffB, accB.gwx0);

@@ -509,10 +509,12 @@ struct Slot {
   float *acc_gc[2] = {nullptr, nullptr}, *acc_gx[2] = {nullptr, nullptr}, *acc_gy[2] = {nullptr, nullptr},
         *acc_gb[2] = {nullptr, nullptr};
   int acc_cur = 0;   // set of the shared accumulators (gc, gx, gy) the next adjoint launch reads
+  bool acc_fresh = false;  // the next pair launch starts a segment: its accumulators are zero, read from `zeros` (the pair that ended the segment before wrote none)
   int accb_cur = 0;  // set of the per-channel accumulator (gb) the next adjoint step reads
   double *tot_gc = nullptr, *tot_gx = nullptr, *tot_gy = nullptr, *tot_gb = nullptr;
   // strip path: one fp32 record per segment and tensor, added into the totals after the last segment
   float *seg_gc = nullptr, *seg_gx = nullptr, *seg_gy = nullptr, *seg_gb = nullptr;
+  float* zeros = nullptr;  // one field of zeros, never written after the slot is made: the accumulators a segment's first pair starts from
   int seg_cur = 0;  // segment the backward pass is in
   GuardState* guard = nullptr;      // device
   double pending_av[5] = {0, 0, 0, 0, 0};  // running means to upload when the arena is (re)made
@@ -557,7 +559,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   s.ring_rows = ring_rows;
   const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)ring_rows;
   size_t need = 0;
-  need += Arena::padded(F, 4) * (2 + 2 + 2 * nck + ring + 2 + 2 + 1 + 2);
+  need += Arena::padded(F, 4) * (2 + 2 + 2 * nck + ring + 2 + 2 + 1 + 2 + 1);
   need += Arena::padded(P, 4) * 6;
   need += Arena::padded(P, 8) * 3 + Arena::padded(F, 8);
   need += Arena::padded(P * nck, 4) * 3 + Arena::padded(F * nck, 4);
@@ -579,8 +581,10 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   s.tot_gb = a.take<double>(F);
   s.seg_gc = a.take<float>(P * nck); s.seg_gx = a.take<float>(P * nck); s.seg_gy = a.take<float>(P * nck);
   s.seg_gb = a.take<float>(F * nck);
+  s.zeros = a.take<float>(F);
   s.guard = a.take<GuardState>(1);
   if (!s.guard) return fail(INPAINT_ERR_HIP, "arena layout overflow");
+  hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, s.zeros, (long long)F);
   GuardState init;
   memset(&init, 0, sizeof(init));
   for (int k = 0; k < 5; k++) { init.av[k] = s.pending_av[k]; init.scale[k] = 1.0; }
@@ -810,14 +814,15 @@ void launch_adjoint_pair_strip(const Slot& s, hipStream_t stream, const float* d
                                const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                                float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const bool zf = s.acc_fresh;  // first pair of a segment: zero accumulators, read from the field of zeros
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip2<C, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2<C, BEND, false, TRUE_ADJ>;
   const int R = strip_rows(s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_adj_rows, 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long waves = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
-                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, zf ? s.zeros : s.acc_gc[i], s.acc_gc[o], zf ? s.zeros : s.acc_gb[ib], s.acc_gb[ob],
+                     zf ? s.zeros : s.acc_gx[i], s.acc_gx[o], zf ? s.zeros : s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
@@ -847,14 +852,15 @@ void launch_adjoint_pair_split(const Slot& s, hipStream_t stream, const float* d
                                const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                                float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const bool zf = s.acc_fresh;  // first pair of a segment: zero accumulators, read from the field of zeros
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip2w<C, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2w<C, BEND, false, TRUE_ADJ>;
   const int R = pair_split_rows(s.n, s.ih, s.iw);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long strips = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(128);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
-                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, zf ? s.zeros : s.acc_gc[i], s.acc_gc[o], zf ? s.zeros : s.acc_gb[ib], s.acc_gb[ob],
+                     zf ? s.zeros : s.acc_gx[i], s.acc_gx[o], zf ? s.zeros : s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
@@ -882,14 +888,15 @@ void launch_adjoint_pair_quad(const Slot& s, hipStream_t stream, const float* dx
                               const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                               float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const bool zf = s.acc_fresh;  // first pair of a segment: zero accumulators, read from the field of zeros
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip4w<CM, C1, BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip4w<CM, C1, BEND, false, TRUE_ADJ>;
   const int R = pair_quad_rows(s.n, s.ih, s.iw);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long strips = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(256);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
-                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, zf ? s.zeros : s.acc_gc[i], s.acc_gc[o], zf ? s.zeros : s.acc_gb[ib], s.acc_gb[ob],
+                     zf ? s.zeros : s.acc_gx[i], s.acc_gx[o], zf ? s.zeros : s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
@@ -911,14 +918,15 @@ void launch_adjoint_pair_channels(const Slot& s, hipStream_t stream, const float
                                   const float* b, const float* xa, const float* xb, const float* xc, const float* g05_in,
                                   float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float tA, float tB) {
   const int i = s.acc_cur, o = 1 - s.acc_cur, ib = s.accb_cur, ob = 1 - s.accb_cur;
+  const bool zf = s.acc_fresh;  // first pair of a segment: zero accumulators, read from the field of zeros
   const size_t sP = (size_t)s.seg_cur * plane_count(s), sF = (size_t)s.seg_cur * field_count(s);  // this segment's records
   auto kern = gx_final ? tvstrip::tv_adjoint_strip2c<BEND, true, TRUE_ADJ> : tvstrip::tv_adjoint_strip2c<BEND, false, TRUE_ADJ>;
   const int R = strip_rows(2 * s.n, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_adj_rows, 9);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
   const long long strips = (long long)sx * sy * s.n;
   const dim3 grid((unsigned)((strips + 7) / 8 * 8)), block(128);
-  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, s.acc_gc[i], s.acc_gc[o], s.acc_gb[ib], s.acc_gb[ob],
-                     s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
+  hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xa, xb, xc, zf ? s.zeros : s.acc_gc[i], s.acc_gc[o], zf ? s.zeros : s.acc_gb[ib], s.acc_gb[ob],
+                     zf ? s.zeros : s.acc_gx[i], s.acc_gx[o], zf ? s.zeros : s.acc_gy[i], s.acc_gy[o], g05_in, g05_out, gxk, gxk_m1, gx_final, s.seg_gc + sP,
                      s.seg_gb + sF, s.seg_gx + sP, s.seg_gy + sP, s.n, s.ih, s.iw, tA, tB, R, sx, sy, s.ic);
 }
 
@@ -1274,6 +1282,10 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
         const float* xa = ring + (size_t)j * F;
         const float* xb = ring + (size_t)(j - 1) * F;
         float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
+        // A pair that ends a segment stores the segment's sums as a record; it does not write the zeros the next segment
+        // starts from (only the sweep's very last launch clears the accumulators): a segment's first pair reads zeros
+        // from the slot's field of zeros instead, which stays in the cache.
+        s.acc_fresh = outer < nseg - 1 && j == len - 1;
         if (j - 1 > 0) {
           const float* xc = ring + (size_t)(j - 2) * F;
           if (timed_run == 0) g_timer.begin(stream);
@@ -1290,6 +1302,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
         }
         pp_src = 1 - pp_src;
       }
+      s.acc_fresh = false;
     } else
     for (int j = len - 1; j >= 0; j--) {
       const float t = s.steps[k0 + j];
