@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "../../include/tvinpaint.h"
+#include "../../include/inpaint_diagnostics.h"
 
 namespace inpaint {
 

@@ -81,20 +81,7 @@ int tgvinpaint_lipschitz(int id, double* L_host, int n);
  * TGVInpaintFistaHelp.cu:119-151). */
 int tgvinpaint_guard_decide(int run, double av_gc, double av_running, double* mult_out, double* av_out);
 
-/* Diagnostic, as tvinpaint_selftest_guard with this layer's guard (check_gradUpdate + update_correct_av_step_host,
- * TGVInpaintFistaHelp.cu:119-216: an entry above the tolerance enters the mean as the tolerance and is clamped to it,
- * not zeroed). */
-int tgvinpaint_selftest_guard(const void* values, long long n, int is_f32, int run, double running_mean, float* out,
-                              double* result7);
-
-/* HIP-event timing of the main adjoint kernel, as tvinpaint_profile / tvinpaint_profile_read. */
-int tgvinpaint_profile(int enable);
-int tgvinpaint_profile_read(double* total_ms, int* launches);
-
-/* Diagnostic, like inpaint_selftest_math: the TGV strip kernels' 1/sqrt(x), x/0.2f, the reciprocal 1/m over [2^-40, 2^40) and w/h^2
- * against the compiler's IEEE expansions on the GPU (host array of four mismatch counts, all 0). */
-int inpaint_selftest_rsqrt(unsigned long long* mismatches4_host, unsigned int pair_rounds);
-
+/* Text of the last error on the calling thread ("" if none; the same text as tvinpaint_last_error). */
 const char* tgvinpaint_last_error(void);
 
 #ifdef __cplusplus
