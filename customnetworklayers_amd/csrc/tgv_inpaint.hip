@@ -659,52 +659,65 @@ __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
   gwy_[smp * 2 * HW + HW + p] = gwy1;
 }
 
-// Upstream check (TGV.cu:2686-2703): counts[0] = non-finite entries, counts[1] = non-zero finite ones.
+// Upstream check (TGV.cu:2686-2703): counts[0] = non-finite entries, counts[1] != 0 if any finite entry is non-zero.
+// One atomic per block and only for non-finite entries; the non-zero flag is a plain store of the same value from
+// whichever blocks see one (a counter bumped by every block of the launch would queue up at the memory side).
 __global__ __launch_bounds__(256) void tgv_upstream_check(const float* __restrict__ g, long long n,
                                                           unsigned int* __restrict__ counts) {
+  typedef float vec4 __attribute__((ext_vector_type(4)));
   unsigned int bad = 0, nz = 0;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (long long)gridDim.x * blockDim.x) {
-    const float v = g[i];
+  auto look = [&](float v) {
     if (!finite_value(v)) bad++;
     else if (v != 0.f) nz++;
+  };
+  const long long n4 = ((reinterpret_cast<uintptr_t>(g) & 15) == 0) ? (n >> 2) : 0;  // whole 16-byte groups
+  const vec4* __restrict__ g4 = reinterpret_cast<const vec4*>(g);
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (long long)gridDim.x * blockDim.x) {
+    const vec4 v = g4[i];
+    look(v.x); look(v.y); look(v.z); look(v.w);
   }
+  for (long long i = 4 * n4 + (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+    look(g[i]);
   bad = wave_sum_u(bad);
   nz = wave_sum_u(nz);
   __shared__ unsigned int s_bad[4], s_nz[4];
   if ((threadIdx.x & 63) == 0) { s_bad[threadIdx.x >> 6] = bad; s_nz[threadIdx.x >> 6] = nz; }
   __syncthreads();
-  if (threadIdx.x == 0) {  // one pair of atomics per block, and only when there is something to report
+  if (threadIdx.x == 0) {
     bad = s_bad[0] + s_bad[1] + s_bad[2] + s_bad[3];
     nz = s_nz[0] + s_nz[1] + s_nz[2] + s_nz[3];
     if (bad) atomicAdd(&counts[0], bad);
-    if (nz && counts[1] == 0) atomicAdd(&counts[1], 1u);
+    if (nz) counts[1] = 1u;
   }
 }
 
 // The guard on the gradient wrt the starting point inspects only the u block (TGV.cu:3014-3021):
 // gather the u blocks of all samples into one contiguous tensor ...
 __global__ __launch_bounds__(256) void tgv_gather_u(const float* __restrict__ src, float* __restrict__ dst,
-                                                    long long CHW, long long total) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= total) return;
-  const long long s = i / CHW, r = i - s * CHW;
-  dst[i] = src[s * 3 * CHW + r];
+                                                    long long CHW) {
+  // grid (blocks, n): blockIdx.y is the sample
+  const float* __restrict__ sp = src + (long long)blockIdx.y * 3 * CHW;
+  float* __restrict__ dp = dst + (long long)blockIdx.y * CHW;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < CHW; i += (long long)gridDim.x * blockDim.x)
+    dp[i] = sp[i];
 }
 // ... and apply its verdict to the u blocks only; v1 / v2 gradients pass through (TGV.cu:3047).
 __global__ __launch_bounds__(256) void tgv_finalize_init(const float* __restrict__ src, float* __restrict__ out,
-                                                         long long CHW, long long total,
-                                                         const GuardState* __restrict__ gs, GuardParams p) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= total) return;
-  const long long r = i % (3 * CHW);
-  float v = src[i];
-  if (r < CHW) {
-    const double mult = gs->scale[4];
-    v = guard_limit(v, p);
-    if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
+                                                         long long CHW, const GuardState* __restrict__ gs, GuardParams p) {
+  // grid (blocks, n, 3): blockIdx.y is the sample, blockIdx.z the variable (0 = u)
+  const long long base = ((long long)blockIdx.y * 3 + blockIdx.z) * CHW;
+  const float* __restrict__ sp = src + base;
+  float* __restrict__ op = out + base;
+  const bool is_u = blockIdx.z == 0;
+  const double mult = gs->scale[4];
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < CHW; i += (long long)gridDim.x * blockDim.x) {
+    float v = sp[i];
+    if (is_u) {
+      v = guard_limit(v, p);
+      if (mult != 1.0) v = (mult == 0.0) ? 0.f : (float)((double)v * mult);
+    }
+    op[i] = v;
   }
-  out[i] = v;
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -1280,7 +1293,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     ZeroList z;
     z.ptr[0] = s.counts; z.bytes[0] = 8;
     hipLaunchKernelGGL(fill_zero_many, dim3(1, 1), dim3(256), 0, stream, z);
-    hipLaunchKernelGGL(tgv_upstream_check, dim3(std::min(gS, 1024)), dim3(256), 0, stream, gin, (long long)S3, s.counts);
+    hipLaunchKernelGGL(tgv_upstream_check, dim3(std::min(grid_stride((long long)S3 / 4 + 1), 2048)), dim3(256), 0, stream, gin, (long long)S3, s.counts);
     unsigned int host_counts[2] = {0, 0};
     INPAINT_HIP(hipMemcpyAsync(host_counts, s.counts, 8, hipMemcpyDeviceToHost, stream));
     INPAINT_HIP(hipStreamSynchronize(stream));
@@ -1521,8 +1534,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   }
   // output guard on the device (TGV.cu:2990-3021), then scale and store (TGV.cu:3024-3050)
   hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(64), 0, stream, s.guard);
-  hipLaunchKernelGGL(tgv_gather_u, dim3(grid1d((long long)F)), dim3(256), 0, stream, gi_src, s.gi_u,
-                     (long long)ic * ih * iw, (long long)F);
+  {
+    const long long CHW = (long long)ic * ih * iw;
+    hipLaunchKernelGGL(tgv_gather_u, dim3(std::min(grid_stride(CHW), 1024), n), dim3(256), 0, stream, gi_src, s.gi_u, CHW);
+  }
   const double* tots[4] = {s.tot_gc, s.tot_gx, s.tot_gy, s.tot_gb};
   const long long cnts[5] = {(long long)P, (long long)(2 * P), (long long)(2 * P), (long long)F, (long long)F};
   GuardJobs jobs;
@@ -1548,8 +1563,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     fin.per_sample[k] = weights ? HW2 : 1;
   }
   hipLaunchKernelGGL(finalize_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, fin, s.guard, kGuard, corr ? 1.f : kGlobalGMult);
-  hipLaunchKernelGGL(tgv_finalize_init, dim3(grid1d((long long)S3)), dim3(256), 0, stream, gi_src, gi,
-                     (long long)ic * ih * iw, (long long)S3, s.guard, kGuard);
+  {
+    const long long CHW = (long long)ic * ih * iw;
+    hipLaunchKernelGGL(tgv_finalize_init, dim3(std::min(grid_stride(CHW), 1024), n, 3), dim3(256), 0, stream, gi_src, gi, CHW,
+                       s.guard, kGuard);
+  }
   INPAINT_HIP(hipGetLastError());
   s.run++;  // TGV.cu:3061
   return 0;
