@@ -1283,8 +1283,8 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
         const float* xb = ring + (size_t)(j - 1) * F;
         float *g_in = s.g05[pp_src], *g_out = s.g05[1 - pp_src], *x_in = s.gxk[pp_src], *x_out = s.gxk[1 - pp_src];
         // A pair that ends a segment stores the segment's sums as a record; it does not write the zeros the next segment
-        // starts from (only the sweep's very last launch clears the accumulators): a segment's first pair reads zeros
-        // from the slot's field of zeros instead, which stays in the cache.
+        // starts from: a segment's first pair reads zeros from the slot's field of zeros instead, which stays in the
+        // cache (and the next backward pass clears the accumulators itself, or starts with a launch that does not read them).
         s.acc_fresh = outer < nseg - 1 && j == len - 1;
         if (j - 1 > 0) {
           const float* xc = ring + (size_t)(j - 2) * F;

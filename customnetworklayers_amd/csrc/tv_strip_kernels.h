@@ -839,10 +839,11 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip(
 }
 
 // -------------------------------------------------------------------------------------------------
-// Accumulators at a segment end, in all pair kernels below: a BEND launch stores the segment's sums as a record; the
-// zeros the reference leaves in the accumulators (TV.cu:178-218) are written by the very last launch of the sweep only
-// (FINAL).  After any other BEND launch the accumulator set it would have written holds stale values, and the caller
-// hands the next launch a field of zeros as gc_in / gb_in / gwx_in / gwy_in instead.
+// Accumulators at a segment end, in all pair kernels below: a BEND launch stores the segment's sums as a record and
+// does not write the zeros the reference leaves in the accumulators (TV.cu:178-218).  The accumulator set it would have
+// written holds stale values afterwards: the caller hands the next segment's first launch a field of zeros as
+// gc_in / gb_in / gwx_in / gwy_in instead, and a later backward pass starts by clearing the accumulators or from a
+// launch that does not read them.
 // -------------------------------------------------------------------------------------------------
 // Two adjoint steps per launch (A = local iteration j, B = j-1), same arithmetic as tv_adjoint_strip
 // applied twice.  B runs one row behind A in the same wavefront: A's outputs g05[j] (B's incoming
@@ -1098,7 +1099,6 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
             stg(g05o_p, roffB + chs[ch], g05v);
             if (BEND) {  // segment flush, fused (TV.cu:178-218)
               __builtin_nontemporal_store(gbv, &seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)]);
-              if (FINAL) stg(gbo_p, roffB + chs[ch], 0.f);
             } else {
               stg(gbo_p, roffB + chs[ch], gbv);
             }
@@ -1111,9 +1111,6 @@ __global__ __launch_bounds__(256) void tv_adjoint_strip2(
           __builtin_nontemporal_store(gcB, &seg_gc[e]);
           __builtin_nontemporal_store(gwxB, &seg_gwx[e]);
           __builtin_nontemporal_store(gwyB, &seg_gwy[e]);
-          if (FINAL) stg(gco_p, roffB, 0.f);
-          if (FINAL) stg(gwxo_p, roffB, 0.f);
-          if (FINAL) stg(gwyo_p, roffB, 0.f);
         } else {
           stg(gco_p, roffB, gcB);
           stg(gwxo_p, roffB, gwxB);
@@ -1434,7 +1431,6 @@ __global__ __launch_bounds__(128) void tv_adjoint_strip2c(
               stg(g05o_p, roffB + chs[ch], g05v);
               if (BEND) {  // segment flush, fused (TV.cu:178-218)
                 __builtin_nontemporal_store(gbv, &seg_gb[((size_t)g.n * Ct + wave + ch) * HW + (roffB >> 2)]);
-                if (FINAL) stg(gbo_p, roffB + chs[ch], 0.f);
               } else {
                 stg(gbo_p, roffB + chs[ch], gbv);
               }
@@ -1447,9 +1443,6 @@ __global__ __launch_bounds__(128) void tv_adjoint_strip2c(
             __builtin_nontemporal_store(gcB, &seg_gc[e]);
             __builtin_nontemporal_store(gwxB, &seg_gwx[e]);
             __builtin_nontemporal_store(gwyB, &seg_gwy[e]);
-            if (FINAL) stg(gco_p, roffB, 0.f);
-            if (FINAL) stg(gwxo_p, roffB, 0.f);
-            if (FINAL) stg(gwyo_p, roffB, 0.f);
           } else {
             stg(gco_p, roffB, gcB);
             stg(gwxo_p, roffB, gwxB);
@@ -1847,7 +1840,6 @@ __global__ __launch_bounds__(128) void tv_adjoint_strip2w(
               stg(g05o_p, roffB + chs[ch], g05v);
               if (BEND) {  // segment flush, fused (TV.cu:178-218)
                 __builtin_nontemporal_store(gbv, &seg_gb[((size_t)g.n * Ct + ch) * HW + (roffB >> 2)]);
-                if (FINAL) stg(gbo_p, roffB + chs[ch], 0.f);
               } else {
                 stg(gbo_p, roffB + chs[ch], gbv);
               }
@@ -1860,9 +1852,6 @@ __global__ __launch_bounds__(128) void tv_adjoint_strip2w(
             __builtin_nontemporal_store(gcB, &seg_gc[e]);
             __builtin_nontemporal_store(gwxB, &seg_gwx[e]);
             __builtin_nontemporal_store(gwyB, &seg_gwy[e]);
-            if (FINAL) stg(gco_p, roffB, 0.f);
-            if (FINAL) stg(gwxo_p, roffB, 0.f);
-            if (FINAL) stg(gwyo_p, roffB, 0.f);
           } else {
             stg(gco_p, roffB, gcB);
             stg(gwxo_p, roffB, gwxB);
@@ -2291,7 +2280,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
               stg(g05o_p, roffB + plane4 * ch, g05v);
               if (BEND) {  // segment flush, fused (TV.cu:178-218)
                 __builtin_nontemporal_store(gbv, &seg_gb[((size_t)g.n * Ct + ch0 + ch) * HW + (roffB >> 2)]);
-                if (FINAL) stg(gbo_p, roffB + plane4 * ch, 0.f);
               } else {
                 stg(gbo_p, roffB + plane4 * ch, gbv);
               }
@@ -2304,9 +2292,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             __builtin_nontemporal_store(gcB, &seg_gc[e]);
             __builtin_nontemporal_store(gwxB, &seg_gwx[e]);
             __builtin_nontemporal_store(gwyB, &seg_gwy[e]);
-            if (FINAL) stg(gco_p, roffB, 0.f);
-            if (FINAL) stg(gwxo_p, roffB, 0.f);
-            if (FINAL) stg(gwyo_p, roffB, 0.f);
           } else {
             stg(gco_p, roffB, gcB);
             stg(gwxo_p, roffB, gwxB);
