@@ -970,7 +970,8 @@ void launch_forward(const Slot& s, hipStream_t stream, const float* c, const flo
 template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin,
                                const float* xin_aux, float* xout, const float* yin, float* yout, float* x05a, float* x05b,
-                               bool store_x_aux, float tA, float tB, bool ring, float tP, int groups = 1) {
+                               bool store_x_aux, float tA, float tB, bool ring, float tP, int groups = 1,
+                               float* keep_x = nullptr, float* keep_y = nullptr) {
   auto kern = tgvstrip::tgv_forward_strip2<C, false>;
   if (x05a && ring) kern = tgvstrip::tgv_forward_strip2<C, true, true>;
   else if (x05a) kern = tgvstrip::tgv_forward_strip2<C, true>;
@@ -979,7 +980,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* c
   const long long waves = (long long)sx * sy * s.n * groups;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   hipLaunchKernelGGL(kern, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b,
-                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic, groups);
+                     store_x_aux ? 1 : 0, s.n, s.ih, s.iw, tA, tB, (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic, groups, keep_x, keep_y);
 }
 
 // One channel per wavefront, all channels in one launch (the C = 1 instantiation with the channel as a grid dimension;
@@ -1003,18 +1004,22 @@ bool forward_pairs(const Slot& s) {
 // extrapolation factor of the iteration that made it); such a launch writes x05 rows only.
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                          const float* yin, float* yout, float* x05a, float* x05b, float tA, float tB,
-                         const float* xin_aux = nullptr, bool store_x_aux = true, bool ring = false, float tP = 0.f) {
+                         const float* xin_aux = nullptr, bool store_x_aux = true, bool ring = false, float tP = 0.f,
+                         float* keep_x = nullptr, float* keep_y = nullptr) {
+  // keep_x / keep_y: where the launch leaves a copy of its input iterate (checkpoint 0 = the starting point)
   if (forward_split_channels(s)) {
-    launch_forward_pair_strip<1>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP, s.ic);
+    launch_forward_pair_strip<1>(s, stream, c, b, xin, xin_aux, xout, yin, yout, x05a, x05b, store_x_aux, tA, tB, ring, tP, s.ic,
+                                 keep_x, keep_y);
     return;
   }
   for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
     const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gxa = at_channel(s, xin_aux, ch0), *gyi = at_channel(s, yin, ch0);
     float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *ga = at_channel(s, x05a, ch0), *gbb = at_channel(s, x05b, ch0);
+    float *kx = at_channel(s, keep_x, ch0), *ky = at_channel(s, keep_y, ch0);
     if (s.ic - ch0 == 1)
-      launch_forward_pair_strip<1>(s, stream, c, gb, gxi, gxa, gxo, gyi, gyo, ga, gbb, store_x_aux, tA, tB, ring, tP);
+      launch_forward_pair_strip<1>(s, stream, c, gb, gxi, gxa, gxo, gyi, gyo, ga, gbb, store_x_aux, tA, tB, ring, tP, 1, kx, ky);
     else
-      launch_forward_pair_strip<2>(s, stream, c, gb, gxi, gxa, gxo, gyi, gyo, ga, gbb, store_x_aux, tA, tB, ring, tP);
+      launch_forward_pair_strip<2>(s, stream, c, gb, gxi, gxa, gxo, gyi, gyo, ga, gbb, store_x_aux, tA, tB, ring, tP, 1, kx, ky);
   }
 }
 
@@ -1225,8 +1230,12 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
     }
   } else {
     scale_weights(s, stream, dx, dy);
-    hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)S3)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
-                       (long long)S3);  // checkpoint 0 = init
+    // checkpoint 0 = the starting point: the first pair launch reads `init` itself and leaves the two copies as it
+    // goes; one-iteration launches (and a caller that iterates in place) get them from a copy kernel
+    const bool copy_in_pair = forward_pairs(s) && out != init;
+    if (!copy_in_pair)
+      hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)S3)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
+                         (long long)S3);
     // first iteration whose x05 row is kept, and the ring row of iteration k
     const int kl = s.iterations.empty() ? K : (keep == 2 ? 0 : (keep == 1 ? s.iterations.back() : K));
     auto ring_row = [&](int k) { return s.x05 + (size_t)(keep == 2 ? k : k - kl) * S3; };
@@ -1250,7 +1259,10 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
           launch_forward_pair(s, stream, c, b, ring_row(k - 2), wanted ? Xp(k + 2) : nullptr, ring_row(k - 1),
                               wanted ? Yp(k + 2) : nullptr, h0, h0 + S3, s.steps[k], s.steps[k + 1], nullptr, true, true,
                               s.steps[k - 1]);
-        } else
+        } else if (k == 0 && copy_in_pair)
+          launch_forward_pair(s, stream, c, b, init, Xp(2), init, Yp(2), h0, h0 ? h0 + S3 : nullptr, s.steps[0], s.steps[1],
+                              nullptr, true, false, 0.f, s.ckpt_x, s.ckpt_y);
+        else
           launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + S3 : nullptr, s.steps[k],
                               s.steps[k + 1]);
       }

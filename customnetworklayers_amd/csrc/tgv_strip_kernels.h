@@ -262,7 +262,9 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const float* __restrict__ xin, const float* __restrict__ xin_aux, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
     int store_x_aux, int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct,
-    int groups) {
+    int groups, float* __restrict__ keep_x = nullptr, float* __restrict__ keep_y = nullptr) {
+  // keep_x / keep_y (optional, not with RING): the input iterate is copied there on the strip's own rows as it passes
+  // through -- how the starting point reaches checkpoint 0 without a copy launch
   // groups > 1: the launch covers `groups` consecutive channel groups of C channels each, every strip once per group
   // (forward channels never couple)
   StripGeom g;
@@ -281,7 +283,8 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
   const float *const wx_p = wx + poff, *const wy_p = wy + poff, *const bx_p = bx + poff, *const by_p = by + poff,
                      *const cf_p = cf + poff;
   const float *y_p[3][C], *x_p[3][C], *b_p[C];
-  float *yo_p[3][C], *xo_p[3][C], *xa_p[3][C], *xb_p[3][C];
+  float *yo_p[3][C], *xo_p[3][C], *xa_p[3][C], *xb_p[3][C], *kx_p[3][C], *ky_p[3][C];
+  const bool keep_in = !RING && keep_x != nullptr;
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
     b_p[ch] = b + ((size_t)g.n * Ct + ch_first + ch) * HW;
@@ -293,6 +296,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
       y_p[v][ch] = yin + q; x_p[v][ch] = ((v > 0 && xin_aux) ? xin_aux : xin) + q;
       yo_p[v][ch] = yout + q; xo_p[v][ch] = xout + q;
       xa_p[v][ch] = X05 ? x05a + q : nullptr; xb_p[v][ch] = X05 ? x05b + q : nullptr;
+      kx_p[v][ch] = keep_in ? keep_x + q : nullptr; ky_p[v][ch] = keep_in ? keep_y + q : nullptr;
     }
   }
   const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
@@ -451,6 +455,13 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
           stg(xa_p[0][ch], roffA, u.xh);
           stg(xa_p[1][ch], roffA, u.y1n);
           stg(xa_p[2][ch], roffA, u.y2n);
+        }
+        if (!RING && keep_in && storeA) {  // (own rows are inside the image: cur.y is the loaded value there)
+#pragma unroll
+          for (int v = 0; v < 3; v++) {
+            stg(kx_p[v][ch], roffA, cur.x[v][ch]);
+            stg(ky_p[v][ch], roffA, cur.y[v][ch]);
+          }
         }
       }
     }

@@ -662,7 +662,8 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* dx, co
 template <int C>
 void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                                const float* b, const float* xin, float* xout, const float* yin, float* yout,
-                               float* x05a, float* x05b, float tA, float tB, bool ring, float tP, int groups = 1) {
+                               float* x05a, float* x05b, float tA, float tB, bool ring, float tP, int groups = 1,
+                               float* keep_x = nullptr, float* keep_y = nullptr) {
   auto kern = tvstrip::tv_forward_strip2<C, false>;
   if (x05a && ring) kern = tvstrip::tv_forward_strip2<C, true, true>;
   else if (x05a) kern = tvstrip::tv_forward_strip2<C, true>;
@@ -671,7 +672,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* d
   const long long waves = (long long)sx * sy * s.n * groups;
   const dim3 grid((unsigned)(((waves + 3) / 4 + 7) / 8 * 8)), block(256);
   hipLaunchKernelGGL(kern, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, s.n, s.ih, s.iw, tA, tB,
-                     (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic, groups);
+                     (x05a && ring) ? tP : 0.f, R, sx, sy, s.ic, groups, keep_x, keep_y);
 }
 
 // A launch that cannot give every SIMD of the chip a wavefront lasts as long as one wavefront needs for its strip, and
@@ -696,19 +697,22 @@ bool forward_pairs(const Slot& s) {
 // (tP: extrapolation factor of the iteration that made it); such a launch writes x05 rows only
 void launch_forward_pair(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                          const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05a,
-                         float* x05b, float tA, float tB, bool ring = false, float tP = 0.f) {
+                         float* x05b, float tA, float tB, bool ring = false, float tP = 0.f, float* keep_x = nullptr,
+                         float* keep_y = nullptr) {
+  // keep_x / keep_y: where the launch leaves a copy of its input iterate (checkpoint 0 = the starting point)
   if (forward_split_channels(s)) {
-    launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP, s.ic);
+    launch_forward_pair_strip<1>(s, stream, dx, dy, c, b, xin, xout, yin, yout, x05a, x05b, tA, tB, ring, tP, s.ic, keep_x, keep_y);
     return;
   }
   for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
     const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
     float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *ga = at_channel(s, x05a, ch0), *gbb = at_channel(s, x05b, ch0);
+    float *kx = at_channel(s, keep_x, ch0), *ky = at_channel(s, keep_y, ch0);
     switch (std::min(kGroup, s.ic - ch0)) {
-      case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
-      case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
-      case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
-      default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP); break;
+      case 1: launch_forward_pair_strip<1>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP, 1, kx, ky); break;
+      case 2: launch_forward_pair_strip<2>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP, 1, kx, ky); break;
+      case 3: launch_forward_pair_strip<3>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP, 1, kx, ky); break;
+      default: launch_forward_pair_strip<4>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, ga, gbb, tA, tB, ring, tP, 1, kx, ky); break;
     }
   }
 }
@@ -1040,8 +1044,12 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
       hipLaunchKernelGGL(fill_zero_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, s.ckpt_x, (long long)F);
     }
   } else {
-    hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
-                       (long long)F);  // checkpoint 0 = init
+    // checkpoint 0 = the starting point: the first pair launch reads `init` itself and leaves the two copies as it
+    // goes; one-iteration launches get them from a copy kernel
+    const bool copy_in_pair = forward_pairs(s) && out != init;  // (a caller that iterates in place keeps the copy launch)
+    if (!copy_in_pair)
+      hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
+                         (long long)F);
     // first iteration whose x05 row is kept, and the ring row of iteration k
     const int kl = s.iterations.empty() ? K : (keep == 2 ? 0 : (keep == 1 ? s.iterations.back() : K));
     auto ring_row = [&](int k) { return s.x05 + (size_t)(keep == 2 ? k : k - kl) * F; };
@@ -1065,7 +1073,10 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
           const bool wanted = k + 2 == K || ck_index(k + 2) >= 0;
           launch_forward_pair(s, stream, dx, dy, c, b, ring_row(k - 2), wanted ? Xp(k + 2) : nullptr, ring_row(k - 1),
                               wanted ? Yp(k + 2) : nullptr, h0, h0 + F, s.steps[k], s.steps[k + 1], true, s.steps[k - 1]);
-        } else
+        } else if (k == 0 && copy_in_pair)
+          launch_forward_pair(s, stream, dx, dy, c, b, init, Xp(2), init, Yp(2), h0, h0 ? h0 + F : nullptr, s.steps[0],
+                              s.steps[1], false, 0.f, s.ckpt_x, s.ckpt_y);
+        else
           launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + F : nullptr,
                               s.steps[k], s.steps[k + 1]);
       }

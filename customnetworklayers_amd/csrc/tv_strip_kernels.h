@@ -301,7 +301,10 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
     const float* __restrict__ yin, float* __restrict__ yout, float* __restrict__ x05a, float* __restrict__ x05b,
-    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct, int groups) {
+    int N, int H, int W, float tA, float tB, float tP, int R, int strips_x, int strips_y, int Ct, int groups,
+    float* __restrict__ keep_x = nullptr, float* __restrict__ keep_y = nullptr) {
+  // keep_x / keep_y (optional, not with RING): the input iterate is copied there on the strip's own rows as it passes
+  // through -- how the starting point reaches checkpoint 0 without a copy launch
   // groups > 1: the launch covers `groups` consecutive channel groups of C channels each, every strip once per group
   // (forward channels never couple): small images then spread over more wavefronts, each with a shorter row step
   StripGeom g;
@@ -320,13 +323,15 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
   const float* const wy_p = wy + (size_t)g.n * HW;
   const float* const cf_p = cf + (size_t)g.n * HW;
   const float *y_p[C], *x_p[C], *b_p[C];
-  float *yo_p[C], *xo_p[C], *xa_p[C], *xb_p[C];
+  float *yo_p[C], *xo_p[C], *xa_p[C], *xb_p[C], *kx_p[C], *ky_p[C];
+  const bool keep_in = !RING && keep_x != nullptr;
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
     const size_t q = ((size_t)g.n * Ct + ch_first + ch) * HW;
     y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
     yo_p[ch] = yout + q; xo_p[ch] = xout + q;
     xa_p[ch] = X05 ? x05a + q : nullptr; xb_p[ch] = X05 ? x05b + q : nullptr;
+    kx_p[ch] = keep_in ? keep_x + q : nullptr; ky_p[ch] = keep_in ? keep_y + q : nullptr;
   }
   const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
 
@@ -429,6 +434,10 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
         nyB[ch] = in_img ? yn : 0.f;  // B reads zero padding outside the image (TV.cu:1229,1237)
         nxB[ch] = x_loc;
         if (X05 && storeA) stg(xa_p[ch], roffA, xh);
+        if (!RING && keep_in && storeA) {  // (own rows are inside the image: cur.y is the loaded value there)
+          stg(kx_p[ch], roffA, cur.x[ch]);
+          stg(ky_p[ch], roffA, cur.y[ch]);
+        }
       }
     }
     if (tri_b.value) {
