@@ -1259,9 +1259,13 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
           launch_forward_pair(s, stream, c, b, ring_row(k - 2), wanted ? Xp(k + 2) : nullptr, ring_row(k - 1),
                               wanted ? Yp(k + 2) : nullptr, h0, h0 + S3, s.steps[k], s.steps[k + 1], nullptr, true, true,
                               s.steps[k - 1]);
-        } else if (k == 0 && copy_in_pair)
-          launch_forward_pair(s, stream, c, b, init, Xp(2), init, Yp(2), h0, h0 ? h0 + S3 : nullptr, s.steps[0], s.steps[1],
-                              nullptr, true, false, 0.f, s.ckpt_x, s.ckpt_y);
+        } else if (k == 0 && copy_in_pair) {
+          // (with every x05 row kept the next pair rebuilds its input from those rows: the iterate is stored only where
+          // somebody reads it)
+          const bool wanted = keep != 2 || 2 == K || ck_index(2) >= 0;
+          launch_forward_pair(s, stream, c, b, init, wanted ? Xp(2) : nullptr, init, wanted ? Yp(2) : nullptr, h0,
+                              h0 ? h0 + S3 : nullptr, s.steps[0], s.steps[1], nullptr, true, false, 0.f, s.ckpt_x, s.ckpt_y);
+        }
         else
           launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + S3 : nullptr, s.steps[k],
                               s.steps[k + 1]);
