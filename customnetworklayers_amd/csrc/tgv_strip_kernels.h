@@ -255,7 +255,8 @@ struct Fwd2Row {
 // the two iterations before it, which the ring holds anyway -- u: x = prox(x05[j-1]), y = x + tP (x - prox(x05[j-2]));
 // v1, v2: x = x05[j-1], y = x + tP (x - x05[j-2]), the forward pass's own expressions -- and no iterate is written.
 // yin / xin then point at those two rows.
-template <int C, bool X05, bool RING = false>
+// STORE = false: the launch stores no iterate at all (xout, yout ignored), and its row loop carries no code for it.
+template <int C, bool X05, bool RING = false, bool STORE = true>
 __global__ __launch_bounds__(256) void tgv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ bx,
     const float* __restrict__ by, const float* __restrict__ cf, const float* __restrict__ b,
@@ -271,7 +272,9 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
   if (!strip_geometry(g, kCols2, R, W, strips_x, strips_y, N * groups, 2)) return;
   const int ch_first = (g.n % groups) * C;
   g.n /= groups;
-  const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
+  // the output iterate is stored where the caller wants it: x and y separately, or neither (a launch whose successor
+  // rebuilds its input from the x05 rows)
+  const bool store_x = STORE && xout != nullptr, store_y = STORE && yout != nullptr;
   const size_t HW = (size_t)H * W, CHW = HW * Ct;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
                      *const cf_p = cf + poff;
   const float *y_p[3][C], *x_p[3][C], *b_p[C];
   float *yo_p[3][C], *xo_p[3][C], *xa_p[3][C], *xb_p[3][C], *kx_p[3][C], *ky_p[3][C];
-  const bool keep_in = !RING && keep_x != nullptr;
+  const bool keep_xin = !RING && keep_x != nullptr, keep_yin = !RING && keep_y != nullptr;
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
     b_p[ch] = b + ((size_t)g.n * Ct + ch_first + ch) * HW;
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
       y_p[v][ch] = yin + q; x_p[v][ch] = ((v > 0 && xin_aux) ? xin_aux : xin) + q;
       yo_p[v][ch] = yout + q; xo_p[v][ch] = xout + q;
       xa_p[v][ch] = X05 ? x05a + q : nullptr; xb_p[v][ch] = X05 ? x05b + q : nullptr;
-      kx_p[v][ch] = keep_in ? keep_x + q : nullptr; ky_p[v][ch] = keep_in ? keep_y + q : nullptr;
+      kx_p[v][ch] = keep_xin ? keep_x + q : nullptr; ky_p[v][ch] = keep_yin ? keep_y + q : nullptr;
     }
   }
   const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
@@ -456,11 +459,11 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
           stg(xa_p[1][ch], roffA, u.y1n);
           stg(xa_p[2][ch], roffA, u.y2n);
         }
-        if (!RING && keep_in && storeA) {  // (own rows are inside the image: cur.y is the loaded value there)
+        if (!RING && storeA) {  // (own rows are inside the image: cur.y is the loaded value there)
 #pragma unroll
           for (int v = 0; v < 3; v++) {
-            stg(kx_p[v][ch], roffA, cur.x[v][ch]);
-            stg(ky_p[v][ch], roffA, cur.y[v][ch]);
+            if (keep_xin) stg(kx_p[v][ch], roffA, cur.x[v][ch]);
+            if (keep_yin) stg(ky_p[v][ch], roffA, cur.y[v][ch]);
           }
         }
       }
@@ -476,10 +479,12 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
           const Upd u = update(pyB[0][ch], pyB[1][ch], pyB[2][ch], t, aFa, aG1y, aG2y, pc, rc1B, pbb[ch], pxB[0][ch],
                                pxB[1][ch], pxB[2][ch], tB);
           if (store_lane) {
-            if (store_xy) {
+            if (store_y) {
               stg(yo_p[0][ch], roffB, u.yn);
               stg(yo_p[1][ch], roffB, u.y1o);
               stg(yo_p[2][ch], roffB, u.y2o);
+            }
+            if (store_x) {
               stg(xo_p[0][ch], roffB, u.x_loc);
               if (store_x_aux) {
                 stg(xo_p[1][ch], roffB, u.y1n);

@@ -489,6 +489,10 @@ struct Slot {
   // recomputed from its checkpoint, the reference's order of work), 1 those of the last segment, 2 all of them (no
   // recompute at all; the ring then has one row per iteration).
   int keep_mode = 2;
+  // Which half of a checkpoint behind the first the last forward stored: -1 both; 0 only y (what the reference's backward
+  // reads at a segment start); 1 only x (what the corrected gradient reads).  A forward that keeps every x05 row stores
+  // the half its id's gradient mode needs, since no segment is ever recomputed from the checkpoint.
+  int ckpt_half = -1;
   int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
   // shape and its whose every-row ring (keep mode 2) the device refused: later forwards of that shape go straight
@@ -665,7 +669,7 @@ void launch_forward_pair_strip(const Slot& s, hipStream_t stream, const float* d
                                float* x05a, float* x05b, float tA, float tB, bool ring, float tP, int groups = 1,
                                float* keep_x = nullptr, float* keep_y = nullptr) {
   auto kern = tvstrip::tv_forward_strip2<C, false>;
-  if (x05a && ring) kern = tvstrip::tv_forward_strip2<C, true, true>;
+  if (x05a && ring) kern = (xout || yout) ? tvstrip::tv_forward_strip2<C, true, true> : tvstrip::tv_forward_strip2<C, true, true, false>;
   else if (x05a) kern = tvstrip::tv_forward_strip2<C, true>;
   const int R = strip_rows(s.n * groups, s.ih, s.iw, tvstrip::kFwd2Cols, knobs().tv_fwd_rows, 8);
   const int sx = (s.iw + tvstrip::kFwd2Cols - 1) / tvstrip::kFwd2Cols, sy = (s.ih + R - 1) / R;
@@ -1046,6 +1050,10 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   } else {
     // checkpoint 0 = the starting point: the first pair launch reads `init` itself and leaves the two copies as it
     // goes; one-iteration launches get them from a copy kernel
+    // a forward that keeps every x05 row never recomputes from a checkpoint: behind checkpoint 0 it stores only the half
+    // the backward pass of this id's gradient mode reads at a segment start (y: the reference's; x: the corrected one)
+    const bool want_x = s.grad_mode == 1, want_y = !want_x;
+    s.ckpt_half = (keep == 2 && forward_pairs(s)) ? (want_x ? 1 : 0) : -1;
     const bool copy_in_pair = forward_pairs(s) && out != init;  // (a caller that iterates in place keeps the copy launch)
     if (!copy_in_pair)
       hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, init, s.ckpt_y, s.ckpt_x,
@@ -1070,14 +1078,17 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
           // With every x05 row kept the iterate need not travel through memory either: the pair rebuilds it from the
           // two rows before it, as the recompute launches of the backward pass do, and stores it only where somebody
           // reads it -- at a checkpoint and at the end.
-          const bool wanted = k + 2 == K || ck_index(k + 2) >= 0;
-          launch_forward_pair(s, stream, dx, dy, c, b, ring_row(k - 2), wanted ? Xp(k + 2) : nullptr, ring_row(k - 1),
-                              wanted ? Yp(k + 2) : nullptr, h0, h0 + F, s.steps[k], s.steps[k + 1], true, s.steps[k - 1]);
+          // At the end that is x alone (the result); at a checkpoint the half the backward pass will read.
+          const bool last = k + 2 == K, ck = !last && ck_index(k + 2) >= 0;
+          launch_forward_pair(s, stream, dx, dy, c, b, ring_row(k - 2), (last || (ck && want_x)) ? Xp(k + 2) : nullptr,
+                              ring_row(k - 1), (ck && want_y) ? Yp(k + 2) : nullptr, h0, h0 + F, s.steps[k], s.steps[k + 1], true,
+                              s.steps[k - 1]);
         } else if (k == 0 && copy_in_pair) {
           // (with every x05 row kept the next pair rebuilds its input from those rows: the iterate is stored only where
           // somebody reads it)
-          const bool wanted = keep != 2 || 2 == K || ck_index(2) >= 0;
-          launch_forward_pair(s, stream, dx, dy, c, b, init, wanted ? Xp(2) : nullptr, init, wanted ? Yp(2) : nullptr, h0,
+          const bool last = 2 == K, ck = !last && ck_index(2) >= 0;
+          const bool sx = keep != 2 || last || (ck && want_x), sy = keep != 2 || (ck && want_y);
+          launch_forward_pair(s, stream, dx, dy, c, b, init, sx ? Xp(2) : nullptr, init, sy ? Yp(2) : nullptr, h0,
                               h0 ? h0 + F : nullptr, s.steps[0], s.steps[1], false, 0.f, s.ckpt_x, s.ckpt_y);
         }
         else
@@ -1164,6 +1175,8 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
   const bool corr = s.grad_mode == 1;
+  if (s.ckpt_half >= 0 && s.ckpt_half != (corr ? 1 : 0))
+    return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass, which kept the checkpoints of the other mode: run the forward pass again", id);
   if (corr && force_tile_path())
     return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TV_PATH=tile is set)");
   s.stream = stream;

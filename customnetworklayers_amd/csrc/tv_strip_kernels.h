@@ -296,7 +296,8 @@ struct Fwd2Row {
 // RING (recompute launches after a segment's first): the input iterate is not read but rebuilt from the x05 rows of
 // the two iterations before it, which the ring holds anyway -- x = prox(x05[j-1]), y = x + tP (x - prox(x05[j-2])),
 // the forward pass's own expressions -- and no iterate is written.  yin / xin then point at those two rows.
-template <int C, bool X05, bool RING = false>
+// STORE = false: the launch stores no iterate at all (xout, yout ignored), and its row loop carries no code for it.
+template <int C, bool X05, bool RING = false, bool STORE = true>
 __global__ __launch_bounds__(256) void tv_forward_strip2(
     const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
     const float* __restrict__ b, const float* __restrict__ xin, float* __restrict__ xout,
@@ -311,7 +312,9 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
   if (!strip_geometry(g, kFwd2Cols, R, W, strips_x, strips_y, N * groups, 2)) return;
   const int ch_first = (g.n % groups) * C;
   g.n /= groups;
-  const bool store_xy = xout != nullptr;  // the last recompute launch of a segment only needs the x05 rows
+  // the output iterate is stored where the caller wants it: x and y separately, or neither (a launch whose successor
+  // rebuilds its input from the x05 rows)
+  const bool store_x = STORE && xout != nullptr, store_y = STORE && yout != nullptr;
   const size_t HW = (size_t)H * W;
   const unsigned W4 = 4u * (unsigned)W;
   const unsigned wc = g.col_ok ? 4u * g.w : 0u;
@@ -324,14 +327,14 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
   const float* const cf_p = cf + (size_t)g.n * HW;
   const float *y_p[C], *x_p[C], *b_p[C];
   float *yo_p[C], *xo_p[C], *xa_p[C], *xb_p[C], *kx_p[C], *ky_p[C];
-  const bool keep_in = !RING && keep_x != nullptr;
+  const bool keep_xin = !RING && keep_x != nullptr, keep_yin = !RING && keep_y != nullptr;
 #pragma unroll
   for (int ch = 0; ch < C; ch++) {
     const size_t q = ((size_t)g.n * Ct + ch_first + ch) * HW;
     y_p[ch] = yin + q; x_p[ch] = xin + q; b_p[ch] = b + q;
     yo_p[ch] = yout + q; xo_p[ch] = xout + q;
     xa_p[ch] = X05 ? x05a + q : nullptr; xb_p[ch] = X05 ? x05b + q : nullptr;
-    kx_p[ch] = keep_in ? keep_x + q : nullptr; ky_p[ch] = keep_in ? keep_y + q : nullptr;
+    kx_p[ch] = keep_xin ? keep_x + q : nullptr; ky_p[ch] = keep_yin ? keep_y + q : nullptr;
   }
   const int h_lo = max(g.hs - 1, 0), h_hi = min(g.hs + Reff, H - 1);  // rows A updates
 
@@ -434,9 +437,9 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
         nyB[ch] = in_img ? yn : 0.f;  // B reads zero padding outside the image (TV.cu:1229,1237)
         nxB[ch] = x_loc;
         if (X05 && storeA) stg(xa_p[ch], roffA, xh);
-        if (!RING && keep_in && storeA) {  // (own rows are inside the image: cur.y is the loaded value there)
-          stg(kx_p[ch], roffA, cur.x[ch]);
-          stg(ky_p[ch], roffA, cur.y[ch]);
+        if (!RING && storeA) {  // (own rows are inside the image: cur.y is the loaded value there)
+          if (keep_xin) stg(kx_p[ch], roffA, cur.x[ch]);
+          if (keep_yin) stg(ky_p[ch], roffA, cur.y[ch]);
         }
       }
     }
@@ -451,10 +454,8 @@ __global__ __launch_bounds__(256) void tv_forward_strip2(
           float xh, x_loc, yn;
           update(pyB[ch], e1_above, from_left_lane(e2), e1, e2, pc, rc1B, pbb[ch], pxB[ch], tB, xh, x_loc, yn);
           if (store_lane) {
-            if (store_xy) {
-              stg(yo_p[ch], roffB, yn);
-              stg(xo_p[ch], roffB, x_loc);
-            }
+            if (store_y) stg(yo_p[ch], roffB, yn);
+            if (store_x) stg(xo_p[ch], roffB, x_loc);
             if (X05) stg(xb_p[ch], roffB, xh);
           }
         }

@@ -54,7 +54,7 @@ int tgvinpaint_reset_id(int id);
  * clamp of the adjoint iterates (562-583), the upstream check and the output guard stay.  With them inactive the
  * result is the gradient of the forward pass (tests compare it with the float64 oracle that automatic differentiation
  * pins).  Any channel count; two adjoint steps per launch with two channels (5% slower than the default), one
- * otherwise. */
+ * otherwise.  Set it before the forward pass whose backward it is meant for, as tvinpaint_gradient_mode. */
 int tgvinpaint_gradient_mode(int id, int mode);
 
 /* Which intermediate iterates (the x05 rows of TGVInpaintFista.cu:2775-2814) the next forwards on `id` keep for

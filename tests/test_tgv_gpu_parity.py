@@ -288,6 +288,22 @@ def test_first_step_of_the_sweep_rides_on_the_second(ext, tgv_oracle, c, its, mo
         np.testing.assert_array_equal(x, y)
 
 
+def test_gradient_mode_is_fixed_by_the_forward_pass(ext):
+    # as in the TV layer: a forward that keeps every x05 row stores one half of each checkpoint, the one its mode reads
+    dev = torch.device("cuda:0")
+    d = {k: torch.from_numpy(v).to(dev) for k, v in varying_inputs(1, 2, 24, 70, seed=12).items()}
+    try:
+        ext.reset_id(3)
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 20, 3)
+        ext.gradient_mode(3, 1)
+        with pytest.raises(RuntimeError, match="gradient mode"):
+            ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
+        ext.gradient_mode(3, 0)
+        ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
+    finally:
+        ext.reset_id(3)
+
+
 def test_varying_beta_and_per_sample_lipschitz(ext, tgv_oracle):
     # sample 0: beta up to 9 (bound above 32, data dependent); sample 1: small beta (bound 32)
     d = varying_inputs(2, 2, 40, 56, seed=11)
