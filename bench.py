@@ -24,10 +24,10 @@ HBM_PEAK_GBS = 8000.0
 #             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
 #   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
 COUNTERS = {
-    1: dict(traffic=(2 * 85088 + 68421) * 1024, step=(2 * 6586702 + 5726314) * 1024, lds=0, rocprof_ms=0.05201,
-            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="eb44935"),
-    2: dict(traffic=(2 * 160462 + 148208) * 1024, step=(2 * 13507418 + 13832001) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.11848,
-            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="eb44935"),
+    1: dict(traffic=(2 * 85091 + 68530) * 1024, step=(2 * 6586753 + 5549704) * 1024, lds=0, rocprof_ms=0.05151,
+            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="9dd8973"),
+    2: dict(traffic=(2 * 160472 + 148414) * 1024, step=(2 * 13495066 + 13252795) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.11738,
+            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="9dd8973"),
     5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
             files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
     6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="26d8b66"),
