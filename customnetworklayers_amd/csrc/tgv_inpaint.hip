@@ -1202,6 +1202,7 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   Slot& s = g_slots[id];
   s.forward_done = false;
   s.x05_valid = false;
+  s.ckpt_half = -1;
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
   const long long shape[5] = {n, ic, ih, iw, its};
   if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
