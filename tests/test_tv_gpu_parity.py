@@ -392,6 +392,35 @@ def test_errors(ext):
         ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 10201 + 300, 0)
 
 
+@pytest.mark.parametrize("its", [2, 3, 20])
+def test_forward_in_place_through_the_c_abi(ext, its):
+    # a caller of the C ABI may hand the starting point's buffer in as the output: the forward pass then copies the
+    # starting point aside before its first launch instead of letting that launch read it while the result is written
+    import ctypes
+
+    from customnetworklayers_amd._lib import lib
+
+    dev = torch.device("cuda:0")
+    d = tv_inputs(2, 2, 37, 130, seed=77 + its, conf_density=0.3)
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    ext.reset_id(4)
+    (ref,) = ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], its, 4)
+    gref = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+    buf = t["di"].clone()
+    n, c, h, w = d["db"].shape
+    p = lambda x: ctypes.c_void_p(x.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    ext.reset_id(4)
+    rc = lib.tvinpaint_forward(p(t["dx"]), p(t["dy"]), p(t["dc"]), p(t["db"]), p(buf), p(buf), n, c, h, w, its, 4, stream)
+    assert rc == 0
+    g = ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], its, 4)
+    torch.cuda.synchronize()
+    assert torch.equal(buf, ref)
+    for a, b in zip(g, gref):
+        assert torch.equal(a, b)
+    ext.reset_id(4)
+
+
 def test_gradient_mode_is_fixed_by_the_forward_pass(ext):
     # a forward that keeps every x05 row stores, at each checkpoint, only the half the backward of the id's mode reads;
     # a backward in the other mode says so instead of reading a stale buffer; with recomputed segments both halves exist
