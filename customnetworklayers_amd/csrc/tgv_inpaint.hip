@@ -1237,8 +1237,9 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
     scale_weights(s, stream, dx, dy);
     // checkpoint 0 = the starting point: the first pair launch reads `init` itself and leaves the two copies as it
     // goes; one-iteration launches (and a caller that iterates in place) get them from a copy kernel
-    // a forward that keeps every x05 row never recomputes from a checkpoint: behind checkpoint 0 it stores only the half
-    // the backward pass of this id's gradient mode reads at a segment start (y: the reference's; x: the corrected one)
+    // a forward that keeps every x05 row never recomputes from a checkpoint: it stores only the half of a checkpoint
+    // the backward pass of this id's gradient mode reads at a segment start (y: the reference's; x: the corrected one,
+    // which also reads checkpoint 0's y when it back-propagates iteration 0)
     const bool want_x = s.grad_mode == 1, want_y = !want_x;
     s.ckpt_half = (keep == 2 && forward_pairs(s)) ? (want_x ? 1 : 0) : -1;
     const bool copy_in_pair = forward_pairs(s) && out != init;
@@ -1275,7 +1276,7 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
           const bool last = 2 == K, ck = !last && ck_index(2) >= 0;
           const bool sx = keep != 2 || last || (ck && want_x), sy = keep != 2 || (ck && want_y);
           launch_forward_pair(s, stream, c, b, init, sx ? Xp(2) : nullptr, init, sy ? Yp(2) : nullptr, h0,
-                              h0 ? h0 + S3 : nullptr, s.steps[0], s.steps[1], nullptr, true, false, 0.f, s.ckpt_x, s.ckpt_y);
+                              h0 ? h0 + S3 : nullptr, s.steps[0], s.steps[1], nullptr, true, false, 0.f, (keep != 2 || want_x) ? s.ckpt_x : nullptr, s.ckpt_y);
         }
         else
           launch_forward_pair(s, stream, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + S3 : nullptr, s.steps[k],

@@ -1051,8 +1051,9 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   } else {
     // checkpoint 0 = the starting point: the first pair launch reads `init` itself and leaves the two copies as it
     // goes; one-iteration launches get them from a copy kernel
-    // a forward that keeps every x05 row never recomputes from a checkpoint: behind checkpoint 0 it stores only the half
-    // the backward pass of this id's gradient mode reads at a segment start (y: the reference's; x: the corrected one)
+    // a forward that keeps every x05 row never recomputes from a checkpoint: it stores only the half of a checkpoint
+    // the backward pass of this id's gradient mode reads at a segment start (y: the reference's; x: the corrected one,
+    // which also reads checkpoint 0's y when it back-propagates iteration 0)
     const bool want_x = s.grad_mode == 1, want_y = !want_x;
     s.ckpt_half = (keep == 2 && forward_pairs(s)) ? (want_x ? 1 : 0) : -1;
     const bool copy_in_pair = forward_pairs(s) && out != init;  // (a caller that iterates in place keeps the copy launch)
@@ -1090,7 +1091,7 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
           const bool last = 2 == K, ck = !last && ck_index(2) >= 0;
           const bool sx = keep != 2 || last || (ck && want_x), sy = keep != 2 || (ck && want_y);
           launch_forward_pair(s, stream, dx, dy, c, b, init, sx ? Xp(2) : nullptr, init, sy ? Yp(2) : nullptr, h0,
-                              h0 ? h0 + F : nullptr, s.steps[0], s.steps[1], false, 0.f, s.ckpt_x, s.ckpt_y);
+                              h0 ? h0 + F : nullptr, s.steps[0], s.steps[1], false, 0.f, (keep != 2 || want_x) ? s.ckpt_x : nullptr, s.ckpt_y);
         }
         else
           launch_forward_pair(s, stream, dx, dy, c, b, Xp(k), Xp(k + 2), Yp(k), Yp(k + 2), h0, h0 ? h0 + F : nullptr,
