@@ -261,6 +261,11 @@ struct GuardState {  // lives in device memory, one per id
   double report[25]; // per tensor: mean |g|, max |g|, num_above, num_invalid, action
   GuardStats stats[5];
   unsigned int tickets[5];  // blocks of pass 2 that have added their share of a tail sum (zero between launches)
+  // The TGV layer's verdict on the upstream gradient of the current backward pass (non-finite entries, or zero
+  // everywhere: every output is zero, the running means and the run count stay as they are), and how many backward
+  // passes so far had such an upstream.  The verdict stays on the device, so the host never waits for it: the host
+  // counts every backward pass and the guard subtracts `skipped`.  Always zero in the TV layer.
+  unsigned int upstream_bad, skipped;
   // pass 1 leaves per-block records here; they are combined in a fixed order (no atomics on one address, which
   // this GPU serialises at the memory side, and a mean that does not depend on the order of arrival)
   GuardStats partial[5][kGuardBlocks];
@@ -459,6 +464,8 @@ __device__ __forceinline__ void guard_tail_decide_body(const T* __restrict__ g, 
   c.tail_sum = any_invalid ? atomicAdd(&st->tail_sum, 0.0) : 0.0;
   if (any_invalid) gs->tickets[k] = 0;
   *st = c;
+  if (gs->upstream_bad) return;  // (TGV) this backward pass returns zeros: no decision, running mean and report untouched
+  run -= (int)gs->skipped;       // (TGV) backward passes that did not count
   double av_gc;
   if (n <= 0) {
     av_gc = 0;
@@ -643,6 +650,12 @@ static __global__ __launch_bounds__(256) void finalize_f32(const float* __restri
   }
 }
 
+// (TGV) every output of a backward pass whose upstream gradient was refused is zero
+template <class T>
+__device__ __forceinline__ void finalize_zero(T* __restrict__ out, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) out[i] = T(0);
+}
+
 // Guarded fp64 totals -> fp32 outputs, the four tensors of one backward in one launch (blockIdx.y picks the tensor):
 // limit, kill / rescale, global multiplier, then the chain factor of the weight scaling (TVInpaintFista.cu:1795-1818;
 // TGVInpaintFistaBetas.cu:3024-3050).  The chain factor is chain_const, or chain_per_sample[i / per_sample] when that
@@ -663,6 +676,11 @@ struct FinalizeJobs {
 static __global__ __launch_bounds__(256) void finalize_many(FinalizeJobs jobs, const GuardState* __restrict__ gs, GuardParams p,
                                                             float global_mult) {
   const int k = blockIdx.y;
+  if (gs->upstream_bad) {
+    if (k == 4) finalize_zero(jobs.f32_out, jobs.f32_n);
+    else finalize_zero(jobs.out[k], jobs.n[k]);
+    return;
+  }
   if (k == 4) {  // (finalize_f32)
     const double mult = gs->scale[jobs.f32_scale];
     const float* __restrict__ src = jobs.f32_src;

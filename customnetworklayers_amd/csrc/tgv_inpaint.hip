@@ -108,9 +108,11 @@ __global__ __launch_bounds__(BX* BY) void tgv_lipschitz_kernel(const float* __re
   if (threadIdx.x == 0 && bits > __float_as_uint(32.0f)) atomicMax(&maxbits[blockIdx.z], bits);
 }
 
-static __global__ void tgv_lipschitz_init(unsigned int* maxbits, int n) {
+// (`counts`, when given: the two words of the upstream check that follows, cleared here)
+static __global__ void tgv_lipschitz_init(unsigned int* maxbits, int n, unsigned int* counts) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) maxbits[i] = __float_as_uint((float)(fmax(12., 8. * (double)kBeta) + 0.000001));
+  if (counts && i < 2) counts[i] = 0u;
 }
 
 __device__ __forceinline__ double lipschitz_from_bits(unsigned int bits) {
@@ -691,6 +693,25 @@ __global__ __launch_bounds__(256) void tgv_upstream_check(const float* __restric
   }
 }
 
+// What the upstream check decides (TGV.cu:2698-2703), kept on the device: an upstream gradient with a non-finite entry,
+// or zero everywhere, is scrubbed in the caller's tensor; the verdict is latched in the guard's state, where the
+// guard's decision and the kernels that store the outputs read it (zeros out, running means and run count untouched).
+// The host never learns it and never waits for it.
+__global__ __launch_bounds__(256) void tgv_upstream_verdict(float* __restrict__ g, long long n,
+                                                            const unsigned int* __restrict__ counts,
+                                                            GuardState* __restrict__ gs) {
+  const bool bad = counts[0] != 0u || counts[1] == 0u;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    gs->upstream_bad = bad ? 1u : 0u;
+    if (bad) gs->skipped += 1u;
+  }
+  if (!bad) return;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    const float v = g[i];
+    if (!finite_value(v)) g[i] = 0.f;
+  }
+}
+
 // The guard on the gradient wrt the starting point inspects only the u block (TGV.cu:3014-3021):
 // gather the u blocks of all samples into one contiguous tensor ...
 __global__ __launch_bounds__(256) void tgv_gather_u(const float* __restrict__ src, float* __restrict__ dst,
@@ -709,6 +730,10 @@ __global__ __launch_bounds__(256) void tgv_finalize_init(const float* __restrict
   const float* __restrict__ sp = src + base;
   float* __restrict__ op = out + base;
   const bool is_u = blockIdx.z == 0;
+  if (gs->upstream_bad) {  // a refused upstream gradient: zeros (TGV.cu:2698-2703)
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < CHW; i += (long long)gridDim.x * blockDim.x) op[i] = 0.f;
+    return;
+  }
   const double mult = gs->scale[4];
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < CHW; i += (long long)gridDim.x * blockDim.x) {
     float v = sp[i];
@@ -724,6 +749,8 @@ __global__ __launch_bounds__(256) void tgv_finalize_init(const float* __restrict
 // per-id state (idStructBs, TGVInpaintFista.h:7-50)
 // -------------------------------------------------------------------------------------------------
 struct Slot {
+  // backward passes so far, INCLUDING those whose upstream gradient was refused: the device counts those in
+  // GuardState::skipped, and the reference's `run` is the difference (run_count())
   int run = 0;
   int n = 0, ic = 0, ih = 0, iw = 0, its = -1;
   bool forward_done = false;
@@ -735,6 +762,7 @@ struct Slot {
   // reads at a segment start); 1 only x (what the corrected gradient reads).  A forward that keeps every x05 row stores
   // the half its id's gradient mode needs, since no segment is ever recomputed from the checkpoint.
   int ckpt_half = -1;
+  int fwd_grad_mode = 0;  // the mode the last forward pass ran under: its backward passes must ask for the same one
   int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tgvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
   // shape and its whose every-row ring (keep mode 2) the device refused: later forwards of that shape go straight
@@ -777,12 +805,15 @@ size_t state_count(const Slot& s) { return (size_t)s.n * 3 * s.ic * s.ih * s.iw;
 size_t field_count(const Slot& s) { return (size_t)s.n * s.ic * s.ih * s.iw; }
 size_t plane_count(const Slot& s) { return (size_t)s.n * s.ih * s.iw; }
 
-int fetch_running_means(Slot& s) {
+// Reads the guard's running means back (waits for the id's stream); `skipped` = the backward passes the device refused.
+int fetch_running_means(Slot& s, unsigned int* skipped = nullptr) {
+  if (skipped) *skipped = 0;
   if (s.guard) {
     GuardState host;
     INPAINT_HIP(hipStreamSynchronize(s.stream));
     INPAINT_HIP(hipMemcpy(&host, s.guard, kGuardHeaderBytes, hipMemcpyDeviceToHost));
     for (int k = 0; k < 5; k++) s.pending_av[k] = host.av[k];
+    if (skipped) *skipped = host.skipped;
   }
   return 0;
 }
@@ -798,8 +829,10 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
                     s.iw == iw && s.its == its && s.ring_rows >= ring_rows;  // the ring only grows
   s.stream = stream;
   if (same) return 0;
-  int rc = fetch_running_means(s);
+  unsigned int skipped = 0;
+  int rc = fetch_running_means(s, &skipped);
   if (rc) return rc;
+  s.run -= (int)skipped;  // the new guard state starts counting refused passes from zero
   s.guard = nullptr;  // the arena is about to be released; the means live in pending_av until the new one exists
   s.n = n; s.ic = ic; s.ih = ih; s.iw = iw; s.its = its;
   make_schedule(its, s.iterations, s.max_inter_its);
@@ -882,9 +915,10 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
 
 // Lipschitz reduction + scaled weight copies for the weights of this call (forward and backward both
 // redo it, TGV.cu:2513-2531 and 2667-2679).
-void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const float* dy) {
+void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const float* dy, bool clear_counts = false) {
   const long long P = (long long)plane_count(s), HW = (long long)s.ih * s.iw;
-  hipLaunchKernelGGL(tgv_lipschitz_init, dim3((s.n + 255) / 256), dim3(256), 0, stream, s.maxbits, s.n);
+  hipLaunchKernelGGL(tgv_lipschitz_init, dim3((s.n + 255) / 256), dim3(256), 0, stream, s.maxbits, s.n,
+                     clear_counts ? s.counts : nullptr);
   hipLaunchKernelGGL(tgv_lipschitz_kernel, dim3((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n), dim3(BX, BY), 0, stream,
                      dx, dy, s.ih, s.iw, s.maxbits);
   hipLaunchKernelGGL(tgv_scale_kernel, dim3(grid1d(P)), dim3(256), 0, stream, dx, dy, s.maxbits, s.wx, s.wy, s.bx, s.by,
@@ -1203,6 +1237,7 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   s.forward_done = false;
   s.x05_valid = false;
   s.ckpt_half = -1;
+  s.fwd_grad_mode = s.grad_mode;
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
   const long long shape[5] = {n, ic, ih, iw, its};
   if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
@@ -1307,8 +1342,10 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
   const bool corr = s.grad_mode == 1;
-  if (s.ckpt_half >= 0 && s.ckpt_half != (corr ? 1 : 0))
-    return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass, which kept the checkpoints of the other mode: run the forward pass again", id);
+  // One rule in every keep mode (a forward that keeps every x05 row stores only the checkpoint halves its mode reads,
+  // so there the other mode could not be served at all):
+  if (s.grad_mode != s.fwd_grad_mode)
+    return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass: set it before the forward pass, or run the forward pass again", id);
   if (corr && !use_strip(s))
     return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TGV_PATH=px is set)");
   s.stream = stream;
@@ -1316,32 +1353,14 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   const int gS = grid_stride((long long)S3), gF = grid_stride((long long)F), gP = grid_stride((long long)P),
             g2P = grid_stride((long long)(2 * P));
 
-  // Upstream check (TGV.cu:2686-2703): any non-finite entry, or an upstream that is zero everywhere,
-  // returns all-zero gradients, scrubs the caller's tensor and leaves `run` alone.  The verdict
-  // decides a host-side counter, so this is the one host wait of the call.
-  {
-    ZeroList z;
-    z.ptr[0] = s.counts; z.bytes[0] = 8;
-    hipLaunchKernelGGL(fill_zero_many, dim3(1, 1), dim3(256), 0, stream, z);
-    hipLaunchKernelGGL(tgv_upstream_check, dim3(std::min(grid_stride((long long)S3 / 4 + 1), 2048)), dim3(256), 0, stream, gin, (long long)S3, s.counts);
-    unsigned int host_counts[2] = {0, 0};
-    INPAINT_HIP(hipMemcpyAsync(host_counts, s.counts, 8, hipMemcpyDeviceToHost, stream));
-    INPAINT_HIP(hipStreamSynchronize(stream));
-    if (host_counts[0] != 0 || host_counts[1] == 0) {
-      hipLaunchKernelGGL(scrub_kernel, dim3(gS), dim3(256), 0, stream, gin, (long long)S3);
-      ZeroList o;
-      o.ptr[0] = gi; o.bytes[0] = (long long)S3 * 4;
-      o.ptr[1] = gx; o.bytes[1] = (long long)P * 8;
-      o.ptr[2] = gy; o.bytes[2] = (long long)P * 8;
-      o.ptr[3] = gc; o.bytes[3] = (long long)P * 4;
-      o.ptr[4] = gb; o.bytes[4] = (long long)F * 4;
-      hipLaunchKernelGGL(fill_zero_many, dim3(gS, 5), dim3(256), 0, stream, o);
-      INPAINT_HIP(hipGetLastError());
-      return 0;
-    }
-  }
-
-  scale_weights(s, stream, dx, dy);
+  // (the first of its launches also clears the two words of the upstream check)
+  scale_weights(s, stream, dx, dy, true);
+  // Upstream check (TGV.cu:2686-2703): any non-finite entry, or an upstream that is zero everywhere, returns
+  // all-zero gradients, scrubs the caller's tensor and leaves `run` and the running means alone.  The verdict stays
+  // on the device: the sweep below runs either way (on the scrubbed tensor; its kernels address nothing by value),
+  // the guard's decision and the kernels that store the outputs read the verdict.  No host wait.
+  hipLaunchKernelGGL(tgv_upstream_check, dim3(std::min(grid_stride((long long)S3 / 4 + 1), 2048)), dim3(256), 0, stream, gin, (long long)S3, s.counts);
+  hipLaunchKernelGGL(tgv_upstream_verdict, dim3(std::min(gS, 1024)), dim3(256), 0, stream, gin, (long long)S3, s.counts, s.guard);
   // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
   // totals after the last segment, in the reference's order (TGV.cu:2944 flushes after every segment: same bits,
   // but the totals are not read and rewritten once per segment).
@@ -1599,7 +1618,7 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
                        s.guard, kGuard);
   }
   INPAINT_HIP(hipGetLastError());
-  s.run++;  // TGV.cu:3061
+  s.run++;  // TGV.cu:3061 (a refused upstream gradient is counted on the device and taken off again: Slot::run)
   return 0;
 }
 
@@ -1611,9 +1630,10 @@ int tgvinpaint_selftest_guard(const void* values, long long n, int is_f32, int r
 int tgvinpaint_get_state(int id, double* state6) {
   if (id < 0 || id >= kUniqueIds || !state6) return fail(INPAINT_ERR_ID, "bad id %d", id);
   Slot& s = g_slots[id];
-  int rc = fetch_running_means(s);
+  unsigned int skipped = 0;
+  int rc = fetch_running_means(s, &skipped);
   if (rc) return rc;
-  state6[0] = s.run;
+  state6[0] = s.run - (int)skipped;
   for (int k = 0; k < 5; k++) state6[1 + k] = s.pending_av[k];
   return 0;
 }
@@ -1627,6 +1647,8 @@ int tgvinpaint_set_state(int id, const double* state6) {
     INPAINT_HIP(hipStreamSynchronize(s.stream));
     INPAINT_HIP(hipMemcpy(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, av), s.pending_av, 5 * sizeof(double),
                          hipMemcpyHostToDevice));
+    const unsigned int none = 0;
+    INPAINT_HIP(hipMemcpy(reinterpret_cast<char*>(s.guard) + offsetof(GuardState, skipped), &none, sizeof(none), hipMemcpyHostToDevice));
   }
   return 0;
 }

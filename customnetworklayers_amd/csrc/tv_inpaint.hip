@@ -493,6 +493,7 @@ struct Slot {
   // reads at a segment start); 1 only x (what the corrected gradient reads).  A forward that keeps every x05 row stores
   // the half its id's gradient mode needs, since no segment is ever recomputed from the checkpoint.
   int ckpt_half = -1;
+  int fwd_grad_mode = 0;  // the mode the last forward pass ran under: its backward passes must ask for the same one
   int grad_mode = 0;    // 0: the reference's backward, bit for bit; 1: the corrected gradient (tvinpaint_gradient_mode)
   int ring_rows = 0;    // rows of the x05 ring the arena was laid out for
   // shape and its whose every-row ring (keep mode 2) the device refused: later forwards of that shape go straight
@@ -1016,6 +1017,7 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   s.forward_done = false;
   s.x05_valid = false;
   s.ckpt_half = -1;
+  s.fwd_grad_mode = s.grad_mode;
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
   const long long shape[5] = {n, ic, ih, iw, its};
   if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
@@ -1136,8 +1138,17 @@ int tvinpaint_forward_noalloc(const float* dx, const float* dy, const float* c, 
   float* xpp[2] = {base + 2 * kNoAllocMaxField, base + 3 * kNoAllocMaxField};
   const int K = 2 * (its / 2);
   if (K == 0) {
-    INPAINT_HIP(hipMemcpyAsync(out, init, F * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    if (out != init) INPAINT_HIP(hipMemcpyAsync(out, init, F * sizeof(float), hipMemcpyDeviceToDevice, stream));
     return 0;
+  }
+  // In place (out == init) a launch that both reads the starting point and stores the result would have strips read
+  // halo pixels that their neighbours have already overwritten: that is the single pair launch of its = 2 or 3.  It
+  // then reads a copy of the starting point in the scratch (one copy kernel more, as tvinpaint_forward does in place).
+  const float *x0 = init, *y0 = init;
+  if (out == init && K == 2 && forward_pairs(s)) {
+    hipLaunchKernelGGL(copy_twice_f32, dim3(grid_stride((long long)F)), dim3(256), 0, stream, init, xpp[0], ypp[0], (long long)F);
+    x0 = xpp[0];
+    y0 = ypp[0];
   }
   // extrapolation factors as make_step_sizes produces them (TV.cu:1525-1532), one at a time
   double t = 1, t_prev = 1;
@@ -1150,8 +1161,8 @@ int tvinpaint_forward_noalloc(const float* dx, const float* dy, const float* c, 
     for (int k = 0; k < K; k += 2) {
       const float tA = next_step(), tB = next_step();
       const int i = (k >> 1) & 1;
-      launch_forward_pair(s, stream, dx, dy, c, b, k == 0 ? init : xpp[i], k + 2 == K ? out : xpp[1 - i],
-                          k == 0 ? init : ypp[i], ypp[1 - i], nullptr, nullptr, tA, tB);
+      launch_forward_pair(s, stream, dx, dy, c, b, k == 0 ? x0 : xpp[i], k + 2 == K ? out : xpp[1 - i],
+                          k == 0 ? y0 : ypp[i], ypp[1 - i], nullptr, nullptr, tA, tB);
     }
   } else {
     for (int k = 0; k < K; k++) {
@@ -1177,8 +1188,10 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   if (!s.forward_done || !s.arena.base || s.n != n || s.ic != ic || s.ih != ih || s.iw != iw || s.its != its)
     return fail(INPAINT_ERR_PAIRING, "backward(id=%d) does not match the last forward on this id", id);
   const bool corr = s.grad_mode == 1;
-  if (s.ckpt_half >= 0 && s.ckpt_half != (corr ? 1 : 0))
-    return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass, which kept the checkpoints of the other mode: run the forward pass again", id);
+  // One rule in every keep mode (a forward that keeps every x05 row stores only the checkpoint halves its mode reads,
+  // so there the other mode could not be served at all):
+  if (s.grad_mode != s.fwd_grad_mode)
+    return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass: set it before the forward pass, or run the forward pass again", id);
   if (corr && force_tile_path())
     return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TV_PATH=tile is set)");
   s.stream = stream;

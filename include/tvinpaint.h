@@ -73,9 +73,9 @@ int tvinpaint_guard_stats(int id, double* stats25);
  * wrt the start, 1696-1729, 1816), and the multipliers 0.1 / 0.1 / 1.0 and the global 0.1 (63-69) are 1.  The
  * clamp of the adjoint iterates (797-799), the upstream scrub and the output guard stay.  With them inactive the
  * result is the gradient of the forward pass (tests compare it with automatic differentiation).  Any channel
- * count; same speed as the default.  Set it before the forward pass whose backward it is meant for: a forward that keeps
- * every x05 row stores, at each checkpoint, only the half that the backward of the id's current mode reads, and a
- * backward in the other mode returns INPAINT_ERR_PAIRING. */
+ * count; same speed as the default.  Set it before the forward pass whose backward it is meant for: the forward pass
+ * latches the id's mode (with every x05 row kept it stores, at each checkpoint, only the half that mode's backward
+ * reads), and a backward pass under another mode returns INPAINT_ERR_PAIRING, whatever the keep mode. */
 int tvinpaint_gradient_mode(int id, int mode);
 
 /* Which intermediate iterates (the x05 rows of TVInpaintFista.cu:1678-1687) the next forwards on `id` keep for

@@ -300,6 +300,14 @@ def test_gradient_mode_is_fixed_by_the_forward_pass(ext):
             ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
         ext.gradient_mode(3, 0)
         ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
+        for keep in (0, 1):  # the same rule where both checkpoint halves exist
+            ext.keep_iterates(3, keep)
+            ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 20, 3)
+            ext.gradient_mode(3, 1)
+            with pytest.raises(RuntimeError, match="gradient mode"):
+                ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
+            ext.gradient_mode(3, 0)
+            ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
     finally:
         ext.reset_id(3)
 

@@ -422,8 +422,8 @@ def test_forward_in_place_through_the_c_abi(ext, its):
 
 
 def test_gradient_mode_is_fixed_by_the_forward_pass(ext):
-    # a forward that keeps every x05 row stores, at each checkpoint, only the half the backward of the id's mode reads;
-    # a backward in the other mode says so instead of reading a stale buffer; with recomputed segments both halves exist
+    # the forward pass latches the id's gradient mode (with every x05 row kept it stores, at each checkpoint, only the
+    # half that mode's backward reads); a backward under the other mode says so, and says so in every keep mode
     dev = torch.device("cuda:0")
     d = {k: torch.from_numpy(v).to(dev) for k, v in tv_inputs(1, 2, 24, 70, seed=12).items()}
     try:
@@ -438,10 +438,15 @@ def test_gradient_mode_is_fixed_by_the_forward_pass(ext):
         ext.keep_iterates(3, 0)
         ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 20, 3)
         ext.gradient_mode(3, 1)
-        ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)  # both halves kept: allowed
+        with pytest.raises(RuntimeError, match="gradient mode"):  # (both checkpoint halves exist here: same rule)
+            ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
         ext.gradient_mode(3, 0)
-        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 20, 3)
         b = ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
+        ext.keep_iterates(3, 1)
+        ext.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], 20, 3)
+        ext.gradient_mode(3, 1)
+        with pytest.raises(RuntimeError, match="gradient mode"):
+            ext.backward(d["grad"].clone(), d["dx"], d["dy"], d["dc"], d["db"], 20, 3)
         for x, y in zip(a, b):
             assert torch.equal(x, y)
     finally:
