@@ -56,7 +56,8 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* count
   if (bad3) atomicAdd(&counts[3], (unsigned long long)bad3);
 }
 
-// counts[0]: rsq_exact(x) against 1.0f / sqrtf(x) over 0 and every float in [2^-96, 2^96]
+// counts[0]: rsq_exact(x) against 1.0f / sqrtf(x) over 0 and every float in [2^-96, 2^96]; and every float up to
+//            kHuberQuiet has Huber weight 1 in both forms
 // counts[1]: div_by_fifth(x) against x / 0.2f over the same set (the TGV layer's Huber threshold)
 // counts[2]: exact_rcp(m) against 1 / m over every float m in [2^-40, 2^40): the reciprocal that every division starts
 //            from, and the segment-start kernel's Huber weight
@@ -72,6 +73,13 @@ __global__ __launch_bounds__(256) void selftest_rsqrt_kernel(unsigned long long*
       bad1 += !same_bits(div_by_fifth(x), x / 0.2f);
     }
     if (x >= 9.094947e-13f && x < 1.0995116e12f) bad2 += !same_bits(exact_rcp(x), 1.0f / x);
+    // a Huber argument up to kHuberQuiet has weight exactly 1 and an inactive term, in both arithmetic forms: what the
+    // strip kernels assume when a whole wavefront skips the square root
+    if (x <= tgvstrip::kHuberQuiet) {
+      const float root = exact_sqrt(x);
+      bad0 += tgvstrip::huber_w_full(x, 0.2f) != 1.0f;
+      bad0 += root > 0.2f || exact_rcp(fmaxf(1.f, div_by_fifth(root))) != 1.0f;
+    }
   }
   for (unsigned int k = 0; k < pair_rounds; k++) {
     const unsigned int h1 = mix(tid * 2654435761U + k * 40503U + 29U), h2 = mix(h1 ^ 0x9e3779b9U);

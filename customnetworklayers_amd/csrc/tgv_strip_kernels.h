@@ -53,8 +53,23 @@ __device__ __forceinline__ float rsq_exact(float x) {
   return (x == 0.0f) ? __builtin_inff() : r;
 }
 
+// A wavefront whose 64 lanes all hold a Huber argument A <= kHuberQuiet skips the square root and the reciprocal of that
+// term: the weight is exactly 1 there.  min(1, fl(fl(1 / fl(sqrt(A))) * 0.2f)) is 1 at A = 0.0399f (the product is
+// 1.0012...) and every operation in it is monotone in A, so it is 1 for every A below as well (0 gives +inf * 0.2f);
+// the segment-start form 1 / max(1, sqrt(A) / 0.2f) is 1 there too (sqrt(0.0399f) / 0.2f = 0.9987).  A NaN fails the
+// comparison and takes the full path.  The test is per wavefront, so no lane diverges and the bits cannot change; what
+// changes is the time, which now depends on the data: the smoothness terms of v1, v2 are quiet in whole rows of smooth
+// flow, the coupling term in most of them.  inpaint_selftest_rsqrt checks the claim at the threshold on the device.
+constexpr float kHuberQuiet = 0.0399f;
+__device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
+
 // Huber weight of the main kernels: min(1, rsqrt(A) * delta)  (TGV.cu:1624 and siblings)
-__device__ __forceinline__ float huber_w(float A, float delta) { return fminf(1.f, rsq_exact(A) * delta); }
+__device__ __forceinline__ float huber_w_full(float A, float delta) { return fminf(1.f, rsq_exact(A) * delta); }
+__device__ __forceinline__ float huber_w(float A, float delta) {
+  static_assert(kD0 == 0.2f, "kHuberQuiet is the bound for a threshold of 0.2f");
+  if (!wave_any(A > kHuberQuiet)) return 1.f;
+  return huber_w_full(A, delta);
+}
 
 // -------------------------------------------------------------------------------------------------
 // Forward iteration, TGV.cu:1546-1776 (and 2005-2235 when x05 is given).
@@ -726,6 +741,10 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip(
 
   // Huber weight, activity and weight derivative of one term in the kernel's own form
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2) {
+    if (!wave_any(A > kHuberQuiet)) {  // no lane of the wavefront is near the threshold: weight 1, term inactive
+      Wt = 1.f; act = false; dW = 0.f; hub2 = 1.f;
+      return;
+    }
     if (END) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
       Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
@@ -1101,6 +1120,10 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
 
   // Huber weight, activity and weight derivative of one term, in the main or the segment-start form
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
+    if (!wave_any(A > kHuberQuiet)) {  // no lane of the wavefront is near the threshold: weight 1, term inactive
+      Wt = 1.f; act = false; dW = 0.f; hub2 = 1.f;
+      return;
+    }
     if (end_form.value) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
       Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
@@ -1518,6 +1541,10 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
 
   // Huber weight, activity and weight derivative of one term, in the main or the segment-start form
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
+    if (!wave_any(A > kHuberQuiet)) {  // no lane of the wavefront is near the threshold: weight 1, term inactive
+      Wt = 1.f; act = false; dW = 0.f; hub2 = 1.f;
+      return;
+    }
     if (end_form.value) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
       Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
@@ -2118,6 +2145,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   // Huber weight, activity and weight derivative of one term, in the main or the segment-start form
   auto huber = [&](float A, float delta, float& Wt, bool& act, float& dW, float& hub2, auto end_form) {
+    if (!wave_any(A > kHuberQuiet)) {  // no lane of the wavefront is near the threshold: weight 1, term inactive
+      Wt = 1.f; act = false; dW = 0.f; hub2 = 1.f;
+      return;
+    }
     if (end_form.value) {  // TGV.cu:1132-1138
       const float hub = exact_sqrt(A);
       Wt = exact_rcp(fmaxf(1.f, div_by_fifth(hub)));  // delta is 0.2f for all three terms
