@@ -15,26 +15,66 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# Counter figures that no bench run can take itself (rocprofv3 --pmc needs a run of its own); each names the file under
-# profiles/ that holds it and the commit of the library it was read at.
-#   traffic   HBM bytes per launch of the dominant kernel: FETCH_SIZE (scaled by the copy-kernel calibration of the
-#             same run) + WRITE_SIZE
-#   step      HBM bytes of one whole forward+backward (every kernel and copy)
-#   lds       LDS bytes per launch of the dominant kernel (SQ_INSTS_LDS x 64 lanes x 8 B; the TV strip kernels issue
-#             no LDS instruction at all -- neighbours are exchanged through DPP in registers)
-#   rocprof_ms  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
-COUNTERS = {
-    1: dict(traffic=(2 * 85091 + 68530) * 1024, step=(2 * 6586753 + 5549704) * 1024, lds=0, rocprof_ms=0.05151,
-            files="profiles/tv_strip_headline_hbm_traffic.txt, profiles/tv_headline_kernel_stats.txt", commit="9dd8973"),
-    2: dict(traffic=(2 * 160472 + 148414) * 1024, step=(2 * 13495066 + 13252795) * 1024, lds=1001952 * 64 * 8, rocprof_ms=0.11738,
-            files="profiles/tgv_strip_config2_hbm_traffic.txt, profiles/tgv_config2_kernel_stats.txt", commit="9dd8973"),
-    5: dict(traffic=(2 * 186980 + 239670) * 1024, sources_traffic=(2 * 289480 + 345100) * 1024,
-            files="profiles/quadfit_config5_kernel_stats_and_traffic.txt", commit="f053591"),
-    6: dict(traffic=(2 * 140091 + 247104) * 1024, files="profiles/median_config6_kernel_stats_and_traffic.txt", commit="26d8b66"),
-}
-MEASURED_TRAFFIC_BYTES = {k: v["traffic"] for k, v in COUNTERS.items()}
 # Peak LDS rate: 128 B per clock and CU x 256 CUs x 2.4 GHz.
 LDS_PEAK_GBS = 128 * 256 * 2.4
+
+
+def sources_sha16(files):
+    """First 16 hex digits of the SHA-256 over the named source files (paths relative to the repository root)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in sorted(files):
+        with open(os.path.join(ROOT, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def load_counters(config):
+    """Counter figures that no bench run can take itself (rocprofv3 --pmc needs a run of its own), from
+    profiles/counters.json -- the same file the text summaries under profiles/ are written from.  Per workload:
+      traffic_bytes   HBM bytes per launch of the dominant kernel: FETCH_SIZE (scaled by the copy-kernel calibration
+                      of the same run) + WRITE_SIZE
+      step_bytes      HBM bytes of one whole forward+backward (every kernel and copy)
+      lds_bytes       LDS bytes per launch of the dominant kernel (SQ_INSTS_LDS x 64 lanes x 8 B; the TV strip kernels
+                      issue no LDS instruction at all -- neighbours are exchanged through DPP in registers)
+      rocprof_avg_us  average duration of the dominant kernel in the rocprofv3 --kernel-trace --stats summary
+      sources, sources_sha16   the kernel sources the figures were read at; `stale` is set when they have changed since
+    Returns None when the file has no entry for the workload."""
+    path = os.path.join(ROOT, "profiles", "counters.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as fh:
+        entry = json.load(fh).get("configs", {}).get(str(config))
+    if entry is None:
+        return None
+    entry = dict(entry)
+    entry["stale"] = sources_sha16(entry["sources"]) != entry["sources_sha16"]
+    return entry
+
+
+def physical_roofline(roof, cnt, kernel_ms, key="traffic_bytes"):
+    """Fills the roofline entry: `achieved` / `frac` are the bytes the kernel really moves (counters) over its launch
+    time, a rate that cannot exceed the peak; `model_achieved` / `model_frac` are the algorithmic bytes (what
+    `bytes_per_launch` counts) over the same time, which can: a launch that fuses two steps keeps the value between them
+    in registers, and the model charges it a round trip.  Without counters only the model figures are given."""
+    model = roof["bytes_per_launch"] / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
+    roof["model_achieved"] = round(model, 1)
+    roof["model_frac"] = round(model / HBM_PEAK_GBS, 4)
+    if cnt and key in cnt and kernel_ms > 0:
+        gbs = cnt[key] / (kernel_ms * 1e-3) / 1e9
+        roof["achieved"] = round(gbs, 1)
+        roof["frac"] = round(gbs / HBM_PEAK_GBS, 4)
+        roof["traffic"] = cnt[key]
+        roof["counters_from"] = {"files": cnt["files"], "library_commit": cnt["library_commit"]}
+        roof["counters_stale"] = cnt["stale"]
+    else:
+        roof["achieved"] = None
+        roof["frac"] = None
+        roof["traffic"] = None
+    roof["basis"] = ("achieved, frac: HBM bytes per launch read off FETCH_SIZE + WRITE_SIZE (profiles/counters.json) / launch time; "
+                     "model_achieved, model_frac: algorithmic bytes per launch (bytes_per_launch) / the same time")
+    return roof
 
 
 def algorithmic_bytes_per_pixel(c, kind="tv"):
@@ -58,9 +98,10 @@ def layer_of(kind):
     return ext, "tvinpaint", workloads.tv_inputs, "TVOracle", "tvstrip::tv_adjoint_strip2<2,false,false>"
 
 
-def cpu_baseline(cfg, seconds_hint=20.0):
+def cpu_baseline(cfg, whole=False):
     """The CPU oracle on a bounded sample of the same workload: ONE sample of the batch, all
-    iterations, forward + backward, all host cores (best of 2 after a warm-up) and one core."""
+    iterations, forward + backward, all host cores (best of 2 after a warm-up) and one core.
+    `whole`: the workload has one sample, so the sample is the workload."""
     import oracle.oracle_lib as oracle_lib
 
     _, _, make_inputs, oracle_name, _ = layer_of(cfg["kind"])
@@ -87,8 +128,8 @@ def cpu_baseline(cfg, seconds_hint=20.0):
     t_one = once()
     o.set_threads(cores)
     return dict(value=round(pxit / t_all / 1e6, 3), unit="Mpixel-iter/s", cores=cores, kind="port",
-                sample="1 of %d samples (%dx%dx%d), %d iterations, fwd+bwd, best of 2"
-                       % (cfg["n"], cfg["c"], cfg["h"], cfg["w"], its),
+                sample=("the whole workload (1 x %dx%dx%d), %d iterations, fwd+bwd, best of 2" % (cfg["c"], cfg["h"], cfg["w"], its)) if whole
+                       else "1 of %d samples (%dx%dx%d), %d iterations, fwd+bwd, best of 2" % (cfg["n"], cfg["c"], cfg["h"], cfg["w"], its),
                 one_core_value=round(pxit / t_one / 1e6, 3), host_cpu_count=os.cpu_count())
 
 
@@ -186,27 +227,26 @@ def bench_flowaux(args, cfg, d):
     k_ms, launches_timed = kernel_ms(2 if cfg["kind"] == "quadfit" else 1)
     src_ms = kernel_ms(1)[0] if cfg["kind"] == "quadfit" else None
     value = px / (elapsed / args.steps) / 1e6
-    achieved = bpp["kernel"] * px / (k_ms * 1e-3) / 1e9 if k_ms > 0 else 0.0
+    cnt = load_counters(args.config)
     out = {
         "metric": "%s fwd+bwd Mpixel/s at %d x %s; achieved HBM GB/s vs peak" % (cfg["kind"], n, shape),
         "value": round(value, 2), "unit": "Mpixel/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s fwd+bwd, N=%d, %s fp32 (config %d)" % (cfg["kind"], n, shape, args.config), "pixels_per_step": px},
-        "whole_job": {"model_bytes_per_pixel": bpp["total"], "achieved_GBps": round(bpp["total"] * px / (elapsed / args.steps) / 1e9, 1),
+        "whole_job": {"model_bytes_per_pixel": bpp["total"], "model_GBps": round(bpp["total"] * px / (elapsed / args.steps) / 1e9, 1),
                       "forward_ms": round(f_ms, 4), "backward_ms": round(b_ms, 4),
-                      "forward_GBps": round(bpp["forward"] * px / (f_ms * 1e-3) / 1e9, 1),
-                      "backward_GBps": round(bpp["backward"] * px / (b_ms * 1e-3) / 1e9, 1)},
-        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config),
-                     "bytes_per_launch": bpp["kernel"] * px, "avg_launch_ms": round(k_ms, 5), "launches_timed": launches_timed,
-                     "counters_from": COUNTERS[args.config]["files"] + " @ " + COUNTERS[args.config]["commit"]},
+                      "forward_model_GBps": round(bpp["forward"] * px / (f_ms * 1e-3) / 1e9, 1),
+                      "backward_model_GBps": round(bpp["backward"] * px / (b_ms * 1e-3) / 1e9, 1)},
+        "roofline": physical_roofline({"bound": "hbm", "kernel": kernel, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                       "bytes_per_launch": bpp["kernel"] * px, "avg_launch_ms": round(k_ms, 5),
+                                       "launches_timed": launches_timed}, cnt, k_ms),
     }
     if src_ms is not None:  # the second kernel of the backward pass
-        cnt = COUNTERS[args.config]
-        out["roofline"]["per_source_pass"] = {
-            "kernel": "quadfit_sources_resident<32,true>", "avg_launch_ms": round(src_ms, 5), "bytes_per_launch": bpp["sources"] * px,
-            "achieved": round(bpp["sources"] * px / (src_ms * 1e-3) / 1e9, 1), "traffic": cnt["sources_traffic"]}
+        out["roofline"]["per_source_pass"] = physical_roofline(
+            {"kernel": "quadfit_sources_resident<32,true>", "avg_launch_ms": round(src_ms, 5), "bytes_per_launch": bpp["sources"] * px},
+            cnt, src_ms, key="sources_traffic_bytes")
+        out["roofline"]["per_source_pass"].pop("basis")
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = flowaux_cpu_baseline(cfg, d)
     print(json.dumps(out))
@@ -307,7 +347,10 @@ def bench_hierarchy(args, cfg):
     h, w = cfg["levels"][-1]
     k_ms = top_ms / max(top_cnt, 1)
     k_bytes = 2 * bpp["adjoint"] * n * h * w
-    achieved = k_bytes / (k_ms * 1e-3) / 1e9 if k_ms > 0 else 0.0
+    # the finest level runs the headline's dominant kernel: its counter bytes per pixel, times this level's pixels
+    cnt = load_counters(1)
+    if cnt:
+        cnt = dict(cnt, traffic_bytes=int(cnt["traffic_bytes"] / cnt["pixels"] * n * h * w))
     sec = elapsed / args.steps
     out = {
         "metric": "TV-FISTA hierarchy fwd+bwd Mpixel-iter/s, %d levels up to %dx%dx%dx%d; achieved HBM GB/s vs peak" % (nl, n, c, h, w),
@@ -316,14 +359,15 @@ def bench_hierarchy(args, cfg):
         "data": "synthetic",
         "config": {"workload": "three TV layers coarse to fine with device glue, N=%d, C=%d, levels %s, %d iterations each (config 3)"
                                % (n, c, "/".join("%dx%d" % l for l in cfg["levels"]), its), "pixel_iterations_per_step": pxit},
-        "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "achieved_GBps": round(bpp["total"] * pxit / sec / 1e9, 1),
-                      "frac_of_hbm_peak": round(bpp["total"] * pxit / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "whole_job": {"model_bytes_per_pixel_iteration": bpp["total"], "model_GBps": round(bpp["total"] * pxit / sec / 1e9, 1),
+                      "model_frac_of_hbm_peak": round(bpp["total"] * pxit / sec / 1e9 / HBM_PEAK_GBS, 4),
                       "glue_forward_ms": round(glue_ms["fwd"], 4), "glue_backward_ms": round(glue_ms["bwd"], 4),
                       "glue_forward_GBps": round(glue_bytes["fwd"] / (glue_ms["fwd"] * 1e-3) / 1e9, 1),
                       "glue_backward_GBps": round(glue_bytes["bwd"] / (glue_ms["bwd"] * 1e-3) / 1e9, 1)},
-        "roofline": {"bound": "hbm", "kernel": "tvstrip::tv_adjoint_strip2<2,false,false> at the finest level", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "bytes_per_launch": k_bytes, "adjoint_steps_per_launch": 2, "avg_launch_ms": round(k_ms, 5), "launches_timed": top_cnt},
+        "roofline": physical_roofline({"bound": "hbm", "kernel": "tvstrip::tv_adjoint_strip2<2,false,false> at the finest level",
+                                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "bytes_per_launch": k_bytes, "adjoint_steps_per_launch": 2,
+                                       "avg_launch_ms": round(k_ms, 5), "launches_timed": top_cnt,
+                                       "traffic_scaled_from": "the same kernel on the headline workload, per pixel"}, cnt, k_ms),
     }
     if not args.no_cpu_baseline:
         import oracle.oracle_lib as oracle_lib
@@ -446,32 +490,31 @@ def bench_layer(config, steps, warmup, corrected=False, keep=None, detail=True):
     bpp = algorithmic_bytes_per_pixel(c, cfg["kind"])
     kernel_ms = tot_ms.value / max(launches.value, 1)
     steps_per_launch = 1 if kernel_name.split("<")[0].endswith("_strip") else 2  # the pair kernels run two adjoint steps
-    cnt = COUNTERS.get(config) if not corrected and keep is None else None  # the counters were read on the default path
+    cnt = load_counters(config) if not corrected and keep is None else None  # the counters were read on the default path
     kernel_bytes = steps_per_launch * bpp["adjoint"] * n * h * w
-    achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
     model_gbs = bpp["total"] * pxit / sec / 1e9
+    have_step = bool(cnt) and "step_bytes" in cnt
     out["whole_job"] = {
-        # the one-round-trip-per-iteration model counts a recompute this build does not execute (keep mode 2) and one
-        # round trip per iteration where a pair launch makes one per two, so its rate may exceed the HBM peak
+        # what the job really moves (every kernel and copy of a step, from the counters) ...
+        "effective_bytes_per_pixel_iteration": round(cnt["step_bytes"] / pxit, 1) if have_step else None,
+        "effective_GBps": round(cnt["step_bytes"] / sec / 1e9, 1) if have_step else None,
+        "effective_frac_of_hbm_peak": round(cnt["step_bytes"] / sec / 1e9 / HBM_PEAK_GBS, 4) if have_step else None,
+        # ... and the one-round-trip-per-iteration model, which counts a recompute this build does not execute (keep
+        # mode 2) and one round trip per iteration where a pair launch makes one per two: its rate may exceed the peak
         "model_bytes_per_pixel_iteration": bpp["total"], "model_GBps": round(model_gbs, 1),
-        "model_frac_of_hbm_peak": round(model_gbs / HBM_PEAK_GBS, 4),
-        "effective_bytes_per_pixel_iteration": round(cnt["step"] / pxit, 1) if cnt and "step" in cnt else None,
-        "effective_GBps": round(cnt["step"] / sec / 1e9, 1) if cnt and "step" in cnt else None,
-        "effective_frac_of_hbm_peak": round(cnt["step"] / sec / 1e9 / HBM_PEAK_GBS, 4) if cnt and "step" in cnt else None}
-    roof = {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": cnt["traffic"] if cnt else None,
-            "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
-            "avg_launch_ms_events": round(kernel_ms, 5), "launches_timed": launches.value}
+        "model_frac_of_hbm_peak": round(model_gbs / HBM_PEAK_GBS, 4)}
+    roof = physical_roofline({"bound": "hbm", "kernel": kernel_name, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "bytes_per_launch": kernel_bytes, "adjoint_steps_per_launch": steps_per_launch,
+                              "avg_launch_ms_events": round(kernel_ms, 5), "launches_timed": launches.value}, cnt, kernel_ms)
     if cnt:
-        roof["traffic_GBps"] = round(cnt["traffic"] / (kernel_ms * 1e-3) / 1e9, 1) if kernel_ms > 0 else None
-        roof["traffic_frac"] = round(cnt["traffic"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if kernel_ms > 0 else None
-        roof["counters_from"] = {"files": cnt["files"], "library_commit": cnt["commit"]}
-        if "rocprof_ms" in cnt:
-            r_gbs = kernel_bytes / (cnt["rocprof_ms"] * 1e-3) / 1e9
-            roof["rocprof"] = {"avg_launch_ms": cnt["rocprof_ms"], "achieved": round(r_gbs, 1), "frac": round(r_gbs / HBM_PEAK_GBS, 4)}
-        if "lds" in cnt and kernel_ms > 0:
-            lds_gbs = cnt["lds"] / (kernel_ms * 1e-3) / 1e9
-            roof["lds"] = {"bytes_per_launch": cnt["lds"], "achieved_GBps": round(lds_gbs, 1), "peak_GBps": round(LDS_PEAK_GBS, 1),
+        if "rocprof_avg_us" in cnt:
+            r_ms = cnt["rocprof_avg_us"] * 1e-3
+            roof["rocprof"] = {"avg_launch_ms": round(r_ms, 5), "achieved": round(cnt["traffic_bytes"] / (r_ms * 1e-3) / 1e9, 1),
+                               "frac": round(cnt["traffic_bytes"] / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                               "model_frac": round(kernel_bytes / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        if "lds_bytes" in cnt and kernel_ms > 0:
+            lds_gbs = cnt["lds_bytes"] / (kernel_ms * 1e-3) / 1e9
+            roof["lds"] = {"bytes_per_launch": cnt["lds_bytes"], "achieved_GBps": round(lds_gbs, 1), "peak_GBps": round(LDS_PEAK_GBS, 1),
                            "frac": round(lds_gbs / LDS_PEAK_GBS, 4)}
     out["roofline"] = roof
     return out, cfg
@@ -575,6 +618,8 @@ def main():
         out["other_configs"] = other
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
+        if args.config == 1:  # the reference's own CPU-sized case, whole (milliseconds)
+            out["cpu_baseline_config0"] = cpu_baseline(CONFIGS[0], whole=True)
     print(json.dumps(out))
 
 
