@@ -36,7 +36,10 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
  *                    (TVInpaintFista.cu:1609-1623)
  *   gx, gy, gc     : (n,1,ih,iw) gradients wrt dx, dy, c   (overwritten)
  *   gb, gi         : (n,ic,ih,iw) gradients wrt b and init (overwritten)
- * Must follow a tvinpaint_forward with the same shape, its and id. */
+ * Must follow a tvinpaint_forward with the same shape, its and id.
+ * Range: the gradients are those of the reference's arithmetic bit for bit while they stay normal floats (tested for
+ * upstream gradients from 1e-30 to 1e30 times N(0,1)); results that fall into the denormal range (upstream around
+ * 1e-36 and below) agree to their last bits only.  The same holds for tgvinpaint_backward. */
 int tvinpaint_backward(const float* dx, const float* dy, const float* c, const float* b, float* gin,
                        float* gx, float* gy, float* gc, float* gb, float* gi, int n, int ic, int ih,
                        int iw, int its, int id, void* stream);

@@ -76,6 +76,39 @@ def test_tgv_full_length_sample_matches_oracle(ext):
     assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3
 
 
+@pytest.mark.parametrize("c,lively", [(3, False), (3, True), (2, True)])
+def test_tgv_pair_kernels_match_the_oracle_at_full_image_size(ext, c, lively):
+    # 1 x C x 384 x 1248, 20 iterations against the oracle: three channels take the adjoint pairs in four wavefronts at the
+    # strip heights and strip counts of config 2's image.  `lively`: auxiliary variables that start far from smooth and a
+    # larger beta, so that all three Huber terms are active in many wavefronts and quiet in others (config 2's own data
+    # keeps the two smoothness terms below their threshold everywhere, the path on which a wavefront skips their roots)
+    from oracle.oracle_lib import TGVOracle
+
+    o = TGVOracle()
+    o.set_quirks()
+    cfg = CONFIGS[2]
+    its = 20
+    d = tgv_inputs(1, c, cfg["h"], cfg["w"], seed=30 + c, **cfg["gen"])
+    if lively:
+        rng = np.random.default_rng(7)
+        d["di"][:, c:] = rng.normal(0, 3.0, d["di"][:, c:].shape).astype(np.float32)
+        d["di"][:, c:, : cfg["h"] // 2] *= 0.01  # (the upper half stays quiet)
+        d["dx"][:, 1] *= 4.0
+        d["dy"][:, 1] *= 4.0
+    print("case 1x%dx%dx%d its=%d lively=%s" % (c, cfg["h"], cfg["w"], its, lively), flush=True)
+    got = gpu_layer(ext, d, its, 3)
+    o.reset_id(3)
+    sol = o.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], its, 3)
+    grads = o.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], its, 3)
+    rel = lambda a, r: float(np.abs(a - r).max() / max(np.abs(r).max(), 1e-30))
+    errs = [rel(a, r) for a, r in zip(got, [sol] + list(grads))]
+    print("\n[tgv 1x%dx384x1248 its=%d] out %.2e grads %s" % (c, its, errs[0], ["%.2e" % e for e in errs[1:]]), flush=True)
+    assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3  # (the layer's tolerances; the kernels give the oracle's bits)
+    for a, r in zip(got, [sol] + list(grads)):
+        np.testing.assert_array_equal(a, r)
+    ext.reset_id(3)
+
+
 @pytest.mark.parametrize("c,parts", [(4, ((0, 2), (2, 4))), (3, ((0, 2), (2, 3)))])
 def test_tgv_wider_runs_contain_the_narrower_ones(ext, c, parts):
     # 2 x C x 384 x 1248, 100 iterations with three and four channels (adjoint pairs in four wavefronts, two channel groups):

@@ -222,6 +222,25 @@ def test_unusual_magnitudes_stay_bit_equal(ext, tv_oracle, regime, c):
         assert np.array_equal(a, b, equal_nan=True)
 
 
+@pytest.mark.parametrize("scale,bit_equal", [(1e-20, True), (1e-30, True), (1e-36, False), (1e20, True), (1e30, True)])
+def test_upstream_gradients_of_extreme_magnitude(ext, tv_oracle, scale, bit_equal):
+    # The short division (reciprocal refined once, quotient corrected once, no range fix-ups) returns the compiler's bits
+    # while the correction's residual stays a normal number.  The adjoint's numerators scale with the upstream gradient:
+    # down to 1e-30 and up to 1e30 (where the clamps of the adjoint iterates act) every gradient is the oracle's, bit for
+    # bit; at 1e-36 the results (1e-38 and below) are denormal and agree to their last bits only (1e-7 of the largest).
+    from customnetworklayers_amd.workloads import tv_inputs as make
+
+    d = make(1, 2, 40, 130, seed=3, conf_density=0.4)
+    d["grad"] = (d["grad"].astype(np.float64) * scale).astype(np.float32)
+    got, ref = run_gpu(ext, d, 12, 2), run_oracle(tv_oracle, d, 12, 2)
+    for a, b in zip(got[1], ref[1]):
+        if bit_equal:
+            assert np.array_equal(a, b, equal_nan=True)
+        else:
+            assert float(np.abs(a.astype(np.float64) - b).max()) <= 1e-6 * float(np.abs(b).max())
+    ext.reset_id(2)
+
+
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
 def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
     # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first

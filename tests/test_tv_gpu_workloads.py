@@ -82,6 +82,44 @@ def test_stress_shape_matches_oracle(ext, tv_oracle):
     assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3
 
 
+def test_stress_batch_equals_its_samples_run_alone(ext):
+    # the quoted stress workload whole: 16 x 2 x 256 x 512, 200 iterations (the launch grid of sixteen samples): finite,
+    # the same bits on another id, and samples 0 and 15 equal to runs on those samples alone
+    cfg = CONFIGS[4]
+    d = tv_inputs(cfg["n"], cfg["c"], cfg["h"], cfg["w"], seed=0, **cfg["gen"])
+    full = gpu_layer(ext, d, cfg["its"], 0)
+    assert all(np.isfinite(a).all() for a in full)
+    again = gpu_layer(ext, d, cfg["its"], 1)
+    for a, b in zip(full, again):
+        np.testing.assert_array_equal(a, b)
+    for s in (0, 15):
+        one = gpu_layer(ext, {k: v[s:s + 1] for k, v in d.items()}, cfg["its"], 2)
+        for a, b in zip(full, one):
+            np.testing.assert_array_equal(a[s:s + 1], b)
+    for pid in (0, 1, 2):
+        ext.reset_id(pid)
+
+
+@pytest.mark.parametrize("c", [3, 5, 8])
+def test_wide_pair_kernels_match_the_oracle_at_full_image_size(ext, tv_oracle, c):
+    # 1 x C x 384 x 1248 with 3, 5 and 8 channels -- the adjoint pairs in two and in four wavefronts at the strip heights
+    # and strip counts of the headline's image -- against the oracle, 20 iterations
+    cfg = CONFIGS[1]
+    its = 20
+    d = tv_inputs(1, c, cfg["h"], cfg["w"], seed=20 + c, **cfg["gen"])
+    got = gpu_layer(ext, d, its, 3)
+    tv_oracle.reset_id(3)
+    sol = tv_oracle.forward(d["dx"], d["dy"], d["dc"], d["db"], d["di"], its, 3)
+    grads = tv_oracle.backward(d["grad"].copy(), d["dx"], d["dy"], d["dc"], d["db"], its, 3)
+    rel = lambda a, r: float(np.abs(a - r).max() / max(np.abs(r).max(), 1e-30))
+    errs = [rel(a, r) for a, r in zip(got, [sol] + list(grads))]
+    print("\n[1x%dx384x1248 its=%d] out %.2e grads %s" % (c, its, errs[0], ["%.2e" % e for e in errs[1:]]), flush=True)
+    assert errs[0] <= 1e-4 and max(errs[1:]) <= 1e-3  # (the layer's tolerances; the kernels give the oracle's bits)
+    for a, r in zip(got, [sol] + list(grads)):
+        np.testing.assert_array_equal(a, r)
+    ext.reset_id(3)
+
+
 def up2(t):
     """x2 bilinear upsampling with doubled values (flow vectors scale with the resolution)."""
     return 2.0 * F.interpolate(t, scale_factor=2, mode="bilinear", align_corners=False)
