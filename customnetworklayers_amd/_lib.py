@@ -28,6 +28,8 @@ def _load():
     lib.tvinpaint_gradient_mode.argtypes = [_int, _int]
     lib.tvinpaint_slot_bytes.argtypes = [_int]
     lib.tvinpaint_slot_bytes.restype = ctypes.c_longlong
+    lib.tvinpaint_set_allocator.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.tgvinpaint_set_allocator.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.tvinpaint_schedule.argtypes = [_int, ctypes.POINTER(_int), ctypes.POINTER(_int)]
     lib.tvinpaint_step_sizes.argtypes = [_int, ctypes.POINTER(ctypes.c_float)]
     lib.tvinpaint_step_sizes.restype = None
@@ -77,6 +79,47 @@ def _load():
 
 
 lib = _load()
+
+
+# ---- the slots' device memory out of PyTorch's caching allocator (t[g]vinpaint_set_allocator) -------------------
+_ALLOC_FN = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_ulonglong, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p)
+_RELEASE_FN = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_void_p)
+
+
+def _torch_alloc(nbytes, device, stream, user):
+    try:
+        import torch
+
+        return torch.cuda.caching_allocator_alloc(int(nbytes), device, int(stream or 0))
+    except Exception:  # out of memory: the library falls back (keep mode 1) or reports the failure itself
+        return None
+
+
+def _torch_release(ptr, user):
+    import torch
+
+    torch.cuda.caching_allocator_delete(ptr)
+
+
+# (kept alive for as long as the library may call them)
+_torch_alloc_c, _torch_release_c = _ALLOC_FN(_torch_alloc), _RELEASE_FN(_torch_release)
+_torch_allocator_on = False
+
+
+def use_torch_allocator(enable=True):
+    """Take the per-id device blocks of both layers from PyTorch's caching allocator (on by default for the modules of
+    this package), so that they show up in torch.cuda.memory_allocated() and return to the pool PyTorch reuses;
+    enable=False goes back to hipMalloc / hipFree.  Blocks already handed out stay with the allocator that made them."""
+    global _torch_allocator_on
+    a, r = (ctypes.cast(_torch_alloc_c, ctypes.c_void_p), ctypes.cast(_torch_release_c, ctypes.c_void_p)) if enable else (None, None)
+    for fn in (lib.tvinpaint_set_allocator, lib.tgvinpaint_set_allocator):
+        if fn(a, r, None) != 0:
+            raise RuntimeError(last_error())
+    _torch_allocator_on = bool(enable)
+
+
+def torch_allocator_in_use():
+    return _torch_allocator_on
 
 
 def reload_env():

@@ -9,6 +9,7 @@
 // PyTorch on ROCm presents its HIP devices under the device type "cuda"; these are the guard and stream of that view
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPCachingAllocator.h>
 
 #include <vector>
 
@@ -39,6 +40,17 @@ void check_shapes(const at::Tensor& d_x, const at::Tensor& d_y, const at::Tensor
 }
 
 void* current_stream(const at::Tensor& t) { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream(); }
+
+// The per-id device blocks out of PyTorch's caching allocator (tgvinpaint_set_allocator): the reference callocs and frees
+// its checkpoints on the host in every forward; here one block per id and shape lives in the pool PyTorch can see.
+void* torch_alloc(unsigned long long bytes, int /*device: the current one*/, void* stream, void* /*user*/) {
+  try {
+    return c10::hip::HIPCachingAllocator::raw_alloc_with_stream((size_t)bytes, (hipStream_t)stream);
+  } catch (const std::exception&) {  // out of memory: the library falls back to fewer kept rows or reports the failure
+    return nullptr;
+  }
+}
+void torch_release(void* ptr, void* /*user*/) { c10::hip::HIPCachingAllocator::raw_delete(ptr); }
 
 }  // namespace
 
@@ -78,6 +90,10 @@ std::vector<at::Tensor> tgvInpaint_backward(at::Tensor d_iGf, at::Tensor d_x, at
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  tgvinpaint_set_allocator(torch_alloc, torch_release, nullptr);
+  m.def("use_torch_allocator", [](bool enable) {
+    TORCH_CHECK(tgvinpaint_set_allocator(enable ? torch_alloc : nullptr, enable ? torch_release : nullptr, nullptr) == 0, tgvinpaint_last_error());
+  }, "take the ids' device blocks from PyTorch's caching allocator (default) or from hipMalloc");
   m.def("forward", &tgvInpaint_forward, "tgvInpaint forward (HIP)");
   m.def("backward", &tgvInpaint_backward, "tgvInpaint backward (HIP)");
   m.def("dummy", &tgvInpaint_dummy, "tgvInpaint dummy");

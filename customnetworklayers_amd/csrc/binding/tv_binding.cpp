@@ -10,6 +10,7 @@
 // PyTorch on ROCm presents its HIP devices under the device type "cuda"; these are the guard and stream of that view
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPCachingAllocator.h>
 
 #include <string>
 #include <vector>
@@ -37,6 +38,17 @@ void check_shapes(const at::Tensor& d_x, const at::Tensor& d_y, const at::Tensor
 }
 
 void* current_stream(const at::Tensor& t) { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream(); }
+
+// The per-id device blocks out of PyTorch's caching allocator (tvinpaint_set_allocator): the reference callocs and frees
+// its checkpoints on the host in every forward; here one block per id and shape lives in the pool PyTorch can see.
+void* torch_alloc(unsigned long long bytes, int /*device: the current one*/, void* stream, void* /*user*/) {
+  try {
+    return c10::hip::HIPCachingAllocator::raw_alloc_with_stream((size_t)bytes, (hipStream_t)stream);
+  } catch (const std::exception&) {  // out of memory: the library falls back to fewer kept rows or reports the failure
+    return nullptr;
+  }
+}
+void torch_release(void* ptr, void* /*user*/) { c10::hip::HIPCachingAllocator::raw_delete(ptr); }
 
 }  // namespace
 
@@ -77,6 +89,10 @@ std::vector<at::Tensor> tvInpaint_backward(at::Tensor d_iGf, at::Tensor d_x, at:
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  tvinpaint_set_allocator(torch_alloc, torch_release, nullptr);
+  m.def("use_torch_allocator", [](bool enable) {
+    TORCH_CHECK(tvinpaint_set_allocator(enable ? torch_alloc : nullptr, enable ? torch_release : nullptr, nullptr) == 0, tvinpaint_last_error());
+  }, "take the ids' device blocks from PyTorch's caching allocator (default) or from hipMalloc");
   m.def("forward", &tvInpaint_forward, "tvInpaint forward (HIP)");
   m.def("backward", &tvInpaint_backward, "tvInpaint backward (HIP)");
   m.def("dummy", &tvInpaint_dummy, "tvInpaint dummy");

@@ -69,6 +69,7 @@ struct Knobs {
   int tgv_pair_waves = 0;         // INPAINT_TGV_PAIR_WAVES=1|2 (0 = by channel count)
   int keep = -1;                  // INPAINT_KEEP=0|1|2 (INPAINT_KEEP_LAST=0 is INPAINT_KEEP=0); -1 = the id's own mode
   double keep_gb = 32.0;          // INPAINT_KEEP_GB: budget of keep mode 2
+  bool keep_gb_set = false;       // (the variable is set: the budget is the caller's, free device memory is not consulted)
   bool quadfit_px_path = false;   // INPAINT_QUADFIT_PATH=px: one pixel per lane, no LDS windows
   bool median_tile_per_wave = false;  // INPAINT_MEDIAN_PATH=tile: one tile of 64 pixels per wavefront for every bin count
   bool quadfit_reread = false;    // INPAINT_QUADFIT_PATH=reread: backward pass A reads the second map twice (any channel count)
@@ -104,7 +105,7 @@ struct Knobs {
       const int v = atoi(e);
       if (v >= 0 && v <= 2) keep = v;
     }
-    if (const char* e = getenv("INPAINT_KEEP_GB")) keep_gb = atof(e);
+    if (const char* e = getenv("INPAINT_KEEP_GB")) { keep_gb = atof(e); keep_gb_set = true; }
     quadfit_px_path = is("INPAINT_QUADFIT_PATH", "px");
     quadfit_reread = is("INPAINT_QUADFIT_PATH", "reread");
     median_tile_per_wave = is("INPAINT_MEDIAN_PATH", "tile");
@@ -156,16 +157,26 @@ inline void make_step_sizes(int its, std::vector<float>& s) {
 // ---------------------------------------------------------------------------------------------
 // device arena: one hipMalloc per slot, re-made only when the shape changes
 // ---------------------------------------------------------------------------------------------
+// Where a slot's block comes from: hipMalloc / hipFree, or the caller's pool (t[g]vinpaint_set_allocator).
+struct Allocator {
+  inpaint_alloc_fn alloc = nullptr;
+  inpaint_release_fn release = nullptr;
+  void* user = nullptr;
+};
+
 struct Arena {
   char* base = nullptr;
   size_t bytes = 0, used = 0;
   int device = -1;
+  Allocator owner;  // the pair that made `base` also takes it back
   int release() {
     if (base) {
       int cur = -1;
       (void)hipGetDevice(&cur);
       if (cur != device && device >= 0) (void)hipSetDevice(device);
-      hipError_t e = hipFree(base);
+      hipError_t e = hipSuccess;
+      if (owner.release) owner.release(base, owner.user);
+      else e = hipFree(base);
       if (cur != device && cur >= 0) (void)hipSetDevice(cur);
       base = nullptr;
       bytes = used = 0;
@@ -173,14 +184,26 @@ struct Arena {
     }
     return 0;
   }
-  int reserve(size_t need) {
+  int reserve(size_t need, const Allocator& from, hipStream_t stream) {
     int rc = release();
     if (rc) return rc;
     INPAINT_HIP(hipGetDevice(&device));
-    const hipError_t e = hipMalloc((void**)&base, need);
-    if (e != hipSuccess) {
-      base = nullptr;
-      return fail(INPAINT_ERR_HIP, "hipMalloc of %zu bytes failed: %s", need, hipGetErrorString(e));
+    if (from.alloc && from.release) {
+      base = static_cast<char*>(from.alloc((unsigned long long)need, device, (void*)stream, from.user));
+      if (!base) return fail(INPAINT_ERR_HIP, "the caller's allocator returned no memory for %zu bytes", need);
+      if (reinterpret_cast<uintptr_t>(base) & 255) {
+        from.release(base, from.user);
+        base = nullptr;
+        return fail(INPAINT_ERR_HIP, "the caller's allocator returned a block that is not aligned to 256 bytes");
+      }
+      owner = from;
+    } else {
+      const hipError_t e = hipMalloc((void**)&base, need);
+      if (e != hipSuccess) {
+        base = nullptr;
+        return fail(INPAINT_ERR_HIP, "hipMalloc of %zu bytes failed: %s", need, hipGetErrorString(e));
+      }
+      owner = Allocator();
     }
     bytes = need;
     used = 0;
@@ -194,6 +217,19 @@ struct Arena {
   }
   static size_t padded(size_t count, size_t elem) { return ((count * elem + 255) & ~size_t(255)) + 256; }
 };
+
+// Keep mode 2 asks for one x05 row per iteration.  When the slot has to grow for them and nobody stated a budget
+// (INPAINT_KEEP_GB), rows that would take more than a quarter of what the device has free right now are not asked for:
+// the forward pass keeps the last segment's rows instead (mode 1).  One hipMemGetInfo per (re)allocation, none per call.
+inline bool rows_exceed_free_memory(double ring_bytes) {
+  if (knobs().keep_gb_set) return false;
+  size_t free_b = 0, total_b = 0;
+  if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return ring_bytes > 0.25 * (double)free_b;
+}
 
 // ---------------------------------------------------------------------------------------------
 // strip height

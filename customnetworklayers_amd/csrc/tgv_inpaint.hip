@@ -799,6 +799,7 @@ struct Slot {
 };
 
 Slot g_slots[kUniqueIds];
+Allocator g_allocator;  // tgvinpaint_set_allocator
 KernelTimer g_timer;
 
 size_t state_count(const Slot& s) { return (size_t)s.n * 3 * s.ic * s.ih * s.iw; }
@@ -849,7 +850,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   need += Arena::padded((size_t)n, 8) + Arena::padded((size_t)n, 4) + Arena::padded(2, 4);
   need += Arena::padded(std::max(F, 2 * P), 4);  // the field of zeros
   need += Arena::padded(1, sizeof(GuardState));
-  rc = s.arena.reserve(need);
+  rc = s.arena.reserve(need, g_allocator, stream);
   if (rc) return rc;
   Arena& a = s.arena;
   s.wx = a.take<float>(P); s.wy = a.take<float>(P); s.bx = a.take<float>(P); s.by = a.take<float>(P);
@@ -1241,6 +1242,9 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
   const long long shape[5] = {n, ic, ih, iw, its};
   if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
+  if (keep == 2 && !(s.arena.base && s.n == n && s.ic == ic && s.ih == ih && s.iw == iw && s.its == its && s.ring_rows >= its) &&
+      rows_exceed_free_memory(4.0 * 3 * n * ic * (double)ih * iw * its))
+    keep = 1;  // (the slot would have to grow by more than a quarter of the free device memory)
   rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
   if (rc && keep == 2) {  // no room for every x05 row: keep the last segment's instead and recompute the others
     (void)hipGetLastError();
@@ -1685,6 +1689,14 @@ int tgvinpaint_keep_iterates(int id, int mode) {
   if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
   if (mode < 0 || mode > 2) return fail(INPAINT_ERR_ARG, "keep mode %d is not 0, 1 or 2", mode);
   g_slots[id].keep_mode = mode;
+  return 0;
+}
+
+int tgvinpaint_set_allocator(inpaint_alloc_fn alloc, inpaint_release_fn release, void* user) {
+  if ((alloc == nullptr) != (release == nullptr)) return fail(INPAINT_ERR_ARG, "tgvinpaint_set_allocator: give both callbacks or neither");
+  g_allocator.alloc = alloc;
+  g_allocator.release = release;
+  g_allocator.user = alloc ? user : nullptr;
   return 0;
 }
 

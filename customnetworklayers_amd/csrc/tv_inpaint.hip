@@ -527,6 +527,7 @@ struct Slot {
 };
 
 Slot g_slots[kUniqueIds];
+Allocator g_allocator;  // tvinpaint_set_allocator
 
 KernelTimer g_timer;
 
@@ -569,7 +570,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   need += Arena::padded(P, 8) * 3 + Arena::padded(F, 8);
   need += Arena::padded(P * nck, 4) * 3 + Arena::padded(F * nck, 4);
   need += Arena::padded(1, sizeof(GuardState));
-  rc = s.arena.reserve(need);
+  rc = s.arena.reserve(need, g_allocator, stream);
   if (rc) return rc;
   Arena& a = s.arena;
   s.ypp[0] = a.take<float>(F); s.ypp[1] = a.take<float>(F);
@@ -1021,6 +1022,9 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   int keep = resolve_keep_mode(s, n, ic, ih, iw, its);
   const long long shape[5] = {n, ic, ih, iw, its};
   if (keep == 2 && std::equal(shape, shape + 5, s.refused)) keep = 1;
+  if (keep == 2 && !(s.arena.base && s.n == n && s.ic == ic && s.ih == ih && s.iw == iw && s.its == its && s.ring_rows >= its) &&
+      rows_exceed_free_memory(4.0 * n * ic * (double)ih * iw * its))
+    keep = 1;  // (the slot would have to grow by more than a quarter of the free device memory)
   rc = prepare_slot(s, n, ic, ih, iw, its, keep, stream);
   if (rc && keep == 2) {  // no room for every x05 row: keep the last segment's instead and recompute the others
     (void)hipGetLastError();
@@ -1499,6 +1503,14 @@ int tvinpaint_keep_iterates(int id, int mode) {
   if (id < 0 || id >= kUniqueIds) return fail(INPAINT_ERR_ID, "bad id %d", id);
   if (mode < 0 || mode > 2) return fail(INPAINT_ERR_ARG, "keep mode %d is not 0, 1 or 2", mode);
   g_slots[id].keep_mode = mode;
+  return 0;
+}
+
+int tvinpaint_set_allocator(inpaint_alloc_fn alloc, inpaint_release_fn release, void* user) {
+  if ((alloc == nullptr) != (release == nullptr)) return fail(INPAINT_ERR_ARG, "tvinpaint_set_allocator: give both callbacks or neither");
+  g_allocator.alloc = alloc;
+  g_allocator.release = release;
+  g_allocator.user = alloc ? user : nullptr;
   return 0;
 }
 

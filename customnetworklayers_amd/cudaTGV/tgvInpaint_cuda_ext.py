@@ -9,10 +9,17 @@ the 3*c channels the layer really writes (the reference binding allocates only c
 TGVInpaintFista_cuda.cpp:91,157); failures raise instead of returning an empty list.
 """
 import ctypes
+import os
 
 import torch
 
-from .._lib import last_error, lib
+from .._lib import last_error, lib, torch_allocator_in_use, use_torch_allocator
+
+# The per-id device blocks come out of PyTorch's caching allocator (t[g]vinpaint_set_allocator), so that
+# torch.cuda.memory_allocated() counts them and reset_id() returns them to the pool; INPAINT_TORCH_ALLOCATOR=0 leaves
+# them with hipMalloc.
+if os.environ.get("INPAINT_TORCH_ALLOCATOR", "1") != "0" and not torch_allocator_in_use():
+    use_torch_allocator(True)
 from ..cudaTV.tvInpaint_cuda_ext import _check_input, _ERRORS, _stream
 
 

@@ -8,10 +8,17 @@ TVInpaintFista_cuda.cpp:61-65), and failures raise instead of returning an empty
 (TVInpaintFista_cuda.cpp:80-87).
 """
 import ctypes
+import os
 
 import torch
 
-from .._lib import last_error, lib
+from .._lib import last_error, lib, torch_allocator_in_use, use_torch_allocator
+
+# The per-id device blocks come out of PyTorch's caching allocator (t[g]vinpaint_set_allocator), so that
+# torch.cuda.memory_allocated() counts them and reset_id() returns them to the pool; INPAINT_TORCH_ALLOCATOR=0 leaves
+# them with hipMalloc.
+if os.environ.get("INPAINT_TORCH_ALLOCATOR", "1") != "0" and not torch_allocator_in_use():
+    use_torch_allocator(True)
 
 _ERRORS = {1: IndexError, 2: ValueError, 3: ValueError, 4: RuntimeError, 5: RuntimeError}
 

@@ -73,6 +73,10 @@ int tgvinpaint_guard_stats(int id, double* stats25);
 
 long long tgvinpaint_slot_bytes(int id);
 
+/* Who owns the TGV slots' device memory: as tvinpaint_set_allocator (the reference's per-forward calloc / free of the
+ * checkpoints: TGVInpaintFistaBetas.cu:2534-2546, TGVInpaintFista.h:18-37). */
+int tgvinpaint_set_allocator(inpaint_alloc_fn alloc, inpaint_release_fn release, void* user);
+
 /* The per-sample step scale L = 1 / (max(32, max_p s_p) + 0.01) the last call on this id used
  * (host array of n doubles).  Waits for the slot's stream. */
 int tgvinpaint_lipschitz(int id, double* L_host, int n);

@@ -86,12 +86,29 @@ int tvinpaint_gradient_mode(int id, int mode);
  * of work and its memory footprint (2 sqrt(its) + sqrt(its) fields).  1: those of the last segment.  2 (default):
  * all of them -- its fields of memory, no recompute, and the fastest backward.  The gradients are the same bits
  * in every mode.  A forward whose gradients are never asked for is fastest with 0.  Mode 2 falls back to 1 when
- * the rows would need more than INPAINT_KEEP_GB (default 32) GiB or the device cannot allocate them; INPAINT_KEEP=0|1|2 overrides this call.
+ * the rows would need more than INPAINT_KEEP_GB GiB (when the variable is not set: more than 32 GiB, or more than a
+ * quarter of the device's free memory at the moment the slot has to grow) or the device cannot allocate them;
+ * INPAINT_KEEP=0|1|2 overrides this call.
  * No counterpart in the reference, which always recomputes. */
 int tvinpaint_keep_iterates(int id, int mode);
 
 /* Bytes of device memory the slot currently owns (0 if none). */
 long long tvinpaint_slot_bytes(int id);
+
+/* Who owns the slots' device memory.  The reference callocs and frees its checkpoints on the host in every forward
+ * (TVInpaintFista.cu:1510-1521, TVInpaintFista.h:18-37); here each id holds ONE device block per shape, and by default
+ * the library takes it from hipMalloc.  A host program that runs its own pool (PyTorch's caching allocator) hands over
+ * two callbacks instead, so that the block comes out of, and goes back to, the pool it can see and reuse:
+ *   alloc(bytes, device, stream, user) -> device pointer aligned to 256 bytes, or NULL when it cannot (the call then
+ *                                         fails with INPAINT_ERR_HIP, or falls back from keep mode 2 to 1)
+ *   release(ptr, user)                    called once per block: when the id's shape changes, by tvinpaint_reset_id,
+ *                                         never while work on the block is still in flight (the id's stream is
+ *                                         synchronised first)
+ * Both NULL restores hipMalloc / hipFree.  A block is always released by the callback pair that made it, so the
+ * allocator may be changed while ids hold memory.  Not thread safe against concurrent forwards. */
+typedef void* (*inpaint_alloc_fn)(unsigned long long bytes, int device, void* stream, void* user);
+typedef void (*inpaint_release_fn)(void* ptr, void* user);
+int tvinpaint_set_allocator(inpaint_alloc_fn alloc, inpaint_release_fn release, void* user);
 
 /* Host-only: checkpoint schedule and FISTA extrapolation factors the layer uses for `its`
  * (TVInpaintFista.cu:1499-1508,1523 and 1525-1532).  iterations_out holds floor(sqrt(its)) ints. */

@@ -15,6 +15,7 @@ def declared_symbols():
     names = []
     for path in sorted(glob.glob(os.path.join(ROOT, "include", "*.h"))):
         text = re.sub(r"/\*.*?\*/", "", open(path).read(), flags=re.S)
+        text = re.sub(r"\btypedef\b[^;]*;", "", text)  # (callback types are not symbols)
         names += re.findall(r"\b([a-z_0-9]+)\s*\([^;{]*\)\s*;", text)
     return sorted(set(names))
 
