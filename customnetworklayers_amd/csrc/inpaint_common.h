@@ -70,6 +70,7 @@ struct Knobs {
   int keep = -1;                  // INPAINT_KEEP=0|1|2 (INPAINT_KEEP_LAST=0 is INPAINT_KEEP=0); -1 = the id's own mode
   double keep_gb = 32.0;          // INPAINT_KEEP_GB: budget of keep mode 2
   bool keep_gb_set = false;       // (the variable is set: the budget is the caller's, free device memory is not consulted)
+  int stats_every = 0;            // INPAINT_STATS_EVERY=N: the guard's statistics on stderr every Nth backward pass of an id (a host wait; off by default)
   bool quadfit_px_path = false;   // INPAINT_QUADFIT_PATH=px: one pixel per lane, no LDS windows
   bool median_tile_per_wave = false;  // INPAINT_MEDIAN_PATH=tile: one tile of 64 pixels per wavefront for every bin count
   bool quadfit_reread = false;    // INPAINT_QUADFIT_PATH=reread: backward pass A reads the second map twice (any channel count)
@@ -106,6 +107,7 @@ struct Knobs {
       if (v >= 0 && v <= 2) keep = v;
     }
     if (const char* e = getenv("INPAINT_KEEP_GB")) { keep_gb = atof(e); keep_gb_set = true; }
+    if (const char* e = getenv("INPAINT_STATS_EVERY")) stats_every = std::max(0, atoi(e));
     quadfit_px_path = is("INPAINT_QUADFIT_PATH", "px");
     quadfit_reread = is("INPAINT_QUADFIT_PATH", "reread");
     median_tile_per_wave = is("INPAINT_MEDIAN_PATH", "tile");
@@ -798,6 +800,25 @@ inline int guard_selftest(const void* values, long long n, bool is_f32, int run,
   const int rc = run_all();
   release();
   return rc;
+}
+
+// The guard's statistics of the backward pass just enqueued, on stderr in the reference's wording (TVInpaintFista.cu:1766-1790
+// prints them on every 75th run of an id, TGVInpaintFistaBetas.cu:2996-3021 with the id in front).  Waits for the stream:
+// only called when INPAINT_STATS_EVERY asks for it.  Nothing is printed for a backward pass whose upstream was refused.
+inline int print_guard_report(const GuardState* dev, hipStream_t stream, int id, bool with_id) {
+  GuardState host;
+  INPAINT_HIP(hipStreamSynchronize(stream));
+  INPAINT_HIP(hipMemcpy(&host, dev, kGuardHeaderBytes, hipMemcpyDeviceToHost));
+  if (host.upstream_bad) return 0;
+  static const char* const names[5] = {"conf ", "gradX ", "gradY ", "gradB ", "gradI "};
+  for (int k = 0; k < 5; k++) {
+    if (with_id) fprintf(stderr, "\nL %d Output gradient to %s %d %g  vs  %g vs %g ", id, names[k], (int)host.report[5 * k + 2],
+                         host.report[5 * k + 0], host.av[k], host.report[5 * k + 1]);
+    else fprintf(stderr, "\nOutput gradient to %s %d %g  vs  %g vs %g ", names[k], (int)host.report[5 * k + 2], host.report[5 * k + 0],
+                 host.av[k], host.report[5 * k + 1]);
+  }
+  fprintf(stderr, "\n\n");
+  return 0;
 }
 
 // Optional timing of a layer's dominant kernel with HIP events on the launch stream.  An event

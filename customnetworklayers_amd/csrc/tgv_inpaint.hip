@@ -29,9 +29,7 @@ using namespace inpaint;
 // TGV.cu:58-60,70,78,87-93; TGVH.cu:24-41
 constexpr float kD0 = 0.2f, kD1 = 0.2f, kD2 = 0.2f;
 constexpr float kBeta = 4.0f;
-constexpr float kClipLocalGrad = 2000.0f;
 constexpr float kLocalGCMult = 0.1f;
-constexpr float kLocalGXMult = 0.1f;
 constexpr float kLocalGBMult = 1.0f;
 constexpr float kGlobalGMult = 0.1f;
 const GuardParams kGuard = {5000000., 5000000., 35., 10., 0.95};
@@ -138,141 +136,6 @@ __global__ __launch_bounds__(256) void tgv_scale_kernel(const float* __restrict_
   by[i] = (float)(L * (double)dy[s * 2 * HW + HW + p]);
 }
 
-// -------------------------------------------------------------------------------------------------
-// forward iteration: TGV.cu:1546-1776; with x05 != nullptr also TGV.cu:2005-2235
-// -------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(BX* BY) void tgv_forward_px(
-    const float* __restrict__ wx_, const float* __restrict__ wy_, const float* __restrict__ bx_,
-    const float* __restrict__ by_, const float* __restrict__ cf_, const float* __restrict__ b_,
-    const float* __restrict__ xin_, float* __restrict__ xout_, const float* __restrict__ yin_,
-    float* __restrict__ yout_, float* __restrict__ x05_, int C, int H, int W, float t) {
-  const int w = blockIdx.x * BX + threadIdx.x, h = blockIdx.y * BY + threadIdx.y;
-  if (w >= W || h >= H) return;
-  const size_t HW = (size_t)H * W, CHW = HW * C, S = 3 * CHW;
-  const size_t smp = blockIdx.z;
-  const float *wx = wx_ + smp * HW, *wy = wy_ + smp * HW, *bx = bx_ + smp * HW, *by = by_ + smp * HW;
-  const size_t p = (size_t)h * W + w;
-  const float conf = cf_[smp * HW + p];
-  const float wx_0 = (w > 0) ? wx[p - 1] : 0.f;
-  const float wx_1 = (w < W - 1) ? wx[p] : 0.f;
-  const float wy_0 = (h > 0) ? wy[p - W] : 0.f;
-  const float wy_1 = (h < H - 1) ? wy[p] : 0.f;
-  const float wx_2 = (h > 0 && w < W - 1) ? wx[p - W] : 0.f;
-  const float wy_2 = (w > 0 && h < H - 1) ? wy[p - 1] : 0.f;
-  const float bX_u = (h > 0) ? bx[p - W] : 0.f, bY_u = (h > 0) ? by[p - W] : 0.f;
-  const float bX_l = (w > 0) ? bx[p - 1] : 0.f, bY_l = (w > 0) ? by[p - 1] : 0.f;
-  const float bX_c = bx[p], bY_c = by[p];
-  const float oneL = 1.0f;  // TGV.cu:2527
-  for (int ch = 0; ch < C; ch++) {
-    const size_t o = smp * S + (size_t)ch * HW;
-    const Plane Y0{yin_ + o, H, W}, Y1{yin_ + o + CHW, H, W}, Y2{yin_ + o + 2 * CHW, H, W};
-    const float x_ = xin_[o + p];
-    const float bb = b_[smp * CHW + (size_t)ch * HW + p];
-    float yc = Y0.f[p];
-    float yt = yc;
-    float y1_new = Y1.f[p], y2_new = Y2.f[p];
-    const float y1_c = y1_new, y2_c = y2_new;
-    if (h > 0) {  // TGV.cu:1613-1640
-      const float betaTX = bX_u, betaTY = bY_u;
-      const float zij_1 = (w < W - 1) ? ((Y0.at(h - 1, w + 1) - Y0.at(h - 1, w)) - Y1.at(h - 1, w)) : 0.f;
-      const float zij_2 = ((yc - Y0.at(h - 1, w)) - Y2.at(h - 1, w));
-      const float hwx = fminf(1.f, rsq(zij_2 * zij_2 * wy_0 + zij_1 * zij_1 * wx_2) * kD0);
-      const float uij1_2 = (y1_c - Y1.at(h - 1, w));
-      const float uij1_1 = (w < W - 1) ? (Y1.at(h - 1, w + 1) - Y1.at(h - 1, w)) : 0.f;
-      const float hwy1 = fminf(1.f, rsq(betaTX * (uij1_2 * uij1_2 + uij1_1 * uij1_1)) * kD1);
-      const float uij2_1 = (w < W - 1) ? (Y2.at(h - 1, w + 1) - Y2.at(h - 1, w)) : 0.f;
-      const float uij2_2 = (y2_c - Y2.at(h - 1, w));
-      const float hwy2 = fminf(1.f, rsq(betaTY * (uij2_2 * uij2_2 + uij2_1 * uij2_1)) * kD2);
-      yt -= wy_0 * oneL * (zij_2 * hwx);
-      y1_new -= (betaTX * oneL) * (uij1_2 * hwy1);
-      y2_new -= (betaTY * oneL) * (uij2_2 * hwy2);
-    }
-    if (w > 0) {  // TGV.cu:1641-1668
-      const float betaTX = bX_l, betaTY = bY_l;
-      const float zij_1 = ((yc - Y0.at(h, w - 1)) - Y1.at(h, w - 1));
-      const float zij_2 = (h < H - 1) ? ((Y0.at(h + 1, w - 1) - Y0.at(h, w - 1)) - Y2.at(h, w - 1)) : 0.f;
-      const float hwx = fminf(1.f, rsq(zij_2 * zij_2 * wy_2 + zij_1 * zij_1 * wx_0) * kD0);
-      const float uij1_1 = (y1_c - Y1.at(h, w - 1));
-      const float uij1_2 = (h < H - 1) ? (Y1.at(h + 1, w - 1) - Y1.at(h, w - 1)) : 0.f;
-      const float hwy1 = fminf(1.f, rsq(betaTX * (uij1_2 * uij1_2 + uij1_1 * uij1_1)) * kD1);
-      const float uij2_1 = (y2_c - Y2.at(h, w - 1));
-      const float uij2_2 = (h < H - 1) ? (Y2.at(h + 1, w - 1) - Y2.at(h, w - 1)) : 0.f;
-      const float hwy2 = fminf(1.f, rsq(betaTY * (uij2_2 * uij2_2 + uij2_1 * uij2_1)) * kD2);
-      yt -= wx_0 * oneL * (zij_1 * hwx);
-      y1_new -= (betaTX * oneL) * (uij1_1 * hwy1);
-      y2_new -= (betaTY * oneL) * (uij2_1 * hwy2);
-    }
-    {  // TGV.cu:1669-1691
-      const float betaTX = bX_c, betaTY = bY_c;
-      const float zij_1 = (w < W - 1) ? ((yc - Y0.at(h, w + 1)) + y1_c) : 0.f;
-      const float zij_2 = (h < H - 1) ? ((yc - Y0.at(h + 1, w)) + y2_c) : 0.f;
-      const float hwx = fminf(1.f, rsq(zij_2 * zij_2 * wy_1 + zij_1 * zij_1 * wx_1) * kD0);
-      const float uij1_1 = (w < W - 1) ? (y1_c - Y1.at(h, w + 1)) : 0.f;
-      const float uij1_2 = (h < H - 1) ? (y1_c - Y1.at(h + 1, w)) : 0.f;
-      const float hwy1 = fminf(1.f, rsq(betaTX * (uij1_2 * uij1_2 + uij1_1 * uij1_1)) * kD1);
-      const float uij2_1 = (w < W - 1) ? (y2_c - Y2.at(h, w + 1)) : 0.f;
-      const float uij2_2 = (h < H - 1) ? (y2_c - Y2.at(h + 1, w)) : 0.f;
-      const float hwy2 = fminf(1.f, rsq(betaTY * (uij2_2 * uij2_2 + uij2_1 * uij2_1)) * kD2);
-      yt -= wy_1 * oneL * (zij_2 * hwx);
-      y1_new -= (betaTX * oneL) * (uij1_2 * hwy1);
-      y2_new -= (betaTY * oneL) * (uij2_2 * hwy2) + wy_1 * oneL * (zij_2 * hwx);
-      yt -= wx_1 * oneL * (zij_1 * hwx);
-      y1_new -= (betaTX * oneL) * (uij1_1 * hwy1) + wx_1 * oneL * (zij_1 * hwx);
-      y2_new -= (betaTY * oneL) * (uij2_1 * hwy2);
-    }
-    // aux variables: momentum only (TGV.cu:1686-1690)
-    yout_[o + CHW + p] = y1_new + t * (y1_new - xin_[o + CHW + p]);
-    yout_[o + 2 * CHW + p] = y2_new + t * (y2_new - xin_[o + 2 * CHW + p]);
-    xout_[o + CHW + p] = y1_new;
-    xout_[o + 2 * CHW + p] = y2_new;
-    if (x05_) {  // TGV.cu:2146-2147,2196
-      x05_[o + p] = yt;
-      x05_[o + CHW + p] = y1_new;
-      x05_[o + 2 * CHW + p] = y2_new;
-    }
-    // Huber-1 prox on u (TGV.cu:1740-1744)
-    float x_loc = (conf * bb + yt) / (1.f + conf);
-    yc = yt - conf;
-    yt = yt + conf;
-    if (yc > 1.f + bb) x_loc = yc;
-    if (yt < bb - 1.f) x_loc = yt;
-    yout_[o + p] = x_loc + t * (x_loc - x_);
-    xout_[o + p] = x_loc;
-  }
-}
-
-// y_{k+1} from x05[k] (xa), x05[k-1] (xb): TGV.cu:1478-1541; aux variables are x05[k] itself.
-__global__ __launch_bounds__(256) void tgv_getyk_kernel(const float* __restrict__ cf, const float* __restrict__ b,
-                                                        const float* __restrict__ xa, const float* __restrict__ xb,
-                                                        float* __restrict__ yk, int C, long long HW, long long total,
-                                                        float t) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // over n*HW pixels
-  if (i >= total) return;
-  const long long s = i / HW, p = i - s * HW;
-  const long long CHW = HW * C;
-  const float conf = cf[i];
-  for (int ch = 0; ch < C; ch++) {
-    const long long q = s * 3 * CHW + ch * HW + p;
-    const float bb = b[s * CHW + ch * HW + p];
-    float diff = bb - xa[q];
-    float sign = (diff < 0) ? -1.f : 1.f;
-    float v;
-    if (1. + (double)conf >= (double)(sign * diff)) {
-      const float xk = (conf * bb + xa[q]) / (1.f + conf);
-      const float xkm = (conf * bb + xb[q]) / (1.f + conf);
-      v = xk + t * (xk - xkm);
-    } else {
-      const float xk = (conf <= sign * diff) ? bb - diff + sign * conf : bb;
-      diff = bb - xb[q];
-      sign = (diff < 0) ? -1.f : 1.f;
-      v = xk + t * (xk - ((conf <= sign * diff) ? bb - diff + sign * conf : bb));
-    }
-    yk[q] = v;
-    yk[q + CHW] = xa[q + CHW];
-    yk[q + 2 * CHW] = xa[q + 2 * CHW];
-  }
-}
-
 // Prox adjoint + confidence / rhs gradient: TGV.cu:592-612, 1418-1442 (and 166-182 for the first step).
 template <bool FIRST, bool TRUE_ADJ = false>
 __device__ __forceinline__ void prox_adjoint(float df_dxk, float bb, float x05v, float conf, float& g05,
@@ -323,46 +186,32 @@ __global__ __launch_bounds__(256) void tgv_adjoint_first(const float* __restrict
   gc[i] = gcv;
 }
 
-// Huber weight of the segment-start kernel: (float)(1. / (double)max(1, hub / delta)), TGV.cu:1133.
-// For a float m >= 1 the double quotient rounded to float equals the float quotient: a
-// double-rounding slip needs 1/m within 2^-54 (relative) of a 25-bit number M, but 1 - m*M is a
-// multiple of 2^-49 and cannot be that small unless it is zero.
-__device__ __forceinline__ float huber_w_end(float hub, float delta) { return 1.0f / fmaxf(1.f, hub / delta); }
-
-// Main adjoint step (TGV.cu:224-644) and, with END, the segment-start variant (TGV.cu:1061-1472)
-// that linearises at the checkpoint y and writes the same Jacobian with sqrt and divisions.
-// y is y_{k+1} rebuilt by tgv_getyk_kernel, or the checkpoint y.
-// JT0 (corrected gradient only): the gradient step of iteration 0, which the reference never back-propagates
-// (TGV.cu:2851-2933 ends after producing g05[0]; TGV.cu:3047 returns g_x[1]).  Only the transposed Jacobian is applied,
-// in the main kernel's form with the v2 block's division (TGV.cu:355) replaced by its siblings' product and
-// multiplier 1: g05_out receives J^T g05_in + gxk (the gradient wrt the start), the weight gradients are added to
-// gwx / gwy; gc, gb, gxk, gxk_m1 are left alone and y is the starting point.
-template <bool END, bool JT0 = false>
-__global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
+// Corrected gradient only: the gradient step of iteration 0, which the reference never back-propagates
+// (TGV.cu:2851-2933 ends after producing g05[0]; TGV.cu:3047 returns g_x[1]).  One thread per pixel applies the
+// transposed Jacobian of the step at the starting point y_0 -- the main adjoint kernel's form (TGV.cu:304-507), every
+// Huber weight derivative as weight x rsqrt^2, multipliers 1 -- to g05[0] and adds the partial g_x[0]:
+// gi = J^T g05[0] + g_x[0] is the gradient wrt the starting point; the weight gradients of iteration 0 are added to the
+// fp32 accumulators gwx / gwy (two planes each: edge weight, beta), which the caller flushes into the totals.
+__global__ __launch_bounds__(BX* BY) void tgv_adjoint_iter0(
     const float* __restrict__ wx_, const float* __restrict__ wy_, const float* __restrict__ bx_,
-    const float* __restrict__ by_, const float* __restrict__ cf_, const float* __restrict__ b_,
-    const float* __restrict__ x05_, float* __restrict__ gc_, float* __restrict__ gb_, float* __restrict__ gwx_,
-    float* __restrict__ gwy_, const float* __restrict__ g05_in_, float* __restrict__ g05_out_, float* __restrict__ gxk_,
-    float* __restrict__ gxk_m1_, const float* __restrict__ y_, int C, int H, int W, float t) {
+    const float* __restrict__ by_, const float* __restrict__ y_, const float* __restrict__ g05_in_,
+    const float* __restrict__ gx0_, float* __restrict__ gi_, float* __restrict__ gwx_, float* __restrict__ gwy_,
+    int C, int H, int W) {
   const int w = blockIdx.x * BX + threadIdx.x, h = blockIdx.y * BY + threadIdx.y;
   if (w >= W || h >= H) return;
   const size_t HW = (size_t)H * W, CHW = HW * C, S = 3 * CHW;
   const size_t smp = blockIdx.z;
   const float *wx = wx_ + smp * HW, *wy = wy_ + smp * HW, *bx = bx_ + smp * HW, *by = by_ + smp * HW;
   const size_t p = (size_t)h * W + w;
-  const float conf = cf_[smp * HW + p];
   const float wx_0 = (w > 0) ? wx[p - 1] : 0.f;
   const float wx_1 = (w < W - 1) ? wx[p] : 0.f;
   const float wy_0 = (h > 0) ? wy[p - W] : 0.f;
   const float wy_1 = (h < H - 1) ? wy[p] : 0.f;
   const float wx_2 = (h > 0 && w < W - 1) ? wx[p - W] : 0.f;
   const float wy_2 = (w > 0 && h < H - 1) ? wy[p - 1] : 0.f;
-  const float bX_u = (h > 0) ? bx[p - W] : 0.f, bY_u = (h > 0) ? by[p - W] : 0.f;
-  const float bX_l = (w > 0) ? bx[p - 1] : 0.f, bY_l = (w > 0) ? by[p - 1] : 0.f;
-  const float bX_c = bx[p], bY_c = by[p];
-  const float oneL = 1.0f;
-  const float gxm = JT0 ? 1.f : kLocalGXMult;
-  float gcv = gc_[smp * HW + p];
+  const float b1u = (h > 0) ? bx[p - W] : 0.f, b2u = (h > 0) ? by[p - W] : 0.f;
+  const float b1l = (w > 0) ? bx[p - 1] : 0.f, b2l = (w > 0) ? by[p - 1] : 0.f;
+  const float b1c = bx[p], b2c = by[p];
   float gwx0 = gwx_[smp * 2 * HW + p], gwx1 = gwx_[smp * 2 * HW + HW + p];
   float gwy0 = gwy_[smp * 2 * HW + p], gwy1 = gwy_[smp * 2 * HW + HW + p];
   for (int ch = 0; ch < C; ch++) {
@@ -371,290 +220,155 @@ __global__ __launch_bounds__(BX* BY) void tgv_adjoint_px(
     const Plane G{g05_in_ + o, H, W}, G1{g05_in_ + o + CHW, H, W}, G2{g05_in_ + o + 2 * CHW, H, W};
 #define QY(F, dh, dw) F.at(h + (dh), w + (dw))
     const float yk = Y.f[p];
-    const float df_dy = G.f[p], df_dy1 = G1.f[p], df_dy2 = G2.f[p];
-    float df_dy_t = df_dy, df_dy1_t = df_dy1, df_dy2_t = df_dy2;
+    const float g0 = G.f[p], g1 = G1.f[p], g2 = G2.f[p];
+    float t0 = g0, t1 = g1, t2 = g2;
     if (h > 0) {  // triangles owned by the pixel above: TGV.cu:304-360 / 1118-1171
-      const float betaTX = bX_u, betaTY = bY_u;
+      const float beta1 = b1u, beta2 = b2u;
       {
-        const float zij_1 = (w < W - 1) ? ((QY(Y, -1, 1) - QY(Y, -1, 0)) - QY(Y1, -1, 0)) : 0.f;
-        const float zij_2 = ((yk - QY(Y, -1, 0)) - QY(Y2, -1, 0));
-        const float A = zij_2 * zij_2 * wy_0 + zij_1 * zij_1 * wx_2;
-        float W_TIJ, dW_TIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(A);
-          W_TIJ = huber_w_end(hub, kD0);
-          active = hub > kD0;
-          dW_TIJ = W_TIJ / (hub * hub);
-        } else {
-          const float hub = rsq(A);
-          W_TIJ = fminf(1.f, hub * kD0);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ * (hub * hub);
-        }
-        df_dy_t -= oneL * W_TIJ * ((df_dy - QY(G, -1, 0)) - QY(G2, -1, 0)) * wy_0;
+        const float z1 = (w < W - 1) ? ((QY(Y, -1, 1) - QY(Y, -1, 0)) - QY(Y1, -1, 0)) : 0.f;
+        const float z2 = ((yk - QY(Y, -1, 0)) - QY(Y2, -1, 0));
+        const float A = z2 * z2 * wy_0 + z1 * z1 * wx_2;
+        const float hub = rsq(A), hw = fminf(1.f, hub * kD0), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        t0 -= hw * ((g0 - QY(G, -1, 0)) - QY(G2, -1, 0)) * wy_0;
         if (active) {
-          const float a2 = zij_2 * wy_0;
-          const float a1 = zij_1 * wx_2;
-          df_dy_t += oneL * (dW_TIJ * a2) * (a1 * (QY(G, -1, 1) - QY(G, -1, 0) - QY(G1, -1, 0)) +
+          const float a2 = z2 * wy_0;
+          const float a1 = z1 * wx_2;
+          t0 += (dhw * a2) * (a1 * (QY(G, -1, 1) - QY(G, -1, 0) - QY(G1, -1, 0)) +
                                             a2 * (QY(G, 0, 0) - QY(G, -1, 0) - QY(G2, -1, 0)));
         }
       }
       {
-        const float uij_1 = (w < W - 1) ? (QY(Y1, -1, 1) - QY(Y1, -1, 0)) : 0.f;
-        const float uij_2 = (QY(Y1, 0, 0) - QY(Y1, -1, 0));
-        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTX;
-        float W_TIJ, dW_TIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(B);
-          W_TIJ = huber_w_end(hub, kD1);
-          active = hub > kD1;
-          dW_TIJ = W_TIJ / (hub * hub);
-        } else {
-          const float hub = rsq(B);
-          W_TIJ = fminf(1.f, hub * kD1);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ * (hub * hub);
-        }
-        df_dy1_t -= betaTX * oneL * W_TIJ * (df_dy1 - QY(G1, -1, 0));
+        const float u1 = (w < W - 1) ? (QY(Y1, -1, 1) - QY(Y1, -1, 0)) : 0.f;
+        const float u2 = (QY(Y1, 0, 0) - QY(Y1, -1, 0));
+        const float B = (u1 * u1 + u2 * u2) * beta1;
+        const float hub = rsq(B), hw = fminf(1.f, hub * kD1), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        t1 -= beta1 * hw * (g1 - QY(G1, -1, 0));
         if (active)
-          df_dy1_t += betaTX * oneL * (dW_TIJ * betaTX * uij_2) * (uij_1 * (QY(G1, -1, 1) - QY(G1, -1, 0)) +
-                                                                  uij_2 * (QY(G1, 0, 0) - QY(G1, -1, 0)));
+          t1 += beta1 * (dhw * beta1 * u2) * (u1 * (QY(G1, -1, 1) - QY(G1, -1, 0)) +
+                                                                  u2 * (QY(G1, 0, 0) - QY(G1, -1, 0)));
       }
       {
-        const float uij_1 = (w < W - 1) ? (QY(Y2, -1, 1) - QY(Y2, -1, 0)) : 0.f;
-        const float uij_2 = (QY(Y2, 0, 0) - QY(Y2, -1, 0));
-        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTY;
-        float W_TIJ, dW_TIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(B);
-          W_TIJ = huber_w_end(hub, kD2);
-          active = hub > kD2;
-          dW_TIJ = W_TIJ / (hub * hub);
-        } else {
-          const float hub = rsq(B);
-          W_TIJ = fminf(1.f, hub * kD2);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = JT0 ? W_TIJ * (hub * hub) : W_TIJ / (hub * hub);  // TGV.cu:355: a division where every sibling block multiplies
-        }
-        df_dy2_t -= betaTY * oneL * W_TIJ * (df_dy2 - QY(G2, -1, 0));
+        const float u1 = (w < W - 1) ? (QY(Y2, -1, 1) - QY(Y2, -1, 0)) : 0.f;
+        const float u2 = (QY(Y2, 0, 0) - QY(Y2, -1, 0));
+        const float B = (u1 * u1 + u2 * u2) * beta2;
+        const float hub = rsq(B), hw = fminf(1.f, hub * kD2), dhw = hw * (hub * hub);  // (the reference divides here, TGV.cu:355, where every sibling block multiplies)
+        const bool active = hw < 1.0f;
+        t2 -= beta2 * hw * (g2 - QY(G2, -1, 0));
         if (active)
-          df_dy2_t += betaTY * oneL * (dW_TIJ * betaTY * uij_2) * (uij_1 * (QY(G2, -1, 1) - QY(G2, -1, 0)) +
-                                                                  uij_2 * (QY(G2, 0, 0) - QY(G2, -1, 0)));
+          t2 += beta2 * (dhw * beta2 * u2) * (u1 * (QY(G2, -1, 1) - QY(G2, -1, 0)) +
+                                                                  u2 * (QY(G2, 0, 0) - QY(G2, -1, 0)));
       }
     }
     if (w > 0) {  // triangles owned by the pixel to the left: TGV.cu:361-418 / 1172-1227
-      const float betaTX = bX_l, betaTY = bY_l;
+      const float beta1 = b1l, beta2 = b2l;
       {
-        const float zij_1 = (yk - QY(Y, 0, -1) - QY(Y1, 0, -1));
-        const float zij_2 = (h < H - 1) ? (QY(Y, 1, -1) - QY(Y, 0, -1) - QY(Y2, 0, -1)) : 0.f;
-        const float A = zij_2 * zij_2 * wy_2 + zij_1 * zij_1 * wx_0;
-        float W_TIJ, dW_TIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(A);
-          W_TIJ = huber_w_end(hub, kD0);
-          active = hub > kD0;
-          dW_TIJ = W_TIJ / (hub * hub);
-        } else {
-          const float hub = rsq(A);
-          W_TIJ = fminf(1.f, hub * kD0);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ * (hub * hub);
-        }
-        df_dy_t -= oneL * W_TIJ * ((df_dy - QY(G, 0, -1)) - QY(G1, 0, -1)) * wx_0;
+        const float z1 = (yk - QY(Y, 0, -1) - QY(Y1, 0, -1));
+        const float z2 = (h < H - 1) ? (QY(Y, 1, -1) - QY(Y, 0, -1) - QY(Y2, 0, -1)) : 0.f;
+        const float A = z2 * z2 * wy_2 + z1 * z1 * wx_0;
+        const float hub = rsq(A), hw = fminf(1.f, hub * kD0), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        t0 -= hw * ((g0 - QY(G, 0, -1)) - QY(G1, 0, -1)) * wx_0;
         if (active) {
-          const float a1 = zij_1 * wx_0;
-          const float a2 = zij_2 * wy_2;
-          df_dy_t += oneL * (dW_TIJ * a1) * (a1 * (QY(G, 0, 0) - QY(G, 0, -1) - QY(G1, 0, -1)) +
+          const float a1 = z1 * wx_0;
+          const float a2 = z2 * wy_2;
+          t0 += (dhw * a1) * (a1 * (QY(G, 0, 0) - QY(G, 0, -1) - QY(G1, 0, -1)) +
                                             a2 * (QY(G, 1, -1) - QY(G, 0, -1) - QY(G2, 0, -1)));
         }
       }
       {
-        const float uij_1 = (QY(Y1, 0, 0) - QY(Y1, 0, -1));
-        const float uij_2 = (h < H - 1) ? (QY(Y1, 1, -1) - QY(Y1, 0, -1)) : 0.f;
-        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTX;
-        float W_TIJ, dW_TIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(B);
-          W_TIJ = huber_w_end(hub, kD1);
-          active = hub > kD1;
-          dW_TIJ = W_TIJ / (hub * hub);
-        } else {
-          const float hub = rsq(B);
-          W_TIJ = fminf(1.f, hub * kD1);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ * (hub * hub);
-        }
-        df_dy1_t -= betaTX * oneL * W_TIJ * (df_dy1 - QY(G1, 0, -1));
+        const float u1 = (QY(Y1, 0, 0) - QY(Y1, 0, -1));
+        const float u2 = (h < H - 1) ? (QY(Y1, 1, -1) - QY(Y1, 0, -1)) : 0.f;
+        const float B = (u1 * u1 + u2 * u2) * beta1;
+        const float hub = rsq(B), hw = fminf(1.f, hub * kD1), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        t1 -= beta1 * hw * (g1 - QY(G1, 0, -1));
         if (active)
-          df_dy1_t += betaTX * oneL * (dW_TIJ * betaTX * uij_1) * (uij_2 * (QY(G1, 1, -1) - QY(G1, 0, -1)) +
-                                                                  uij_1 * (QY(G1, 0, 0) - QY(G1, 0, -1)));
+          t1 += beta1 * (dhw * beta1 * u1) * (u2 * (QY(G1, 1, -1) - QY(G1, 0, -1)) +
+                                                                  u1 * (QY(G1, 0, 0) - QY(G1, 0, -1)));
       }
       {
-        const float uij_1 = (QY(Y2, 0, 0) - QY(Y2, 0, -1));
-        const float uij_2 = (h < H - 1) ? (QY(Y2, 1, -1) - QY(Y2, 0, -1)) : 0.f;
-        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTY;
-        float W_TIJ, dW_TIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(B);
-          W_TIJ = huber_w_end(hub, kD2);
-          active = hub > kD2;
-          dW_TIJ = W_TIJ / (hub * hub);
-        } else {
-          const float hub = rsq(B);
-          W_TIJ = fminf(1.f, hub * kD2);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ * (hub * hub);
-        }
-        df_dy2_t -= betaTY * oneL * W_TIJ * (df_dy2 - QY(G2, 0, -1));
+        const float u1 = (QY(Y2, 0, 0) - QY(Y2, 0, -1));
+        const float u2 = (h < H - 1) ? (QY(Y2, 1, -1) - QY(Y2, 0, -1)) : 0.f;
+        const float B = (u1 * u1 + u2 * u2) * beta2;
+        const float hub = rsq(B), hw = fminf(1.f, hub * kD2), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        t2 -= beta2 * hw * (g2 - QY(G2, 0, -1));
         if (active)
-          df_dy2_t += betaTY * oneL * (dW_TIJ * betaTY * uij_1) * (uij_2 * (QY(G2, 1, -1) - QY(G2, 0, -1)) +
-                                                                  uij_1 * (QY(G2, 0, 0) - QY(G2, 0, -1)));
+          t2 += beta2 * (dhw * beta2 * u1) * (u2 * (QY(G2, 1, -1) - QY(G2, 0, -1)) +
+                                                                  u1 * (QY(G2, 0, 0) - QY(G2, 0, -1)));
       }
     }
     {  // the pixel's own triangles: TGV.cu:419-507 / 1228-1333
-      const float betaTX = bX_c, betaTY = bY_c;
+      const float beta1 = b1c, beta2 = b2c;
       {
-        const float aij_1 = (w < W - 1) ? ((QY(Y, 0, 1) - QY(Y, 0, 0)) - QY(Y1, 0, 0)) : 0.f;
-        const float aij_2 = (h < H - 1) ? ((QY(Y, 1, 0) - QY(Y, 0, 0)) - QY(Y2, 0, 0)) : 0.f;
-        const float A = aij_2 * aij_2 * wy_1 + aij_1 * aij_1 * wx_1;
+        const float z1 = (w < W - 1) ? ((QY(Y, 0, 1) - QY(Y, 0, 0)) - QY(Y1, 0, 0)) : 0.f;
+        const float z2 = (h < H - 1) ? ((QY(Y, 1, 0) - QY(Y, 0, 0)) - QY(Y2, 0, 0)) : 0.f;
+        const float A = z2 * z2 * wy_1 + z1 * z1 * wx_1;
         const float gr = QY(G, 0, 1), gd = QY(G, 1, 0);
-        float W_TIJ, dW_TIJ, dyij_1, dyij_2;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(A);
-          W_TIJ = huber_w_end(hub, kD0);
-          active = hub > kD0;
-          dW_TIJ = W_TIJ / (hub * hub);
-          dyij_1 = df_dy - gr + df_dy1;
-          dyij_2 = df_dy - gd + df_dy2;
-          df_dy_t -= oneL * ((df_dy - gd) + df_dy2) * wy_1 * W_TIJ;
-          df_dy_t -= oneL * ((df_dy - gr) + df_dy1) * wx_1 * W_TIJ;
-          df_dy1_t -= oneL * W_TIJ * (df_dy1 - gr + df_dy) * wx_1;
-          df_dy2_t -= oneL * W_TIJ * (df_dy2 - gd + df_dy) * wy_1;
-          gwx0 = gwx0 + oneL * gxm * dyij_1 * aij_1 * W_TIJ;
-          gwy0 = gwy0 + oneL * gxm * dyij_2 * aij_2 * W_TIJ;
-        } else {
-          const float hub = rsq(A);
-          W_TIJ = fminf(1.f, hub * kD0);
-          active = W_TIJ < 1.0f;
-          dW_TIJ = W_TIJ * (hub * hub);
-          dyij_1 = df_dy - gr + df_dy1;
-          dyij_2 = df_dy - gd + df_dy2;
-          df_dy_t -= oneL * W_TIJ * (dyij_2 * wy_1 + dyij_1 * wx_1);
-          df_dy1_t -= oneL * W_TIJ * dyij_1 * wx_1;
-          df_dy2_t -= oneL * W_TIJ * dyij_2 * wy_1;
-          gwx0 = gwx0 + oneL * gxm * dyij_1 * (aij_1 * W_TIJ);
-          gwy0 = gwy0 + oneL * gxm * dyij_2 * (aij_2 * W_TIJ);
-        }
+        const float hub = rsq(A), hw = fminf(1.f, hub * kD0), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        const float dz1 = g0 - gr + g1, dz2 = g0 - gd + g2;
+        t0 -= hw * (dz2 * wy_1 + dz1 * wx_1);
+        t1 -= hw * dz1 * wx_1;
+        t2 -= hw * dz2 * wy_1;
+        gwx0 = gwx0 + dz1 * (z1 * hw);
+        gwy0 = gwy0 + dz2 * (z2 * hw);
         if (active) {
-          const float a1 = aij_1 * wx_1;
-          const float a2 = aij_2 * wy_1;
-          const float deriv_Tij = (dyij_1 * a1 + dyij_2 * a2) * oneL;
-          df_dy_t += deriv_Tij * ((a1 + a2) * dW_TIJ);
-          df_dy2_t += deriv_Tij * (a2 * dW_TIJ);
-          df_dy1_t += deriv_Tij * (a1 * dW_TIJ);
+          const float a1 = z1 * wx_1;
+          const float a2 = z2 * wy_1;
+          const float dot = (dz1 * a1 + dz2 * a2);
+          t0 += dot * ((a1 + a2) * dhw);
+          t2 += dot * (a2 * dhw);
+          t1 += dot * (a1 * dhw);
           // the literal 0.5 makes these two updates double (TGV.cu:452-453)
-          gwy0 = (float)((double)gwy0 - (double)(gxm * (aij_2 * dW_TIJ * aij_2)) * 0.5 * (double)deriv_Tij);
-          gwx0 = (float)((double)gwx0 - (double)(gxm * (aij_1 * dW_TIJ * aij_1)) * 0.5 * (double)deriv_Tij);
+          gwy0 = (float)((double)gwy0 - (double)((z2 * dhw * z2)) * 0.5 * (double)dot);
+          gwx0 = (float)((double)gwx0 - (double)((z1 * dhw * z1)) * 0.5 * (double)dot);
         }
       }
       {
-        const float uij_1 = (w < W - 1) ? (QY(Y1, 0, 1) - QY(Y1, 0, 0)) : 0.f;
-        const float uij_2 = (h < H - 1) ? (QY(Y1, 1, 0) - QY(Y1, 0, 0)) : 0.f;
-        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTX;
+        const float u1 = (w < W - 1) ? (QY(Y1, 0, 1) - QY(Y1, 0, 0)) : 0.f;
+        const float u2 = (h < H - 1) ? (QY(Y1, 1, 0) - QY(Y1, 0, 0)) : 0.f;
+        const float B = (u1 * u1 + u2 * u2) * beta1;
         const float gr = QY(G1, 0, 1), gd = QY(G1, 1, 0);
-        float W_YIJ, dW_YIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(B);
-          W_YIJ = huber_w_end(hub, kD1);
-          active = hub > kD1;
-          dW_YIJ = W_YIJ / (hub * hub);
-          if (h < H - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gd);  // TGV.cu:1271-1274: y first
-          if (w < W - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gr);
-        } else {
-          const float hub = rsq(B);
-          W_YIJ = fminf(1.f, hub * kD1);
-          active = W_YIJ < 1.0f;
-          dW_YIJ = W_YIJ * (hub * hub);
-          if (w < W - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gr);
-          if (h < H - 1) df_dy1_t -= betaTX * oneL * W_YIJ * (df_dy1 - gd);
-        }
-        gwx1 = gwx1 + oneL * gxm * ((df_dy1 - gr) * uij_1 + (df_dy1 - gd) * uij_2) * W_YIJ;
+        const float hub = rsq(B), hw = fminf(1.f, hub * kD1), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        if (w < W - 1) t1 -= beta1 * hw * (g1 - gr);
+        if (h < H - 1) t1 -= beta1 * hw * (g1 - gd);
+        gwx1 = gwx1 + ((g1 - gr) * u1 + (g1 - gd) * u2) * hw;
         if (active) {
-          const float deriv_Yij = ((df_dy1 - gr) * uij_1 * betaTX + (df_dy1 - gd) * uij_2 * betaTX) * oneL;
-          df_dy1_t += betaTX * dW_YIJ * (uij_1 + uij_2) * deriv_Yij;
+          const float dot = ((g1 - gr) * u1 * beta1 + (g1 - gd) * u2 * beta1);
+          t1 += beta1 * dhw * (u1 + u2) * dot;
           gwx1 = (float)((double)gwx1 -
-                         (double)(gxm * (uij_2 * dW_YIJ * uij_2 + uij_1 * dW_YIJ * uij_1)) * 0.5 * (double)deriv_Yij);
+                         (double)((u2 * dhw * u2 + u1 * dhw * u1)) * 0.5 * (double)dot);
         }
       }
       {
-        const float uij_1 = (w < W - 1) ? (QY(Y2, 0, 1) - QY(Y2, 0, 0)) : 0.f;
-        const float uij_2 = (h < H - 1) ? (QY(Y2, 1, 0) - QY(Y2, 0, 0)) : 0.f;
-        const float B = (uij_1 * uij_1 + uij_2 * uij_2) * betaTY;
+        const float u1 = (w < W - 1) ? (QY(Y2, 0, 1) - QY(Y2, 0, 0)) : 0.f;
+        const float u2 = (h < H - 1) ? (QY(Y2, 1, 0) - QY(Y2, 0, 0)) : 0.f;
+        const float B = (u1 * u1 + u2 * u2) * beta2;
         const float gr = QY(G2, 0, 1), gd = QY(G2, 1, 0);
-        float W_YIJ, dW_YIJ;
-        bool active;
-        if (END) {
-          const float hub = sqrtf(B);
-          W_YIJ = huber_w_end(hub, kD2);
-          active = hub > kD2;
-          dW_YIJ = W_YIJ / (hub * hub);
-        } else {
-          const float hub = rsq(B);
-          W_YIJ = fminf(1.f, hub * kD2);
-          active = W_YIJ < 1.0f;
-          dW_YIJ = W_YIJ * (hub * hub);
-        }
-        if (w < W - 1) df_dy2_t -= betaTY * oneL * W_YIJ * (df_dy2 - gr);
-        if (h < H - 1) df_dy2_t -= betaTY * oneL * W_YIJ * (df_dy2 - gd);
-        gwy1 = gwy1 + oneL * gxm * ((df_dy2 - gr) * uij_1 + (df_dy2 - gd) * uij_2) * W_YIJ;
+        const float hub = rsq(B), hw = fminf(1.f, hub * kD2), dhw = hw * (hub * hub);
+        const bool active = hw < 1.0f;
+        if (w < W - 1) t2 -= beta2 * hw * (g2 - gr);
+        if (h < H - 1) t2 -= beta2 * hw * (g2 - gd);
+        gwy1 = gwy1 + ((g2 - gr) * u1 + (g2 - gd) * u2) * hw;
         if (active) {
-          const float deriv_Yij = ((df_dy2 - gr) * uij_1 * betaTY + (df_dy2 - gd) * uij_2 * betaTY) * oneL;
-          df_dy2_t += betaTY * dW_YIJ * (uij_1 + uij_2) * deriv_Yij;
+          const float dot = ((g2 - gr) * u1 * beta2 + (g2 - gd) * u2 * beta2);
+          t2 += beta2 * dhw * (u1 + u2) * dot;
           gwy1 = (float)((double)gwy1 -
-                         (double)(gxm * (uij_2 * dW_YIJ * uij_2 + uij_1 * dW_YIJ * uij_1)) * 0.5 * (double)deriv_Yij);
+                         (double)((u2 * dhw * u2 + u1 * dhw * u1)) * 0.5 * (double)dot);
         }
       }
     }
 #undef QY
-    // aux variables: momentum adjoint only (TGV.cu:560-577 / 1383-1399); the literal 1. makes the
-    // product double
+    // J^T g05[0] plus the partial g_x[0]: the gradient wrt the starting point, all three variables
     const size_t q = o + p;
-    if (JT0) {
-      g05_out_[q] = df_dy_t + gxk_[q];
-      g05_out_[q + CHW] = df_dy1_t + gxk_[q + CHW];
-      g05_out_[q + 2 * CHW] = df_dy2_t + gxk_[q + 2 * CHW];
-      continue;
-    }
-    gxk_m1_[q + CHW] = -t * df_dy1_t;
-    df_dy1_t = (float)((double)gxk_[q + CHW] + (1. + (double)t) * (double)df_dy1_t);
-    df_dy1_t = fmaxf(-kClipLocalGrad, fminf(df_dy1_t, kClipLocalGrad));
-    g05_out_[q + CHW] = df_dy1_t;
-    gxk_[q + CHW] = df_dy1_t;
-    gxk_m1_[q + 2 * CHW] = -t * df_dy2_t;
-    df_dy2_t = (float)((double)gxk_[q + 2 * CHW] + (1. + (double)t) * (double)df_dy2_t);
-    df_dy2_t = fmaxf(-kClipLocalGrad, fminf(df_dy2_t, kClipLocalGrad));
-    g05_out_[q + 2 * CHW] = df_dy2_t;
-    gxk_[q + 2 * CHW] = df_dy2_t;
-    // u (TGV.cu:579-612 / 1403-1442)
-    float df_dxk = (float)((double)gxk_[q] + (1. + (double)t) * (double)df_dy_t);
-    df_dxk = fmaxf(-kClipLocalGrad, fminf(df_dxk, kClipLocalGrad));
-    gxk_[q] = df_dxk;
-    gxk_m1_[q] = -t * df_dy_t;
-    const size_t qb = smp * CHW + (size_t)ch * HW + p;
-    float g05v, gbv = gb_[qb];
-    prox_adjoint<false>(df_dxk, b_[qb], x05_[q], conf, g05v, gcv, gbv);
-    g05_out_[q] = g05v;
-    gb_[qb] = gbv;
+    gi_[q] = t0 + gx0_[q];
+    gi_[q + CHW] = t1 + gx0_[q + CHW];
+    gi_[q + 2 * CHW] = t2 + gx0_[q + 2 * CHW];
   }
-  if (!JT0) gc_[smp * HW + p] = gcv;
   gwx_[smp * 2 * HW + p] = gwx0;
   gwx_[smp * 2 * HW + HW + p] = gwx1;
   gwy_[smp * 2 * HW + p] = gwy0;
@@ -782,7 +496,7 @@ struct Slot {
   unsigned int* maxbits = nullptr;                                   // per-sample Lipschitz bound (float bits)
   unsigned int* counts = nullptr;                                    // upstream check
   float *ypp[2] = {nullptr, nullptr}, *xpp[2] = {nullptr, nullptr}, *ckpt_y = nullptr, *ckpt_x = nullptr, *x05 = nullptr;
-  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr}, *yk = nullptr, *gi_u = nullptr, *gx_final = nullptr;
+  float *g05[2] = {nullptr, nullptr}, *gxk[2] = {nullptr, nullptr}, *gi_u = nullptr, *gx_final = nullptr;
   // per-segment fp32 accumulators, double-buffered: a strip-kernel step reads one set and writes the other
   float *acc_gc[2] = {nullptr, nullptr}, *acc_gx[2] = {nullptr, nullptr}, *acc_gy[2] = {nullptr, nullptr},
         *acc_gb[2] = {nullptr, nullptr};
@@ -842,7 +556,7 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   s.ring_rows = ring_rows;
   const size_t nck = std::max<size_t>(s.iterations.size(), 1), ring = (size_t)ring_rows;
   size_t need = 0;
-  need += Arena::padded(S3, 4) * (2 + 2 + 2 + 2 + 1 + 1) + Arena::padded(S3 * nck, 4) * 2 + Arena::padded(S3 * ring, 4);
+  need += Arena::padded(S3, 4) * (2 + 2 + 2 + 2 + 1) + Arena::padded(S3 * nck, 4) * 2 + Arena::padded(S3 * ring, 4);
   need += Arena::padded(F, 4) * 3 + Arena::padded(F, 8);
   need += Arena::padded(P, 4) * (4 + 2) + Arena::padded(2 * P, 4) * 4;
   need += Arena::padded(P, 8) + Arena::padded(2 * P, 8) * 2;
@@ -863,7 +577,6 @@ int prepare_slot(Slot& s, int n, int ic, int ih, int iw, int its, int keep_mode,
   s.x05 = a.take<float>(S3 * ring);
   s.g05[0] = a.take<float>(S3); s.g05[1] = a.take<float>(S3);
   s.gxk[0] = a.take<float>(S3); s.gxk[1] = a.take<float>(S3);
-  s.yk = a.take<float>(S3);
   s.gx_final = a.take<float>(S3);
   s.gi_u = a.take<float>(F);
   for (int i = 0; i < 2; i++) {
@@ -905,7 +618,7 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
     if (!ptrs[i]) return fail(INPAINT_ERR_ARG, "null pointer argument (position %d)", i);
   if (n < 1 || ic < 1 || ih < 1 || iw < 1 || its < 0)
     return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
-  if (n > 65535 || (ih + BY - 1) / BY > 65535)
+  if (n > 65535 || (ih + BY - 1) / BY > 65535)  // (the Lipschitz and iteration-0 kernels put rows / BY and n on the grid)
     return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
   if ((long long)ih * iw >= (1ll << 29))  // the strip kernels address two planes of a tensor with one 32-bit byte offset
     return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^29", (long long)ih * iw);
@@ -927,10 +640,14 @@ void scale_weights(const Slot& s, hipStream_t stream, const float* dx, const flo
 }
 
 // -------------------------------------------------------------------------------------------------
-// kernel selection: wave-strip kernels for 1..2 flow channels, the per-pixel kernels otherwise.
-// INPAINT_TGV_PATH=px forces the per-pixel kernels (used by the tests to keep both paths covered).
+// kernel selection: the wave-strip kernels.  INPAINT_TGV_PATH=px used to select the one-pixel-per-thread kernels
+// written first; they are no longer built, and the setting is refused.
 // -------------------------------------------------------------------------------------------------
-bool use_strip(const Slot& s) { return !knobs().tgv_px_path && s.ic >= 1; }
+int refuse_removed_path() {
+  if (knobs().tgv_px_path)
+    return fail(INPAINT_ERR_ARG, "INPAINT_TGV_PATH=px names the per-pixel kernels, which this library no longer contains; unset it (INPAINT_TGV_FUSE=0 selects the one-iteration strip kernels)");
+  return 0;
+}
 
 // Channel groups: the strip kernels are instantiated for one and two flow channels.  More channels run as consecutive
 // launches over groups of two, each getting the per-channel tensors already moved to its first channel and the
@@ -990,18 +707,12 @@ void launch_forward_strip(const Slot& s, hipStream_t stream, const float* c, con
 
 void launch_forward(const Slot& s, hipStream_t stream, const float* c, const float* b, const float* xin, float* xout,
                     const float* yin, float* yout, float* x05, float t) {
-  if (use_strip(s)) {
-    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
-      const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
-      float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *gh = at_channel(s, x05, ch0);
-      if (s.ic - ch0 == 1) launch_forward_strip<1>(s, stream, c, gb, gxi, gxo, gyi, gyo, gh, t);
-      else launch_forward_strip<2>(s, stream, c, gb, gxi, gxo, gyi, gyo, gh, t);
-    }
-    return;
+  for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+    const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
+    float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *gh = at_channel(s, x05, ch0);
+    if (s.ic - ch0 == 1) launch_forward_strip<1>(s, stream, c, gb, gxi, gxo, gyi, gyo, gh, t);
+    else launch_forward_strip<2>(s, stream, c, gb, gxi, gxo, gyi, gyo, gh, t);
   }
-  const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
-  hipLaunchKernelGGL(tgv_forward_px, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xin, xout, yin, yout, x05,
-                     s.ic, s.ih, s.iw, t);
 }
 
 // Two forward iterations in one launch (strip path): (xin, yin) = iterate k, (xout, yout) = iterate k+2;
@@ -1034,8 +745,7 @@ bool forward_split_channels(const Slot& s) {
 }
 
 bool forward_pairs(const Slot& s) {
-  if (!knobs().tgv_fuse) return false;
-  return use_strip(s);
+  return knobs().tgv_fuse;
 }
 
 // xin_aux (optional): where v1, v2 of the input iterate are read from instead of xin; store_x_aux: write v1, v2 of xout.
@@ -1097,35 +807,19 @@ void launch_adjoint_first_two(Slot& s, hipStream_t stream, const float* c, const
   s.accb_cur = 1 - s.accb_cur;
 }
 
-// One adjoint step.  Strip path: y is rebuilt inside the kernel from xa = x05[k], xb = x05[k-1] (END:
-// read from the checkpoint yck); accumulator set acc_cur is read, the other one written, then
-// acc_cur flips; g_x is stored (to gx_final) only when asked.  Per-pixel path: y comes from the yk
-// buffer (or yck), accumulators and g_x are updated in place.
-// ADJ > 0 (strip path only, the caller checks): the corrected gradient; ADJ == 2: xb is the checkpointed x.
+// One adjoint step: y is rebuilt inside the kernel from xa = x05[k], xb = x05[k-1] (END: read from the checkpoint yck);
+// accumulator set acc_cur is read, the other one written, then acc_cur flips; g_x is stored (to gx_final) only when
+// asked.  ADJ > 0: the corrected gradient; ADJ == 2: xb is the checkpointed x.
 template <bool END, int ADJ = 0>
 void launch_adjoint(Slot& s, hipStream_t stream, const float* c, const float* b, const float* xa, const float* xb,
                     const float* yck, const float* g05_in, float* g05_out, float* gxk, float* gxk_m1, float* gx_final,
                     float t) {
-  if (use_strip(s)) {
-    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
-      if (s.ic - ch0 == 1) launch_adjoint_strip<1, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0);
-      else launch_adjoint_strip<2, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0);
-      s.acc_cur = 1 - s.acc_cur;
-    }
-    s.accb_cur = 1 - s.accb_cur;
-    return;
+  for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+    if (s.ic - ch0 == 1) launch_adjoint_strip<1, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0);
+    else launch_adjoint_strip<2, END, ADJ>(s, stream, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0);
+    s.acc_cur = 1 - s.acc_cur;
   }
-  const float* y = yck;
-  if (!END) {
-    const long long P = (long long)plane_count(s);
-    hipLaunchKernelGGL(tgv_getyk_kernel, dim3(grid1d(P)), dim3(256), 0, stream, c, b, xa, xb, s.yk, s.ic,
-                       (long long)s.ih * s.iw, P, t);
-    y = s.yk;
-  }
-  const int a = s.acc_cur;  // (the per-pixel kernels update their accumulators in place: both indices stay put)
-  const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
-  hipLaunchKernelGGL(tgv_adjoint_px<END>, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, xa, s.acc_gc[a],
-                     s.acc_gb[s.accb_cur], s.acc_gx[a], s.acc_gy[a], g05_in, g05_out, gxk, gxk_m1, y, s.ic, s.ih, s.iw, t);
+  s.accb_cur = 1 - s.accb_cur;
 }
 
 // Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
@@ -1232,6 +926,8 @@ int tgvinpaint_forward(const float* dx, const float* dy, const float* c, const f
                        float* out, int n, int ic, int ih, int iw, int its, int id, void* stream_) {
   const void* ptrs[] = {dx, dy, c, b, init, out};
   int rc = check_common(ptrs, 6, n, ic, ih, iw, its, id);
+  if (rc) return rc;
+  rc = refuse_removed_path();
   if (rc) return rc;
   hipStream_t stream = (hipStream_t)stream_;
   Slot& s = g_slots[id];
@@ -1350,11 +1046,9 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   // so there the other mode could not be served at all):
   if (s.grad_mode != s.fwd_grad_mode)
     return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass: set it before the forward pass, or run the forward pass again", id);
-  if (corr && !use_strip(s))
-    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TGV_PATH=px is set)");
   s.stream = stream;
   const size_t S3 = state_count(s), F = field_count(s), P = plane_count(s);
-  const int gS = grid_stride((long long)S3), gF = grid_stride((long long)F), gP = grid_stride((long long)P),
+  const int gS = grid_stride((long long)S3), gF = grid_stride((long long)F),
             g2P = grid_stride((long long)(2 * P));
 
   // (the first of its launches also clears the two words of the upstream check)
@@ -1368,7 +1062,6 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
   // totals after the last segment, in the reference's order (TGV.cu:2944 flushes after every segment: same bits,
   // but the totals are not read and rewritten once per segment).
-  const bool seg_mode = use_strip(s);
   SegmentJobs sj;
   {
     float* segs[4] = {s.seg_gc, s.seg_gx, s.seg_gy, s.seg_gb};
@@ -1386,34 +1079,27 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
   // reading them, and every launch after it reads only what its predecessor wrote in full: nothing to clear.
   const bool corr_pairs_ok = !corr || pair_split(s.ic);
   const int nseg_all = (int)s.iterations.size();
-  const bool first_two = seg_mode && adjoint_pairs(s) && corr_pairs_ok && s.ic <= kGroup && knobs().tgv_fuse_first &&
+  const bool first_two = adjoint_pairs(s) && corr_pairs_ok && s.ic <= kGroup && knobs().tgv_fuse_first &&
                          nseg_all > 0 && 2 * ((its - s.iterations[nseg_all - 1]) / 2) >= 4;
   s.acc_cur = 0;
   s.accb_cur = 0;
   if (!first_two) {
     ZeroList z;
     int k = 0;
-    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.yk, s.gx_final}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
+    for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.gx_final}) { z.ptr[k] = p; z.bytes[k++] = (long long)S3 * 4; }
     z.ptr[k] = s.acc_gb[0]; z.bytes[k++] = (long long)F * 4;
     z.ptr[k] = s.acc_gc[0]; z.bytes[k++] = (long long)P * 4;
     z.ptr[k] = s.acc_gx[0]; z.bytes[k++] = (long long)P * 8;
     z.ptr[k] = s.acc_gy[0]; z.bytes[k++] = (long long)P * 8;
-    if (!seg_mode) {  // (the strip path writes every total when it adds up the segment records)
-      z.ptr[k] = s.tot_gc; z.bytes[k++] = (long long)P * 8;
-      z.ptr[k] = s.tot_gx; z.bytes[k++] = (long long)P * 16;
-      z.ptr[k] = s.tot_gy; z.bytes[k++] = (long long)P * 16;
-      z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
-    }
+    // (the totals need no clearing: every one of them is written when the segment records are added up)
     hipLaunchKernelGGL(fill_zero_many, dim3(gS, k), dim3(256), 0, stream, z);
   }
 
   // buffer roles of TGV.cu:2718-2736: g05[0]/g05[1] and gxk[0]/gxk[1] ping-pong with the parity of the
   // local iteration index (the copy of the upstream gradient into gxk[0], TGV.cu:2729, is overwritten
   // before it is read and is not made).
-  // The strip kernels store g_x only at the very last step (into gx_final); the per-pixel kernels
-  // keep it in gxk[1] as the reference does.
-  const bool strip = use_strip(s);
-  const float* gi_src = strip ? s.gx_final : s.gxk[1];
+  // The kernels store g_x only at the very last step (into gx_final).
+  const float* gi_src = s.gx_final;
   // the corrected gradient has a pair kernel in the two-wavefront form only
   const bool pairs = adjoint_pairs(s) && (!corr || pair_split(s.ic));
   int lastIt = its;
@@ -1548,11 +1234,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
       } else {
         // the very last step's g_x is the gradient wrt the starting point (TGV.cu:3047)
         launch_adjoint<true>(s, stream, c, b, xa, xa, cky, s.g05[1], s.g05[0], s.gxk[1], s.gxk[0],
-                             (strip && outer == 0) ? s.gx_final : nullptr, t);
+                             outer == 0 ? s.gx_final : nullptr, t);
       }
     }
     // fp32 segment sums into the fp64 totals (TGV.cu:2944)
-    if (!flushed && seg_mode) {
+    if (!flushed) {
       SegmentJobs st = sj;
       const int a = s.acc_cur;
       float* accs[4] = {s.acc_gc[a], s.acc_gx[a], s.acc_gy[a], s.acc_gb[s.accb_cur]};
@@ -1561,17 +1247,11 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
         st.seg[k] = sj.seg[k] + (size_t)outer * sj.n[k];
       }
       hipLaunchKernelGGL(segment_store_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, st);
-    } else if (!flushed) {
-      const int a = s.acc_cur;
-      hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[a], s.tot_gc, (long long)P);
-      hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
-      hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
-      hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[s.accb_cur], s.tot_gb, (long long)F);
     }
     lastIt = k0;
   }
 
-  if (seg_mode) hipLaunchKernelGGL(combine_segments_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, sj, nseg);
+  hipLaunchKernelGGL(combine_segments_many, dim3(g2P > gF ? g2P : gF, 4), dim3(256), 0, stream, sj, nseg);
   if (corr && 2 * (its / 2) > 0) {
     // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it).  The last
     // step above left g05[0] and the partial g_x[0] in the halves of the ping-pongs it wrote; checkpoint 0 is y_0; the
@@ -1579,9 +1259,8 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
     const int a = s.acc_cur;
     const dim3 block(BX, BY), grid((s.iw + BX - 1) / BX, (s.ih + BY - 1) / BY, s.n);
     const int last = pairs ? pp_src : 0;
-    hipLaunchKernelGGL((tgv_adjoint_px<false, true>), grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, c, b, s.ckpt_y,
-                       s.acc_gc[a], s.acc_gb[s.accb_cur], s.acc_gx[a], s.acc_gy[a], s.g05[last], s.gx_final, s.gxk[last],
-                       s.gxk[1 - last], s.ckpt_y, s.ic, s.ih, s.iw, 0.f);
+    hipLaunchKernelGGL(tgv_adjoint_iter0, grid, block, 0, stream, s.wx, s.wy, s.bx, s.by, s.ckpt_y, s.g05[last], s.gxk[last],
+                       s.gx_final, s.acc_gx[a], s.acc_gy[a], s.ic, s.ih, s.iw);
     hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gx[a], s.tot_gx, (long long)(2 * P));
     hipLaunchKernelGGL(flush_kernel, dim3(g2P), dim3(256), 0, stream, s.acc_gy[a], s.tot_gy, (long long)(2 * P));
   }
@@ -1622,6 +1301,15 @@ int tgvinpaint_backward(const float* dx, const float* dy, const float* c, const 
                        s.guard, kGuard);
   }
   INPAINT_HIP(hipGetLastError());
+  if (knobs().stats_every > 0) {  // TGV.cu:2996: run % 75 == 0, with the run count the reference would hold
+    unsigned int skipped = 0;
+    INPAINT_HIP(hipStreamSynchronize(stream));
+    INPAINT_HIP(hipMemcpy(&skipped, reinterpret_cast<char*>(s.guard) + offsetof(GuardState, skipped), sizeof(skipped), hipMemcpyDeviceToHost));
+    if ((s.run - (int)skipped) % knobs().stats_every == 0) {
+      rc = print_guard_report(s.guard, stream, id, true);
+      if (rc) return rc;
+    }
+  }
   s.run++;  // TGV.cu:3061 (a refused upstream gradient is counted on the device and taken off again: Slot::run)
   return 0;
 }

@@ -3,11 +3,11 @@
 // What the layer computes is fixed by the reference's kernels
 // (cudaTV/cudaCode/TVInpaintFista.cu, cited per function below as TV.cu).  How it is computed is not:
 //   * samples are a grid dimension (n >= 1), weights are scaled by L = 1/8 and masked at the image
-//     border when they are staged into LDS (no scaled copies, no textures);
+//     border when they are loaded (no scaled copies, no textures);
 //   * checkpoints, the x05 history, the adjoint iterates, the per-segment fp32 accumulators and
 //     their fp64 totals all live in one device arena per id, sized once per shape;
-//   * the y rebuild (get_yk) is fused into the adjoint kernel: y_{k+1} is rebuilt straight into
-//     the LDS tile, halo included, and never written to HBM;
+//   * the y rebuild (get_yk) is fused into the adjoint kernels: y_{k+1} is rebuilt in registers and
+//     never written to HBM;
 //   * the output guard runs on the device (two reductions, a one-thread decision, a finalize
 //     pass), so a backward call enqueues work and returns without a host synchronisation.
 //
@@ -28,146 +28,11 @@ using namespace inpaint;
 
 // TV.cu:44,52,63-69,84-90
 constexpr float kDelta = 0.1f;
-constexpr float kClipLocalGrad = 10000.0f;
 constexpr float kLocalGCMult = 0.1f;
-constexpr float kLocalGXMult = 0.1f;
 constexpr float kLocalGBMult = 1.0f;
 constexpr float kGlobalGMult = 0.1f;
 constexpr float kL = 0.125f;  // 1/Lipschitz, TV.cu:1478 (a power of two: scaling is exact)
 const GuardParams kGuard = {10000000., 0., 50., 10., 0.975};
-
-constexpr int TW = 64;   // tile width  = one wavefront along W
-constexpr int TH = 16;   // tile height
-constexpr int NTY = 4;   // thread rows; each thread owns TH/NTY pixels of one column
-constexpr int NT = TW * NTY;
-constexpr int RPT = TH / NTY;
-constexpr int YS = TW + 2;  // LDS row length of a haloed tile
-
-// -------------------------------------------------------------------------------------------------
-// device helpers
-// -------------------------------------------------------------------------------------------------
-
-// Masked, L-scaled edge weights of the tile whose first interior pixel is (h0, w0), staged with a
-// one-pixel top/left apron.  wxs[ly][lx] = wx(h0-1+ly, w0-1+lx)/8, forced to 0 outside the image and
-// in the last column (no right neighbour); wys likewise with the last row.  With these, the six
-// weights of TV.cu:1204-1211 are plain LDS reads.
-__device__ __forceinline__ void stage_weights(const float* __restrict__ wx, const float* __restrict__ wy,
-                                              float (*wxs)[TW + 1], float (*wys)[TW + 1], int h0, int w0,
-                                              int H, int W, int tid) {
-  for (int e = tid; e < (TH + 1) * (TW + 1); e += NT) {
-    const int ly = e / (TW + 1), lx = e - ly * (TW + 1);
-    const int gh = h0 - 1 + ly, gw = w0 - 1 + lx;
-    const bool in = gh >= 0 && gh < H && gw >= 0 && gw < W;
-    float a = 0.f, b = 0.f;
-    if (in) {
-      const size_t p = (size_t)gh * W + gw;
-      if (gw < W - 1) a = kL * wx[p];
-      if (gh < H - 1) b = kL * wy[p];
-    }
-    wxs[ly][lx] = a;
-    wys[ly][lx] = b;
-  }
-}
-
-// Zero-padded haloed tile of one channel plane (TV.cu:1221-1239).
-__device__ __forceinline__ void stage_plane(const float* __restrict__ f, float (*s)[YS], int h0, int w0,
-                                            int H, int W, int tid) {
-  for (int e = tid; e < (TH + 2) * YS; e += NT) {
-    const int ly = e / YS, lx = e - ly * YS;
-    const int gh = h0 - 1 + ly, gw = w0 - 1 + lx;
-    s[ly][lx] = (gh >= 0 && gh < H && gw >= 0 && gw < W) ? f[(size_t)gh * W + gw] : 0.f;
-  }
-}
-
-// y_{k+1} from x05[k] (xa), x05[k-1] (xb): TV.cu:1149-1165.
-__device__ __forceinline__ float rebuild_y(float bb, float xa, float xb, float conf, float t) {
-  float diff = bb - xa;
-  float sign = (diff < 0) ? -1.f : 1.f;
-  float yk;
-  if (1. + (double)conf >= (double)(sign * diff)) {
-    const float xk = (conf * bb + xa) / (1.f + conf);
-    const float xkm = (conf * bb + xb) / (1.f + conf);
-    yk = xk + t * (xk - xkm);
-  } else {
-    const float xk = (conf <= sign * diff) ? bb - diff + sign * conf : bb;
-    diff = bb - xb;
-    sign = (diff < 0) ? -1.f : 1.f;
-    yk = xk + t * (xk - ((conf <= sign * diff) ? bb - diff + sign * conf : bb));
-  }
-  return yk;
-}
-
-// -------------------------------------------------------------------------------------------------
-// forward iteration: TV.cu:1194-1319; with x05 != nullptr also TV.cu:1321-1455
-// -------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(NT) void tv_forward_iter(
-    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
-    const float* __restrict__ b, const float* xin, float* xout, const float* __restrict__ yin,
-    float* __restrict__ yout, float* __restrict__ x05, int C, int H, int W, float t) {
-  __shared__ float ys[TH + 2][YS];
-  __shared__ float wxs[TH + 1][TW + 1];
-  __shared__ float wys[TH + 1][TW + 1];
-  const int tid = threadIdx.y * TW + threadIdx.x;
-  const int w0 = blockIdx.x * TW, h0 = blockIdx.y * TH;
-  const size_t HW = (size_t)H * W;
-  const size_t sample = (size_t)blockIdx.z;
-  wx += sample * HW;
-  wy += sample * HW;
-  cf += sample * HW;
-  const size_t soff = sample * HW * C;
-  stage_weights(wx, wy, wxs, wys, h0, w0, H, W, tid);
-  const int lx = threadIdx.x, w = w0 + lx;
-  float conf[RPT];
-#pragma unroll
-  for (int r = 0; r < RPT; r++) {
-    const int h = h0 + threadIdx.y + r * NTY;
-    conf[r] = (h < H && w < W) ? cf[(size_t)h * W + w] : 0.f;
-  }
-  for (int ch = 0; ch < C; ch++) {
-    const size_t coff = soff + (size_t)ch * HW;
-    if (ch > 0) __syncthreads();
-    stage_plane(yin + coff, ys, h0, w0, H, W, tid);
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < RPT; r++) {
-      const int ly = threadIdx.y + r * NTY, h = h0 + ly;
-      if (h >= H || w >= W) continue;
-      const size_t q = coff + (size_t)h * W + w;
-      const float wx_0 = wxs[ly + 1][lx], wx_1 = wxs[ly + 1][lx + 1], wx_2 = wxs[ly][lx + 1];
-      const float wy_0 = wys[ly][lx + 1], wy_1 = wys[ly + 1][lx + 1], wy_2 = wys[ly + 1][lx];
-      const float x_ = xin[q];
-      const float bb = b[q];
-      float yc = ys[ly + 1][lx + 1];
-      float yt = yc;
-      if (h > 0) {
-        const float yu = ys[ly][lx + 1], yur = ys[ly][lx + 2];
-        const float hub = sqrtf((yc - yu) * (yc - yu) * wy_0 + (yu - yur) * (yu - yur) * wx_2);
-        yt -= (yc - yu) * (wy_0 / fmaxf(1.f, hub / kDelta));
-      }
-      if (w > 0) {
-        const float yl = ys[ly + 1][lx], yld = ys[ly + 2][lx];
-        const float hub = sqrtf((yc - yl) * (yc - yl) * wx_0 + (yl - yld) * (yl - yld) * wy_2);
-        yt -= (yc - yl) * (wx_0 / fmaxf(1.f, hub / kDelta));
-      }
-      {
-        const float yd = ys[ly + 2][lx + 1], yr = ys[ly + 1][lx + 2];
-        const float hub = sqrtf((yc - yd) * (yc - yd) * wy_1 + (yc - yr) * (yc - yr) * wx_1);
-        const float m = fmaxf(1.f, hub / kDelta);
-        yt -= (yc - yd) * (wy_1 / m);
-        yt -= (yc - yr) * (wx_1 / m);
-      }
-      if (x05) x05[q] = yt;
-      const float c = conf[r];
-      float x_loc = (c * bb + yt) / (1.f + c);
-      yc = yt - c;
-      yt = yt + c;
-      if (yc > 1.f + bb) x_loc = yc;
-      if (yt < bb - 1.f) x_loc = yt;
-      yout[q] = x_loc + t * (x_loc - x_);
-      xout[q] = x_loc;
-    }
-  }
-}
 
 // Prox adjoint + confidence / rhs gradient: TV.cu:806-828 (and 240-255 for the first step).
 // Only g05 continues down the chain; none of these values reaches a switch.
@@ -311,173 +176,6 @@ __global__ __launch_bounds__(256) void tv_adjoint_iter0(const float* __restrict_
   tot_gy[i] += (double)gwy;
 }
 
-// Main adjoint step with the y rebuild fused in: TV.cu:586-859 (+1130-1189), and, with END, the
-// segment-start variant TV.cu:862-1126 that linearises at the checkpoint y.
-template <bool END>
-__global__ __launch_bounds__(NT) void tv_adjoint_iter(
-    const float* __restrict__ wx, const float* __restrict__ wy, const float* __restrict__ cf,
-    const float* __restrict__ b, const float* __restrict__ x05a, const float* __restrict__ x05b,
-    const float* __restrict__ yck, const float* gc_in, float* gc, const float* gb_in, float* gb,
-    const float* gwx_in, float* gwx, const float* gwy_in, float* gwy, const float* __restrict__ g05_in,
-    float* __restrict__ g05_out, const float* gxk, float* gxk_m1, float* gx_final, int C, int H, int W,
-    float t) {
-  __shared__ float ys[TH + 2][YS];
-  __shared__ float gs[TH + 2][YS];
-  __shared__ float wxs[TH + 1][TW + 1];
-  __shared__ float wys[TH + 1][TW + 1];
-  const int tid = threadIdx.y * TW + threadIdx.x;
-  const int w0 = blockIdx.x * TW, h0 = blockIdx.y * TH;
-  const size_t HW = (size_t)H * W;
-  const size_t sample = (size_t)blockIdx.z;
-  wx += sample * HW;
-  wy += sample * HW;
-  cf += sample * HW;
-  gc += sample * HW;
-  gwx += sample * HW;
-  gwy += sample * HW;
-  gc_in += sample * HW;
-  gwx_in += sample * HW;
-  gwy_in += sample * HW;
-  const size_t soff = sample * HW * C;
-  stage_weights(wx, wy, wxs, wys, h0, w0, H, W, tid);
-  const int lx = threadIdx.x, w = w0 + lx;
-  float conf[RPT], gcv[RPT], gwxv[RPT], gwyv[RPT];
-#pragma unroll
-  for (int r = 0; r < RPT; r++) {
-    const int h = h0 + threadIdx.y + r * NTY;
-    const bool in = h < H && w < W;
-    const size_t p = (size_t)h * W + w;
-    conf[r] = in ? cf[p] : 0.f;
-    gcv[r] = in ? gc_in[p] : 0.f;
-    gwxv[r] = in ? gwx_in[p] : 0.f;
-    gwyv[r] = in ? gwy_in[p] : 0.f;
-  }
-  for (int ch = 0; ch < C; ch++) {
-    const size_t coff = soff + (size_t)ch * HW;
-    if (ch > 0) __syncthreads();
-    if (END) {
-      stage_plane(yck + coff, ys, h0, w0, H, W, tid);
-    } else {
-      for (int e = tid; e < (TH + 2) * YS; e += NT) {
-        const int ly = e / YS, lxx = e - ly * YS;
-        const int gh = h0 - 1 + ly, gw = w0 - 1 + lxx;
-        float v = 0.f;
-        if (gh >= 0 && gh < H && gw >= 0 && gw < W) {
-          const size_t p = (size_t)gh * W + gw;
-          v = rebuild_y(b[coff + p], x05a[coff + p], x05b[coff + p], cf[p], t);
-        }
-        ys[ly][lxx] = v;
-      }
-    }
-    stage_plane(g05_in + coff, gs, h0, w0, H, W, tid);
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < RPT; r++) {
-      const int ly = threadIdx.y + r * NTY, h = h0 + ly;
-      if (h >= H || w >= W) continue;
-      const size_t q = coff + (size_t)h * W + w;
-      const float wx_0 = wxs[ly + 1][lx], wx_1 = wxs[ly + 1][lx + 1];
-      const float wy_0 = wys[ly][lx + 1], wy_1 = wys[ly + 1][lx + 1];
-      const float yk = ys[ly + 1][lx + 1];
-      const float df_dy = gs[ly + 1][lx + 1];
-      float df_dy_t = df_dy;
-      if (h > 0) {  // triangle owned by the pixel above, TV.cu:655-686
-        const float wx_2 = wxs[ly][lx + 1];
-        const float yu = ys[ly][lx + 1], yur = ys[ly][lx + 2];
-        const float gu = gs[ly][lx + 1], gur = gs[ly][lx + 2];
-        const float wy_nyy2 = (yk - yu) * (yk - yu) * wy_0;
-        const float wx_nyx2 = (yu - yur) * (yu - yur) * wx_2;
-        const float hub = sqrtf(wx_nyx2 + wy_nyy2);
-        if (hub > kDelta) {
-          const float nom = kDelta / hub;
-          const float denom = nom / (2.f * hub * hub);
-          df_dy_t -= (df_dy - gu) * (wy_0 * nom);
-          const float temp = -denom * 2.0f * (yk - yu) * wy_0;
-          df_dy_t -= (df_dy - gu) * wy_0 * (yk - yu) * temp;
-          df_dy_t -= (gur - gu) * wx_2 * (yur - yu) * temp;
-        } else {
-          df_dy_t -= (df_dy - gu) * wy_0;
-        }
-      }
-      if (w > 0) {  // triangle owned by the pixel to the left, TV.cu:687-720
-        const float wy_2 = wys[ly + 1][lx];
-        const float yl = ys[ly + 1][lx], yld = ys[ly + 2][lx];
-        const float gl = gs[ly + 1][lx], gld = gs[ly + 2][lx];
-        const float wx_nyx2 = (yk - yl) * (yk - yl) * wx_0;
-        const float wy_nyy2 = (yl - yld) * (yl - yld) * wy_2;
-        const float hub = sqrtf(wx_nyx2 + wy_nyy2);
-        if (hub > kDelta) {
-          const float nom = kDelta / hub;
-          const float denom = nom / (2.f * hub * hub);
-          df_dy_t -= (df_dy - gl) * (wx_0 * nom);
-          const float temp = -denom * 2.0f * (yk - yl) * wx_0;
-          df_dy_t -= (df_dy - gl) * wx_0 * (yk - yl) * temp;
-          df_dy_t -= (gld - gl) * wy_2 * (yld - yl) * temp;
-        } else {
-          df_dy_t -= (df_dy - gl) * wx_0;
-        }
-      }
-      {  // the pixel's own triangle, TV.cu:722-771
-        const float yr = ys[ly + 1][lx + 2], yd = ys[ly + 2][lx + 1];
-        const float gr = gs[ly + 1][lx + 2], gd = gs[ly + 2][lx + 1];
-        const float wx_nyx2 = (yk - yr) * (yk - yr) * wx_1;
-        const float wy_nyy2 = (yk - yd) * (yk - yd) * wy_1;
-        const float hub = sqrtf(wx_nyx2 + wy_nyy2);
-        if (hub > kDelta) {
-          const float nom = kDelta / hub;
-          const float denom = nom / (2.f * hub * hub);
-          df_dy_t -= (df_dy - gd) * (wy_1 * nom);
-          df_dy_t -= (df_dy - gr) * (wx_1 * nom);
-          const float temp = denom * 2.0f * ((yd - yk) * wy_1 + (yr - yk) * wx_1);
-          df_dy_t -= (df_dy - gd) * wy_1 * (yk - yd) * temp;
-          df_dy_t -= (df_dy - gr) * wx_1 * (yk - yr) * temp;
-          if (!END) {  // TV.cu:749-759
-            if (w < W - 1)
-              gwxv[r] = gwxv[r] - kLocalGXMult * (yk - yr) *
-                                      ((df_dy - gr) * (nom - wx_nyx2 * denom) -
-                                       (df_dy - gd) * (yk - yr) * (yk - yd) * denom * wy_1);
-            if (h < H - 1)
-              gwyv[r] = gwyv[r] - kLocalGXMult * (yk - yd) *
-                                      ((df_dy - gd) * (nom - wy_nyy2 * denom) -
-                                       (df_dy - gr) * (yk - yd) * (yk - yr) * denom * wx_1);
-          } else {  // TV.cu:1019-1027 (same algebra, other operand order)
-            if (w < W - 1)
-              gwxv[r] = gwxv[r] - kLocalGXMult * ((df_dy - gr) * (yk - yr) * (nom - wx_nyx2 * denom) -
-                                                  (df_dy - gd) * (yk - yr) * (yk - yr) * (yk - yd) * denom * wy_1);
-            if (h < H - 1)
-              gwyv[r] = gwyv[r] - kLocalGXMult * ((df_dy - gd) * (yk - yd) * (nom - wy_nyy2 * denom) -
-                                                  (df_dy - gr) * (yk - yd) * (yk - yd) * (yk - yr) * denom * wx_1);
-          }
-        } else {
-          df_dy_t -= (df_dy - gd) * wy_1;
-          df_dy_t -= (df_dy - gr) * wx_1;
-          if (w < W - 1) gwxv[r] = gwxv[r] - kLocalGXMult * (yk - yr) * (df_dy - gr);
-          if (h < H - 1) gwyv[r] = gwyv[r] - kLocalGXMult * (yk - yd) * (df_dy - gd);
-        }
-      }
-      // momentum adjoint, TV.cu:796-801 (the product is formed in double, as the literal 1. implies)
-      float df_dxk = (float)((double)gxk[q] + (1. + (double)t) * (double)df_dy_t);
-      df_dxk = fmaxf(-kClipLocalGrad, fminf(df_dxk, kClipLocalGrad));
-      if (gx_final) gx_final[q] = df_dxk;  // only the last step's g_x is ever read again (TV.cu:800,1785)
-      gxk_m1[q] = -t * df_dy_t;
-      float g05v, gbv = gb_in[q];
-      prox_adjoint<false>(df_dxk, b[q], x05a[q], conf[r], g05v, gcv[r], gbv);
-      g05_out[q] = g05v;
-      gb[q] = gbv;
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < RPT; r++) {
-    const int h = h0 + threadIdx.y + r * NTY;
-    if (h < H && w < W) {
-      const size_t p = (size_t)h * W + w;
-      gc[p] = gcv[r];
-      gwx[p] = gwxv[r];
-      gwy[p] = gwyv[r];
-    }
-  }
-}
-
 // -------------------------------------------------------------------------------------------------
 // per-id state (idStruct, TVInpaintFista.h:7-50)
 // -------------------------------------------------------------------------------------------------
@@ -607,8 +305,7 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
     if (!ptrs[i]) return fail(INPAINT_ERR_ARG, "null pointer argument (position %d)", i);
   if (n < 1 || ic < 1 || ih < 1 || iw < 1 || its < 0)
     return fail(INPAINT_ERR_ARG, "bad sizes n=%d ic=%d ih=%d iw=%d its=%d", n, ic, ih, iw, its);
-  if (n > 65535 || (ih + TH - 1) / TH > 65535)
-    return fail(INPAINT_ERR_ARG, "n=%d or ih=%d exceed the launch grid", n, ih);
+  if (n > 65535) return fail(INPAINT_ERR_ARG, "n=%d exceeds the launch grid", n);
   // the strip kernels address up to four planes of a tensor with one 32-bit byte offset from a common base pointer
   if ((long long)ih * iw * std::min(std::max(ic, 2), 4) >= (1ll << 30))
     return fail(INPAINT_ERR_ARG, "ih*iw = %lld pixels per plane exceed 2^29 (2^28 with more than 3 channels)", (long long)ih * iw);
@@ -618,10 +315,14 @@ int check_common(const void* const* ptrs, int nptrs, int n, int ic, int ih, int 
 }
 
 // -------------------------------------------------------------------------------------------------
-// kernel selection: the wave-strip kernels (more than 4 channels: in channel groups).
-// INPAINT_TV_PATH=tile forces the LDS-tile kernels written first (used by the tests as a second path).
+// kernel selection: the wave-strip kernels (more than 4 channels: in channel groups).  INPAINT_TV_PATH=tile used to
+// select the LDS-tile kernels written first; they are no longer built, and the setting is refused.
 // -------------------------------------------------------------------------------------------------
-bool force_tile_path() { return knobs().tv_tile_path; }
+int refuse_removed_path() {
+  if (knobs().tv_tile_path)
+    return fail(INPAINT_ERR_ARG, "INPAINT_TV_PATH=tile names the LDS-tile kernels, which this library no longer contains; unset it (INPAINT_TV_FUSE=0 selects the one-iteration strip kernels)");
+  return 0;
+}
 // The x05 rows the forward pass keeps.  INPAINT_KEEP=0|1|2 overrides the id's setting (INPAINT_KEEP_LAST=0 is the
 // older spelling of INPAINT_KEEP=0); keeping all rows needs its * field bytes, at most INPAINT_KEEP_GB (default 32).
 int resolve_keep_mode(const Slot& s, int n, int ic, int ih, int iw, int its) {
@@ -692,11 +393,8 @@ bool forward_split_channels(const Slot& s) {
   return sx * ((s.ih + 1) / 2) * s.n <= 8ll * compute_unit_count();  // strips of two rows: at most two wavefronts per SIMD
 }
 
-bool strip_path(const Slot& s) { return !force_tile_path() && s.ic >= 1; }
-
 bool forward_pairs(const Slot& s) {
-  if (!knobs().tv_fuse) return false;
-  return strip_path(s);
+  return knobs().tv_fuse;
 }
 
 // ring: xin / yin are the x05 rows of the two iterations before this pair and the iterate is rebuilt from them
@@ -726,21 +424,15 @@ void launch_forward_pair(const Slot& s, hipStream_t stream, const float* dx, con
 void launch_forward(const Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
                     const float* b, const float* xin, float* xout, const float* yin, float* yout, float* x05,
                     float t) {
-  if (strip_path(s)) {
-    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
-      const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
-      float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *gh = at_channel(s, x05, ch0);
-      switch (std::min(kGroup, s.ic - ch0)) {
-        case 1: launch_forward_strip<1>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
-        case 2: launch_forward_strip<2>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
-        case 3: launch_forward_strip<3>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
-        default: launch_forward_strip<4>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
-      }
+  for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+    const float *gb = at_channel(s, b, ch0), *gxi = at_channel(s, xin, ch0), *gyi = at_channel(s, yin, ch0);
+    float *gxo = at_channel(s, xout, ch0), *gyo = at_channel(s, yout, ch0), *gh = at_channel(s, x05, ch0);
+    switch (std::min(kGroup, s.ic - ch0)) {
+      case 1: launch_forward_strip<1>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+      case 2: launch_forward_strip<2>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+      case 3: launch_forward_strip<3>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
+      default: launch_forward_strip<4>(s, stream, dx, dy, c, gb, gxi, gxo, gyi, gyo, gh, t); break;
     }
-  } else {
-    const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
-    hipLaunchKernelGGL(tv_forward_iter, grid, block, 0, stream, dx, dy, c, b, xin, xout, yin, yout, x05, s.ic, s.ih,
-                       s.iw, t);
   }
 }
 
@@ -790,31 +482,20 @@ void launch_adjoint_first_two(Slot& s, hipStream_t stream, const float* dx, cons
 // TRUE_ADJ (strip path only, the caller checks): the corrected gradient; with END, yck is the checkpointed x.
 template <bool END, bool TRUE_ADJ = false>
 bool launch_adjoint(Slot& s, hipStream_t stream, const float* dx, const float* dy, const float* c,
-                    const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
-                    float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
-  const bool strip = strip_path(s);
-  if (strip) {
-    for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
-      const bool last = ch0 + kGroup >= s.ic;
-      switch (std::min(kGroup, s.ic - ch0)) {
-        case 1: launch_adjoint_strip<1, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
-        case 2: launch_adjoint_strip<2, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
-        case 3: launch_adjoint_strip<3, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
-        default: launch_adjoint_strip<4, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
-      }
-      s.acc_cur = 1 - s.acc_cur;
+                  const float* b, const float* xa, const float* xb, const float* yck, const float* g05_in,
+                  float* g05_out, const float* gxk, float* gxk_m1, float* gx_final, float t) {
+  for (int ch0 = 0; ch0 < s.ic; ch0 += kGroup) {
+    const bool last = ch0 + kGroup >= s.ic;
+    switch (std::min(kGroup, s.ic - ch0)) {
+      case 1: launch_adjoint_strip<1, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+      case 2: launch_adjoint_strip<2, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+      case 3: launch_adjoint_strip<3, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
+      default: launch_adjoint_strip<4, END, TRUE_ADJ>(s, stream, dx, dy, c, b, xa, xb, yck, g05_in, g05_out, gxk, gxk_m1, gx_final, t, ch0, last); break;
     }
-    s.accb_cur = 1 - s.accb_cur;
-  } else {
-    const dim3 block(TW, NTY), grid((s.iw + TW - 1) / TW, (s.ih + TH - 1) / TH, s.n);
-    const int i = s.acc_cur, o = 1 - s.acc_cur;
-    hipLaunchKernelGGL(tv_adjoint_iter<END>, grid, block, 0, stream, dx, dy, c, b, xa, xb, yck, s.acc_gc[i],
-                       s.acc_gc[o], s.acc_gb[i], s.acc_gb[o], s.acc_gx[i], s.acc_gx[o], s.acc_gy[i], s.acc_gy[o], g05_in,
-                       g05_out, gxk, gxk_m1, gx_final, s.ic, s.ih, s.iw, t);
     s.acc_cur = 1 - s.acc_cur;
-    s.accb_cur = s.acc_cur;
   }
-  return strip;
+  s.accb_cur = 1 - s.accb_cur;
+  return true;
 }
 
 // Two adjoint steps in one launch (strip path): A = local iteration j (x05 slots xa = j, xb = j-1), B = j-1
@@ -1013,6 +694,8 @@ int tvinpaint_forward(const float* dx, const float* dy, const float* c, const fl
   const void* ptrs[] = {dx, dy, c, b, init, out};
   int rc = check_common(ptrs, 6, n, ic, ih, iw, its, id);
   if (rc) return rc;
+  rc = refuse_removed_path();
+  if (rc) return rc;
   hipStream_t stream = (hipStream_t)stream_;
   Slot& s = g_slots[id];
   s.forward_done = false;
@@ -1196,18 +879,15 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   // so there the other mode could not be served at all):
   if (s.grad_mode != s.fwd_grad_mode)
     return fail(INPAINT_ERR_PAIRING, "the gradient mode of id %d was changed after its forward pass: set it before the forward pass, or run the forward pass again", id);
-  if (corr && force_tile_path())
-    return fail(INPAINT_ERR_ARG, "the corrected gradient is built for the strip kernels only (INPAINT_TV_PATH=tile is set)");
   s.stream = stream;
   const size_t F = field_count(s), P = plane_count(s);
-  const int gF = grid_stride((long long)F), gP = grid_stride((long long)P);
+  const int gF = grid_stride((long long)F);
 
   s.acc_cur = 0;
   s.accb_cur = 0;
   // The strip kernels keep one fp32 record of the accumulators per segment; the records are added into the fp64
   // totals after the last segment, in the reference's order (TV.cu:1730 flushes after every segment: same bits,
   // but the totals are not read and rewritten ten times).
-  const bool seg_mode = strip_path(s);
   SegmentJobs sj;
   {
     float* segs[4] = {s.seg_gc, s.seg_gx, s.seg_gy, s.seg_gb};
@@ -1223,7 +903,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   // is then an inner step) and one launch holds every channel.  That launch starts from zero accumulators without
   // reading them, and every launch after it reads only what its predecessor wrote in full: nothing to clear.
   const int nseg = (int)s.iterations.size();
-  const bool first_two = seg_mode && adjoint_pairs(s) && s.ic <= kGroup && knobs().tv_fuse_first && nseg > 0 &&
+  const bool first_two = adjoint_pairs(s) && s.ic <= kGroup && knobs().tv_fuse_first && nseg > 0 &&
                          2 * ((its - s.iterations[nseg - 1]) / 2) >= 4;
   {
     ZeroList z;
@@ -1232,10 +912,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
       for (float* p : {s.g05[0], s.g05[1], s.gxk[0], s.gxk[1], s.gx_final, s.acc_gb[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)F * 4; }
       for (float* p : {s.acc_gc[0], s.acc_gx[0], s.acc_gy[0]}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 4; }
     }
-    if (!seg_mode) {  // (the strip path writes every total when it adds up the segment records)
-      for (double* p : {s.tot_gc, s.tot_gx, s.tot_gy}) { z.ptr[k] = p; z.bytes[k++] = (long long)P * 8; }
-      z.ptr[k] = s.tot_gb; z.bytes[k++] = (long long)F * 8;
-    }
+    // (the totals need no clearing: every one of them is written when the segment records are added up)
     // one launch: these buffers zeroed, the upstream gradient scrubbed (TV.cu:1609-1623), the guard's statistics cleared
     hipLaunchKernelGGL(backward_prologue_many, dim3(gF, k + 2), dim3(256), 0, stream, z, k, gin, (long long)F, s.guard);
   }
@@ -1385,7 +1062,7 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
     }
     // fp32 segment sums into the fp64 totals (TV.cu:1730); the strip kernel of the segment's first
     // iteration has already done it
-    if (!flushed && seg_mode) {
+    if (!flushed) {
       SegmentJobs st = sj;
       float* accs[4] = {s.acc_gc[s.acc_cur], s.acc_gx[s.acc_cur], s.acc_gy[s.acc_cur], s.acc_gb[s.accb_cur]};
       for (int k = 0; k < 4; k++) {
@@ -1393,16 +1070,11 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
         st.seg[k] = sj.seg[k] + (size_t)outer * sj.n[k];
       }
       hipLaunchKernelGGL(segment_store_many, dim3(gF, 4), dim3(256), 0, stream, st);
-    } else if (!flushed) {
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gc[s.acc_cur], s.tot_gc, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gx[s.acc_cur], s.tot_gx, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gP), dim3(256), 0, stream, s.acc_gy[s.acc_cur], s.tot_gy, (long long)P);
-    hipLaunchKernelGGL(flush_kernel, dim3(gF), dim3(256), 0, stream, s.acc_gb[s.accb_cur], s.tot_gb, (long long)F);
     }
     lastIt = k0;
   }
 
-  if (seg_mode) hipLaunchKernelGGL(combine_segments_many, dim3(gF, 4), dim3(256), 0, stream, sj, nseg);
+  hipLaunchKernelGGL(combine_segments_many, dim3(gF, 4), dim3(256), 0, stream, sj, nseg);
   if (corr && 2 * (its / 2) > 0) {
     // corrected gradient: back-propagate through iteration 0 as well (the reference stops before it); the last
     // step above left g05[0] and the partial g_x[0] in the halves of the ping-pongs it wrote, checkpoint 0 is y_0
@@ -1439,6 +1111,10 @@ int tvinpaint_backward(const float* dx, const float* dy, const float* c, const f
   fin.f32_scale = 4;
   hipLaunchKernelGGL(finalize_many, dim3(gF, 5), dim3(256), 0, stream, fin, s.guard, kGuard, corr ? 1.f : kGlobalGMult);
   INPAINT_HIP(hipGetLastError());
+  if (knobs().stats_every > 0 && s.run % knobs().stats_every == 1 % knobs().stats_every) {  // TV.cu:1766: run % 75 == 1
+    rc = print_guard_report(s.guard, stream, id, false);
+    if (rc) return rc;
+  }
   s.run++;  // TV.cu:1829
   return 0;
 }

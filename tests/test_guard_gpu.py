@@ -11,6 +11,7 @@ import ctypes
 
 import numpy as np
 import pytest
+import torch
 
 pytestmark = pytest.mark.gpu
 
@@ -111,3 +112,33 @@ def test_rescale_and_kill(lib, oracles, layer, dtype):
     for run, av in ((10, mean / 20), (10, mean / 60), (9, mean / 60), (10, mean / 2)):
         acts.append(int(check(lib, oracles[layer], layer, g, run, av, "av=mean/%g" % (mean / av))[4]))
     assert acts == [1, 2, 0, 0]
+
+
+def test_guard_statistics_on_stderr_when_asked(monkeypatch, capfd):
+    """INPAINT_STATS_EVERY=N prints the guard's statistics of every Nth backward pass of an id on stderr, in the
+    reference's wording (TVInpaintFista.cu:1766-1790 does so on every 75th run); nothing is printed otherwise."""
+    from customnetworklayers_amd.cudaTV import tvInpaint_cuda_ext as ext
+    from customnetworklayers_amd.workloads import tv_inputs
+
+    d = tv_inputs(1, 2, 24, 70, seed=2, conf_density=0.3)
+    t = {k: torch.from_numpy(v).to("cuda:0") for k, v in d.items()}
+
+    def fwd_bwd():
+        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 8, 6)
+        ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], 8, 6)
+        torch.cuda.synchronize()
+
+    ext.reset_id(6)
+    fwd_bwd()
+    assert "Output gradient" not in capfd.readouterr().err
+    monkeypatch.setenv("INPAINT_STATS_EVERY", "2")
+    try:
+        ext.reset_id(6)  # (re-reads the environment; run count 0)
+        fwd_bwd()        # run 0: silent
+        assert "Output gradient" not in capfd.readouterr().err
+        fwd_bwd()        # run 1: 1 % 2 == 1
+        err = capfd.readouterr().err
+        assert err.count("Output gradient to") == 5 and "gradI" in err
+    finally:
+        monkeypatch.delenv("INPAINT_STATS_EVERY")
+        ext.reset_id(6)

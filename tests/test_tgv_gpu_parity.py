@@ -117,14 +117,21 @@ def test_more_than_two_channels_run_in_channel_groups(ext, tgv_oracle, n, c, h, 
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 1, 33, 64, 9), (1, 3, 20, 64, 6)])
-def test_per_pixel_kernels_when_forced(ext, tgv_oracle, n, c, h, w, its, monkeypatch):
-    # every channel count normally takes the wave-strip kernels; force the per-pixel kernels written first
-    d = varying_inputs(n, c, h, w, seed=77 + c)
-    ref = run_oracle(tgv_oracle, d, its, 2)
-    compare("default path c=%d" % c, run_gpu(ext, d, its, 2), ref)
+def test_removed_kernel_path_is_refused(ext, monkeypatch):
+    # INPAINT_TGV_PATH=px used to select the one-pixel-per-thread kernels written first; the library no longer contains
+    # them and says so
+    d = varying_inputs(1, 2, 20, 64, seed=3)
+    t = {k: torch.from_numpy(v).to("cuda:0") for k, v in d.items()}
     monkeypatch.setenv("INPAINT_TGV_PATH", "px")
-    compare("per-pixel path c=%d" % c, run_gpu(ext, d, its, 2), ref)
+    try:
+        ext.reset_id(2)  # (re-reads the environment)
+        with pytest.raises(ValueError, match="no longer contains"):
+            ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 6, 2)
+    finally:
+        monkeypatch.delenv("INPAINT_TGV_PATH")
+        ext.reset_id(2)
+    ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 6, 2)
+    ext.reset_id(2)
 
 
 @pytest.mark.parametrize("n,c,h,w,its", [
@@ -593,21 +600,11 @@ def test_corrected_gradient_is_the_gradient_of_the_forward_pass(ext, tgv_oracle)
     assert rel_err(plain[3], true[3]) > 0.5  # the reference's gradient is a different vector
 
 
-def test_corrected_gradient_needs_the_strip_kernels(ext, monkeypatch):
-    d = varying_inputs(1, 3, 12, 20, seed=1)
-    dev = torch.device("cuda:0")
-    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
-    monkeypatch.setenv("INPAINT_TGV_PATH", "px")  # the per-pixel kernels have no corrected form
-    try:
-        ext.reset_id(2)
-        ext.gradient_mode(2, 1)
-        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 4, 2)
-        with pytest.raises(ValueError):
-            ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], 4, 2)
-        with pytest.raises(ValueError):
-            ext.gradient_mode(2, 2)
-    finally:
-        ext.reset_id(2)
+def test_gradient_mode_takes_zero_or_one(ext):
+    with pytest.raises(ValueError):
+        ext.gradient_mode(2, 2)
+    with pytest.raises(ValueError):
+        ext.gradient_mode(2, -1)
 
 
 @pytest.mark.parametrize("env,c", [({"INPAINT_TGV_PAIR_WAVES": "2"}, 1), ({"INPAINT_TGV_FUSE_ADJ": "0"}, 2),

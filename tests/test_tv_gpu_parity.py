@@ -241,14 +241,21 @@ def test_upstream_gradients_of_extreme_magnitude(ext, tv_oracle, scale, bit_equa
     ext.reset_id(2)
 
 
-@pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 33, 64, 9), (1, 5, 20, 64, 6)])
-def test_tile_kernels_when_forced(ext, tv_oracle, n, c, h, w, its, monkeypatch):
-    # every channel count normally takes the wave-strip kernels; force the LDS-tile kernels written first
-    d = tv_inputs(n, c, h, w, seed=77 + c, conf_density=0.3)
-    ref = run_oracle(tv_oracle, d, its, 2)
-    compare("default path c=%d" % c, run_gpu(ext, d, its, 2), ref)
+def test_removed_kernel_path_is_refused(ext, monkeypatch):
+    # INPAINT_TV_PATH=tile used to select the LDS-tile kernels written first; the library no longer contains them and
+    # says so instead of silently running something else
+    d = tv_inputs(1, 2, 20, 64, seed=3, conf_density=0.3)
+    t = {k: torch.from_numpy(v).to("cuda:0") for k, v in d.items()}
     monkeypatch.setenv("INPAINT_TV_PATH", "tile")
-    compare("tile path c=%d" % c, run_gpu(ext, d, its, 2), ref)
+    try:
+        ext.reset_id(2)  # (re-reads the environment)
+        with pytest.raises(ValueError, match="no longer contains"):
+            ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 6, 2)
+    finally:
+        monkeypatch.delenv("INPAINT_TV_PATH")
+        ext.reset_id(2)
+    ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 6, 2)
+    ext.reset_id(2)
 
 
 @pytest.mark.parametrize("n,c,h,w,its", [(2, 2, 70, 256, 20), (1, 3, 45, 130, 10)])
@@ -616,21 +623,11 @@ def test_corrected_gradient_is_the_gradient_of_the_forward_pass(ext, tv_oracle):
     assert rel_err(plain[3], true[3]) > 0.5
 
 
-def test_corrected_gradient_needs_the_strip_kernels(ext, monkeypatch):
-    d = tv_inputs(1, 5, 12, 20, seed=1, conf_density=0.3)
-    dev = torch.device("cuda:0")
-    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
-    monkeypatch.setenv("INPAINT_TV_PATH", "tile")  # the LDS-tile kernels have no corrected form
-    try:
-        ext.reset_id(2)
-        ext.gradient_mode(2, 1)
-        ext.forward(t["dx"], t["dy"], t["dc"], t["db"], t["di"], 4, 2)
-        with pytest.raises(ValueError):
-            ext.backward(t["grad"].clone(), t["dx"], t["dy"], t["dc"], t["db"], 4, 2)
-        with pytest.raises(ValueError):
-            ext.gradient_mode(2, 2)
-    finally:
-        ext.reset_id(2)
+def test_gradient_mode_takes_zero_or_one(ext):
+    with pytest.raises(ValueError):
+        ext.gradient_mode(2, 2)
+    with pytest.raises(ValueError):
+        ext.gradient_mode(2, -1)
 
 
 def test_module_with_the_corrected_gradient(ext, tv_oracle):
