@@ -1765,6 +1765,8 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
       in.gwx1_i = ldg(gwx1i_p, off_o);
       in.gwy0_i = ldg(gwy0i_p, off_o);
       in.gwy1_i = ldg(gwy1i_p, off_o);
+      // (the scheduler must not move the row loads that follow in front of these: see the order of the calls below)
+      __builtin_amdgcn_sched_barrier(0);
     };
     auto absorb = [&](int k, Adj2ARow<C>& o) {
       const int h = g.hs - 2 + k;
@@ -1858,12 +1860,14 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     auto publish = [&](int k) {
       if (k % kP == kP - 1) lds_barrier();
     };
+    // (The accumulators of row k+1 are asked for BEFORE the rows prefetched further ahead: loads return in order, so a
+    // wait for the youngest load of the queue would drain every prefetched row with it.)
     Adj2ARow<C> b0, b1, b2;
     Adj2Late<C> late;
     load_row(0, b0);
     load_row(1, b1);
-    load_row(2, b2);
     load_late(1, late);
+    load_row(2, b2);
     absorb(0, b0);
     absorb(1, b1);
     step(0, b0, b1, late, kNo);
@@ -1871,31 +1875,31 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     publish(0);
     absorb(2, b2);
     step(1, b1, b2, late, kYes);
-    load_row(4, b1);
     load_late(2, late);
+    load_row(4, b1);
     publish(1);
     absorb(3, b0);
     step(2, b2, b0, late, kYes);
-    load_row(5, b2);
     load_late(3, late);
+    load_row(5, b2);
     publish(2);
     for (int k = 3; k <= klast; k += 3) {  // cur / next rotate through (b0,b1) (b1,b2) (b2,b0)
       absorb(k + 1, b1);
       step(k, b0, b1, late, kYes);
-      load_row(k + 3, b0);
       load_late(k + 1, late);
+      load_row(k + 3, b0);
       publish(k);
       if (k + 1 > klast) break;
       absorb(k + 2, b2);
       step(k + 1, b1, b2, late, kYes);
-      load_row(k + 4, b1);
       load_late(k + 2, late);
+      load_row(k + 4, b1);
       publish(k + 1);
       if (k + 2 > klast) break;
       absorb(k + 3, b0);
       step(k + 2, b2, b0, late, kYes);
-      load_row(k + 5, b2);
       load_late(k + 3, late);
+      load_row(k + 5, b2);
       publish(k + 2);
     }
     if (klast % kP != kP - 1) lds_barrier();  // the last rows have not been published yet
