@@ -434,7 +434,7 @@ constexpr int kTW = 64;  // tile width: one pixel column per lane
 constexpr int kMaxWinW = 128;  // widest window
 template <int PX>              // PX pixels per lane (rows PX * wave + i): tile height, window capacity in floats
 struct TileCfg {
-  static constexpr int TH = 4 * PX, ELEMS = 96 * (4 * PX + 16);
+  static constexpr int TH = 4 * PX, ELEMS = (96 * (4 * PX + 16) + 255) / 256 * 256;
 };
 constexpr int kPxForward = 2, kPxSources = 2;
 
@@ -869,7 +869,7 @@ constexpr int kPairs = 12;
 constexpr int kPxGather = 2;
 
 template <int PX>
-__global__ __launch_bounds__(256) void quadfit_gather_tiles(const float* __restrict__ im0, float* __restrict__ g1, QfWorkspace ws,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void quadfit_gather_tiles(const float* __restrict__ im0, float* __restrict__ g1, QfWorkspace ws,
                                                             int N, int d, int H, int W, int tiles_x, int tiles_y) {
   constexpr int kTH = TileCfg<PX>::TH;
   __shared__ float win[2][TileCfg<PX>::ELEMS];
@@ -889,6 +889,13 @@ __global__ __launch_bounds__(256) void quadfit_gather_tiles(const float* __restr
   unsigned off[PX][kPairs];  // packed (y << 16 | x) of the source, then its offset in the window
   float cf[PX][kPairs];
   int minx = INT_MAX, maxx = INT_MIN, miny = INT_MAX, maxy = INT_MIN;
+  // (position whose sources reach a pixel, tap they reach it with), as an offset in the plane; a neighbour outside the
+  // image has no list.  Three reads stand behind every pair -- list length, list, coefficient.  They are issued
+  // unconditionally and in batches (an absent list reads the pixel's own, an unused entry coefficient 0 of the sample):
+  // lengths and lists of all pixels of the lane together, then the coefficients of one pixel at a time -- three round
+  // trips to memory; behind `if (cnt > 0)` / `if (s < cnt)` each read waits for the one before it, some fifty in a row.
+  int cnt[PX][5];
+  int4 sl[PX][5];
 #pragma unroll
   for (int i = 0; i < PX; i++) {
     const int y = ty * kTH + wave * PX + i;
@@ -900,28 +907,47 @@ __global__ __launch_bounds__(256) void quadfit_gather_tiles(const float* __restr
       off[i][j] = 0u;
       cf[i][j] = 0.f;
     }
-    if (!valid[i]) continue;
-    // (position whose sources reach this pixel, tap they reach it with); -1: outside the image
-    long long ctr[5];
-    ctr[0] = base + pix[i];
-    ctr[1] = x > 0 ? base + pix[i] - 1 : -1;      // right tap of the left neighbour
-    ctr[2] = x < W - 1 ? base + pix[i] + 1 : -1;  // left tap of the right neighbour
-    ctr[3] = y > 0 ? base + pix[i] - W : -1;      // lower tap of the upper neighbour
-    ctr[4] = y < H - 1 ? base + pix[i] + W : -1;  // upper tap of the lower neighbour
+    const bool has[5] = {valid[i], valid[i] && x > 0, valid[i] && x < W - 1, valid[i] && y > 0, valid[i] && y < H - 1};
+    const int step[5] = {0, -1, 1, -W, W};
 #pragma unroll
     for (int k = 0; k < 5; k++) {
-      const int cnt = ctr[k] >= 0 ? min(ws.count[ctr[k]], kSlots) : 0;
-      int4 sl = make_int4(0, 0, 0, 0);
-      if (cnt > 0) sl = *reinterpret_cast<const int4*>(ws.slots + ctr[k] * kSlots);
-      const int sv[4] = {sl.x, sl.y, sl.z, sl.w};
+      const long long ctr = base + (long long)pix[i] + (has[k] ? step[k] : 0);
+      cnt[i][k] = ws.count[ctr];
+      sl[i][k] = *reinterpret_cast<const int4*>(ws.slots + ctr * kSlots);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PX; i++) {
+    const int y = ty * kTH + wave * PX + i;
+    const bool has[5] = {valid[i], valid[i] && x > 0, valid[i] && x < W - 1, valid[i] && y > 0, valid[i] && y < H - 1};
+    float cv[5][kSlots];
+    unsigned spv[5][kSlots];
+#pragma unroll
+    for (int k = 0; k < 5; k++) {
+      cnt[i][k] = has[k] ? min(cnt[i][k], kSlots) : 0;
+      const int sv[4] = {sl[i][k].x, sl[i][k].y, sl[i][k].z, sl[i][k].w};
 #pragma unroll
       for (int s = 0; s < kSlots; s++) {
-        if (s < cnt) {
-          const unsigned sp = (unsigned)sv[s];  // source pixel, offset in its plane (below 2^24: the float quotient is off by one at most)
+        spv[k][s] = s < cnt[i][k] ? (unsigned)sv[s] : 0u;  // source pixel, offset in its plane
+        cv[k][s] = ws.coef[(long long)k * P + base + spv[k][s]];
+      }
+    }
+    // (the values are pinned here, all of them: left alone, the optimizer moves each read back behind the branch that
+    // uses it)
+#pragma unroll
+    for (int k = 0; k < 5; k++)
+#pragma unroll
+      for (int s = 0; s < kSlots; s++) asm volatile("" : "+v"(cv[k][s]));
+#pragma unroll
+    for (int k = 0; k < 5; k++) {
+#pragma unroll
+      for (int s = 0; s < kSlots; s++) {
+        if (s < cnt[i][k]) {
+          const unsigned sp = spv[k][s];  // (below 2^24: the float quotient is off by one at most)
           int sy = (int)((float)sp * inv_w), sx = (int)sp - sy * W;
           if (sx < 0) { sy--; sx += W; }
           if (sx >= W) { sy++; sx -= W; }
-          const float c = ws.coef[(long long)k * P + base + sp];
+          const float c = cv[k][s];
 #pragma unroll
           for (int j = 0; j < kPairs; j++)
             if (np[i] == j) {
@@ -962,12 +988,17 @@ __global__ __launch_bounds__(256) void quadfit_gather_tiles(const float* __restr
   }
   auto nothing = [](int) { return 0; };
   window_pass<PX>(a, d, HW, W, box, win, nothing, [&](int cc, const float* buf, const float* plane, int, bool live) {
+    // all window reads of a pixel are issued before the first product: a read inside the branch that skips an unused pair
+    // is waited for on the spot, one LDS round trip after the other (an unused pair reads element 0, a broadcast)
 #pragma unroll
     for (int i = 0; i < PX; i++) {
+      float v[kPairs];
+#pragma unroll
+      for (int j = 0; j < kPairs; j++) v[j] = buf[off[i][j]];
       float acc = 0.f;
 #pragma unroll
       for (int j = 0; j < kPairs; j++)
-        if (need & (1u << j)) acc = __builtin_fmaf(buf[off[i][j]], cf[i][j], acc);
+        if (need & (1u << j)) acc = __builtin_fmaf(v[j], cf[i][j], acc);
       if (live && valid[i] && !slow[i]) G1[(size_t)cc * HW + pix[i]] = acc;
     }
   });
