@@ -569,6 +569,60 @@ __device__ __forceinline__ void window_pass(const float* __restrict__ q, int d, 
   }
 }
 
+// The same stream with the windows loaded from memory straight into LDS (global_load_lds: no staging registers) through a
+// ring of kDmaStages buffers: while channel c is consumed, channels c+1 and c+2 are on their way and channel c+3 is asked
+// for as soon as c has been consumed -- three channels in flight per wavefront instead of two, one barrier per channel.
+// Loads return in order, so "at most two channels' worth of loads outstanding" means channel c has arrived (a wavefront's
+// stores in between make the wait a little longer, never shorter); the barrier then makes every wavefront's part of the
+// window visible.  A buffer is overwritten two barriers after its last reader has passed the barrier that follows its
+// consumption.  No `pre` values: for consumers that need the window only.
+// The four buffers are four separate __shared__ arrays, not one: the compiler waits, before a read of LDS, for every load
+// into LDS that may alias it, and it can tell loads into different variables apart, not into parts of one.
+template <int PX, typename Consume>
+__device__ __forceinline__ void window_pass_dma(const float* __restrict__ q, int d, size_t HW, int W, const Box& box,
+                                                float* w0, float* w1, float* w2, float* w3, Consume consume) {
+  constexpr int kElems = TileCfg<PX>::ELEMS, kPer = kElems / 256;
+  static_assert(kElems % 256 == 0, "every thread loads the same number of window elements");
+  typedef const __attribute__((address_space(1))) void* GlobalPtr;
+  typedef __attribute__((address_space(3))) void* LdsPtr;
+  const int count = box.w * box.h;
+  unsigned goff[kPer];
+  const float inv_w = 1.0f / (float)max(box.w, 1);
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    const int e = threadIdx.x + 256 * k;
+    const int r = (int)(((float)e + 0.5f) * inv_w);
+    goff[k] = e < count ? (unsigned)(r * W + (e - r * box.w)) : 0u;
+  }
+  const float* corner = q + (size_t)box.y0 * W + box.x0;
+  const int wave_first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x & ~63u));  // lane l of the wavefront writes element wave_first + l
+  auto fetch = [&](int c, float* buf) {
+    const float* src = corner + (size_t)c * HW;
+#pragma unroll
+    for (int k = 0; k < kPer; k++)
+      __builtin_amdgcn_global_load_lds((GlobalPtr)(src + goff[k]), (LdsPtr)(buf + 256 * k + wave_first), 4, 0, 0);
+  };
+  const int last = d - 1;
+  auto phase = [&](int c, float* buf, float* refill) {
+    // channel c's loads have landed when at most the two younger channels' loads are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * kPer) : "memory");
+    const int cc = min(c, last);
+    consume(cc, buf, q + (size_t)cc * HW, 0, c < d);
+    fetch(min(c + 3, last), refill);
+  };
+  fetch(0, w0);
+  fetch(min(1, last), w1);
+  fetch(min(2, last), w2);
+  for (int c0 = 0; c0 < d; c0 += 4) {
+    phase(c0, w0, w3);
+    phase(c0 + 1, w1, w0);
+    phase(c0 + 2, w2, w1);
+    phase(c0 + 3, w3, w2);
+  }
+  // (the loads still in flight at the end target LDS: they must have landed before the workgroup's LDS is handed on)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // the five taps of every inside pixel of the lane, from the window or (far pixels) from the plane
 template <int PX, typename Body>
 __device__ __forceinline__ void each_pixel_taps(const TilePx (&px)[PX], const float* buf, const float* plane, Body body) {
@@ -868,11 +922,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 constexpr int kPairs = 12;
 constexpr int kPxGather = 2;
 
+// Twelve reads of one LDS buffer at per-lane element offsets, issued together and waited for once, as one block the
+// compiler does not look into: before an LDS read that it sees, it waits for the loads into LDS that may alias it, and
+// with four buffers in a ring it takes that to be all of them -- the whole prefetch queue.  The caller has waited for the
+// buffer's own loads (window_pass_dma).
+static_assert(kPairs == 12, "lds_gather12 reads twelve elements");
+__device__ __forceinline__ void lds_gather12(const float* buf, const unsigned (&off)[kPairs], float (&v)[kPairs]) {
+  const unsigned b = (unsigned)(size_t)(const __attribute__((address_space(3))) float*)buf;
+  unsigned a[kPairs];
+#pragma unroll
+  for (int j = 0; j < kPairs; j++) a[j] = b + 4u * off[j];
+  asm volatile(
+      "ds_read_b32 %0, %12\n\tds_read_b32 %1, %13\n\tds_read_b32 %2, %14\n\tds_read_b32 %3, %15\n\t"
+      "ds_read_b32 %4, %16\n\tds_read_b32 %5, %17\n\tds_read_b32 %6, %18\n\tds_read_b32 %7, %19\n\t"
+      "ds_read_b32 %8, %20\n\tds_read_b32 %9, %21\n\tds_read_b32 %10, %22\n\tds_read_b32 %11, %23\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7]), "=&v"(v[8]),
+        "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11])
+      : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]), "v"(a[8]), "v"(a[9]), "v"(a[10]),
+        "v"(a[11])
+      : "memory");
+}
+
 template <int PX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void quadfit_gather_tiles(const float* __restrict__ im0, float* __restrict__ g1, QfWorkspace ws,
                                                             int N, int d, int H, int W, int tiles_x, int tiles_y) {
   constexpr int kTH = TileCfg<PX>::TH;
-  __shared__ float win[2][TileCfg<PX>::ELEMS];
+  __shared__ float win0[TileCfg<PX>::ELEMS], win1[TileCfg<PX>::ELEMS], win2[TileCfg<PX>::ELEMS], win3[TileCfg<PX>::ELEMS];
   __shared__ int red[16];
   int n, tx, ty;
   if (!tile_of_block(N, tiles_x, tiles_y, n, tx, ty)) return;
@@ -986,15 +1062,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       if (__ballot(!slow[i] && j < np[i]) != 0) need |= 1u << j;  // pairs nobody in the wavefront has are skipped by a uniform branch
     }
   }
-  auto nothing = [](int) { return 0; };
-  window_pass<PX>(a, d, HW, W, box, win, nothing, [&](int cc, const float* buf, const float* plane, int, bool live) {
+  window_pass_dma<PX>(a, d, HW, W, box, win0, win1, win2, win3, [&](int cc, const float* buf, const float* plane, int, bool live) {
     // all window reads of a pixel are issued before the first product: a read inside the branch that skips an unused pair
     // is waited for on the spot, one LDS round trip after the other (an unused pair reads element 0, a broadcast)
 #pragma unroll
     for (int i = 0; i < PX; i++) {
       float v[kPairs];
-#pragma unroll
-      for (int j = 0; j < kPairs; j++) v[j] = buf[off[i][j]];
+      lds_gather12(buf, off[i], v);
       float acc = 0.f;
 #pragma unroll
       for (int j = 0; j < kPairs; j++)

@@ -72,6 +72,9 @@ def check_quadfit(qf, o, d, name):
     (1, 1, 1, 1, 2),        # a single pixel
     (1, 3, 1, 200, 2),      # a single row
     (1, 3, 150, 1, 2),      # a single column
+    (1, 1, 12, 70, 2),      # fewer channels than the backward gather's ring of windows holds
+    (2, 2, 12, 70, 2),
+    (1, 6, 20, 66, 2),      # a channel count that ends in the middle of the ring
 ])
 def test_quadfit_random_inputs_match_oracle(qf, flowaux_oracle, n, c, h, w, fc):
     d = random_quadfit(n, c, h, w, seed=n * 100 + c + h + w, fc=fc)
