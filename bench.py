@@ -561,6 +561,18 @@ def copy_ceiling():
     return round(g.value, 1) if rc == 0 else None
 
 
+def stream_ceiling(planes_read=2, planes_written=1):
+    """What a streaming kernel that reads two bytes for each one it writes (the strip kernels' mix) reaches on this GPU."""
+    import torch
+
+    from customnetworklayers_amd._lib import lib
+
+    g = ctypes.c_double(0)
+    rc = lib.inpaint_stream_bandwidth(1 << 29, planes_read, planes_written, 10, ctypes.byref(g),
+                                      ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return {"planes_read": planes_read, "planes_written": planes_written, "GBps": round(g.value, 1)} if rc == 0 else None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -595,6 +607,7 @@ def main():
         return bench_flowaux(args, cfg, d)
     out, cfg = bench_layer(args.config, args.steps, args.warmup, corrected=args.corrected_gradient, keep=args.keep)
     out["roofline"]["hbm_copy_ceiling_GBps"] = copy_ceiling()
+    out["roofline"]["hbm_stream_ceiling"] = stream_ceiling()
     if args.config == 1 and not args.no_other_configs and not args.corrected_gradient and args.keep is None:
         # after the headline's timed region: short legs of the other workloads, so that one run witnesses them all
         other = {}

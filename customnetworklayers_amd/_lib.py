@@ -43,6 +43,7 @@ def _load():
     lib.inpaint_selftest_division_pairs.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_ulonglong)]
     lib.inpaint_reload_env.restype = None
     lib.inpaint_copy_bandwidth.argtypes = [ctypes.c_longlong, _int, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+    lib.inpaint_stream_bandwidth.argtypes = [ctypes.c_longlong, _int, _int, _int, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     lib.tvinpaint_last_error.restype = ctypes.c_char_p
     lib.tgvinpaint_forward.argtypes = [_f32p] * 6 + [_int] * 6 + [ctypes.c_void_p]
     lib.tgvinpaint_backward.argtypes = [_f32p] * 10 + [_int] * 6 + [ctypes.c_void_p]

@@ -102,6 +102,25 @@ __global__ __launch_bounds__(256) void copy_kernel(const copy_v4* __restrict__ s
     __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// NR planes read and summed, NW planes written: one 16-byte element per thread and plane (the streaming mix of a kernel
+// that reads more than it writes; a plain copy is NR = NW = 1)
+template <int NR, int NW>
+__global__ __launch_bounds__(256) void stream_kernel(const copy_v4* __restrict__ src, copy_v4* __restrict__ dst, long long n16,
+                                                     copy_v4* __restrict__ sink) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n16) return;
+  copy_v4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < NR; r++) a += src[(long long)r * n16 + i];
+#pragma unroll
+  for (int w = 0; w < NW; w++) dst[(long long)w * n16 + i] = a;
+  if (NW == 0 && a.x == 123.456f) *sink = a;  // (never true for the fill value: keeps the reads alive)
+}
+template <int NR, int NW>
+static void launch_stream(int grid, hipStream_t stream, const copy_v4* src, copy_v4* dst, long long n16, copy_v4* sink) {
+  hipLaunchKernelGGL((stream_kernel<NR, NW>), dim3(grid), dim3(256), 0, stream, src, dst, n16, sink);
+}
+
 // Every quotient of ordinary operands is, up to a power of two, n / d with n, d in [1, 2): all 2^23 x 2^23 pairs of
 // mantissas, the library's division (reciprocal refined once, quotient corrected once) against the compiler's IEEE
 // expansion.  One thread per denominator; blockIdx.y selects a sixteenth of the numerators.
@@ -196,6 +215,50 @@ extern "C" int inpaint_copy_bandwidth(long long bytes, int repeats, double* gbps
   INPAINT_HIP(hipEventElapsedTime(&ms, e0, e1));
   INPAINT_HIP(hipGetLastError());
   *gbps_host = ms > 0 ? 2.0 * (double)n16 * 16 * repeats / (ms * 1e-3) / 1e9 : 0.0;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  (void)hipFree(src);
+  (void)hipFree(dst);
+  return 0;
+}
+
+// Diagnostic: the rate of a streaming kernel that reads `planes_read` planes and writes `planes_written` planes of
+// `bytes_per_plane` each (16 bytes per thread and plane), bytes read + written per second in GB/s.  The memory system
+// serves mixes of reads and writes more slowly than reads alone, so this, not the copy, is the practical ceiling of a
+// kernel with that mix.  planes_read 1..4, planes_written 0..2.
+extern "C" int inpaint_stream_bandwidth(long long bytes_per_plane, int planes_read, int planes_written, int repeats,
+                                        double* gbps_host, void* stream_) {
+  if (bytes_per_plane < 16 || repeats < 1 || !gbps_host || planes_read < 1 || planes_read > 4 || planes_written < 0 ||
+      planes_written > 2)
+    return inpaint::fail(INPAINT_ERR_ARG, "bad arguments (1..4 planes read, 0..2 written)");
+  hipStream_t stream = (hipStream_t)stream_;
+  const long long n16 = bytes_per_plane / 16;
+  copy_v4 *src = nullptr, *dst = nullptr;
+  INPAINT_HIP(hipMalloc((void**)&src, (size_t)n16 * 16 * planes_read));
+  if (hipMalloc((void**)&dst, (size_t)n16 * 16 * std::max(planes_written, 1)) != hipSuccess) {
+    (void)hipFree(src);
+    return inpaint::fail(INPAINT_ERR_HIP, "hipMalloc of the stream target failed");
+  }
+  INPAINT_HIP(hipMemsetAsync(src, 0x3c, (size_t)n16 * 16 * planes_read, stream));
+  hipEvent_t e0, e1;
+  INPAINT_HIP(hipEventCreate(&e0));
+  INPAINT_HIP(hipEventCreate(&e1));
+  const int grid = (int)std::min<long long>((n16 + 255) / 256, (1LL << 31) - 1);
+  typedef void (*Launch)(int, hipStream_t, const copy_v4*, copy_v4*, long long, copy_v4*);
+  static const Launch table[4][3] = {{launch_stream<1, 0>, launch_stream<1, 1>, launch_stream<1, 2>},
+                                     {launch_stream<2, 0>, launch_stream<2, 1>, launch_stream<2, 2>},
+                                     {launch_stream<3, 0>, launch_stream<3, 1>, launch_stream<3, 2>},
+                                     {launch_stream<4, 0>, launch_stream<4, 1>, launch_stream<4, 2>}};
+  const Launch go = table[planes_read - 1][planes_written];
+  go(grid, stream, src, dst, n16, dst);
+  INPAINT_HIP(hipEventRecord(e0, stream));
+  for (int r = 0; r < repeats; r++) go(grid, stream, src, dst, n16, dst);
+  INPAINT_HIP(hipEventRecord(e1, stream));
+  INPAINT_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  INPAINT_HIP(hipEventElapsedTime(&ms, e0, e1));
+  INPAINT_HIP(hipGetLastError());
+  *gbps_host = ms > 0 ? (double)(planes_read + planes_written) * (double)n16 * 16 * repeats / (ms * 1e-3) / 1e9 : 0.0;
   (void)hipEventDestroy(e0);
   (void)hipEventDestroy(e1);
   (void)hipFree(src);

@@ -59,6 +59,13 @@ int inpaint_selftest_rsqrt(unsigned long long* mismatches4_host, unsigned int pa
  * copies `repeats` times after a warm-up launch, timed with HIP events on `stream`; waits for the result. */
 int inpaint_copy_bandwidth(long long bytes, int repeats, double* gbps_host, void* stream);
 
+/* The same for a streaming kernel that reads `planes_read` (1..4) planes and writes `planes_written` (0..2) planes of
+ * `bytes_per_plane` each: the memory system serves a mix of reads and writes more slowly than either alone, so this is the
+ * practical ceiling to hold a kernel with that mix against (the strip kernels read about two bytes for each one they
+ * write).  Bytes read + written per second, GB/s. */
+int inpaint_stream_bandwidth(long long bytes_per_plane, int planes_read, int planes_written, int repeats, double* gbps_host,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,3 +42,25 @@ def test_division_is_correctly_rounded_on_every_pair_of_mantissas(first):
     print("slices %d..%d: %d mismatches in %.2e pairs (uncorrected product: %d)" % (first, first + 7, out[0], pairs, out[1]), flush=True)
     assert out[0] == 0
     assert out[1] > pairs // 10  # the comparison does see last-bit errors
+
+
+def test_stream_bandwidth_diagnostics_report_plausible_rates():
+    # the copy and the mixed read / write streams that bench.py quotes beside the published HBM peak: well above what a
+    # mistake in the byte count or the timing would leave (1 TB/s), below the peak; bad plane counts are refused
+    import torch
+
+    from customnetworklayers_amd._lib import last_error, lib
+
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = ctypes.c_double(0)
+    assert lib.inpaint_copy_bandwidth(1 << 30, 5, ctypes.byref(g), st) == 0, last_error()
+    copy = g.value
+    rates = {}
+    for nr, nw in ((1, 0), (2, 1), (4, 2)):
+        assert lib.inpaint_stream_bandwidth(1 << 29, nr, nw, 5, ctypes.byref(g), st) == 0, last_error()  # far beyond the last-level cache
+        rates[(nr, nw)] = g.value
+    print("copy %.0f GB/s, streams %s" % (copy, {k: round(v) for k, v in rates.items()}), flush=True)
+    for v in [copy] + list(rates.values()):
+        assert 1000.0 < v < 8000.0  # (the published peak)
+    assert lib.inpaint_stream_bandwidth(1 << 27, 5, 1, 5, ctypes.byref(g), st) != 0
+    assert lib.inpaint_stream_bandwidth(1 << 27, 1, 3, 5, ctypes.byref(g), st) != 0
