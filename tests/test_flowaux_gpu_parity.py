@@ -81,7 +81,8 @@ def test_quadfit_random_inputs_match_oracle(qf, flowaux_oracle, n, c, h, w, fc):
     check_quadfit(qf, flowaux_oracle, d, "random %dx%dx%dx%d fc=%d" % (n, c, h, w, fc))
 
 
-@pytest.mark.parametrize("n,c,h,w", [(2, 8, 96, 160), (1, 16, 50, 333), (1, 32, 70, 200)])
+@pytest.mark.parametrize("n,c,h,w", [(2, 8, 96, 160), (1, 16, 50, 333), (1, 32, 70, 200),
+                                     (1, 32, 384, 1248)])  # one sample of the benchmark's shape: every block of the chip busy at once
 def test_quadfit_warped_features_match_oracle(qf, flowaux_oracle, n, c, h, w):
     d = workloads.quadfit_inputs(n, c, h, w, seed=3)
     out = check_quadfit(qf, flowaux_oracle, d, "warped %dx%dx%dx%d" % (n, c, h, w))
