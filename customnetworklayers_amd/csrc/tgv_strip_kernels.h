@@ -34,6 +34,15 @@ using tvstrip::from_right_lane;
 using tvstrip::ldg;
 using tvstrip::stg;
 using tvstrip::lds_barrier;
+
+// A copy of a store offset made INSIDE the block that stores.  Instruction selection folds "scalar base + 32-bit vector
+// offset" into a store only if the offset's widening to 64 bits sits in the store's own basic block; the offset of a row is
+// computed before the `if (store_lane)` blocks, its widening lands there too, and every store of a block then computes a
+// 64-bit vector address of its own (19 per row in step B of the pair kernel).  The empty asm pins the copy in the block.
+__device__ __forceinline__ unsigned offset_here(unsigned off) {
+  asm volatile("" : "+v"(off));
+  return off;
+}
 using tvstrip::strip_geometry;
 using tvstrip::strip_geometry_block;
 using tvstrip::StripGeom;
@@ -1322,7 +1331,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
     const int h = g.hs - 2 + k;  // A's row; B's row is h - 1
     const bool in_img = g.col_ok && h >= 0 && h < H;
     const bool dmaskA = h >= 0 && h < H - 1, dmaskB = h - 1 >= 0 && h - 1 < H - 1;
-    const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+    const unsigned roffB_ = (unsigned)max(h - 1, 0) * W4 + wc;
     float nG[3][C], ngxm[3][C], ngb[C];
     float gcv = late.gc_i;
     Acc accA{late.gwx0_i, late.gwx1_i, late.gwy0_i, late.gwy1_i};
@@ -1357,6 +1366,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
           gcB += o.gc_add;
           const float gbv = pgb[ch] + o.gb_add;
           if (store_lane) {
+            const unsigned roffB = offset_here(roffB_);
             if (FINAL) {
               stg(gxf_p[0][ch], roffB, o.df);
               stg(gxf_p[1][ch], roffB, o.d1);
@@ -1378,6 +1388,7 @@ __global__ __launch_bounds__(256) void tgv_adjoint_strip2(
         }
       }
       if (do_b.value && store_lane) {
+        const unsigned roffB = offset_here(roffB_);
         if (BEND) {
           const size_t e1 = poff + (roffB >> 2), e2 = 2 * poff + (roffB >> 2);
           seg_gc[e1] = gcB;
@@ -1967,7 +1978,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
     auto step = [&](int k, const Adj2BRow<C>& cur, auto tri_b, auto do_b) {
       const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
       const bool dmaskB = h - 1 >= 0 && h - 1 < H - 1;
-      const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+      const unsigned roffB_ = (unsigned)max(h - 1, 0) * W4 + wc;
       float (*slot)[64] = hand[k % (2 * kP)];
       float nG[3][C], ngxm[3][C], ngb[C];
 #pragma unroll
@@ -1994,6 +2005,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
             gcB += o.gc_add;
             const float gbv = pgb[ch] + o.gb_add;
             if (store_lane) {
+              const unsigned roffB = offset_here(roffB_);
               if (FINAL) {
                 stg(gxf_p[0][ch], roffB, o.df);
                 stg(gxf_p[1][ch], roffB, o.d1);
@@ -2015,6 +2027,7 @@ __global__ __launch_bounds__(128) void tgv_adjoint_strip2w(
           }
         }
         if (do_b.value && store_lane) {
+          const unsigned roffB = offset_here(roffB_);
           if (BEND) {
             const size_t e1 = poff + (roffB >> 2), e2 = 2 * poff + (roffB >> 2);
             seg_gc[e1] = gcB;
@@ -2632,7 +2645,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     auto step = [&](int k, const Adj2BRow<C>& cur, auto tri_b, auto do_b) {
       const int h = g.hs - 2 + k;  // the row step A handed over; B's row is h - 1
       const bool dmaskB = h - 1 >= 0 && h - 1 < H - 1;
-      const unsigned roffB = (unsigned)max(h - 1, 0) * W4 + wc;
+      const unsigned roffB_ = (unsigned)max(h - 1, 0) * W4 + wc;
       const float (*slot)[64] = handA[G][k % kSlots];
       float (*tf)[64] = termF[k % kSlots];
       double (*td)[64] = termD[k % kSlots];
@@ -2687,6 +2700,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             const float gbv = pgb[ch] + o.gb_add;
             if (store_lane) {
+              const unsigned roffB = offset_here(roffB_);
               if (FINAL) {
                 stg(gxf_p[0][ch], roffB, o.df);
                 stg(gxf_p[1][ch], roffB, o.d1);
@@ -2708,6 +2722,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           }
         }
         if (G == 1 && do_b.value && store_lane) {
+          const unsigned roffB = offset_here(roffB_);
           if (BEND) {
             const size_t e1 = poff + (roffB >> 2), e2 = 2 * poff + (roffB >> 2);
             seg_gc[e1] = gcB;
