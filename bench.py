@@ -608,6 +608,9 @@ def main():
     out, cfg = bench_layer(args.config, args.steps, args.warmup, corrected=args.corrected_gradient, keep=args.keep)
     out["roofline"]["hbm_copy_ceiling_GBps"] = copy_ceiling()
     out["roofline"]["hbm_stream_ceiling"] = stream_ceiling()
+    if out["roofline"]["hbm_stream_ceiling"] and out["roofline"].get("achieved"):
+        # the physical rate of the dominant kernel against what a plain stream with its mix of reads and writes reaches
+        out["roofline"]["frac_of_stream_ceiling"] = round(out["roofline"]["achieved"] / out["roofline"]["hbm_stream_ceiling"]["GBps"], 4)
     if args.config == 1 and not args.no_other_configs and not args.corrected_gradient and args.keep is None:
         # after the headline's timed region: short legs of the other workloads, so that one run witnesses them all
         other = {}
