@@ -33,6 +33,7 @@ using tvstrip::from_left_lane;
 using tvstrip::from_right_lane;
 using tvstrip::ldg;
 using tvstrip::stg;
+using tvstrip::stg_nt;
 using tvstrip::lds_barrier;
 
 // A copy of a store offset made INSIDE the block that stores.  Instruction selection folds "scalar base + 32-bit vector
@@ -503,10 +504,10 @@ __global__ __launch_bounds__(256) void tgv_forward_strip2(
           const Upd u = update(pyB[0][ch], pyB[1][ch], pyB[2][ch], t, aFa, aG1y, aG2y, pc, rc1B, pbb[ch], pxB[0][ch],
                                pxB[1][ch], pxB[2][ch], tB);
           if (store_lane) {
-            if (store_y) {
-              stg(yo_p[0][ch], roffB, u.yn);
-              stg(yo_p[1][ch], roffB, u.y1o);
-              stg(yo_p[2][ch], roffB, u.y2o);
+            if (store_y) {  // (half of a checkpoint: read once, by the backward pass -- it need not stay in the caches)
+              stg_nt(yo_p[0][ch], roffB, u.yn);
+              stg_nt(yo_p[1][ch], roffB, u.y1o);
+              stg_nt(yo_p[2][ch], roffB, u.y2o);
             }
             if (store_x) {
               stg(xo_p[0][ch], roffB, u.x_loc);
