@@ -761,7 +761,7 @@ __global__ __launch_bounds__(256) void quadfit_tiles(const float* __restrict__ i
         g = 0.5 * (t[0] * k[i].k00 + t[1] * k[i].k0p + t[2] * k[i].k0m + t[3] * k[i].kp0 + t[4] * k[i].km0);
       else  // QF.cu:295
         g = t[0] * k[i].dFds;
-      if (live) G0[(size_t)cc * HW + px[i].p] = g;
+      if (live) __builtin_nontemporal_store(g, &G0[(size_t)cc * HW + px[i].p]);
     });
   });
 }
@@ -911,7 +911,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         g = 0.5 * (tap[c][0] * kf.k00 + tap[c][1] * kf.k0p + tap[c][2] * kf.k0m + tap[c][3] * kf.kp0 + tap[c][4] * kf.km0);
       else  // QF.cu:295
         g = tap[c][0] * kf.dFds;
-      G0[(size_t)c * HW + px.p] = g;
+      __builtin_nontemporal_store(g, &G0[(size_t)c * HW + px.p]);  // (the caller reads it, later: kept out of the caches, it leaves them to the windows)
     }
   }
 }
@@ -1073,7 +1073,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
       for (int j = 0; j < kPairs; j++)
         if (need & (1u << j)) acc = __builtin_fmaf(v[j], cf[i][j], acc);
-      if (live && valid[i] && !slow[i]) G1[(size_t)cc * HW + pix[i]] = acc;
+      if (live && valid[i] && !slow[i]) __builtin_nontemporal_store(acc, &G1[(size_t)cc * HW + pix[i]]);
     }
   });
 #pragma unroll
@@ -1449,7 +1449,7 @@ __global__ __launch_bounds__(64) void median_stream_kernel(const float* __restri
       vec4* dst = reinterpret_cast<vec4*>(res) + t * per;
 #pragma unroll
       for (int u = 0; u < NV; u++)
-        if (lane + 64 * u < per) dst[lane + 64 * u] = tile4[lane + 64 * u];
+        if (lane + 64 * u < per) dst[lane + 64 * u] = tile4[lane + 64 * u];  // (plain stores: the non-temporal hint costs this pass 7%)
     }
     lds_only_barrier();  // the next tile overwrites the rows
   }
